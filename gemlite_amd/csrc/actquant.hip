@@ -1,0 +1,307 @@
+// Fused dynamic activation quantisation.
+//
+// per-token (reference: gemlite/quant_utils.py:467-539):
+//   s = max(amax(|row|) / qmax, 1e-6); y = clamp(row / s, qmin, qmax);
+//   int8 rounds with floor(y + 0.5) (reference: gemlite/quant_utils.py:289-296),
+//   fp8 is the round-to-nearest-even e4m3fn cast of the clamped value.
+// MXFP4 (reference: gemlite/quant_utils.py:2005-2135, :697-705):
+//   per 32 values: e = clamp(exp(amax/6) + (mantissa != 0), 97, 254), s = 2^(e-127),
+//   code = #{thresholds < |x/s|} over {.25,.75,1.25,1.75,2.5,3.5,5} (strict, so
+//   ties round toward zero), +8 when x/s < 0; two codes per byte, even k low.
+//
+// Both kernels are HBM-bound: one read of x, one write of the codes.  A wave
+// owns a row (per-token) or a run of 32-value groups (MXFP4); every lane moves
+// 16 bytes per load.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace gla {
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// Load 8 consecutive elements starting at element index k (k % 8 == 0) as floats.
+template <int XDT>
+__device__ __forceinline__ void load8(const void* row, int k, float (&v)[8]) {
+    if constexpr (XDT == GLA_DT_FP32) {
+        const float4 a = ((const float4*)((const float*)row + k))[0];
+        const float4 b = ((const float4*)((const float*)row + k))[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 raw = *(const uint4*)((const uint16_t*)row + k);
+        const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (XDT == GLA_DT_FP16) {
+                v[2 * i] = half_bits_to_float((uint16_t)(r[i] & 0xffffu));
+                v[2 * i + 1] = half_bits_to_float((uint16_t)(r[i] >> 16));
+            } else {
+                v[2 * i] = bf16_bits_to_float((uint16_t)(r[i] & 0xffffu));
+                v[2 * i + 1] = bf16_bits_to_float((uint16_t)(r[i] >> 16));
+            }
+        }
+    }
+}
+
+// float -> OCP e4m3fn byte, round to nearest even, input already clamped to +-448
+__device__ __forceinline__ uint32_t f32_to_fp8_pair(float a, float b) {
+    // v_cvt_pk_fp8_f32 packs two conversions into the low 16 bits
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+}
+
+// Raw 8-element chunk as loaded from memory (16 bytes for 16-bit types, 32 for fp32).
+template <int XDT>
+struct Raw8 {
+    uint4 a;
+};
+template <>
+struct Raw8<GLA_DT_FP32> {
+    uint4 a, b;
+};
+
+template <int XDT>
+__device__ __forceinline__ Raw8<XDT> load_raw8(const void* row, int k) {
+    Raw8<XDT> r;
+    if constexpr (XDT == GLA_DT_FP32) {
+        r.a = ((const uint4*)((const float*)row + k))[0];
+        r.b = ((const uint4*)((const float*)row + k))[1];
+    } else {
+        r.a = *(const uint4*)((const uint16_t*)row + k);
+    }
+    return r;
+}
+
+template <int XDT>
+__device__ __forceinline__ void decode_raw8(const Raw8<XDT>& r, float (&v)[8]) {
+    if constexpr (XDT == GLA_DT_FP32) {
+        const uint32_t w[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __builtin_bit_cast(float, w[i]);
+    } else {
+        const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (XDT == GLA_DT_FP16) {
+                v[2 * i] = half_bits_to_float((uint16_t)(w[i] & 0xffffu));
+                v[2 * i + 1] = half_bits_to_float((uint16_t)(w[i] >> 16));
+            } else {
+                v[2 * i] = bf16_bits_to_float((uint16_t)(w[i] & 0xffffu));
+                v[2 * i + 1] = bf16_bits_to_float((uint16_t)(w[i] >> 16));
+            }
+        }
+    }
+}
+
+template <bool TO_INT8>
+__device__ __forceinline__ uint2 quantise8(float (&v)[8], float s) {
+    const float qmax = TO_INT8 ? 127.0f : 448.0f;
+    const float qmin = TO_INT8 ? -128.0f : -448.0f;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = fminf(fmaxf(v[j] / s, qmin), qmax);
+    if constexpr (TO_INT8) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            lo |= ((uint32_t)(int)floorf(v[j] + 0.5f) & 0xffu) << (8 * j);
+            hi |= ((uint32_t)(int)floorf(v[4 + j] + 0.5f) & 0xffu) << (8 * j);
+        }
+    } else {
+        lo = f32_to_fp8_pair(v[0], v[1]) | (f32_to_fp8_pair(v[2], v[3]) << 16);
+        hi = f32_to_fp8_pair(v[4], v[5]) | (f32_to_fp8_pair(v[6], v[7]) << 16);
+    }
+    return make_uint2(lo, hi);
+}
+
+// 8-element chunks a lane keeps in registers between the two passes
+// (16-bit inputs: rows up to 64*8*16 = 8192 elements stay resident).
+template <int XDT>
+constexpr int row_cache() { return XDT == GLA_DT_FP32 ? 8 : 16; }
+
+// One wave per row.  The amax pass keeps the raw row in registers; the part of a
+// longer row that does not fit is read again (from L2) in the quantise pass.
+template <int XDT, bool TO_INT8>
+__global__ __launch_bounds__(256) void per_token_kernel(const void* __restrict__ x, int64_t xsm, int M, int K,
+                                                        uint8_t* __restrict__ y, float* __restrict__ scales) {
+    constexpr int RC = row_cache<XDT>();
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+    const int chunks = K / 8;  // K % 8 == 0 enforced by the launcher
+
+    Raw8<XDT> cache[RC];
+    float amax = 0.0f;
+#pragma unroll
+    for (int ci = 0; ci < RC; ++ci) {
+        const int c = lane + ci * kWave;
+        if (c < chunks) cache[ci] = load_raw8<XDT>(xrow, c * 8);
+    }
+#pragma unroll
+    for (int ci = 0; ci < RC; ++ci) {
+        const int c = lane + ci * kWave;
+        if (c < chunks) {
+            float v[8];
+            decode_raw8<XDT>(cache[ci], v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+        }
+    }
+    for (int c = lane + RC * kWave; c < chunks; c += kWave) {
+        float v[8];
+        decode_raw8<XDT>(load_raw8<XDT>(xrow, c * 8), v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    }
+    amax = wave_max(amax);
+    const float qmax = TO_INT8 ? 127.0f : 448.0f;
+    const float s = fmaxf(amax / qmax, 1e-6f);
+    if (lane == 0) scales[row] = s;
+
+    uint8_t* yrow = y + (int64_t)row * K;
+#pragma unroll
+    for (int ci = 0; ci < RC; ++ci) {
+        const int c = lane + ci * kWave;
+        if (c < chunks) {
+            float v[8];
+            decode_raw8<XDT>(cache[ci], v);
+            *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
+        }
+    }
+    for (int c = lane + RC * kWave; c < chunks; c += kWave) {
+        float v[8];
+        decode_raw8<XDT>(load_raw8<XDT>(xrow, c * 8), v);
+        *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
+    }
+}
+
+// e2m1 code of v (already divided by the block scale): ties toward zero, -0 keeps its sign bit
+// only through the v >= 0 test, exactly like the reference's threshold path.
+__device__ __forceinline__ uint32_t e2m1_code(float v) {
+    const float a = fabsf(v);
+    uint32_t idx = (a > 0.25f) + (a > 0.75f) + (a > 1.25f) + (a > 1.75f) + (a > 2.5f) + (a > 3.5f) + (a > 5.0f);
+    return (v >= 0.0f) ? idx : (idx + 8u);
+}
+
+// Four lanes share one 32-value group (8 values each): a wave covers 16 groups = 512 values.
+template <int XDT>
+__global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, int64_t xsm, int M, int M_pad, int K,
+                                                    uint8_t* __restrict__ y, uint8_t* __restrict__ scales) {
+    const int groups = K / 32;
+    const int gpr = (groups + 15) / 16;  // wave-chunks per row
+    const int64_t wave_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int row = (int)(wave_id / gpr);
+    const int g = (int)(wave_id % gpr) * 16 + (lane >> 2);
+    if (row >= M_pad) return;
+    if (row >= M) {  // padding rows carry the identity scale and no codes
+        if ((lane & 3) == 0 && g < groups) scales[(int64_t)row * groups + g] = 127;
+        return;
+    }
+    const bool active = g < groups;
+    const int k = g * 32 + (lane & 3) * 8;
+    float v[8];
+    if (active) {
+        const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+        load8<XDT>(xrow, k, v);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = 0.0f;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
+
+    const uint32_t bits = __builtin_bit_cast(uint32_t, amax / 6.0f);
+    uint32_t e = (bits >> 23) & 0xffu;
+    e += (bits & 0x7fffffu) ? 1u : 0u;
+    e = e > 254u ? 254u : e;
+    e = e < 97u ? 97u : e;
+    const float s = __builtin_bit_cast(float, e << 23);
+
+    if (!active) return;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) packed |= e2m1_code(v[j] / s) << (4 * j);
+    *(uint32_t*)(y + (int64_t)row * (K / 2) + k / 2) = packed;
+    if ((lane & 3) == 0) scales[(int64_t)row * groups + g] = (uint8_t)e;
+}
+
+}  // namespace
+
+int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
+                         float* scales, hipStream_t stream) {
+    if (x == nullptr || y == nullptr || scales == nullptr || M < 0 || K <= 0) {
+        set_error("scale_activations_per_token: null pointer or bad size");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (K % 8 != 0 || x_stride_m % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)y & 7)) {
+        set_error("scale_activations_per_token: K and the row stride must be multiples of 8, x 16-byte aligned");
+        return GLA_ERR_MISALIGNED_SHAPE;
+    }
+    if (y_dtype != GLA_DT_INT8 && y_dtype != GLA_DT_FP8) {
+        set_error("scale_activations_per_token: output type %d not supported (int8 or fp8-e4m3fn)", y_dtype);
+        return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (M == 0) return GLA_OK;
+    dim3 grid(ceil_div(M, 4)), block(256);
+    const bool i8 = (y_dtype == GLA_DT_INT8);
+#define GLA_PT(XDT)                                                                                         \
+    do {                                                                                                    \
+        if (i8) hipLaunchKernelGGL((per_token_kernel<XDT, true>), grid, block, 0, stream, x, x_stride_m, M, K, \
+                                   (uint8_t*)y, scales);                                                    \
+        else hipLaunchKernelGGL((per_token_kernel<XDT, false>), grid, block, 0, stream, x, x_stride_m, M, K,  \
+                                (uint8_t*)y, scales);                                                       \
+    } while (0)
+    switch (x_dtype) {
+        case GLA_DT_FP16: GLA_PT(GLA_DT_FP16); break;
+        case GLA_DT_BF16: GLA_PT(GLA_DT_BF16); break;
+        case GLA_DT_FP32: GLA_PT(GLA_DT_FP32); break;
+        default:
+            set_error("scale_activations_per_token: input type %d not supported", x_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+#undef GLA_PT
+    return check_hip(hipGetLastError(), "per-token activation quant launch");
+}
+
+int launch_act_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
+                     hipStream_t stream) {
+    if (x == nullptr || y == nullptr || scales == nullptr || M < 0 || K <= 0) {
+        set_error("scale_activations_mxfp4: null pointer or bad size");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (K % 32 != 0 || x_stride_m % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)y & 3)) {
+        set_error("scale_activations_mxfp4: K must be a multiple of 32, the row stride of 8, x 16-byte aligned");
+        return GLA_ERR_MISALIGNED_SHAPE;
+    }
+    if (M == 0) return GLA_OK;
+    const int M_pad = (M + 31) / 32 * 32;
+    const int groups = K / 32;
+    const int gpr = (groups + 15) / 16;
+    const int64_t waves = (int64_t)M_pad * gpr;
+    dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    switch (x_dtype) {
+        case GLA_DT_FP16:
+            hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP16>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            break;
+        case GLA_DT_BF16:
+            hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_BF16>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            break;
+        case GLA_DT_FP32:
+            hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP32>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            break;
+        default:
+            set_error("scale_activations_mxfp4: input type %d not supported", x_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    return check_hip(hipGetLastError(), "MXFP4 activation quant launch");
+}
+
+}  // namespace gla

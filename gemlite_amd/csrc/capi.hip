@@ -1,0 +1,222 @@
+// C ABI of the library: argument validation, kernel-family choice, error strings.
+// Entry points are declared and documented in include/gemlite_amd.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace gla {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return GLA_OK;
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return GLA_ERR_LAUNCH_FAILED;
+}
+
+namespace {
+
+bool is_mx(int dt) { return dt >= 14 && dt <= 18; }
+
+int closest_m(int M) {
+    // {2^i} plus 0.75*2^i and 1.5*2^i for 2^i >= 32, capped at 4096; next value >= M
+    if (M > 4096) return 4096;
+    int best = 4096;
+    for (int i = 0; i <= 12; ++i) {
+        const int p = 1 << i;
+        const int cands[3] = {p, (p >= 32 && 2 * p <= 4096) ? (3 * p) / 4 : p, (p >= 32 && 2 * p <= 4096) ? (3 * p) / 2 : p};
+        for (int c : cands)
+            if (c >= M && c < best) best = c;
+    }
+    return best;
+}
+
+int matmul_type_for(int M, int W_nbits, int mx) {
+    if (M >= 64) return GLA_MATMUL_GEMM;
+    const int gemv_limit = (W_nbits < 8 && !mx) ? 4 : 2;
+    if (M > gemv_limit) return GLA_MATMUL_GEMM_SPLITK;
+    if (mx) return GLA_MATMUL_GEMM_SPLITK;
+    return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
+}
+
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4 };
+
+int validate(const gla_matmul_args* p) {
+    if (p == nullptr) {
+        set_error("matmul: args is NULL");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (p->struct_size != sizeof(gla_matmul_args)) {
+        set_error("matmul: struct_size %u does not match the library's %zu", p->struct_size, sizeof(gla_matmul_args));
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (p->M < 0 || p->N <= 0 || p->K <= 0) {
+        set_error("matmul: bad shape M=%d N=%d K=%d", p->M, p->N, p->K);
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (p->x == nullptr || p->w == nullptr || p->out == nullptr) {
+        if (p->M == 0) return GLA_OK;
+        set_error("matmul: x, w and out must not be NULL");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (p->matmul_type < GLA_MATMUL_AUTO || p->matmul_type > GLA_MATMUL_GEMM) {
+        set_error("matmul: matmul_type %d out of range", p->matmul_type);
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    if (p->elements_per_sample < 1 || p->K % p->elements_per_sample != 0) {
+        set_error("matmul: K=%d not divisible by elements_per_sample=%d", p->K, p->elements_per_sample);
+        return GLA_ERR_MISALIGNED_SHAPE;
+    }
+    if (p->input_dtype == GLA_DT_MXFP4) {
+        if (p->K % 32 != 0) {
+            set_error("matmul: MXFP4 needs K %% 32 == 0 (K=%d)", p->K);
+            return GLA_ERR_MISALIGNED_SHAPE;
+        }
+        return GLA_OK;
+    }
+    if (is_mx(p->input_dtype)) {
+        set_error("matmul: micro-scaled input type %d is not supported (MXFP4 x MXFP4 only)", p->input_dtype);
+        return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    switch (p->input_dtype) {
+        case GLA_DT_FP32: case GLA_DT_FP16: case GLA_DT_BF16: case GLA_DT_FP8: case GLA_DT_INT8: break;
+        default:
+            set_error("matmul: input type %d not supported", p->input_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    switch (p->output_dtype) {
+        case GLA_DT_FP32: case GLA_DT_FP16: case GLA_DT_BF16: case GLA_DT_INT32: break;
+        default:
+            set_error("matmul: output type %d not supported", p->output_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (p->acc_dtype != GLA_DT_FP32 && p->acc_dtype != GLA_DT_INT32) {
+        set_error("matmul: accumulator type %d not supported (fp32 or int32)", p->acc_dtype);
+        return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (p->acc_dtype == GLA_DT_INT32 && p->input_dtype != GLA_DT_INT8) {
+        set_error("matmul: int32 accumulation needs int8 activations");
+        return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (p->W_group_mode < GLA_WGM_NONE || p->W_group_mode > GLA_WGM_FMA) {
+        set_error("matmul: W_group_mode %d out of range", p->W_group_mode);
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    if (p->channel_scale_mode < GLA_CSM_NONE || p->channel_scale_mode > GLA_CSM_BOTH) {
+        set_error("matmul: channel_scale_mode %d not supported for this input type", p->channel_scale_mode);
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    const bool need_s = p->W_group_mode >= GLA_WGM_SCALE || (p->channel_scale_mode & 1);
+    const bool need_z = p->W_group_mode == GLA_WGM_SHIFT || p->W_group_mode >= GLA_WGM_SHIFT_SCALE;
+    if ((need_s && p->scales == nullptr) || (need_z && p->zeros == nullptr) ||
+        ((p->channel_scale_mode & 2) && p->scales_x == nullptr)) {
+        set_error("matmul: mode (W_group_mode=%d, channel_scale_mode=%d) needs a tensor that is NULL",
+                  p->W_group_mode, p->channel_scale_mode);
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (p->W_group_mode != GLA_WGM_NONE && !(p->W_group_mode == GLA_WGM_SHIFT && p->zero_is_scalar)) {
+        if (p->group_size < 1 || p->K % p->group_size != 0) {
+            set_error("matmul: K=%d not divisible by group_size=%d", p->K, p->group_size);
+            return GLA_ERR_MISALIGNED_SHAPE;
+        }
+    }
+    return GLA_OK;
+}
+
+Family choose(const gla_matmul_args& p, int type) {
+    if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : F_GENERIC;
+    const bool want_gemv = type <= GLA_MATMUL_GEMV_SPLITK;
+    if (want_gemv) {
+        if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
+        if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
+        return F_GENERIC;
+    }
+    if (gemm_wn_eligible(p)) return F_GEMM_WN;
+    if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;
+    return F_GENERIC;
+}
+
+int resolve_type(const gla_matmul_args& p) {
+    return p.matmul_type == GLA_MATMUL_AUTO ? matmul_type_for(p.M, p.W_nbits, is_mx(p.input_dtype)) : p.matmul_type;
+}
+
+}  // namespace
+}  // namespace gla
+
+using namespace gla;
+
+extern "C" {
+
+int gla_abi_version(void) { return GLA_ABI_VERSION; }
+
+const char* gla_last_error(void) { return g_error; }
+
+int gla_get_matmul_type(int M, int W_nbits, int is_mx_) { return matmul_type_for(M, W_nbits, is_mx_); }
+
+int gla_get_closest_m(int M) { return closest_m(M); }
+
+int gla_select_config(const gla_matmul_args* args) {
+    const int rc = validate(args);
+    if (rc != GLA_OK) return rc;
+    const Family f = choose(*args, resolve_type(*args));
+    if (f == F_GEMV_PACKED) return gemv_packed_default_config(*args);
+    return 0;
+}
+
+int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
+    const int rc = validate(args);
+    if (rc != GLA_OK) return rc;
+    if (args->M == 0) return 0;
+    switch (choose(*args, resolve_type(*args))) {
+        case F_GEMV_PACKED: return gemv_packed_workspace_bytes(*args);
+        case F_GEMM_WN: return gemm_wn_workspace_bytes(*args);
+        default: return 0;
+    }
+}
+
+int gla_matmul(const gla_matmul_args* args, void* stream) {
+    const int rc = validate(args);
+    if (rc != GLA_OK) return rc;
+    if (args->M == 0) return GLA_OK;
+    hipStream_t s = (hipStream_t)stream;
+    switch (choose(*args, resolve_type(*args))) {
+        case F_GEMV_PACKED: return launch_gemv_packed(*args, s);
+        case F_GEMV_KMAJOR: return launch_gemv_kmajor(*args, s);
+        case F_GEMM_WN: return launch_gemm_wn(*args, s);
+        case F_GEMM_8BIT: return launch_gemm_8bit(*args, s);
+        case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
+        default: return launch_generic(*args, s);
+    }
+}
+
+int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y,
+                                    int y_dtype, float* scales, void* stream) {
+    return launch_act_per_token(x, x_dtype, x_stride_m, M, K, y, y_dtype, scales, (hipStream_t)stream);
+}
+
+int gla_scale_activations_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y,
+                                uint8_t* scales, void* stream) {
+    return launch_act_mxfp4(x, x_dtype, x_stride_m, M, K, y, scales, (hipStream_t)stream);
+}
+
+int gla_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t cols, int W_nbits,
+                       int packing_bitwidth, void* stream) {
+    return launch_pack_over_cols(codes, out, rows, cols, W_nbits, packing_bitwidth, (hipStream_t)stream);
+}
+
+int gla_unpack_over_cols(const void* packed, uint8_t* out, int64_t rows, int64_t packed_cols, int W_nbits,
+                         int packing_bitwidth, void* stream) {
+    return launch_unpack_over_cols(packed, out, rows, packed_cols, W_nbits, packing_bitwidth, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,45 @@
+// Host-side declarations shared by the C ABI and the kernel-family launchers.
+#pragma once
+
+#include "common.hpp"
+
+namespace gla {
+
+// ---- layout-agnostic path (generic.hip) -----------------------------------
+int launch_generic(const gla_matmul_args& p, hipStream_t stream);
+
+// ---- streaming GEMV on 32-bit packed words, N fastest (gemv_packed.hip) ----
+// tile_config (when >= 0) = number of 128-word-row slabs each workgroup owns.
+bool gemv_packed_eligible(const gla_matmul_args& p);
+int64_t gemv_packed_workspace_bytes(const gla_matmul_args& p);
+int gemv_packed_default_config(const gla_matmul_args& p);
+int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream);
+
+// ---- GEMV on K-contiguous 8/16-bit weights (gemv_kmajor.hip) ---------------
+bool gemv_kmajor_eligible(const gla_matmul_args& p);
+int launch_gemv_kmajor(const gla_matmul_args& p, hipStream_t stream);
+
+// ---- MFMA GEMM with in-register dequant of packed words (gemm_wn.hip) ------
+bool gemm_wn_eligible(const gla_matmul_args& p);
+int64_t gemm_wn_workspace_bytes(const gla_matmul_args& p);
+int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream);
+
+// ---- MFMA GEMM on 8-bit operands, both K-contiguous (gemm_8bit.hip) --------
+bool gemm_8bit_eligible(const gla_matmul_args& p);
+int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream);
+
+// ---- block-scaled MXFP4 MFMA GEMM (gemm_mxfp4.hip) -------------------------
+bool gemm_mxfp4_eligible(const gla_matmul_args& p);
+int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream);
+
+// ---- activation quantisation (actquant.hip) and bit packing (bitpack.hip) --
+int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
+                         float* scales, hipStream_t stream);
+int launch_act_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
+                     hipStream_t stream);
+int launch_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t cols, int nbits, int width,
+                          hipStream_t stream);
+int launch_unpack_over_cols(const void* packed, uint8_t* out, int64_t rows, int64_t pcols, int nbits, int width,
+                            hipStream_t stream);
+
+}  // namespace gla

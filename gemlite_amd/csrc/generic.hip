@@ -1,0 +1,206 @@
+// Layout-agnostic quantized matmul: one lane per output column, a loop over K.
+//
+// This kernel accepts every operand layout, packing width, element type and
+// mode combination the C ABI admits.  It is the path for shapes the tuned
+// kernels do not cover (odd packing widths, strided views, N not a multiple of
+// 4, ...); the tuned kernels are checked against the same arithmetic contract:
+//
+//   w(k,n)   = dequant(code(k,n))            per W_group_mode, in fp32
+//   acc(m,n) = sum_k x(m,k) * w(k,n)         fp32, or exact int32
+//   out(m,n) = cast(acc * channel scales)    per channel_scale_mode
+//
+// (reference: gemlite/triton_kernels/utils.py:73-105 for dequant,
+//  gemlite/triton_kernels/gemm_kernels.py:405-496 for the loop and epilogue,
+//  gemlite/triton_kernels/gemm_kernels.py:696-726 for the micro-scaled form).
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace gla {
+
+namespace {
+
+constexpr int kRows = 4;  // output rows per thread
+
+struct GenericArgs {
+    const void* x;
+    const void* w;
+    const void* scales;
+    const void* zeros;
+    const void* scales_x;
+    void* out;
+    int M, N, K;
+    int64_t xsm, xsk, wsk, wsn, osm, osn, msg, msn, sxm, sxg;
+    int nbits, gs, mask, e;
+    int in_dt, out_dt, acc_dt, meta_dt, csm, wgm;
+    int w_dt, z_dt, z_scalar, sx_dt;
+};
+
+__device__ __forceinline__ int64_t load_word(const void* p, int dt, int64_t idx) {
+    switch (dt) {
+        case GLA_DT_UINT8: return ((const uint8_t*)p)[idx];
+        case GLA_DT_INT8: return ((const int8_t*)p)[idx];
+        case GLA_DT_INT16: return ((const int16_t*)p)[idx];
+        case GLA_DT_INT32: return ((const int32_t*)p)[idx];
+        case GLA_DT_INT64: return ((const int64_t*)p)[idx];
+        default: return 0;
+    }
+}
+
+__device__ __forceinline__ bool is_float_dt(int dt) {
+    return dt == GLA_DT_FP32 || dt == GLA_DT_FP16 || dt == GLA_DT_BF16 || dt == GLA_DT_FP8;
+}
+
+// Integer and float grouped-dequant matmul.
+__global__ __launch_bounds__(64) void generic_int_kernel(GenericArgs a) {
+    const int n = blockIdx.x * 64 + threadIdx.x;
+    const int m0 = blockIdx.y * kRows;
+    if (n >= a.N) return;
+
+    const bool int_acc = (a.acc_dt == GLA_DT_INT32);
+    const bool w_is_float = is_float_dt(a.w_dt);
+    const int groups = (a.wgm == GLA_WGM_NONE) ? 1 : (a.K / a.gs);
+    const int klen = (a.wgm == GLA_WGM_NONE) ? a.K : a.gs;
+    const bool has_scale = (a.wgm == GLA_WGM_SCALE || a.wgm == GLA_WGM_SHIFT_SCALE || a.wgm == GLA_WGM_FMA);
+    const bool has_zero = (a.wgm == GLA_WGM_SHIFT || a.wgm == GLA_WGM_SHIFT_SCALE || a.wgm == GLA_WGM_FMA);
+
+    float facc[kRows] = {0.f, 0.f, 0.f, 0.f};
+    int iacc[kRows] = {0, 0, 0, 0};
+
+    for (int g = 0; g < groups; ++g) {
+        float s = 1.0f, z = 0.0f;
+        if (has_scale) s = load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + (int64_t)n * a.msn);
+        if (has_zero)
+            z = a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0)
+                           : load_as_float(a.zeros, a.z_dt, (int64_t)g * a.msg + (int64_t)n * a.msn);
+        const int k0 = g * klen;
+        for (int kk = 0; kk < klen; ++kk) {
+            const int k = k0 + kk;
+            const int64_t widx = (int64_t)(k / a.e) * a.wsk + (int64_t)n * a.wsn;
+            float qf;
+            int qi = 0;
+            if (w_is_float) {
+                qf = load_as_float(a.w, a.w_dt, widx);
+            } else {
+                int64_t word = load_word(a.w, a.w_dt, widx);
+                if (a.e > 1) word = (word >> ((k % a.e) * a.nbits)) & (int64_t)a.mask;
+                qi = (int)word;
+                qf = (float)qi;
+            }
+            if (int_acc) {
+                const int wi = has_zero ? (qi - (int)z) : qi;
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const int m = m0 + r;
+                    if (m < a.M)
+                        iacc[r] += (int)((const int8_t*)a.x)[(int64_t)m * a.xsm + (int64_t)k * a.xsk] * wi;
+                }
+            } else {
+                float wv;
+                switch (a.wgm) {
+                    case GLA_WGM_SHIFT: wv = qf - z; break;
+                    case GLA_WGM_SCALE: wv = qf * s; break;
+                    case GLA_WGM_SHIFT_SCALE: wv = (qf - z) * s; break;
+                    case GLA_WGM_FMA: wv = __builtin_fmaf(qf, s, z); break;
+                    default: wv = qf; break;
+                }
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) {
+                    const int m = m0 + r;
+                    if (m < a.M)
+                        facc[r] = __builtin_fmaf(
+                            load_as_float(a.x, a.in_dt, (int64_t)m * a.xsm + (int64_t)k * a.xsk), wv, facc[r]);
+                }
+            }
+        }
+    }
+
+    float sb = 1.0f;
+    if (a.csm == GLA_CSM_WEIGHT || a.csm == GLA_CSM_BOTH) sb = load_as_float(a.scales, a.meta_dt, n);
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        const int m = m0 + r;
+        if (m >= a.M) continue;
+        const int64_t oidx = (int64_t)m * a.osm + (int64_t)n * a.osn;
+        if (int_acc && a.csm == GLA_CSM_NONE && a.out_dt == GLA_DT_INT32) {
+            ((int32_t*)a.out)[oidx] = iacc[r];
+            continue;
+        }
+        float v = int_acc ? (float)iacc[r] : facc[r];
+        float sa = 1.0f;
+        if (a.csm == GLA_CSM_ACTIVATION || a.csm == GLA_CSM_BOTH)
+            sa = load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
+        if (a.csm == GLA_CSM_WEIGHT) v *= sb;
+        else if (a.csm == GLA_CSM_ACTIVATION) v *= sa;
+        else if (a.csm == GLA_CSM_BOTH) v *= (sa * sb);
+        store_from_float(a.out, a.out_dt, oidx, v);
+    }
+}
+
+// e2m1 x e2m1 with e8m0 block scales on both operands (block = 32 along K).
+__global__ __launch_bounds__(64) void generic_mxfp4_kernel(GenericArgs a) {
+    const int n = blockIdx.x * 64 + threadIdx.x;
+    const int m0 = blockIdx.y * kRows;
+    if (n >= a.N) return;
+    float acc[kRows] = {0.f, 0.f, 0.f, 0.f};
+    const int blocks = a.K / 32;
+    for (int b = 0; b < blocks; ++b) {
+        const float sw = e8m0_to_float(((const uint8_t*)a.scales)[(int64_t)b * a.msg + (int64_t)n * a.msn]);
+        float part[kRows] = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < 16; ++j) {
+            const int kb = b * 16 + j;  // byte index along K
+            const uint32_t wb = ((const uint8_t*)a.w)[(int64_t)kb * a.wsk + (int64_t)n * a.wsn];
+            const float w0 = e2m1_to_float(wb & 15u), w1 = e2m1_to_float(wb >> 4);
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                const int m = m0 + r;
+                if (m < a.M) {
+                    const uint32_t xb = ((const uint8_t*)a.x)[(int64_t)m * a.xsm + (int64_t)kb * a.xsk];
+                    part[r] += e2m1_to_float(xb & 15u) * w0 + e2m1_to_float(xb >> 4) * w1;
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+            const int m = m0 + r;
+            if (m < a.M) {
+                const float sa =
+                    e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)b * a.sxg]);
+                acc[r] = __builtin_fmaf(part[r], sa * sw, acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        const int m = m0 + r;
+        if (m < a.M) store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, acc[r]);
+    }
+}
+
+}  // namespace
+
+int launch_generic(const gla_matmul_args& p, hipStream_t stream) {
+    GenericArgs a;
+    a.x = p.x; a.w = p.w; a.scales = p.scales; a.zeros = p.zeros; a.scales_x = p.scales_x; a.out = p.out;
+    a.M = p.M; a.N = p.N; a.K = p.K;
+    a.xsm = p.x_stride_m; a.xsk = p.x_stride_k; a.wsk = p.w_stride_k; a.wsn = p.w_stride_n;
+    a.osm = p.out_stride_m; a.osn = p.out_stride_n; a.msg = p.meta_stride_g; a.msn = p.meta_stride_n;
+    a.sxm = p.sx_stride_m; a.sxg = p.sx_stride_g;
+    a.nbits = p.W_nbits; a.gs = p.group_size; a.mask = p.unpack_mask; a.e = p.elements_per_sample;
+    a.in_dt = p.input_dtype; a.out_dt = p.output_dtype; a.acc_dt = p.acc_dtype; a.meta_dt = p.meta_dtype;
+    a.csm = p.channel_scale_mode; a.wgm = p.W_group_mode;
+    a.w_dt = p.w_dtype; a.z_dt = p.zeros_dtype; a.z_scalar = p.zero_is_scalar; a.sx_dt = p.sx_dtype;
+
+    dim3 grid(ceil_div(p.N, 64), ceil_div(p.M, kRows));
+    if (p.input_dtype == GLA_DT_MXFP4) {
+        if (p.channel_scale_mode != GLA_CSM_MX || p.scales == nullptr || p.scales_x == nullptr) {
+            set_error("MXFP4 activations need channel_scale_mode 4 with both block-scale tensors");
+            return GLA_ERR_UNSUPPORTED_MODE;
+        }
+        hipLaunchKernelGGL(generic_mxfp4_kernel, grid, dim3(64), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL(generic_int_kernel, grid, dim3(64), 0, stream, a);
+    }
+    return check_hip(hipGetLastError(), "generic matmul launch");
+}
+
+}  // namespace gla

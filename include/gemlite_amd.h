@@ -1,0 +1,187 @@
+/*
+ * gemlite_amd.h - C ABI of the MI355X (gfx950) quantized-matmul library.
+ *
+ * Every entry point takes plain pointers, sizes and integer ids only.  Device
+ * pointers are owned by the caller; the library never allocates, frees or
+ * retains them, never synchronises the host with the device, and launches on
+ * the stream it is given (a hipStream_t passed as void*; NULL = default
+ * stream).  All functions return GLA_OK (0) or a negative GLA_ERR_* code and
+ * never throw; gla_last_error() returns a thread-local description of the
+ * last failure.
+ *
+ * Element-type ids are the integers of the reference's DType enumeration
+ * (reference: gemlite/dtypes.py:8-29).
+ */
+#ifndef GEMLITE_AMD_H
+#define GEMLITE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GLA_ABI_VERSION 1
+
+/* status codes */
+#define GLA_OK 0
+#define GLA_ERR_INVALID_ARGUMENT (-1) /* NULL pointer, bad size, inconsistent strides */
+#define GLA_ERR_UNSUPPORTED_DTYPE (-2)
+#define GLA_ERR_UNSUPPORTED_MODE (-3) /* W_group_mode / channel_scale_mode / matmul_type */
+#define GLA_ERR_MISALIGNED_SHAPE (-4) /* K not a multiple of group size / word size */
+#define GLA_ERR_WORKSPACE_TOO_SMALL (-5)
+#define GLA_ERR_LAUNCH_FAILED (-6)    /* HIP runtime reported an error */
+#define GLA_ERR_NO_DEVICE (-7)
+
+/* element-type ids (subset used on the hot path) */
+#define GLA_DT_FP32 0
+#define GLA_DT_FP16 1
+#define GLA_DT_BF16 2
+#define GLA_DT_FP8 3 /* OCP e4m3fn */
+#define GLA_DT_INT8 4
+#define GLA_DT_UINT8 5
+#define GLA_DT_INT32 6
+#define GLA_DT_INT16 9
+#define GLA_DT_INT64 11
+#define GLA_DT_MXFP8 16
+#define GLA_DT_MXFP4 17
+#define GLA_DT_E8M0 19
+
+/* matmul kernel families; the ids index the reference's kernel list
+ * (reference: gemlite/core.py:57-67). */
+#define GLA_MATMUL_AUTO (-1)
+#define GLA_MATMUL_GEMV 0
+#define GLA_MATMUL_GEMV_REVSPLITK 1
+#define GLA_MATMUL_GEMV_SPLITK 2
+#define GLA_MATMUL_GEMM_SPLITK 3
+#define GLA_MATMUL_GEMM 4
+
+/* weight dequantisation modes (reference: gemlite/triton_kernels/utils.py:73-105) */
+#define GLA_WGM_NONE 0          /* w = q                */
+#define GLA_WGM_SHIFT 1         /* w = q - zero         */
+#define GLA_WGM_SCALE 2         /* w = q * scale        */
+#define GLA_WGM_SHIFT_SCALE 3   /* w = (q - zero)*scale */
+#define GLA_WGM_FMA 4           /* w = q*scale + zero   */
+
+/* post-accumulation scaling (reference: gemlite/core.py:647-703,
+ * gemlite/triton_kernels/gemm_kernels.py:471-485) */
+#define GLA_CSM_NONE 0
+#define GLA_CSM_WEIGHT 1     /* out *= scales[n]                       */
+#define GLA_CSM_ACTIVATION 2 /* out *= scales_x[m]                     */
+#define GLA_CSM_BOTH 3       /* out *= scales_x[m] * scales[n]         */
+#define GLA_CSM_MX 4         /* per-32 e8m0 micro-scales on both sides */
+
+/*
+ * Arguments of one quantized matmul  out[M,N] = x[M,K] * dequant(w)[K,N].
+ *
+ * Replaces the argument list of the reference's per-family launchers
+ *   gemv_forward            gemlite/triton_kernels/gemv_kernels.py:608-701
+ *   gemv_revsplitK_forward  gemlite/triton_kernels/gemv_revsplitK_kernels.py:446-531
+ *   gemv_splitK_forward     gemlite/triton_kernels/gemv_splitK_kernels.py:480-542
+ *   gemm_splitK_forward     gemlite/triton_kernels/gemm_splitK_kernels.py:772-837
+ *   gemm_forward            gemlite/triton_kernels/gemm_kernels.py:741-799
+ * All strides are in elements of the tensor they belong to.  `w` is the
+ * [K/e, N] view the reference hands to its kernels (e = elements_per_sample):
+ * packed integer words are row-major with N fastest (w_stride_k = N,
+ * w_stride_n = 1); unpacked 8/16-bit weights are the transposed view of the
+ * row-major [N, K] tensor (w_stride_k = 1, w_stride_n = K).
+ */
+typedef struct gla_matmul_args {
+    uint32_t struct_size; /* sizeof(gla_matmul_args), for ABI checking */
+    int32_t matmul_type;  /* GLA_MATMUL_*; AUTO applies gla_get_matmul_type */
+
+    const void* x;        /* [M, K] activations (MXFP4: [M, K/2] bytes) */
+    const void* w;        /* weights, see above */
+    const void* scales;   /* weight scales or NULL */
+    const void* zeros;    /* weight zero points or NULL */
+    const void* scales_x; /* activation scales or NULL */
+    void* out;            /* [M, N] */
+    void* workspace;      /* scratch of >= gla_matmul_workspace_bytes() bytes, or NULL if 0 */
+    uint64_t workspace_bytes;
+
+    int32_t M, N, K;
+
+    int64_t x_stride_m, x_stride_k;
+    int64_t w_stride_k, w_stride_n;
+    int64_t out_stride_m, out_stride_n;
+    int64_t meta_stride_g, meta_stride_n; /* scales / zeros: [K/group_size, N] */
+    int64_t sx_stride_m, sx_stride_g;     /* scales_x: [M, 1] or [M_pad, K/32] */
+
+    /* the reference's meta_args (reference: gemlite/core.py:804-817) */
+    int32_t W_nbits;
+    int32_t group_size;
+    int32_t unpack_mask;
+    int32_t elements_per_sample;
+    int32_t input_dtype;  /* element type of x as the kernel sees it */
+    int32_t output_dtype;
+    int32_t acc_dtype;    /* GLA_DT_FP32 or GLA_DT_INT32 */
+    int32_t meta_dtype;   /* element type of scales */
+    int32_t channel_scale_mode;
+    int32_t W_group_mode;
+    int32_t data_contiguous;
+
+    int32_t w_dtype;        /* storage type of w (word type for packed data) */
+    int32_t zeros_dtype;    /* element type of zeros */
+    int32_t zero_is_scalar; /* zeros holds a single element */
+    int32_t sx_dtype;       /* element type of scales_x (FP32 or UINT8/E8M0) */
+    int32_t tile_config;    /* -1 = library heuristic, else an id from gla_select_config */
+} gla_matmul_args;
+
+/* Library identification.  No reference counterpart. */
+int gla_abi_version(void);
+const char* gla_last_error(void);
+
+/* Kernel-family choice from the batch size (reference: gemlite/core.py:163-179). */
+int gla_get_matmul_type(int M, int W_nbits, int is_mx);
+
+/* Batch-size bucketing used in config-cache keys
+ * (reference: gemlite/triton_kernels/utils.py:185-220). */
+int gla_get_closest_m(int M);
+
+/* Shape-based tile choice for a problem; the returned id is meaningful only to
+ * gla_matmul (replaces the Triton autotuner's config pruning,
+ * reference: gemlite/triton_kernels/gemm_kernels.py:31-145). */
+int gla_select_config(const gla_matmul_args* args);
+
+/* Scratch bytes gla_matmul needs for these arguments (0 if none).  The scratch
+ * must be zero-filled once when it is allocated; the library leaves it zeroed
+ * where it needs zeros.  (Plays the role of the reference's pre-zeroed output
+ * ring, gemlite/triton_kernels/config.py:31-34.) */
+int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args);
+
+/* Launch one quantized matmul (reference: the five launchers listed above). */
+int gla_matmul(const gla_matmul_args* args, void* stream);
+
+/* Per-token dynamic activation quantisation to fp8-e4m3fn or int8:
+ *   s[m] = max(amax(|x[m,:]|) / qmax, 1e-6);  y = clamp(x / s, qmin, qmax);
+ *   int8 rounds with floor(y + 0.5).
+ * x: [M, K] fp16/bf16/fp32 with row stride x_stride_m; y: [M, K] contiguous;
+ * scales: [M] fp32.
+ * (reference: gemlite/quant_utils.py:467-539, rounding :289-296) */
+int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K,
+                                    void* y, int y_dtype, float* scales, void* stream);
+
+/* MXFP4 dynamic activation quantisation: per 32 consecutive k one e8m0 scale
+ * 2^ceil(log2(amax/6)) (exponent clamped to [97, 254]) and 32 e2m1 codes, two
+ * per byte, even k in the low nibble.  y: [M, K/2] bytes; scales: [M_pad, K/32]
+ * bytes with M_pad = M rounded up to 32; rows M..M_pad-1 are set to 127.
+ * (reference: gemlite/quant_utils.py:2005-2135, exponent trick :697-705) */
+int gla_scale_activations_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K,
+                                uint8_t* y, uint8_t* scales, void* stream);
+
+/* Pack rows x cols 8-bit codes into words of packing_bitwidth bits along the
+ * column axis; out is [rows, cols/e] contiguous
+ * (reference: gemlite/bitpack.py:77-144). */
+int gla_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t cols, int W_nbits,
+                       int packing_bitwidth, void* stream);
+
+/* Inverse of gla_pack_over_cols; out is [rows, packed_cols*e] bytes
+ * (reference: gemlite/bitpack.py:164-205). */
+int gla_unpack_over_cols(const void* packed, uint8_t* out, int64_t rows, int64_t packed_cols,
+                         int W_nbits, int packing_bitwidth, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GEMLITE_AMD_H */

@@ -1,0 +1,277 @@
+"""GPU parity tests: every call goes through the C ABI (gemlite_amd._ext) and is compared with
+the CPU oracle on the same seeded inputs.  Integer / code outputs must match bit for bit; float
+outputs are gated at 1e-2 relative Frobenius error (and a tighter bound that a correct kernel
+with fp32 accumulation meets with room to spare)."""
+import numpy as np
+import pytest
+import torch
+
+import gemlite_amd
+from gemlite_amd import DType, GemLiteLinear, helper
+from gemlite_amd.bitpack import pack_weights_over_cols_hip, unpack_over_cols_hip
+from oracle import oracle as orc
+from parity import FROB_TOL, gen_int_case, gen_x, oracle_forward, rel_frob, round_like, to_np
+
+pytestmark = pytest.mark.gpu
+
+ALL_TYPES = ["GEMV_REVSPLITK", "GEMV", "GEMV_SPLITK", "GEMM_SPLITK", "GEMM"]
+TIGHT = {torch.float16: 1.5e-3, torch.bfloat16: 6e-3, torch.float32: 2e-4}
+
+
+def check_layer(layer, x, tol_dtype, types=ALL_TYPES, exact=False):
+    y_ref = oracle_forward(layer, x)
+    for mt in types:
+        M = x.numel() // x.shape[-1]
+        if M > 16 and "GEMV" in mt:
+            continue
+        print(f"case: {mt} M={M} N={layer.out_features} K={layer.in_features}", flush=True)
+        y = layer.forward_manual(x, matmul_type=mt)
+        torch.cuda.synchronize()
+        y_np = to_np(y).reshape(y_ref.shape)
+        if exact:
+            assert np.array_equal(y_np, y_ref), mt
+        else:
+            err = rel_frob(y_np, y_ref)
+            assert err <= FROB_TOL, (mt, err)
+            assert err <= TIGHT[tol_dtype], (mt, err)
+    y_auto = layer(x)
+    torch.cuda.synchronize()
+    if exact:
+        assert np.array_equal(to_np(y_auto).reshape(y_ref.shape), y_ref)
+    else:
+        assert rel_frob(to_np(y_auto).reshape(y_ref.shape), y_ref) <= TIGHT[tol_dtype]
+
+
+# ------------------------------------------------------------------ bit packing
+@pytest.mark.parametrize("nbits", [1, 2, 4, 8])
+@pytest.mark.parametrize("width", [8, 16, 32, 64])
+def test_pack_unpack_bit_exact(device, nbits, width):
+    rng = np.random.default_rng(nbits * 7 + width)
+    e = width // nbits
+    W = rng.integers(0, 2 ** nbits, size=(37, 6 * e), dtype=np.uint8)
+    packed, e_out = pack_weights_over_cols_hip(torch.from_numpy(W).to(device), nbits, width, transpose=False)
+    assert e_out == e
+    assert np.array_equal(packed.cpu().numpy(), orc.pack_over_cols(W, nbits, width))
+    back = unpack_over_cols_hip(packed, nbits, 6 * e)
+    assert np.array_equal(back.cpu().numpy(), W)
+
+
+def test_pack_large_matches_torch(device):
+    g = torch.Generator().manual_seed(0)
+    W = torch.randint(0, 16, (2032, 3968), generator=g, dtype=torch.int32).to(torch.uint8)
+    ref, _ = gemlite_amd.pack_weights_over_cols_torch(W, 4, 32, transpose=True)
+    out, _ = pack_weights_over_cols_hip(W.to(device), 4, 32, transpose=True)
+    assert torch.equal(out.cpu(), ref)
+
+
+# ------------------------------------------------------------------ activation quant
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 64), (5, 4224), (33, 8192), (7, 16384 + 64)])
+def test_per_token_quant_bit_exact(device, dtype, shape):
+    x = gen_x(shape[0], shape[1], dtype, seed=shape[1]) * 3
+    x[0, 0] = 0.0
+    for w_dtype, to_int8 in ((torch.int8, True), (torch.float8_e4m3fn, False)):
+        y, s = gemlite_amd.scale_activations_per_token(x.to(device), w_dtype)
+        q_ref, s_ref = orc.scale_activations_per_token(to_np(x), to_int8)
+        assert s.shape == (shape[0], 1) and np.array_equal(s.cpu().numpy(), s_ref)
+        y_bits = y.cpu().numpy() if to_int8 else y.view(torch.uint8).cpu().numpy()
+        assert np.array_equal(y_bits, q_ref)
+
+
+def test_per_token_quant_edge_rows(device):
+    x = torch.zeros((3, 128), dtype=torch.bfloat16)
+    x[1, 5] = -7.0
+    x[2, :8] = torch.tensor([127.0, 0.5, 1.5, -0.5, -1.5, 2.5, -2.5, 0.0]).bfloat16()
+    y, s = gemlite_amd.scale_activations_per_token(x.to(device), torch.int8)
+    q_ref, s_ref = orc.scale_activations_per_token(to_np(x), True)
+    assert np.array_equal(y.cpu().numpy(), q_ref) and np.array_equal(s.cpu().numpy(), s_ref)
+    assert y.cpu()[2, :8].tolist() == [127, 1, 2, 0, -1, 3, -2, 0]
+    # 3-D input keeps its shape
+    y3, s3 = gemlite_amd.scale_activations_per_token(x.view(3, 2, 64).to(device), torch.int8)
+    assert y3.shape == (3, 2, 64) and s3.shape == (6, 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 32), (3, 4224), (32, 1024), (45, 16384)])
+def test_mxfp4_quant_bit_exact(device, dtype, shape):
+    x = gen_x(shape[0], shape[1], dtype, seed=shape[0]) * (2.0 ** torch.randint(-6, 6, (shape[0], 1)).float()).to(dtype)
+    x[0, :8] = torch.tensor([0.25, -0.25, 0.75, 2.5, -0.0, 0.0, 5.0, -6.0]).to(dtype)
+    y, s = gemlite_amd.scale_activations_mxfp4(x.to(device))
+    y_ref, s_ref = orc.scale_activations_mxfp4(to_np(x))
+    assert y.shape == (shape[0], shape[1] // 2) and s.shape == ((shape[0] + 31) // 32 * 32, shape[1] // 32)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(y.cpu().numpy(), y_ref)
+
+
+def test_mxfp4_quant_zero_and_tiny_groups(device):
+    x = torch.zeros((2, 64), dtype=torch.bfloat16)
+    x[1, 32:] = 1e-30
+    y, s = gemlite_amd.scale_activations_mxfp4(x.to(device))
+    y_ref, s_ref = orc.scale_activations_mxfp4(to_np(x))
+    assert np.array_equal(s.cpu().numpy(), s_ref) and np.array_equal(y.cpu().numpy(), y_ref)
+    assert s.cpu()[0].tolist() == [97, 97]
+
+
+# ------------------------------------------------------------------ A16Wn
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("fma_mode", [True, False])
+def test_a16w4_grouped_reference_test_shape(device, dtype, fma_mode):
+    # the reference's own test shape: K = 3968, N = 2032 (edge tiles), 4-bit, group 128
+    N, K, gs = 2032, 3968, 128
+    W_q, scales, zeros = gen_int_case(N, K, 4, gs, dtype)
+    dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
+    layer = GemLiteLinear(4, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device), fma_mode=fma_mode)
+    assert layer.W_group_mode == (4 if fma_mode else 3) and layer.channel_scale_mode == 0 and layer.data_contiguous
+    for M in (1, 3, 5, 16, 30, 65):
+        check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("shape", [(4096, 4096), (14336, 4096), (4096, 14336)])
+def test_a16w4_benchmark_shapes(device, M, shape):
+    N, K = shape
+    W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16, seed=N + K)
+    layer = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    x = gen_x(M, K, torch.float16, seed=M)
+    y_ref = oracle_forward(layer, x)
+    y = layer(x.to(device))
+    torch.cuda.synchronize()
+    err = rel_frob(to_np(y), y_ref)
+    assert err <= TIGHT[torch.float16], err
+    # against the baseline's CPU path on the unpacked tensors: fp32 (W_q - z) * s, then matmul
+    y_hqq = orc.hqq_dequant_matmul(to_np(x), W_q.numpy(), to_np(scales), to_np(zeros), 128)
+    assert rel_frob(to_np(y), y_hqq) <= FROB_TOL
+
+
+@pytest.mark.parametrize("nbits,gs", [(2, 64), (1, 64), (4, 32), (4, 64), (8, 128), (2, 32), (4, 16)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
+    N, K = 1024, 2048
+    W_q, scales, zeros = gen_int_case(N, K, nbits, gs, dtype, seed=nbits * 10 + gs)
+    dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
+    layer = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    for M in (1, 4, 7, 64):
+        check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
+
+
+@pytest.mark.parametrize("post_scale", [True, False])
+@pytest.mark.parametrize("nbits", [8, 4])
+def test_a16wn_channelwise(device, nbits, post_scale):
+    N, K = 768, 1536
+    W_q, scales, zeros = gen_int_case(N, K, nbits, K, torch.bfloat16, seed=nbits, scale_std=0.01, channelwise=True)
+    layer = helper.A16Wn(device=device, post_scale=post_scale).from_weights(W_q, scales, zeros, nbits, K)
+    assert (layer.W_group_mode, layer.channel_scale_mode) == ((1, 1) if post_scale else (3, 0))
+    for M in (1, 2, 16, 65):
+        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16)
+
+
+def test_symmetric_and_shift_only_modes(device):
+    N, K, gs = 512, 1024, 128
+    W_q, scales, _ = gen_int_case(N, K, 4, gs, torch.float16)
+    # mode 2: scales only
+    l2 = GemLiteLinear(4, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), None)
+    assert l2.W_group_mode == 2
+    # mode 3 with an integer zero point
+    l3 = GemLiteLinear(4, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), 8)
+    assert l3.W_group_mode == 3 and l3.zeros.numel() == 1
+    # mode 1: shift only, fp32 output
+    l1 = GemLiteLinear(4, gs, K, N, DType.FP16, DType.FP32).pack(W_q.to(device), None, 7)
+    assert l1.W_group_mode == 1
+    for layer, dt in ((l2, torch.float16), (l3, torch.float16), (l1, torch.float32)):
+        for M in (1, 5):
+            check_layer(layer, (gen_x(M, K, torch.float16, seed=M) / 10).to(device), dt)
+
+
+def test_unpacked_fp16_weights_and_bias(device):
+    N, K = 1000, 2048
+    W = gen_x(N, K, torch.float16, seed=3, std=0.05)
+    bias = gen_x(1, N, torch.float16, seed=4).view(N)
+    layer = GemLiteLinear(16, None, K, N, DType.FP16, DType.FP16).pack(W.to(device), None, None, bias.to(device))
+    assert layer.W_group_mode == 0 and layer.elements_per_sample == 1 and not layer.data_contiguous
+    for M in (1, 3, 17):
+        x = gen_x(M, K, torch.float16, seed=M).to(device)
+        check_layer(layer, x, torch.float16)
+    # 3-D activations keep their leading dims
+    y = layer(gen_x(6, K, torch.float16).view(2, 3, K).to(device))
+    assert y.shape == (2, 3, N)
+
+
+@pytest.mark.parametrize("width", [8, 16, 64])
+def test_other_packing_widths(device, width):
+    N, K, gs = 256, 512, 64
+    W_q, scales, zeros = gen_int_case(N, K, 4, gs, torch.float16, seed=width)
+    layer = GemLiteLinear(4, gs, K, N, DType.FP16, DType.FP16).pack(
+        W_q.to(device), scales.to(device), zeros.to(device), packing_bitwidth=width)
+    assert layer.W_q.element_size() * 8 == width
+    check_layer(layer, gen_x(3, K, torch.float16).to(device), torch.float16)
+
+
+# ------------------------------------------------------------------ 8-bit activations
+def test_int8_x_int8_accumulators_bit_exact(device):
+    N, K = 520, 1024
+    g = torch.Generator().manual_seed(0)
+    W = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    layer = GemLiteLinear(8, None, K, N, DType.INT8, DType.INT32).pack(W.to(device), None, None)
+    assert layer.acc_dtype == DType.INT32 and layer.W_group_mode == 0 and layer.channel_scale_mode == 0
+    for M in (1, 2, 9, 70, 256):
+        x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+        ref = (x.long() @ W.long().t()).numpy()
+        for mt in ALL_TYPES:
+            y = layer.forward_manual(x.to(device), matmul_type=mt)
+            assert y.dtype == torch.int32 and np.array_equal(y.cpu().numpy(), ref), (mt, M)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_a8w8_dynamic(device, fp8):
+    N, K = 1032, 2048
+    W = gen_x(N, K, torch.bfloat16, seed=5, std=0.02)
+    proc = helper.A8W8_FP8_dynamic(device=device) if fp8 else helper.A8W8_INT8_dynamic(device=device)
+    layer = proc.from_weights(W)
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 3) and layer.scales.dtype == torch.float32
+    assert layer.W_q.stride() == (1, K)
+    # the weight codes are the oracle's
+    q_ref, s_ref = orc.quantize_per_channel(to_np(W), not fp8)
+    got = layer.W_q.t().contiguous()
+    got = got.view(torch.uint8).cpu().numpy() if fp8 else got.cpu().numpy()
+    assert np.array_equal(got, q_ref) and np.array_equal(layer.scales.cpu().numpy().reshape(-1, 1), s_ref)
+    for M in (1, 2, 33, 128):
+        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16)
+
+
+def test_int8_activations_packed_weights(device):
+    # int8 x 4-bit with an integer zero and channel-wise scales (reference: tests/test_int.py:146-171)
+    N, K = 400, 1024
+    W_q, _, _ = gen_int_case(N, K, 4, 128, torch.bfloat16)
+    scales = (gen_x(N, 1, torch.bfloat16, seed=9) * 1e-2)
+    layer = GemLiteLinear(4, 128, K, N, DType.INT8, DType.FP32).pack(W_q.to(device), scales.to(device), 7)
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (1, 1)
+    g = torch.Generator().manual_seed(1)
+    for M in (1, 5, 65):
+        x = torch.randint(-10, 10, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+        check_layer(layer, x.to(device), torch.float32)
+    # dynamic int8 activations x shifted 4-bit weights (reference: tests/test_int.py:173-199)
+    layer = GemLiteLinear(4, 128, K, N, DType.INT8, DType.FP32, scaled_activations=True).pack(W_q.to(device), None, 7)
+    layer.meta_dtype = DType.FP32
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (1, 2)
+    for M in (1, 5, 65):
+        check_layer(layer, (gen_x(M, K, torch.float16, seed=M) / 20).to(device), torch.float32)
+
+
+# ------------------------------------------------------------------ MXFP4
+@pytest.mark.parametrize("M", [1, 3, 32, 100, 128])
+def test_a4w4_mxfp4(device, M):
+    N, K = 512, 4224  # K of the reference's MX tests (reference: tests/test_mxfp.py:31)
+    W = gen_x(N, K, torch.bfloat16, seed=6, std=0.02)
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+    lin.weight.data = W
+    layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 4)
+    codes_ref, e_ref = orc.quantize_mxfp4_weights(to_np(W))
+    assert np.array_equal(orc.unpack_fp4_bytes(layer.W_q.t().contiguous().cpu().numpy()), codes_ref)
+    assert np.array_equal(layer.scales.contiguous().cpu().numpy(), e_ref)
+    x = gen_x(M, K, torch.bfloat16, seed=M)
+    check_layer(layer, x.to(device), torch.bfloat16, types=["GEMM", "GEMM_SPLITK"])
+    # and close to the unquantised product (format error only)
+    y = to_np(layer(x.to(device)))
+    y_fp = to_np(x) @ to_np(W).T
+    assert rel_frob(y, y_fp) < 0.2

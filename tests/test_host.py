@@ -1,0 +1,257 @@
+"""CPU-side tests of the host layer: layout, mode logic, dispatcher, C-ABI surface, errors."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import gemlite_amd
+from gemlite_amd import DType, GemLiteLinear, _ext
+from gemlite_amd.bitpack import pack_weights_over_cols_torch, unpack_over_cols_torch
+from gemlite_amd.dtypes import PACKING_BITWIDTH_TO_TORCH_DTYPE
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_dtype_enum_values():
+    # serialised integer ids (reference: gemlite/dtypes.py:8-29)
+    expect = dict(FP32=0, FP16=1, BF16=2, FP8=3, FP8e4=3, INT8=4, UINT8=5, INT32=6, UINT32=7, FP8e5=8, INT16=9,
+                  UINT16=10, INT64=11, FP8e4nuz=12, FP8e5nuz=13, MXFP16=14, MXBF16=15, MXFP8=16, MXFP4=17, NVFP4=18,
+                  E8M0=19)
+    for name, v in expect.items():
+        assert DType[name].value == v
+    assert gemlite_amd.is_mx_dtype(DType.MXFP4) and gemlite_amd.is_mx_dtype(17) and not gemlite_amd.is_mx_dtype(DType.FP8)
+
+
+@pytest.mark.parametrize("nbits", [1, 2, 4, 8])
+@pytest.mark.parametrize("width", [8, 16, 32, 64])
+def test_torch_pack_matches_oracle(nbits, width):
+    rng = np.random.default_rng(nbits + width)
+    e = width // nbits
+    W = rng.integers(0, 2 ** nbits, size=(6, 4 * e), dtype=np.uint8)
+    packed, e_out = pack_weights_over_cols_torch(torch.from_numpy(W), nbits, width, transpose=False)
+    assert e_out == e and packed.dtype == PACKING_BITWIDTH_TO_TORCH_DTYPE[width]
+    assert np.array_equal(packed.numpy(), orc.pack_over_cols(W, nbits, width))
+    packed_t, _ = pack_weights_over_cols_torch(torch.from_numpy(W), nbits, width, transpose=True)
+    assert packed_t.shape == (4, 6) and not packed_t.is_contiguous()
+    assert np.array_equal(unpack_over_cols_torch(packed, nbits, 4 * e).numpy(), W)
+
+
+def _layer(nbits=4, gs=128, K=256, N=64, in_dt=DType.FP16, out_dt=DType.FP16, **kw):
+    return GemLiteLinear(nbits, gs, K, N, in_dt, out_dt, **kw)
+
+
+def test_pack_layout_a16w4():
+    N, K, gs = 64, 256, 128
+    g = torch.Generator().manual_seed(0)
+    W_q = torch.randint(0, 16, (N, K), generator=g, dtype=torch.int32).to(torch.uint8)
+    scales = torch.rand((N * K // gs, 1), generator=g).half()
+    zeros = (torch.rand((N * K // gs, 1), generator=g) * 8).half()
+    layer = _layer().pack(W_q, scales, zeros)
+    # physical [K/8, N] int32, N fastest
+    assert layer.W_q.shape == (K // 8, N) and layer.W_q.dtype == torch.int32 and layer.W_q.is_contiguous()
+    assert layer.elements_per_sample == 8 and layer.data_contiguous is True
+    k8, n = 5, 17
+    word = sum(int(W_q[n, 8 * k8 + i]) << (4 * i) for i in range(8))
+    assert int(layer.W_q[k8, n]) & 0xFFFFFFFF == word
+    # scales [K/gs, N]; zeros pre-multiplied: z' = fp16(-z * s); mode 4
+    assert layer.scales.shape == (K // gs, N) and layer.scales.is_contiguous()
+    assert layer.W_group_mode == 4 and layer.channel_scale_mode == 0
+    assert torch.equal(layer.scales, scales.view(N, -1).t())
+    assert torch.equal(layer.zeros, (-zeros.float() * scales.float()).half().view(N, -1).t())
+    assert layer.get_meta_args() == [0, 4, 128, 15, 8, 1, 1, 0, 1, 0, 4, 1]
+    assert layer.metadata.tolist() == layer.get_meta_args() and layer.orig_shape.tolist() == [N, K]
+    # fma_mode=False keeps the raw zeros and uses mode 3
+    layer3 = _layer().pack(W_q, scales, zeros, fma_mode=False)
+    assert layer3.W_group_mode == 3 and torch.equal(layer3.zeros, zeros.view(N, -1).t())
+
+
+def test_pack_modes_like_reference_tests():
+    N, K = 48, 256
+    W_q = torch.randint(0, 15, (N, K)).to(torch.uint8)
+    W = torch.randn(N, K).to(torch.bfloat16)
+    # fp16 x fp16 (reference: tests/test_int.py:99-113)
+    l = _layer(16, None, K, N, DType.BF16, DType.BF16).pack(W, None, None, None)
+    assert (l.W_group_mode, l.channel_scale_mode, l.data_contiguous) == (0, 0, False)
+    assert l.W_q.shape == (K, N) and l.W_q.stride() == (1, K) and l.elements_per_sample == 1
+    # int8 x Wn, channel-wise scales + integer zero (reference: tests/test_int.py:146-163)
+    l = _layer(4, 128, K, N, DType.INT8, DType.FP32).pack(W_q, torch.randn(N, 1).bfloat16() * 1e-4, 7)
+    assert (l.W_group_mode, l.channel_scale_mode) == (1, 1) and l.zeros.item() == 7 and l.zeros.dtype == torch.int32
+    assert l.acc_dtype == DType.INT32
+    # dynamic activations only (reference: tests/test_int.py:173-190)
+    l = _layer(4, 128, K, N, DType.INT8, DType.FP32, scaled_activations=True).pack(W_q, None, 7)
+    assert (l.W_group_mode, l.channel_scale_mode) == (1, 2)
+    assert l.meta_dtype == DType.INT32  # placeholder scales tensor is int32
+    # both scaled (reference: tests/test_int.py:201-218)
+    l = _layer(8, 128, K, N, DType.INT8, DType.FP32, scaled_activations=True).pack(W_q, torch.rand(N, 1), 7)
+    assert (l.W_group_mode, l.channel_scale_mode) == (1, 3)
+    # fp8 x fp8, no scales / both scaled (reference: tests/test_int.py:226-271)
+    W8 = W.float().to(torch.float8_e4m3fn)
+    l = _layer(8, None, K, N, DType.FP8, DType.BF16, scaled_activations=True).pack(W8, None, None)
+    assert (l.W_group_mode, l.channel_scale_mode) == (0, 2) and l.W_q.stride() == (1, K)
+    l = _layer(8, K, K, N, DType.FP8, DType.BF16, scaled_activations=True).pack(W8, torch.rand(N, 1), None)
+    assert (l.W_group_mode, l.channel_scale_mode) == (0, 3)
+    # float inputs never get dynamic activation quantisation
+    assert _layer(4, 128, K, N, DType.FP16, DType.FP16, scaled_activations=True).scaled_activations is False
+
+
+def test_pack_mxfp4_layout():
+    N, K = 64, 256
+    codes = torch.randint(0, 16, (N, K)).to(torch.uint8)
+    e8 = torch.randint(110, 130, (N, K // 32)).to(torch.uint8).view(torch.float8_e8m0fnu)
+    l = gemlite_amd.helper.A4W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16).from_weights(codes, scales=e8)
+    # bytes [N, K/2] (low nibble = even k) handed over as the [K/2, N] view; e8m0 scales as the [N, K/32] view
+    assert l.W_q.shape == (K // 2, N) and l.W_q.stride() == (1, K // 2) and l.W_q.dtype == torch.uint8
+    assert int(l.W_q[3, 5]) == int(codes[5, 6]) | (int(codes[5, 7]) << 4)
+    assert l.scales.shape == (N, K // 32) and l.scales.dtype == torch.uint8 and l.scales.stride() == (1, N)
+    assert (l.W_group_mode, l.channel_scale_mode, l.elements_per_sample) == (0, 4, 2)
+    assert l.W_q.numel() == N * K // 2  # packed byte count (reference: tests/test_mxfp.py:96)
+
+
+def test_packing_widths_and_dtypes():
+    # W_q storage dtype per packing width (reference: tests/test_serialization.py:334-356)
+    N, K = 32, 128
+    W_q = torch.randint(0, 16, (N, K)).to(torch.uint8)
+    s, z = torch.rand(N * K // 64, 1).half(), torch.rand(N * K // 64, 1).half()
+    for width, dt in ((8, torch.uint8), (16, torch.int16), (32, torch.int32)):
+        l = _layer(4, 64, K, N).pack(W_q, s, z, packing_bitwidth=width)
+        assert l.W_q.dtype == dt and l.W_q.shape == (K * 4 // width, N)
+
+
+def test_constructor_errors():
+    with pytest.raises(NotImplementedError):
+        GemLiteLinear(3, 64, 128, 128)
+    with pytest.raises(NotImplementedError):
+        GemLiteLinear(4, 64, 100, 128)  # K % 32
+    with pytest.raises(NotImplementedError):
+        GemLiteLinear(4, 96, 128, 128)  # K % group_size
+    with pytest.raises(NotImplementedError):
+        GemLiteLinear(4, 8, 128, 128)   # group_size < 16
+    with pytest.raises(NotImplementedError):
+        GemLiteLinear(4, 64, 128, 128, input_dtype=DType.INT32)
+    with pytest.raises(Exception, match="floating-point zeros"):
+        _layer(4, 128, 256, 64, DType.INT8, DType.FP32).pack(
+            torch.zeros(64, 256, dtype=torch.uint8), torch.rand(64, 1), torch.rand(128, 1) + 0.3)
+    with pytest.raises(Exception, match="not packed"):
+        _layer().pack(torch.zeros(64, 256, dtype=torch.int32), None, None)
+
+
+def test_state_dict_roundtrip():
+    N, K, gs = 64, 256, 64
+    W_q = torch.randint(0, 16, (N, K)).to(torch.uint8)
+    s, z = torch.rand(N * K // gs, 1).half(), torch.rand(N * K // gs, 1).half()
+    fresh = _layer(4, gs, K, N)
+    assert set(fresh.state_dict().keys()) == {"W_q", "scales", "zeros", "metadata", "orig_shape", "meta_scale"}
+    a = _layer(4, gs, K, N).pack(W_q, s, z, bias=torch.rand(N).half())
+    sd = a.state_dict()
+    assert set(sd.keys()) == {"W_q", "scales", "zeros", "metadata", "orig_shape", "meta_scale", "bias"}
+    b = GemLiteLinear()
+    b.load_state_dict(dict(sd))
+    assert b.get_meta_args() == a.get_meta_args() and (b.in_features, b.out_features) == (K, N)
+    for ta, tb in zip(a.get_tensor_args(), b.get_tensor_args()):
+        assert torch.equal(ta, tb)
+    # through a parent module, strict
+    seq_a = torch.nn.Sequential(a)
+    seq_b = torch.nn.Sequential(GemLiteLinear())
+    seq_b.load_state_dict(seq_a.state_dict(), strict=True)
+    assert seq_b[0].get_meta_args() == a.get_meta_args() and torch.equal(seq_b[0].bias, a.bias)
+    # overridden modes are what gets saved
+    a.W_group_mode, a.channel_scale_mode = 3, 0
+    assert a.state_dict()["metadata"].tolist()[9:11] == [0, 3]
+    with pytest.raises(RuntimeError, match="missing required keys"):
+        GemLiteLinear().load_state_dict({"scales": s})
+
+
+def test_dispatcher_host_and_library_agree():
+    for nbits in (1, 2, 4, 8, 16):
+        for mx in (False, True):
+            for M in (1, 2, 3, 4, 5, 8, 16, 32, 63, 64, 65, 512, 4096, 8192):
+                name = gemlite_amd.get_matmul_type(M, nbits, mx)
+                assert name == orc.get_matmul_type(M, nbits, mx)
+                assert gemlite_amd.GEMLITE_MATMUL_TYPES[_ext.get_matmul_type_id(M, nbits, mx)] == name
+    for M in list(range(0, 300)) + [1000, 3000, 4096, 4097, 100000]:
+        assert gemlite_amd.get_closest_m(M) == orc.get_closest_m(M) == _ext.get_closest_m(M)
+    assert gemlite_amd.get_type_id(DType.BF16.value, 4) == 104 and gemlite_amd.get_type_id(DType.MXFP4.value, 4) == 1704
+    assert gemlite_amd.config_key(3, 4096, 4096, 128, 8, 104) == "(4, 4096, 4096, 128, 8, 104)"
+
+
+def test_config_cache_roundtrip(tmp_path):
+    gemlite_amd.reset_config()
+    gemlite_amd.GEMLITE_CONFIG_CACHE.setdefault("GEMV_REVSPLITK", {})["(1, 4096, 4096, 128, 8, 104)"] = {"tile_config": 2}
+    f = str(tmp_path / "cfg.json")
+    gemlite_amd.cache_config(f)
+    gemlite_amd.reset_config()
+    assert gemlite_amd.GEMLITE_CONFIG_CACHE == {}
+    assert gemlite_amd.load_config(f) is True
+    assert gemlite_amd.GEMLITE_CONFIG_CACHE["GEMV_REVSPLITK"]["(1, 4096, 4096, 128, 8, 104)"] == {"tile_config": 2}
+    assert gemlite_amd.load_config(str(tmp_path / "missing.json"), print_error=False) is False
+    gemlite_amd.reset_config()
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "gemlite_amd.h")).read()
+    declared = set(re.findall(r"\b(gla_[a-z0-9_]+)\s*\(", header))
+    assert declared and declared == set(_ext.SYMBOLS)
+    lib = ctypes.CDLL(_ext.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _ext.load_library().gla_abi_version() == 1
+
+
+def test_abi_struct_matches_header():
+    header = open(os.path.join(ROOT, "include", "gemlite_amd.h")).read()
+    body = header[header.index("typedef struct gla_matmul_args {"): header.index("} gla_matmul_args;")]
+    names = []
+    for line in body.splitlines()[1:]:
+        line = line.split("/*")[0].strip()
+        if not line.endswith(";"):
+            continue
+        decl = line[:-1]
+        for part in decl.split(",") if "*" not in decl else [decl]:
+            names.append(part.strip().split()[-1].lstrip("*"))
+    assert names == [f[0] for f in _ext.MatmulArgs._fields_]
+
+
+def test_abi_rejects_bad_arguments_without_a_gpu():
+    lib = _ext.load_library()
+    a = _ext.MatmulArgs()
+    assert lib.gla_matmul(None, None) == -1 and b"NULL" in lib.gla_last_error()
+    a.struct_size = 4
+    assert lib.gla_matmul(ctypes.byref(a), None) == -1 and b"struct_size" in lib.gla_last_error()
+    a.struct_size = ctypes.sizeof(_ext.MatmulArgs)
+    a.M, a.N, a.K = 1, 0, 64
+    assert lib.gla_matmul(ctypes.byref(a), None) == -1
+    a.N = 64
+    assert lib.gla_matmul(ctypes.byref(a), None) == -1  # NULL operands
+    a.x = a.w = a.out = 4096  # never dereferenced: validation fails first
+    a.elements_per_sample, a.W_nbits = 8, 4
+    a.input_dtype = DType.NVFP4.value
+    assert lib.gla_matmul(ctypes.byref(a), None) == -2
+    a.input_dtype, a.output_dtype, a.acc_dtype = DType.FP16.value, DType.FP16.value, DType.FP32.value
+    a.W_group_mode = 7
+    assert lib.gla_matmul(ctypes.byref(a), None) == -3
+    a.W_group_mode, a.group_size = 4, 48
+    a.scales = a.zeros = 4096
+    assert lib.gla_matmul(ctypes.byref(a), None) == -4  # K % group_size
+    a.group_size, a.scales = 64, None
+    assert lib.gla_matmul(ctypes.byref(a), None) == -1  # mode needs scales
+    a.matmul_type = 9
+    assert lib.gla_matmul(ctypes.byref(a), None) == -3
+    # activation-quant and packing entry points validate before launching
+    assert lib.gla_scale_activations_per_token(None, 1, 64, 1, 64, None, 4, None, None) == -1
+    assert lib.gla_scale_activations_per_token(4096, 1, 60, 1, 60, 4096, 4, 4096, None) == -4
+    assert lib.gla_scale_activations_per_token(4096, 1, 64, 1, 64, 4096, 2, 4096, None) == -2
+    assert lib.gla_scale_activations_mxfp4(4096, 1, 48, 1, 48, 4096, 4096, None) == -4
+    assert lib.gla_pack_over_cols(4096, 4096, 4, 30, 4, 32, None) == -4
+    assert lib.gla_pack_over_cols(4096, 4096, 4, 32, 3, 32, None) == -3
+
+
+def test_forward_requires_gpu_and_library():
+    l = _layer().pack(torch.zeros(64, 256, dtype=torch.uint8), torch.ones(128, 1).half(), torch.ones(128, 1).half())
+    with pytest.raises(RuntimeError, match="GPU only"):
+        l(torch.zeros(1, 256).half())
+    with pytest.raises(RuntimeError, match="not found"):
+        _ext.load_library(os.path.join(ROOT, "no_such_dir", "libgemlite_amd.so"))

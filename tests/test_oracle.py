@@ -1,0 +1,364 @@
+"""Pins the CPU oracle (oracle/oracle.py, oracle/oracle_c.c) without the reference:
+hand-computed answers, brute force, closed forms, library routines (torch's own
+low-precision casts), and the assertions the reference's tests make."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ------------------------------------------------------------------ bit packing
+def test_pack_known_words():
+    row = np.arange(8, dtype=np.uint8).reshape(1, 8)
+    assert orc.pack_over_cols(row, 4, 32)[0, 0] == 0x76543210
+    # a code >= 8 in the top nibble sets the sign bit of the int32 word
+    row = np.array([[0, 0, 0, 0, 0, 0, 0, 15]], dtype=np.uint8)
+    w = orc.pack_over_cols(row, 4, 32)
+    assert w.dtype == np.int32 and w[0, 0] == -268435456  # 0xF0000000
+    # 2-bit codes, 8-bit words: 3,2,1,0 -> 0b00_01_10_11
+    assert orc.pack_over_cols(np.array([[3, 2, 1, 0]], dtype=np.uint8), 2, 8)[0, 0] == 0b00011011
+    # 8-bit codes, 32-bit words: little-endian bytes
+    assert orc.pack_over_cols(np.array([[0x11, 0x22, 0x33, 0x84]], dtype=np.uint8), 8, 32)[0, 0] == 0x84332211 - (1 << 32)
+
+
+@pytest.mark.parametrize("nbits", [1, 2, 4, 8])
+@pytest.mark.parametrize("width", [8, 16, 32, 64])
+def test_pack_bruteforce_and_roundtrip(nbits, width):
+    rng = np.random.default_rng(nbits * 100 + width)
+    e = width // nbits
+    W = rng.integers(0, 2 ** nbits, size=(5, 3 * e), dtype=np.uint8)
+    packed = orc.pack_over_cols(W, nbits, width)
+    assert packed.shape == (5, 3) and packed.dtype == orc._WORD_DTYPES[width]
+    # brute force with python ints
+    for r in range(5):
+        for c in range(3):
+            word = 0
+            for i in range(e):
+                word |= int(W[r, c * e + i]) << (nbits * i)
+            assert int(packed[r, c]) & ((1 << width) - 1) == word
+    assert np.array_equal(orc.unpack_over_cols(packed, nbits, 3 * e), W)
+
+
+def test_c_pack_matches_numpy():
+    lib = ctypes.CDLL(os.path.join(ROOT, "oracle", "liboracle_c.so"))
+    rng = np.random.default_rng(0)
+    for nbits in (1, 2, 4, 8):
+        W = rng.integers(0, 2 ** nbits, size=(7, 64), dtype=np.uint8)
+        out = np.zeros((7, 64 * nbits // 32), dtype=np.int32)
+        lib.orc_pack_over_cols_32(
+            W.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(7), ctypes.c_int64(64), ctypes.c_int(nbits),
+            out.ctypes.data_as(ctypes.c_void_p),
+        )
+        assert np.array_equal(out, orc.pack_over_cols(W, nbits, 32))
+
+
+# ------------------------------------------------------------------ codecs
+def test_e2m1_table():
+    assert list(orc.e2m1_decode(np.arange(8))) == [0, 0.5, 1, 1.5, 2, 3, 4, 6]
+    assert list(orc.e2m1_decode(np.arange(8, 16))[1:]) == [-0.5, -1, -1.5, -2, -3, -4, -6]
+    assert np.signbit(orc.e2m1_decode(8))
+
+
+def test_e2m1_against_torch_fp4_dtype():
+    # torch's packed fp4 dtype decodes the same nibbles (low nibble first), where this torch build converts it
+    if hasattr(torch, "float4_e2m1fn_x2"):
+        b = torch.arange(256, dtype=torch.uint8)
+        try:
+            vals = b.view(torch.float4_e2m1fn_x2).to(torch.float32)
+        except Exception:
+            pytest.skip("torch cannot convert float4_e2m1fn_x2 on this build")
+        vals = vals.numpy().reshape(256, -1)
+        if vals.shape[1] == 2:
+            assert np.array_equal(vals[:, 0], orc.e2m1_decode(np.arange(256) & 15))
+            assert np.array_equal(vals[:, 1], orc.e2m1_decode(np.arange(256) >> 4))
+
+
+def test_e8m0_against_torch():
+    b = torch.arange(255, dtype=torch.uint8)
+    ref = b.view(torch.float8_e8m0fnu).to(torch.float32).numpy().astype(np.float64)
+    mine = orc.e8m0_decode(np.arange(255))
+    # torch returns fp32: 2^-127 is subnormal there but exact
+    assert np.array_equal(mine.astype(np.float32), ref.astype(np.float32))
+    assert np.isnan(orc.e8m0_decode(255))
+    assert orc.e8m0_decode(127) == 1.0 and orc.e8m0_decode(128) == 2.0
+
+
+def test_e4m3_codec_against_torch():
+    b = torch.arange(256, dtype=torch.uint8)
+    ref = b.view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    mine = orc.e4m3fn_decode(np.arange(256))
+    ok = ~np.isnan(ref)
+    assert np.array_equal(mine[ok], ref[ok]) and np.all(np.isnan(mine[~ok]))
+    assert mine[0x7E] == 448.0
+    # encode: random values, exact midpoints and the range ends, against torch's RNE cast
+    rng = np.random.default_rng(1)
+    x = np.concatenate([
+        rng.normal(0, 50, 20000), rng.uniform(-448, 448, 20000), rng.normal(0, 0.01, 5000),
+        [0.0, -0.0, 448.0, -448.0, 2 ** -9, 2 ** -10, 3 * 2 ** -10],
+        (ref[ok][:-1].astype(np.float64) + ref[ok][1:].astype(np.float64))[np.abs(ref[ok][:-1]) < 400] / 2,
+    ]).astype(np.float32)
+    x = np.clip(x, -448, 448)
+    t = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    mine = orc.e4m3fn_encode(x)
+    # +-0 may differ in sign bit handling only when x == -0.0
+    assert np.array_equal(mine, t)
+
+
+def test_round_to_bf16_against_torch():
+    rng = np.random.default_rng(2)
+    x = rng.normal(0, 3, 10000).astype(np.float32)
+    assert np.array_equal(orc.round_to_bf16(x), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+
+
+# ------------------------------------------------------------------ dequant / matmul
+def test_dequantize_closed_forms():
+    q = np.array([[0, 5, 15]], dtype=np.uint8)
+    s = np.array([[0.5]], dtype=np.float32)
+    z = np.array([[7.0]], dtype=np.float32)
+    assert np.array_equal(orc.dequantize(q, None, None, 0), [[0, 5, 15]])
+    assert np.array_equal(orc.dequantize(q, None, z, 1), [[-7, -2, 8]])
+    assert np.array_equal(orc.dequantize(q, None, 7, 1), [[-7, -2, 8]])
+    assert np.array_equal(orc.dequantize(q, s, None, 2), [[0, 2.5, 7.5]])
+    assert np.array_equal(orc.dequantize(q, s, z, 3), [[-3.5, -1, 4]])
+    assert np.array_equal(orc.dequantize(q, s, -z * s, 4), [[-3.5, -1, 4]])  # fma form, z' = -z*s
+
+
+def test_mode4_is_single_rounding():
+    # q*s + z' where the double-rounded fp32 result differs from the fused one
+    q = np.array([[3.0]], dtype=np.float32)
+    s = np.array([[1.0 + 2 ** -23]], dtype=np.float32)
+    z = np.array([[-3.0]], dtype=np.float32)
+    fused = orc.dequantize(q, s, z, 4)[0, 0]
+    assert fused == np.float32(3 * 2.0 ** -23)  # exact: 3*(1+2^-23) - 3
+    assert np.float32(np.float32(q * s) + z)[0, 0] != fused  # q*s rounds to 3+2^-21 first
+
+
+def test_matmul_reduces_to_library_matmul():
+    rng = np.random.default_rng(3)
+    M, K, N, gs = 3, 64, 8, 32
+    x = rng.normal(size=(M, K)).astype(np.float32)
+    q = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    ones = np.ones((K // gs, N), dtype=np.float32)
+    zeros = np.zeros((K // gs, N), dtype=np.float32)
+    ref = x.astype(np.float64) @ q.astype(np.float64)
+    # scales = 1, zeros = 0 in every mode is the plain integer matmul
+    for mode, s, z in [(0, None, None), (1, None, zeros), (2, ones, None), (3, ones, zeros), (4, ones, zeros)]:
+        out = orc.matmul_int(x, q, s, z, None, mode, 0, gs)
+        assert np.allclose(out, ref, rtol=1e-6), mode
+    # a one-hot activation picks out one dequantised row
+    s = rng.uniform(0.5, 2, size=(K // gs, N)).astype(np.float32)
+    z = rng.uniform(0, 15, size=(K // gs, N)).astype(np.float32)
+    onehot = np.zeros((1, K), dtype=np.float32)
+    onehot[0, 37] = 1.0
+    out = orc.matmul_int(onehot, q, s, z, None, 3, 0, gs)
+    assert np.allclose(out[0], (q[37].astype(np.float32) - z[37 // gs]) * s[37 // gs], rtol=1e-6)
+    # channel scaling is linear in each scale
+    sx = rng.uniform(0.5, 2, size=(M, 1)).astype(np.float32)
+    sn = rng.uniform(0.5, 2, size=(N,)).astype(np.float32)
+    base = orc.matmul_int(x, q, None, None, None, 0, 0, gs).astype(np.float64)
+    assert np.allclose(orc.matmul_int(x, q, None, None, sx, 0, 3, gs, scales_n=sn), base * sx * sn, rtol=1e-6)
+    assert np.allclose(orc.matmul_int(x, q, None, None, sx, 0, 2, gs), base * sx, rtol=1e-6)
+    assert np.allclose(orc.matmul_int(x, q, None, None, None, 0, 1, gs, scales_n=sn), base * sn, rtol=1e-6)
+
+
+def test_int_acc_is_exact():
+    rng = np.random.default_rng(4)
+    x = rng.integers(-128, 128, size=(5, 256), dtype=np.int8)
+    w = rng.integers(-128, 128, size=(256, 7), dtype=np.int8)
+    out = orc.matmul_int(x, w, None, None, None, 0, 0, 256, int_acc=True)
+    assert np.array_equal(out, (torch.from_numpy(x).long() @ torch.from_numpy(w).long()).numpy())
+    out = orc.matmul_int(x, w.view(np.uint8) & 15, None, 7, None, 1, 0, 256, int_acc=True)
+    assert np.array_equal(out, x.astype(np.int64) @ ((w.view(np.uint8) & 15).astype(np.int64) - 7))
+
+
+def test_hqq_path_matches_grouped_matmul_and_c_port():
+    rng = np.random.default_rng(5)
+    M, N, K, gs = 2, 24, 256, 128
+    x = rng.normal(size=(M, K)).astype(np.float32)
+    Wq = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    scales = np.abs(rng.normal(0, 0.02, size=(N * K // gs, 1))).astype(np.float32)
+    zeros = rng.uniform(6, 9, size=(N * K // gs, 1)).astype(np.float32)
+    y = orc.hqq_dequant_matmul(x, Wq, scales, zeros, gs)
+    # same thing through the kernel-side layout: [K, N] codes, [K/gs, N] metadata, mode 3
+    y2 = orc.matmul_int(x, Wq.T, scales.reshape(N, -1).T, zeros.reshape(N, -1).T, None, 3, 0, gs)
+    assert np.allclose(y, y2, rtol=1e-4, atol=1e-5)
+    # C port
+    lib = ctypes.CDLL(os.path.join(ROOT, "oracle", "liboracle_c.so"))
+    W = np.zeros((N, K), dtype=np.float32)
+    yc = np.zeros((M, N), dtype=np.float32)
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    lib.orc_hqq_dequantize(p(Wq), p(scales), p(zeros), ctypes.c_int64(N), ctypes.c_int64(K), ctypes.c_int64(gs), p(W), 2)
+    lib.orc_matmul_nt_f32(p(x), p(W), ctypes.c_int64(M), ctypes.c_int64(N), ctypes.c_int64(K), p(yc), 2)
+    assert np.allclose(yc, y, rtol=1e-4, atol=1e-5)
+
+
+def test_matmul_mx_special_cases():
+    rng = np.random.default_rng(6)
+    M, N, K = 3, 5, 64
+    a = rng.integers(0, 16, size=(M, K), dtype=np.uint8)
+    b = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    unit = np.full((M, K // 32), 127, dtype=np.uint8)
+    unit_b = np.full((N, K // 32), 127, dtype=np.uint8)
+    ref = orc.e2m1_decode(a).astype(np.float64) @ orc.e2m1_decode(b).astype(np.float64).T
+    assert np.array_equal(orc.matmul_mx(a, unit, b, unit_b), ref.astype(np.float32))
+    # raising one block scale by one doubles that block's contribution only
+    sa = unit.copy()
+    sa[:, 1] = 128
+    ref2 = ref + orc.e2m1_decode(a[:, 32:]).astype(np.float64) @ orc.e2m1_decode(b[:, 32:]).astype(np.float64).T
+    assert np.array_equal(orc.matmul_mx(a, sa, b, unit_b), ref2.astype(np.float32))
+    assert np.array_equal(orc.unpack_fp4_bytes(np.array([[0x21, 0xF8]], dtype=np.uint8)), [[1, 2, 8, 15]])
+
+
+# ------------------------------------------------------------------ activation quant
+def test_per_token_int8_properties():
+    rng = np.random.default_rng(7)
+    x = rng.normal(size=(6, 128)).astype(np.float32)
+    q, s = orc.scale_activations_per_token(x, True)
+    assert s.shape == (6, 1) and s.dtype == np.float32
+    assert np.allclose(s[:, 0], np.abs(x).max(axis=1) / 127, rtol=1e-6)
+    assert np.abs(q).max() <= 127 and np.all(np.abs(q).max(axis=1) == 127)
+    assert np.all(np.abs(x - q.astype(np.float32) * s) <= s / 2 * (1 + 1e-5))
+    # floor(y + 0.5): halves go up, also for negatives (-0.5 -> 0, -1.5 -> -1)
+    x2 = np.array([[127.0, 0.5, 1.5, -0.5, -1.5, 2.5, -2.5, 0.0]], dtype=np.float32)
+    q2, s2 = orc.scale_activations_per_token(x2, True)
+    assert s2[0, 0] == 1.0 and list(q2[0]) == [127, 1, 2, 0, -1, 3, -2, 0]
+    # all-zero row: scale floor 1e-6
+    q3, s3 = orc.scale_activations_per_token(np.zeros((1, 8), dtype=np.float32), True)
+    assert s3[0, 0] == np.float32(1e-6) and not q3.any()
+
+
+def test_per_token_fp8_against_torch_formula():
+    rng = np.random.default_rng(8)
+    x = (rng.normal(size=(5, 256)) * rng.uniform(0.01, 10, size=(5, 1))).astype(np.float32)
+    q, s = orc.scale_activations_per_token(x, False)
+    t = torch.from_numpy(x)
+    ts = (t.abs().amax(dim=1, keepdim=True) / 448.0).clamp_(min=1e-6)
+    tq = (t / ts).clamp_(-448.0, 448.0).to(torch.float8_e4m3fn)
+    assert np.array_equal(s, ts.numpy())
+    assert np.array_equal(q, tq.view(torch.uint8).numpy())
+
+
+def test_mxfp4_exponent_rule():
+    # exponent = ceil(log2(v)) + 127 for normal v, clamped to [97, 254]
+    v = np.array([1.0, 1.0000001, 2.0, 3.0, 0.75, 0.5, 2.0 ** -40, 0.0, 2.0 ** 127, 3e38], dtype=np.float32)
+    assert list(orc.next_power_of_2_exponent(v)) == [127, 128, 128, 129, 127, 126, 97, 97, 254, 254]
+
+
+def test_mxfp4_exhaustive_binade():
+    # every bf16 value in [1, 2) and [4, 8) (both signs), scaled so that the group maximum fixes
+    # the scale at 1: codes must follow the strict-threshold rule
+    mant = np.arange(128, dtype=np.uint32)
+    vals = []
+    for e in (127, 128, 129):
+        bits = (e << 23) | (mant << 16)
+        vals.append(bits.astype(np.uint32).view(np.float32))
+    vals = np.concatenate(vals)
+    vals = np.concatenate([vals, -vals, [0.0, -0.0, 0.25, -0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 0.1, -0.1]]).astype(np.float32)
+    vals = vals[np.abs(vals) <= 6.0]
+    pad = (-len(vals)) % 31
+    vals = np.concatenate([vals, np.zeros(pad, dtype=np.float32)])
+    groups = vals.reshape(-1, 31)
+    x = np.concatenate([np.full((groups.shape[0], 1), 6.0, dtype=np.float32), groups], axis=1).reshape(1, -1)
+    packed, scales = orc.scale_activations_mxfp4(x)
+    assert np.all(scales[0] == 127) and np.all(scales[1:] == 127) and scales.shape[0] == 32
+    codes = orc.unpack_fp4_bytes(packed)[0]
+    flat = x[0]
+    for v, c in zip(flat, codes):
+        a = abs(float(v))
+        mag = sum(a > t for t in (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0))
+        assert c == (mag if v >= 0 else mag + 8), (v, c)
+    # ties go toward zero; a negative value that rounds to zero keeps the sign bit; -0.0 does not
+    look = {float(v): int(c) for v, c in zip(flat, codes)}
+    assert look[0.25] == 0 and look[0.75] == 1 and look[2.5] == 4 and look[5.0] == 6
+    assert look[-0.25] == 8 and look[float(np.float32(-0.1))] == 8
+    neg_zero = [int(c) for v, c in zip(flat, codes) if v == 0 and np.signbit(v)]
+    assert neg_zero and all(c == 0 for c in neg_zero)
+
+
+def test_mxfp4_scale_and_error_bound():
+    rng = np.random.default_rng(9)
+    x = (rng.normal(size=(40, 256)) * rng.uniform(1e-3, 1e3, size=(40, 1))).astype(np.float32)
+    packed, scales = orc.scale_activations_mxfp4(x)
+    assert packed.shape == (40, 128) and scales.shape == (64, 8)
+    assert np.all(scales[40:] == 127)
+    amax = np.abs(x.reshape(40, 8, 32)).max(axis=2)
+    s = orc.e8m0_decode(scales[:40])
+    assert np.all(s >= amax / 6 * (1 - 1e-6)) and np.all(s / 2 < amax / 6)  # smallest power of two >= amax/6
+    deq = orc.e2m1_decode(orc.unpack_fp4_bytes(packed)).reshape(40, 8, 32) * s[:, :, None]
+    # e2m1 grid spacing is at most 2 (between 4 and 6): error <= 1 * s
+    assert np.all(np.abs(deq - x.reshape(40, 8, 32)) <= s[:, :, None] * (1 + 1e-6))
+
+
+# ------------------------------------------------------------------ weight quantisers
+def test_quantize_mxfp4_weights():
+    rng = np.random.default_rng(10)
+    W = rng.normal(0, 0.02, size=(16, 128)).astype(np.float32)
+    codes, e = orc.quantize_mxfp4_weights(W)
+    assert codes.shape == (16, 128) and e.shape == (16, 4) and codes.max() <= 15
+    s = orc.e8m0_decode(e)
+    amax = np.abs(W.reshape(16, 4, 32)).max(axis=2)
+    assert np.all(s >= amax / 6 * (1 - 1e-6)) and np.all(s / 2 < amax / 6)
+    deq = orc.e2m1_decode(codes).reshape(16, 4, 32) * s[:, :, None]
+    assert np.all(np.abs(deq - W.reshape(16, 4, 32)) <= s[:, :, None] * (1 + 1e-6))
+    assert not np.any(codes == 8)  # -0 is never produced on the weight side
+    # the torch-side quantiser of the product makes the same codes
+    from gemlite_amd.quant_utils import WeightQuantizerMXFP
+
+    q, sc = WeightQuantizerMXFP().quantize_mxfp4(torch.from_numpy(W), index=True)
+    assert np.array_equal(q.view(16, 128).numpy(), codes)
+    assert np.array_equal(sc.view(torch.uint8).view(16, 4).numpy(), e)
+
+
+def test_quantize_per_channel():
+    rng = np.random.default_rng(11)
+    W = rng.normal(0, 0.02, size=(8, 64)).astype(np.float32)
+    q, s = orc.quantize_per_channel(W, True)
+    assert np.all(np.abs(q).max(axis=1) == 127)
+    assert np.all(np.abs(W - q.astype(np.float32) * s) <= s / 2 * (1 + 1e-5))
+    from gemlite_amd.quant_utils import quantize_weights_per_channel
+
+    tq, ts = quantize_weights_per_channel(torch.from_numpy(W), torch.int8)
+    assert np.array_equal(tq.numpy(), q) and np.array_equal(ts.numpy(), s)
+    q8, s8 = orc.quantize_per_channel(W, False)
+    tq8, ts8 = quantize_weights_per_channel(torch.from_numpy(W), torch.float8_e4m3fn)
+    assert np.array_equal(tq8.view(torch.uint8).numpy(), q8) and np.array_equal(ts8.numpy(), s8)
+
+
+# ------------------------------------------------------------------ host logic
+def test_matmul_type_table():
+    # the decision table in the reference's source, including every batch size of the benchmark configs
+    t = orc.get_matmul_type
+    assert [t(m, 4) for m in (1, 2, 4, 5, 8, 16, 63, 64, 4096)] == [
+        "GEMV_REVSPLITK", "GEMV_REVSPLITK", "GEMV_REVSPLITK", "GEMM_SPLITK", "GEMM_SPLITK", "GEMM_SPLITK",
+        "GEMM_SPLITK", "GEMM", "GEMM"]
+    assert [t(m, 8) for m in (1, 2, 3, 16, 64, 512)] == [
+        "GEMV_SPLITK", "GEMV_SPLITK", "GEMM_SPLITK", "GEMM_SPLITK", "GEMM", "GEMM"]
+    assert [t(m, 2) for m in (1, 16, 64, 512)] == ["GEMV_REVSPLITK", "GEMM_SPLITK", "GEMM", "GEMM"]
+    assert [t(m, 4, True) for m in (1, 32, 1024, 8192)] == ["GEMM_SPLITK", "GEMM_SPLITK", "GEMM", "GEMM"]
+
+
+def test_closest_m_table():
+    g = orc.get_closest_m
+    assert [g(m) for m in (0, 1, 2, 3, 5, 9, 17, 24, 25, 33, 48, 49, 65, 97, 129, 250, 1000, 3000, 4096, 5000)] == [
+        1, 1, 2, 4, 8, 16, 24, 24, 32, 48, 48, 64, 96, 128, 192, 256, 1024, 3072, 4096, 4096]
+
+
+def test_select_modes_like_reference_tests():
+    s = orc.select_modes
+    N = 2032
+    assert s(False, 0, None, N, False) == (0, 0)                       # fp16 x fp16  (tests/test_int.py:111-113)
+    assert s(True, N * 31, "tensor", N, False) == (4, 0)               # A16W4 grouped, fma (tests/test_int.py:136-139)
+    assert s(True, N * 31, "tensor", N, False, fma_mode=False) == (3, 0)
+    assert s(True, N, "int", N, False) == (1, 1)                       # int8 x Wn channelwise (tests/test_int.py:161-163)
+    assert s(False, 0, "int", N, True) == (1, 2)                       # dynamic activations only (tests/test_int.py:188-190)
+    assert s(True, N, "int", N, True) == (1, 3)                        # both scaled (tests/test_int.py:216-218)
+    assert s(False, 0, None, N, True) == (0, 2)                        # fp8 x fp8 dynamic (tests/test_int.py:241-243)
+    assert s(True, N, None, N, True) == (0, 3)                         # fp8 both scaled (tests/test_int.py:269-271)
+    assert s(True, N, None, N, False) == (0, 1)                        # weight-only channelwise
+    assert s(True, N * 132, None, N, True, mx=True) == (2, 0)          # micro-scaled formats
