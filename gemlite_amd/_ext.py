@@ -12,7 +12,7 @@ from typing import Optional
 
 import torch
 
-from .dtypes import DType, TORCH_TO_DTYPE
+from .dtypes import DType, TORCH_TO_DTYPE, is_mx_dtype
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgemlite_amd.so")
@@ -216,8 +216,12 @@ def build_matmul_args(
     a.x_stride_m, a.x_stride_k = x.stride(0), x.stride(1)
     a.w_stride_k, a.w_stride_n = W_q.stride(0), W_q.stride(1)
     a.out_stride_m, a.out_stride_n = out.stride(0), out.stride(1)
+    mx = is_mx_dtype(int(input_dtype))
     if has_scales and scales.dim() == 2:
-        a.meta_stride_g, a.meta_stride_n = scales.stride(0), scales.stride(1)
+        if mx:  # micro-scaled formats hand the scales over as the [N, K/group] view
+            a.meta_stride_n, a.meta_stride_g = scales.stride(0), scales.stride(1)
+        else:   # [K/group, N]
+            a.meta_stride_g, a.meta_stride_n = scales.stride(0), scales.stride(1)
     elif has_zeros and zeros.dim() == 2:
         a.meta_stride_g, a.meta_stride_n = zeros.stride(0), zeros.stride(1)
     else:
@@ -242,7 +246,47 @@ def build_matmul_args(
     a.zero_is_scalar = int(has_zeros and zeros.numel() == 1)
     a.sx_dtype = _dt(scales_x, DType.FP32.value)
     a.tile_config = int(tile_config)
+    _check_operand_bounds(a, x, W_q, scales if has_scales else None, zeros if has_zeros else None, scales_x, out, mx)
     return a
+
+
+def _span(t: torch.Tensor) -> int:
+    """Elements addressable from the tensor's first element to the end of its storage."""
+    return t.untyped_storage().nbytes() // t.element_size() - t.storage_offset()
+
+
+def _check_operand_bounds(a, x, W_q, scales, zeros, scales_x, out, mx):
+    """The kernels trust strides: refuse any operand whose last addressed element would fall
+    outside the memory its tensor owns."""
+    def need(*terms):
+        return 1 + sum((n - 1) * abs(s) for n, s in terms if n > 0)
+
+    def check(name, t, required):
+        if t is not None and required > _span(t):
+            raise ValueError(
+                f"{name}: kernel would address {required} elements but the tensor spans {_span(t)} "
+                f"(shape {tuple(t.shape)}, strides {t.stride()})"
+            )
+
+    M, N, K, e = a.M, a.N, a.K, a.elements_per_sample
+    kx = K // 2 if a.input_dtype == DType.MXFP4.value else K
+    check("x", x, need((M, a.x_stride_m), (kx, a.x_stride_k)))
+    check("W_q", W_q, need((K // e, a.w_stride_k), (N, a.w_stride_n)))
+    check("out", out, need((M, a.out_stride_m), (N, a.out_stride_n)))
+    wgm, csm = a.W_group_mode, a.channel_scale_mode
+    groups = K // 32 if mx else (K // a.group_size if a.group_size > 0 else 1)
+    if scales is not None:
+        if mx or wgm >= 2:
+            check("scales", scales, need((groups, a.meta_stride_g), (N, a.meta_stride_n)))
+        if csm in (1, 3):
+            check("scales", scales, N)
+    if zeros is not None and not a.zero_is_scalar and wgm in (1, 3, 4):
+        check("zeros", zeros, need((groups, a.meta_stride_g), (N, a.meta_stride_n)))
+    if scales_x is not None:
+        if csm == 4:
+            check("scales_x", scales_x, need((M, a.sx_stride_m), (K // 32, a.sx_stride_g)))
+        elif csm in (2, 3):
+            check("scales_x", scales_x, need((M, a.sx_stride_m)))
 
 
 def matmul(args: MatmulArgs, device: torch.device):

@@ -33,6 +33,7 @@ constexpr int kThreads = kWaves * kWave;
 constexpr int kTileN = 64;       // output columns per workgroup
 constexpr int kBatch = 8;        // 128-bit loads in flight per lane
 constexpr int kSlabRows = kWaves * kBatch * 4;  // 128: granularity of RW
+constexpr int64_t kCounterBytes = 256 * 1024;   // fixed ticket-counter region at the start of the workspace
 
 struct GemvArgs {
     const uint32_t* w;
@@ -297,14 +298,16 @@ __global__ __launch_bounds__(kThreads) void gemv_packed_kernel(GemvArgs a) {
                 __hip_atomic_store(a.partials + ((size_t)split * a.Mp + (m0 + m)) * a.N + n_out, total[t],
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __threadfence();
+        // The partials were stored with agent scope (written through to the point every XCD reads
+        // from), so waiting for their acknowledgement orders them before the ticket; a full release
+        // fence would also write back the whole L2 and is far too expensive here.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0)
-            ticket = __hip_atomic_fetch_add(a.counters + blockIdx.y * a.tiles + tile, 1u, __ATOMIC_ACQ_REL,
+            ticket = __hip_atomic_fetch_add(a.counters + blockIdx.y * a.tiles + tile, 1u, __ATOMIC_RELAXED,
                                             __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (ticket != (unsigned)(a.S - 1)) return;
-        __threadfence();
 #pragma unroll
         for (int t = 0; t < (MT + kWaves - 1) / kWaves; ++t) {
             const int m = wv + t * kWaves;
@@ -382,6 +385,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g) {
         if (per_wg == 1) return false;
     }
     g.S = ceil_div(g.R, g.RW);
+    if (g.S > 1 && (int64_t)g.tiles * g.mchunks * 4 > kCounterBytes) return false;
     const int nl = g.RW / kWaves / 4;
     int fl = 1;
     if (g.gr >= 4 && g.gr % 4 == 0) {
@@ -461,9 +465,7 @@ int64_t gemv_packed_workspace_bytes(const gla_matmul_args& p) {
     Geometry g;
     if (!geometry(p, g)) return 0;
     if (g.S <= 1) return 0;
-    const int64_t counters = (int64_t)g.tiles * g.mchunks * 4;
-    const int64_t counters_pad = (counters + 255) / 256 * 256;
-    return counters_pad + (int64_t)g.S * g.Mp * p.N * 4;
+    return kCounterBytes + (int64_t)g.S * g.Mp * p.N * 4;
 }
 
 int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
@@ -482,9 +484,8 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
                       (unsigned long long)p.workspace_bytes);
             return GLA_ERR_WORKSPACE_TOO_SMALL;
         }
-        const int64_t counters = (int64_t)g.tiles * g.mchunks * 4;
         a.counters = (unsigned*)p.workspace;
-        a.partials = (float*)((char*)p.workspace + (counters + 255) / 256 * 256);
+        a.partials = (float*)((char*)p.workspace + kCounterBytes);
     }
     a.M = p.M; a.N = p.N; a.K = p.K; a.R = g.R; a.RW = g.RW; a.S = g.S; a.tiles = g.tiles; a.Mp = g.Mp;
     a.gr = g.gr; a.G = g.G; a.GW = g.GW; a.FL = g.FL;

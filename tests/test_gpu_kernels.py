@@ -226,7 +226,10 @@ def test_a8w8_dynamic(device, fp8):
     N, K = 1032, 2048
     W = gen_x(N, K, torch.bfloat16, seed=5, std=0.02)
     proc = helper.A8W8_FP8_dynamic(device=device) if fp8 else helper.A8W8_INT8_dynamic(device=device)
-    layer = proc.from_weights(W)
+    # weights are quantised once on the host (CPU torch), then handed over pre-quantised
+    W_q_cpu, s_cpu = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+    proc.dtype = torch.bfloat16
+    layer = proc.from_weights(W_q_cpu, scales=s_cpu)
     assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 3) and layer.scales.dtype == torch.float32
     assert layer.W_q.stride() == (1, K)
     # the weight codes are the oracle's

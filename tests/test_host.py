@@ -255,3 +255,32 @@ def test_forward_requires_gpu_and_library():
         l(torch.zeros(1, 256).half())
     with pytest.raises(RuntimeError, match="not found"):
         _ext.load_library(os.path.join(ROOT, "no_such_dir", "libgemlite_amd.so"))
+
+
+def test_operand_bounds_are_checked_on_the_host():
+    # strides that would walk outside a tensor are refused before any launch
+    N, K, M = 64, 256, 2
+    x = torch.zeros(M, K, dtype=torch.float16)
+    W = torch.zeros(K // 8, N, dtype=torch.int32)
+    s = torch.zeros(K // 128, N, dtype=torch.float16)
+    out = torch.zeros(M, N, dtype=torch.float16)
+    kw = dict(W_nbits=4, group_size=128, unpack_mask=15, elements_per_sample=8, input_dtype=1, output_dtype=1,
+              acc_dtype=0, meta_dtype=1, channel_scale_mode=0, W_group_mode=4, data_contiguous=1)
+    _ext.build_matmul_args(x, W, s, s, None, out, **kw)  # consistent: accepted
+    with pytest.raises(ValueError, match="scales"):
+        _ext.build_matmul_args(x, W, s.t(), s, None, out, **kw)   # [N, G] view read as [G, N]
+    with pytest.raises(ValueError, match="W_q"):
+        _ext.build_matmul_args(x, W[: K // 16], s, s, None, out, **dict(kw, elements_per_sample=16))
+    with pytest.raises(ValueError, match="out"):
+        _ext.build_matmul_args(x, W, s, s, None, out[:1], **kw)
+    # micro-scaled layers hand their scales over as the [N, K/32] view of a [K/32, N] buffer
+    codes = torch.randint(0, 16, (N, K)).to(torch.uint8)
+    e8 = torch.randint(110, 130, (N, K // 32)).to(torch.uint8)
+    l = gemlite_amd.helper.A4W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16).from_weights(codes, scales=e8)
+    m = l.get_meta_args()
+    a = _ext.build_matmul_args(
+        torch.zeros(M, K // 2, dtype=torch.uint8), l.W_q, l.scales, l.zeros, torch.zeros(32, K // 32, dtype=torch.uint8),
+        torch.zeros(M, N, dtype=torch.bfloat16), W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+        elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
+        channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11])
+    assert (a.meta_stride_g, a.meta_stride_n) == (N, 1) and (a.w_stride_k, a.w_stride_n) == (1, K // 2)
