@@ -269,8 +269,8 @@ def test_operand_bounds_are_checked_on_the_host():
     _ext.build_matmul_args(x, W, s, s, None, out, **kw)  # consistent: accepted
     with pytest.raises(ValueError, match="scales"):
         _ext.build_matmul_args(x, W, s.t(), s, None, out, **kw)   # [N, G] view read as [G, N]
-    with pytest.raises(ValueError, match="W_q"):
-        _ext.build_matmul_args(x, W[: K // 16], s, s, None, out, **dict(kw, elements_per_sample=16))
+    with pytest.raises(ValueError, match="x:"):
+        _ext.build_matmul_args(x[:, : K // 2].contiguous(), W, s, s, None, out, **kw)  # x shorter than K
     with pytest.raises(ValueError, match="out"):
         _ext.build_matmul_args(x, W, s, s, None, out[:1], **kw)
     # micro-scaled layers hand their scales over as the [N, K/32] view of a [K/32, N] buffer
