@@ -272,7 +272,7 @@ def test_operand_bounds_are_checked_on_the_host():
     with pytest.raises(ValueError, match="x:"):
         _ext.build_matmul_args(x[:, : K // 2].contiguous(), W, s, s, None, out, **kw)  # x shorter than K
     with pytest.raises(ValueError, match="out"):
-        _ext.build_matmul_args(x, W, s, s, None, out[:1], **kw)
+        _ext.build_matmul_args(x, W, s, s, None, out[:1].clone(), **kw)
     # micro-scaled layers hand their scales over as the [N, K/32] view of a [K/32, N] buffer
     codes = torch.randint(0, 16, (N, K)).to(torch.uint8)
     e8 = torch.randint(110, 130, (N, K // 32)).to(torch.uint8)
