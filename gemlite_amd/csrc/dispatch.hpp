@@ -9,7 +9,7 @@ namespace gla {
 int launch_generic(const gla_matmul_args& p, hipStream_t stream);
 
 // ---- streaming GEMV on 32-bit packed words, N fastest (gemv_packed.hip) ----
-// tile_config (when >= 0) = number of 128-word-row slabs each workgroup owns.
+// tile_config (when >= 1000) = waves per workgroup * 1000 + load batches per wave.
 bool gemv_packed_eligible(const gla_matmul_args& p);
 int64_t gemv_packed_workspace_bytes(const gla_matmul_args& p);
 int gemv_packed_default_config(const gla_matmul_args& p);

@@ -1,26 +1,27 @@
-// Streaming GEMV for 32-bit packed weight words stored [K/e, N], N fastest.
+// Streaming small-batch matmul (M <= 16 per pass) for 32-bit packed weight words stored
+// [K/e, N], N fastest: the decode path.
 //
-// Takes the place of the reference's GEMV / RevSplit-K kernels for packed data
-// (reference: gemlite/triton_kernels/gemv_revsplitK_kernels.py:248-443 and
-// gemlite/triton_kernels/gemv_kernels.py:245-426), with a different
-// decomposition:
+// Takes the place of the reference's GEMV / RevSplit-K kernels and of its split-K GEMM at
+// small batch (reference: gemlite/triton_kernels/gemv_revsplitK_kernels.py:248-443,
+// gemlite/triton_kernels/gemv_kernels.py:245-426,
+// gemlite/triton_kernels/gemm_splitK_kernels.py:300-523) with a different decomposition:
 //
-//  * A workgroup (4 waves) owns 64 output columns and a slab of RW word rows.
-//    In every wave a lane owns 4 adjacent columns (one 128-bit load) and the
-//    four 16-lane quarters own four consecutive word rows, so one wave load
-//    covers 4 rows x 256 contiguous bytes.
-//  * Codes are never dequantised one by one.  Within a quantisation group the
-//    lane accumulates dq = sum_k x_k * (OFF + q_k) with v_dot2 on fp16/bf16
-//    pairs built by OR-ing the code bits into the mantissa of the constant
-//    OFF (1024 in fp16, 128 in bf16), and sx = sum_k x_k.  At the group end
-//    acc += s * dq + zz * sx, where (s, zz) folds the scale, the zero point
-//    and -OFF*s in fp32.  All five dequant modes reduce to a choice of (s, zz).
-//  * The activation slab, its per-row sums and the (s, zz) table of the slab
-//    are staged in LDS once per workgroup, so every global load of the kernel
-//    is issued up front.
-//  * The K reduction is deterministic: quarters by wave shuffles, waves through
-//    LDS, slabs by fp32 partials in a workspace that the last-arriving
-//    workgroup of a column tile sums in slab order (no float atomics).
+//  * A workgroup (4 waves) owns 64 output columns and a slab of RW word rows; its waves split
+//    the slab.  A lane owns 4 adjacent columns (one 128-bit load) and the four 16-lane quarters
+//    own four consecutive "super rows" (8 codes along K, i.e. one word for <= 4-bit codes, two
+//    words for 8-bit codes), so a wave load covers 4 rows x 256 contiguous bytes.
+//  * The lane's word is exactly one B operand of v_mfma_f32_16x16x32 (8 K-values of one
+//    column).  Codes are turned into fp16/bf16 numbers OFF+q by OR-ing their bits into the
+//    mantissa of the constant OFF (1024 in fp16, 128 in bf16): two codes per VALU op, in the
+//    pair order (j, j + e/2).  The activation rows are staged in LDS in the same pair order
+//    and are the A operand (up to 16 rows, so every batch size up to 16 costs the same).
+//  * Scales and zero points are applied per quantisation group, not per weight: with
+//    C = sum_k x_k (OFF + q_k) and SX = sum_k x_k (one more MFMA against a B of ones) the
+//    group adds s*C + zz*SX, where (s, zz) folds scale, zero point and -OFF*s in fp32.  All
+//    five dequant modes are a choice of (s, zz), staged per slab in LDS.
+//  * The K reduction is deterministic: k-blocks inside the MFMA, waves through LDS, slabs by
+//    fp32 partials in a workspace that the last-arriving workgroup of a column tile sums in
+//    slab order (no float atomics).
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -28,14 +29,23 @@ namespace gla {
 
 namespace {
 
-constexpr int kWaves = 4;        // waves per workgroup
-constexpr int kThreads = kWaves * kWave;
-constexpr int kTileN = 64;       // output columns per workgroup
-constexpr int kBatch = 8;        // 128-bit loads in flight per lane
-constexpr int kSlabRows = kWaves * kBatch * 4;  // 128: granularity of RW
-constexpr int64_t kCounterBytes = 256 * 1024;   // fixed ticket-counter region at the start of the workspace
+constexpr int kTileN = 64;  // output columns per workgroup
+constexpr int kBatch = 8;   // 128-bit loads in flight per lane
+constexpr int64_t kCounterBytes = 256 * 1024;  // fixed ticket-counter region at the start of the workspace
+
+#ifndef GLA_EXP
+#define GLA_EXP 0  // lab-only experiment switches; 0 in every product build
+#endif
+#ifdef GLA_TRACE
+#define GLA_STAMP(i) do { if (threadIdx.x == 0) a.trace[((size_t)blockIdx.x) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define GLA_STAMP(i) do { } while (0)
+#endif
 
 struct GemvArgs {
+#ifdef GLA_TRACE
+    long long* trace;
+#endif
     const uint32_t* w;
     const void* x;
     const void* scales;
@@ -45,15 +55,18 @@ struct GemvArgs {
     float* partials;
     unsigned* counters;
     int M, N, K;
-    int R;        // word rows = K / E
-    int RW;       // word rows per workgroup (multiple of kSlabRows)
-    int S;        // number of slabs along K
-    int tiles;    // column tiles
-    int Mp;       // M rounded up to the row-tile
-    int gr;       // word rows per quantisation group (>= 1)
-    int G;        // number of groups along K
-    int GW;       // (s, zz) table rows staged per workgroup
-    int FL;       // loads per flush
+    int R;      // word rows = K / E
+    int RW;     // word rows per workgroup
+    int S;      // number of slabs along K
+    int tiles;  // column tiles
+    int Mp;     // M rounded up to the row tile
+    int gr;     // word rows per quantisation group
+    int G;      // number of groups along K
+    int GW;     // (s, zz) table rows staged per workgroup
+    int FL;     // wave iterations per flush
+    int waves;  // waves per workgroup (4, 8 or 16)
+    int nfb;      // direct variant: flush blocks per batch of loads
+    int fl_log2;  // log2(FL)
     int wgm, csm, meta_dt, z_dt, z_scalar, out_dt, sx_dt;
     int64_t wsk, xsm, osm, msg, sxm;
 };
@@ -63,238 +76,108 @@ struct Magic;
 template <>
 struct Magic<false> {
     static constexpr uint32_t bits = 0x64006400u;  // fp16 1024.0 twice
+    static constexpr uint32_t ones = 0x3c003c00u;  // fp16 1.0 twice
     static constexpr float off = 1024.0f;
 };
 template <>
 struct Magic<true> {
     static constexpr uint32_t bits = 0x43004300u;  // bf16 128.0 twice
+    static constexpr uint32_t ones = 0x3f803f80u;  // bf16 1.0 twice
     static constexpr float off = 128.0f;
 };
 
 template <bool BF16>
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+__device__ __forceinline__ float4_t mfma16(const uint4& a, const uint4& b, float4_t c) {
     if constexpr (BF16) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c,
-                                               false);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                       c, 0, 0, 0);
     } else {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c,
+                                                      0, 0, 0);
     }
 }
 
-__device__ __forceinline__ float elem16_to_float(uint16_t v, bool bf16) {
-    return bf16 ? bf16_bits_to_float(v) : half_bits_to_float(v);
+__device__ __forceinline__ float meta_to_float(uint16_t v, int dt) {
+    return dt == GLA_DT_BF16 ? bf16_bits_to_float(v) : half_bits_to_float(v);
 }
 
-// BITS: code width.  BF16: activation type.  MT: rows of x per workgroup.
-// F32: convert codes and activations to fp32 and use FMAs (8-bit codes with
-// bf16 activations, where OFF + q is not exact in bf16).
-template <int BITS, bool BF16, int MT, bool F32>
-__global__ __launch_bounds__(kThreads) void gemv_packed_kernel(GemvArgs a) {
-    constexpr int E = 32 / BITS;       // codes per word
-    constexpr int XW = F32 ? E : E / 2;  // 32-bit LDS words per staged activation row
-    constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
-    constexpr float OFF = F32 ? 0.0f : Magic<BF16>::off;
+__device__ __forceinline__ float2 fold_meta(float s, float z, int wgm, float OFF) {
+    float zz;
+    switch (wgm) {
+        case GLA_WGM_SHIFT: zz = -z - OFF; break;
+        case GLA_WGM_SCALE: zz = -OFF * s; break;
+        case GLA_WGM_SHIFT_SCALE: zz = -(z + OFF) * s; break;
+        case GLA_WGM_FMA: zz = __builtin_fmaf(-OFF, s, z); break;
+        default: zz = -OFF; break;
+    }
+    return make_float2(s, zz);
+}
 
-    extern __shared__ __align__(16) unsigned char smem[];
-    uint32_t* xs = (uint32_t*)smem;                        // [MT][RW][XW]
-    float* rs = (float*)(xs + (size_t)MT * a.RW * XW);       // [MT][RW]
-    float2* mt = (float2*)(rs + (size_t)MT * a.RW);          // [GW][64]
-    float* red = (float*)(mt + (size_t)a.GW * kTileN);       // [kWaves][MT][64]
-    __shared__ unsigned ticket;
+// Geometry shared by kernel and host: per code width, a "super row" is the run of word rows
+// that holds the 8..32 K-values one lane feeds to the MFMAs of one wave iteration.
+template <int BITS>
+struct Shape {
+    static constexpr int E = 32 / BITS;             // codes per word
+    static constexpr int LW = (E < 8) ? 8 / E : 1;  // word rows per super row (2 for 8-bit codes)
+    static constexpr int KPS = E * LW;              // K-values per super row (8, 16 or 32)
+    static constexpr int T = KPS / 8;               // MFMA K-steps per super row
+};
 
+// (w & mask) | magic.  Callers keep `mask` and `magic` in registers (made opaque to constant
+// folding) so that the compiler can select the single-instruction v_and_or_b32, which takes no
+// literal operands on this target.  Plain C on purpose: an inline-asm VALU op is invisible to the
+// compiler's MFMA hazard tracking.
+__device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t magic) {
+    return (w & mask) | magic;
+}
+
+__device__ __forceinline__ uint32_t pick(const uint4& v, int j) {
+    return j == 0 ? v.x : (j == 1 ? v.y : (j == 2 ? v.z : v.w));
+}
+
+// Shared end of both kernels: sum the waves of the workgroup through LDS, combine the K slabs
+// (last-arriving workgroup of a column tile sums the partials in slab order), apply the channel
+// scales and store.  Lane (cg, kb) holds rows 4*kb + i of columns 4*cg + j in acc[j][i].
+template <int RT, int kWaves, int RI>
+__device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI], float* red, unsigned& ticket,
+                                          int tile, int split, int m0, int n0) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
-    const int cg = lane & 15, rg = lane >> 4;
-    const int tile = blockIdx.x % a.tiles;
-    const int split = blockIdx.x / a.tiles;
-    const int m0 = blockIdx.y * MT;
-    const int n0 = tile * kTileN;
-    const int r0 = split * a.RW;
-    const int RWW = a.RW / kWaves;
-    const int nl = RWW / 4;  // loads per lane (multiple of kBatch)
-
-    // ---- weight stream: first batch of loads goes out before anything else
-    int col = n0 + cg * 4;
-    if (col > a.N - 4) col = a.N - 4;  // clamped lanes are never stored
-    const uint32_t* wbase = a.w + col;
-    const int lrow0 = wv * RWW + rg;  // local row of load 0
-    uint4 buf[kBatch];
+    const int cg = lane & 15, kb = lane >> 4;
+    GLA_STAMP(2);
+    // ---- reduce the waves: lane (cg, kb) holds rows 4*kb + i of columns 4*cg + j
+    if (RT == 16 || kb == 0) {
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-        int row = r0 + lrow0 + 4 * u;
-        if (row > a.R - 1) row = a.R - 1;  // activation rows there are staged as zeros
-        buf[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
-    }
-
-    // ---- stage the activation slab (permuted for the pair extraction) and row sums
-    for (int idx = tid; idx < MT * a.RW; idx += kThreads) {
-        const int m = idx / a.RW, rl = idx - m * a.RW;
-        const int row = r0 + rl;
-        uint32_t* dst = xs + (size_t)idx * XW;
-        float sum = 0.0f;
-        if (row < a.R && (m0 + m) < a.M) {
-            const uint16_t* src = (const uint16_t*)a.x + (int64_t)(m0 + m) * a.xsm + (int64_t)row * E;
-            uint16_t v[E];
-            if constexpr (E == 4) {
-                *(uint2*)v = *(const uint2*)src;
-            } else {
-#pragma unroll
-                for (int q = 0; q < E / 8; ++q) ((uint4*)v)[q] = ((const uint4*)src)[q];
-            }
-#pragma unroll
-            for (int j = 0; j < E; ++j) sum += elem16_to_float(v[j], BF16);
-            if constexpr (F32) {
-#pragma unroll
-                for (int j = 0; j < E; ++j) dst[j] = __builtin_bit_cast(uint32_t, elem16_to_float(v[j], BF16));
-            } else {
-#pragma unroll
-                for (int j = 0; j < E / 2; ++j) dst[j] = (uint32_t)v[j] | ((uint32_t)v[j + E / 2] << 16);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < XW; ++j) dst[j] = 0u;
+        for (int i = 0; i < RI; ++i) {
+            const int m = 4 * kb + i;
+            *(float4*)(red + ((size_t)wv * RT + m) * kTileN + cg * 4) =
+                make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
         }
-        rs[idx] = sum;
-    }
-
-    // ---- stage the (s, zz) table of this slab
-    const int g0 = r0 / a.gr;
-    for (int idx = tid; idx < a.GW * kTileN; idx += kThreads) {
-        const int gl = idx / kTileN, c = idx - gl * kTileN;
-        int g = g0 + gl;
-        if (g > a.G - 1) g = a.G - 1;
-        int n = n0 + c;
-        if (n > a.N - 1) n = a.N - 1;
-        float s = 1.0f, z = 0.0f;
-        if (a.wgm >= GLA_WGM_SCALE) s = load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + n);
-        if (a.wgm == GLA_WGM_SHIFT || a.wgm >= GLA_WGM_SHIFT_SCALE)
-            z = a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0) : load_as_float(a.zeros, a.z_dt, (int64_t)g * a.msg + n);
-        float zz;
-        switch (a.wgm) {
-            case GLA_WGM_SHIFT: zz = -z - OFF; break;
-            case GLA_WGM_SCALE: zz = -OFF * s; break;
-            case GLA_WGM_SHIFT_SCALE: zz = -(z + OFF) * s; break;
-            case GLA_WGM_FMA: zz = __builtin_fmaf(-OFF, s, z); break;
-            default: zz = -OFF; break;
-        }
-        mt[idx] = make_float2(s, zz);
     }
     __syncthreads();
 
-    // ---- main loop
-    float acc[4][MT], dq[4][MT], sx[MT];
+    constexpr int NT = (RT + kWaves - 1) / kWaves;  // output rows per thread
+    const int n_out = n0 + lane;
+    const bool col_ok = n_out < a.N;
+    float total[NT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        sx[m] = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) { acc[c][m] = 0.0f; dq[c][m] = 0.0f; }
-    }
-
-    for (int ib = 0; ib < nl; ib += kBatch) {
-        uint4 cur[kBatch];
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) cur[u] = buf[u];
-        if (ib + kBatch < nl) {
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                int row = r0 + lrow0 + 4 * (ib + kBatch + u);
-                if (row > a.R - 1) row = a.R - 1;
-                buf[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const int i = ib + u;
-            const int rl = lrow0 + 4 * i;
-            uint32_t xv[MT][XW];
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const uint32_t* src = xs + ((size_t)m * a.RW + rl) * XW;
-                if constexpr (XW == 2) {
-                    *(uint2*)xv[m] = *(const uint2*)src;
-                } else {
-#pragma unroll
-                    for (int q = 0; q < XW / 4; ++q) ((uint4*)xv[m])[q] = ((const uint4*)src)[q];
-                }
-                sx[m] += rs[m * a.RW + rl];
-            }
-            const uint32_t wq[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if constexpr (F32) {
-#pragma unroll
-                    for (int j = 0; j < E; ++j) {
-                        const float q = (float)((wq[c] >> (j * BITS)) & ((1u << BITS) - 1u));
-#pragma unroll
-                        for (int m = 0; m < MT; ++m)
-                            dq[c][m] = __builtin_fmaf(q, __builtin_bit_cast(float, xv[m][j]), dq[c][m]);
-                    }
-                } else {
-#pragma unroll
-                    for (int j = 0; j < E / 2; ++j) {
-                        const uint32_t t = ((wq[c] >> (j * BITS)) & kPairMask) | Magic<BF16>::bits;
-#pragma unroll
-                        for (int m = 0; m < MT; ++m) dq[c][m] = dot2<BF16>(t, xv[m][j], dq[c][m]);
-                    }
-                }
-            }
-            if ((i + 1) % a.FL == 0) {
-                int gl = (r0 + rl) / a.gr - g0;
-                if (gl > a.GW - 1) gl = a.GW - 1;
-                const float2* mrow = mt + gl * kTileN + cg * 4;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float2 sz = mrow[c];
-#pragma unroll
-                    for (int m = 0; m < MT; ++m) {
-                        acc[c][m] = __builtin_fmaf(sz.x, dq[c][m], __builtin_fmaf(sz.y, sx[m], acc[c][m]));
-                        dq[c][m] = 0.0f;
-                    }
-                }
-#pragma unroll
-                for (int m = 0; m < MT; ++m) sx[m] = 0.0f;
-            }
-        }
-    }
-
-    // ---- reduce the four row quarters of each wave, then the waves
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-#pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            float v = acc[c][m];
-            v += wave_xor(v, 16);
-            v += wave_xor(v, 32);
-            acc[c][m] = v;
-        }
-    if (rg == 0) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-            *(float4*)(red + ((size_t)wv * MT + m) * kTileN + cg * 4) =
-                make_float4(acc[0][m], acc[1][m], acc[2][m], acc[3][m]);
-    }
-    __syncthreads();
-
-    const int n_out = n0 + (tid & 63);
-    float total[(MT + kWaves - 1) / kWaves];
-#pragma unroll
-    for (int t = 0; t < (MT + kWaves - 1) / kWaves; ++t) {
+    for (int t = 0; t < NT; ++t) {
         const int m = wv + t * kWaves;
         float v = 0.0f;
-        if (m < MT) {
+        if (m < RT) {
 #pragma unroll
-            for (int w2 = 0; w2 < kWaves; ++w2) v += red[((size_t)w2 * MT + m) * kTileN + (tid & 63)];
+            for (int w2 = 0; w2 < kWaves; ++w2) v += red[((size_t)w2 * RT + m) * kTileN + lane];
         }
         total[t] = v;
     }
 
-    const bool col_ok = n_out < a.N;
+    GLA_STAMP(3);
     if (a.S > 1) {
         // publish this slab's partial, then take a ticket; the last slab to arrive sums all
 #pragma unroll
-        for (int t = 0; t < (MT + kWaves - 1) / kWaves; ++t) {
+        for (int t = 0; t < NT; ++t) {
             const int m = wv + t * kWaves;
-            if (m < MT && col_ok)
+            if (m < RT && col_ok)
                 __hip_atomic_store(a.partials + ((size_t)split * a.Mp + (m0 + m)) * a.N + n_out, total[t],
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -307,15 +190,27 @@ __global__ __launch_bounds__(kThreads) void gemv_packed_kernel(GemvArgs a) {
             ticket = __hip_atomic_fetch_add(a.counters + blockIdx.y * a.tiles + tile, 1u, __ATOMIC_RELAXED,
                                             __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
+        GLA_STAMP(4);
         if (ticket != (unsigned)(a.S - 1)) return;
 #pragma unroll
-        for (int t = 0; t < (MT + kWaves - 1) / kWaves; ++t) {
+        for (int t = 0; t < NT; ++t) {
             const int m = wv + t * kWaves;
             float v = 0.0f;
-            if (m < MT && col_ok) {
-                for (int s = 0; s < a.S; ++s)
-                    v += __hip_atomic_load(a.partials + ((size_t)s * a.Mp + (m0 + m)) * a.N + n_out, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
+            if (m < RT && col_ok) {
+                const float* p = a.partials + (size_t)(m0 + m) * a.N + n_out;
+                const size_t stride = (size_t)a.Mp * a.N;
+                int s = 0;
+                for (; s + 8 <= a.S; s += 8) {  // loads of a batch are independent; the sum keeps slab order
+                    float q[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        q[u] = __hip_atomic_load(p + (size_t)(s + u) * stride, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) v += q[u];
+                }
+                for (; s < a.S; ++s)
+                    v += __hip_atomic_load(p + (size_t)s * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             total[t] = v;
         }
@@ -326,9 +221,9 @@ __global__ __launch_bounds__(kThreads) void gemv_packed_kernel(GemvArgs a) {
 
     // ---- epilogue: channel scales, cast, store
 #pragma unroll
-    for (int t = 0; t < (MT + kWaves - 1) / kWaves; ++t) {
+    for (int t = 0; t < NT; ++t) {
         const int m = wv + t * kWaves;
-        if (m >= MT || !col_ok || (m0 + m) >= a.M) continue;
+        if (m >= RT || !col_ok || (m0 + m) >= a.M) continue;
         float v = total[t];
         if (a.csm == GLA_CSM_WEIGHT) {
             v *= load_as_float(a.scales, a.meta_dt, n_out);
@@ -340,86 +235,616 @@ __global__ __launch_bounds__(kThreads) void gemv_packed_kernel(GemvArgs a) {
         }
         store_from_float(a.out, a.out_dt, (int64_t)(m0 + m) * a.osm + n_out, v);
     }
+    GLA_STAMP(5);
 }
 
-int row_tile(int M) { return M >= 8 ? 8 : (M >= 3 ? 4 : (M == 2 ? 2 : 1)); }
+// BITS: code width.  BF16: activation type.  RT: rows of x per pass (1, 2, 4 or 16).
+// kWaves: waves per workgroup; 16 lets one workgroup own all of K with every load in flight at once.
+template <int BITS, bool BF16, int RT, int kWaves>
+__global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
+    constexpr int kThreads = kWaves * kWave;
+    using SH = Shape<BITS>;
+    constexpr int E = SH::E, LW = SH::LW, KPS = SH::KPS, T = SH::T;
+    constexpr int RI = RT < 4 ? RT : 4;  // accumulator rows a lane folds
+    constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
+    constexpr float OFF = Magic<BF16>::off;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int SRW = a.RW / LW;                          // super rows per workgroup
+    uint4* xs = (uint4*)smem;                           // [SRW][RT][T] A-operand chunks
+    float2* mt = (float2*)(xs + (size_t)SRW * RT * T);  // [GW][64] (s, zz)
+    float* red = (float*)(mt + (size_t)a.GW * kTileN);  // [kWaves][RT][64]
+    __shared__ unsigned ticket;
+
+    GLA_STAMP(0);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wv = tid >> 6;
+    const int cg = lane & 15, kb = lane >> 4;
+    const int tile = blockIdx.x % a.tiles;
+    const int split = blockIdx.x / a.tiles;
+    const int m0 = blockIdx.y * RT;
+    const int n0 = tile * kTileN;
+    const int r0 = split * a.RW;
+    const int SRWW = SRW / kWaves;  // super rows per wave
+    const int nit = SRWW / 4;       // wave iterations (multiple of kBatch / LW)
+
+    // ---- phase A: small loads first (activation chunk and metadata of the first staging pass)
+    const int x_items = SRW * RT;
+    const int sr_a = tid / RT, m_a = tid - sr_a * RT;
+    uint4 xraw[T];
+    const bool x_first = tid < x_items;
+    bool x_valid = false;
+    {
+        // unconditional, clamped load: validity is applied when the chunk is written to LDS
+        int row = r0 + sr_a * LW;
+        int mrow = m0 + m_a;
+        x_valid = x_first && row < a.R && mrow < a.M;
+        if (row > a.R - LW) row = a.R - LW;
+        if (mrow > a.M - 1) mrow = a.M - 1;
+        const uint4* src = (const uint4*)((const uint16_t*)a.x + (int64_t)mrow * a.xsm + (int64_t)row * E);
+#pragma unroll
+        for (int t = 0; t < T; ++t) xraw[t] = src[t];
+    }
+    const int g0 = r0 / a.gr;
+    const bool fast_meta = (a.meta_dt == GLA_DT_FP16 || a.meta_dt == GLA_DT_BF16) && !a.z_scalar &&
+                           (a.z_dt == a.meta_dt) && a.wgm >= GLA_WGM_SHIFT_SCALE;
+    uint2 sraw = make_uint2(0, 0), zraw = make_uint2(0, 0);
+    const int gl_a = tid >> 4, c4_a = (tid & 15) * 4;
+    const bool meta_first = fast_meta && gl_a < a.GW;
+    if (fast_meta) {  // uniform branch; lanes past the table load a clamped row and drop it
+        int g = g0 + gl_a;
+        if (g > a.G - 1) g = a.G - 1;
+        int n = n0 + c4_a;
+        if (n > a.N - 4) n = a.N - 4;
+        sraw = *(const uint2*)((const uint16_t*)a.scales + (int64_t)g * a.msg + n);
+        zraw = *(const uint2*)((const uint16_t*)a.zeros + (int64_t)g * a.msg + n);
+    }
+
+    // ---- phase B: first batch of the weight stream
+    int col = n0 + cg * 4;
+    if (col > a.N - 4) col = a.N - 4;  // clamped lanes are never stored
+    const uint32_t* wbase = a.w + col;
+    const int lsr0 = wv * SRWW + kb;  // local super row of iteration 0
+    uint4 buf[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+        int row = r0 + (lsr0 + 4 * (u / LW)) * LW + (u % LW);
+        if (row > a.R - 1) row = a.R - 1;  // activation rows there are staged as zeros
+        buf[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
+    }
+    // keep every load above in flight before anything below consumes one of them
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase C: fill LDS
+    auto stage_x = [&](int sr, int m, bool valid, const uint4(&raw)[T]) {
+        uint4* dst = xs + ((size_t)sr * RT + m) * T;
+        if (!valid) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) dst[t] = make_uint4(0, 0, 0, 0);
+            return;
+        }
+        uint16_t v[KPS];
+#pragma unroll
+        for (int t = 0; t < T; ++t) ((uint4*)v)[t] = raw[t];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            uint32_t o[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                int lo, hi;
+                if constexpr (E >= 8) {
+                    lo = 4 * t + r;
+                    hi = lo + E / 2;
+                } else {  // 8-bit codes: register r pairs (j, j + 2) of word r / 2
+                    lo = 4 * (r / 2) + (r % 2);
+                    hi = lo + 2;
+                }
+                o[r] = (uint32_t)v[lo] | ((uint32_t)v[hi] << 16);
+            }
+            dst[t] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    };
+    if (x_first) stage_x(sr_a, m_a, x_valid, xraw);
+    for (int idx = tid + kThreads; idx < x_items; idx += kThreads) {
+        const int sr = idx / RT, m = idx - sr * RT;
+        const int row = r0 + sr * LW;
+        const bool valid = row < a.R && (m0 + m) < a.M;
+        uint4 raw[T];
+        if (valid) {
+            const uint4* src = (const uint4*)((const uint16_t*)a.x + (int64_t)(m0 + m) * a.xsm + (int64_t)row * E);
+#pragma unroll
+            for (int t = 0; t < T; ++t) raw[t] = src[t];
+        }
+        stage_x(sr, m, valid, raw);
+    }
+
+    if (fast_meta) {
+        auto stage_meta = [&](int gl, int c4, uint2 sr_, uint2 zr_) {
+            const uint16_t sv[4] = {(uint16_t)(sr_.x & 0xffff), (uint16_t)(sr_.x >> 16), (uint16_t)(sr_.y & 0xffff),
+                                    (uint16_t)(sr_.y >> 16)};
+            const uint16_t zv[4] = {(uint16_t)(zr_.x & 0xffff), (uint16_t)(zr_.x >> 16), (uint16_t)(zr_.y & 0xffff),
+                                    (uint16_t)(zr_.y >> 16)};
+            float2 o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                o[j] = fold_meta(meta_to_float(sv[j], a.meta_dt), meta_to_float(zv[j], a.meta_dt), a.wgm, OFF);
+            float4* dst = (float4*)(mt + gl * kTileN + c4);
+            dst[0] = make_float4(o[0].x, o[0].y, o[1].x, o[1].y);
+            dst[1] = make_float4(o[2].x, o[2].y, o[3].x, o[3].y);
+        };
+        if (meta_first) stage_meta(gl_a, c4_a, sraw, zraw);
+        for (int idx = tid + kThreads; idx < a.GW * 16; idx += kThreads) {
+            const int gl = idx >> 4, c4 = (idx & 15) * 4;
+            int g = g0 + gl;
+            if (g > a.G - 1) g = a.G - 1;
+            int n = n0 + c4;
+            if (n > a.N - 4) n = a.N - 4;
+            const uint2 s2 = *(const uint2*)((const uint16_t*)a.scales + (int64_t)g * a.msg + n);
+            const uint2 z2 = *(const uint2*)((const uint16_t*)a.zeros + (int64_t)g * a.msg + n);
+            stage_meta(gl, c4, s2, z2);
+        }
+    } else {
+        for (int idx = tid; idx < a.GW * kTileN; idx += kThreads) {
+            const int gl = idx / kTileN, c = idx - gl * kTileN;
+            int g = g0 + gl;
+            if (g > a.G - 1) g = a.G - 1;
+            int n = n0 + c;
+            if (n > a.N - 1) n = a.N - 1;
+            float s = 1.0f, z = 0.0f;
+            if (a.wgm >= GLA_WGM_SCALE) s = load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + n);
+            if (a.wgm == GLA_WGM_SHIFT || a.wgm >= GLA_WGM_SHIFT_SCALE)
+                z = a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0)
+                               : load_as_float(a.zeros, a.z_dt, (int64_t)g * a.msg + n);
+            mt[idx] = fold_meta(s, z, a.wgm, OFF);
+        }
+    }
+    __syncthreads();
+    GLA_STAMP(1);
+
+    // ---- main loop
+    float acc[4][RI];
+    float4_t c[4], csx;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        c[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < RI; ++i) acc[j][i] = 0.0f;
+    }
+    csx = float4_t{0.f, 0.f, 0.f, 0.f};
+    const uint4 ones = make_uint4(Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones);
+    const int mA = (RT == 16) ? cg : (cg & (RT - 1));  // rows >= RT of the A operand may hold anything
+    constexpr int IPB = kBatch / LW;                   // wave iterations per batch of loads
+    uint32_t pair_mask = kPairMask, magic = Magic<BF16>::bits;
+    asm volatile("" : "+s"(pair_mask), "+v"(magic));  // keep both in registers, not literals
+    const int fl_mask = a.FL - 1;                      // FL is a power of two
+
+    for (int ib = 0; ib < nit; ib += IPB) {
+        uint4 cur[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) cur[u] = buf[u];
+        if (ib + IPB < nit) {
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                int row = r0 + (lsr0 + 4 * (ib + IPB + u / LW)) * LW + (u % LW);
+                if (row > a.R - 1) row = a.R - 1;
+                buf[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
+            }
+        }
+#pragma unroll
+        for (int ii = 0; ii < IPB; ++ii) {
+            const int it = ib + ii;
+            const int lsr = lsr0 + 4 * it;
+            const uint4* xa = xs + ((size_t)lsr * RT + mA) * T;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const uint4 av = xa[t];
+                csx = mfma16<BF16>(av, ones, csx);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t b[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if constexpr (E >= 8) {
+                            b[r] = and_or(pick(cur[ii], j) >> ((4 * t + r) * BITS), pair_mask, magic);
+                        } else {
+                            b[r] = and_or(pick(cur[ii * LW + r / 2], j) >> ((r % 2) * 8), pair_mask, magic);
+                        }
+                    }
+                    c[j] = mfma16<BF16>(av, make_uint4(b[0], b[1], b[2], b[3]), c[j]);
+                }
+            }
+            if (((it + 1) & fl_mask) == 0) {
+                // group of this iteration: the four quarters' super rows lie in one group
+                int gl = (r0 + (wv * SRWW + 4 * it) * LW) / a.gr - g0;
+                if (gl > a.GW - 1) gl = a.GW - 1;
+                const float4* mrow = (const float4*)(mt + gl * kTileN + cg * 4);
+                const float4 m01 = mrow[0], m23 = mrow[1];
+                const float sj[4] = {m01.x, m01.z, m23.x, m23.z};
+                const float zj[4] = {m01.y, m01.w, m23.y, m23.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int i = 0; i < RI; ++i)
+                        acc[j][i] = __builtin_fmaf(sj[j], c[j][i], __builtin_fmaf(zj[j], csx[i], acc[j][i]));
+                    c[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+                csx = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    }
+
+    wg_finish<RT, kWaves, RI>(a, acc, red, ticket, tile, split, m0, n0);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Direct variant for 4- and 8-bit codes at M <= 4: no workgroup staging and no barrier before the
+// stream.  Every wave loads, right ahead of its own weight words, the activation chunks those
+// words meet (from L2) and the scales / zero points of its own groups (into a wave-private LDS
+// table), so waves run independently until the final reduction and compute overlaps the stream.
+// LOOP = false: exactly one batch of kBatch loads per lane (everything in flight at once).
+// ---------------------------------------------------------------------------------------------
+template <int BITS, bool BF16, int RT, int kWaves, bool LOOP>
+__global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
+    using SH = Shape<BITS>;
+    constexpr int E = SH::E, LW = SH::LW;
+    static_assert(SH::T == 1, "direct variant handles one MFMA K-step per super row");
+    constexpr int IPB = kBatch / LW;  // wave iterations per batch
+    constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
+    constexpr float OFF = Magic<BF16>::off;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int nfb = a.nfb;                                        // flush blocks per batch
+    float2* mtw = (float2*)smem + (size_t)(threadIdx.x >> 6) * nfb * kTileN;  // [nfb][64], this wave's
+    float* red = (float*)((float2*)smem + (size_t)kWaves * nfb * kTileN);     // [kWaves][RT][64]
+    __shared__ unsigned ticket;
+
+    GLA_STAMP(0);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wv = tid >> 6;
+    const int cg = lane & 15, kb = lane >> 4;
+    const int tile = blockIdx.x % a.tiles;
+    const int split = blockIdx.x / a.tiles;
+    const int m0 = blockIdx.y * RT;
+    const int n0 = tile * kTileN;
+    const int r0 = split * a.RW;
+    const int SRWW = a.RW / LW / kWaves;  // super rows per wave
+    const int nit = SRWW / 4;             // wave iterations
+    const int lsr0 = wv * SRWW + kb;
+    const int g0w = (r0 + wv * SRWW * LW) / a.gr;  // first group this wave touches
+
+    int col = n0 + cg * 4;
+    if (col > a.N - 4) col = a.N - 4;  // clamped lanes are never stored
+    const uint32_t* wbase = a.w + col;
+    int mrow = m0 + (cg & (RT - 1));  // rows >= RT of the A operand may hold anything
+    if (mrow > a.M - 1) mrow = a.M - 1;
+    const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)mrow * a.xsm;
+    const bool fast_meta = (a.meta_dt == GLA_DT_FP16 || a.meta_dt == GLA_DT_BF16) && !a.z_scalar &&
+                           (a.z_dt == a.meta_dt) && a.wgm >= GLA_WGM_SHIFT_SCALE;
+
+    struct Batch {
+        uint2 sr[2], zr[2];
+        uint4 xr[IPB];
+        uint4 wr[kBatch];
+    };
+
+    // group (relative to g0w) whose fold closes flush block `fbl` of the batch starting at iteration ib
+    auto block_group = [&](int ib, int fbl) {
+        const int it_f = (a.FL <= IPB) ? (ib + (fbl + 1) * a.FL - 1) : (ib + IPB - 1);
+        int g = (r0 + (wv * SRWW + 4 * it_f) * LW) / a.gr;
+        if (g > a.G - 1) g = a.G - 1;
+        return g;
+    };
+
+    auto issue = [&](int ib, Batch& b) {
+        if (fast_meta && !(GLA_EXP & 4)) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int item = lane + 64 * p;
+                int fbl = item >> 4;
+                if (fbl > nfb - 1) fbl = nfb - 1;  // surplus lanes reload the last block and drop it
+                const int g = block_group(ib, fbl);
+                int n = n0 + (item & 15) * 4;
+                if (n > a.N - 4) n = a.N - 4;
+                if (p == 0 || nfb > 4) {
+                    b.sr[p] = *(const uint2*)((const uint16_t*)a.scales + (int64_t)g * a.msg + n);
+                    b.zr[p] = *(const uint2*)((const uint16_t*)a.zeros + (int64_t)g * a.msg + n);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < IPB; ++u) {
+            int row = r0 + (lsr0 + 4 * (ib + u)) * LW;
+            if (row > a.R - LW) row = a.R - LW;
+            if (GLA_EXP & 1) b.xr[u] = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
+            else b.xr[u] = *(const uint4*)(xbase + (int64_t)row * E);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            int row = r0 + (lsr0 + 4 * (ib + u / LW)) * LW + (u % LW);
+            if (row > a.R - 1) row = a.R - 1;
+            b.wr[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
+        }
+    };
+
+    float acc[4][RT];
+    float4_t c[4], csx;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        c[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < RT; ++i) acc[j][i] = 0.0f;
+    }
+    csx = float4_t{0.f, 0.f, 0.f, 0.f};
+    const uint4 ones = make_uint4(Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones);
+    uint32_t pair_mask = kPairMask, magic = Magic<BF16>::bits;
+    asm volatile("" : "+s"(pair_mask), "+v"(magic));  // keep both in registers, not literals
+    const int fl_mask = a.FL - 1;                      // FL is a power of two
+
+    auto stage_meta = [&](int ib, const Batch& b) {
+        if (fast_meta) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int item = lane + 64 * p;
+                if ((p == 0 || nfb > 4) && item < nfb * 16) {
+                    const uint32_t sw[2] = {b.sr[p].x, b.sr[p].y}, zw[2] = {b.zr[p].x, b.zr[p].y};
+                    float2 o[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint16_t sv = (uint16_t)(sw[j >> 1] >> (16 * (j & 1)));
+                        const uint16_t zv = (uint16_t)(zw[j >> 1] >> (16 * (j & 1)));
+                        o[j] = fold_meta(meta_to_float(sv, a.meta_dt), meta_to_float(zv, a.meta_dt), a.wgm, OFF);
+                    }
+                    float4* dst = (float4*)(mtw + (item >> 4) * kTileN + (item & 15) * 4);
+                    dst[0] = make_float4(o[0].x, o[0].y, o[1].x, o[1].y);
+                    dst[1] = make_float4(o[2].x, o[2].y, o[3].x, o[3].y);
+                }
+            }
+        } else {
+            for (int idx = lane; idx < nfb * kTileN; idx += kWave) {
+                const int fbl = idx / kTileN, cc = idx - fbl * kTileN;
+                const int g = block_group(ib, fbl);
+                int n = n0 + cc;
+                if (n > a.N - 1) n = a.N - 1;
+                float s = 1.0f, z = 0.0f;
+                if (a.wgm >= GLA_WGM_SCALE) s = load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + n);
+                if (a.wgm == GLA_WGM_SHIFT || a.wgm >= GLA_WGM_SHIFT_SCALE)
+                    z = a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0)
+                                   : load_as_float(a.zeros, a.z_dt, (int64_t)g * a.msg + n);
+                mtw[idx] = fold_meta(s, z, a.wgm, OFF);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    auto process = [&](int ib, const Batch& b) {
+        stage_meta(ib, b);
+#pragma unroll
+        for (int ii = 0; ii < IPB; ++ii) {
+            const int it = ib + ii;
+            // activation chunk -> the pair order of the code extraction
+            const uint4 xr = b.xr[ii];
+            uint4 av;
+            if constexpr (E == 8) {  // pairs (j, j + 4)
+                av.x = __builtin_amdgcn_perm(xr.z, xr.x, 0x05040100u);
+                av.y = __builtin_amdgcn_perm(xr.z, xr.x, 0x07060302u);
+                av.z = __builtin_amdgcn_perm(xr.w, xr.y, 0x05040100u);
+                av.w = __builtin_amdgcn_perm(xr.w, xr.y, 0x07060302u);
+            } else {  // two words of 4 codes: pairs (j, j + 2) inside each word
+                av.x = __builtin_amdgcn_perm(xr.y, xr.x, 0x05040100u);
+                av.y = __builtin_amdgcn_perm(xr.y, xr.x, 0x07060302u);
+                av.z = __builtin_amdgcn_perm(xr.w, xr.z, 0x05040100u);
+                av.w = __builtin_amdgcn_perm(xr.w, xr.z, 0x07060302u);
+            }
+            if (GLA_EXP & 2) {
+#pragma unroll
+                for (int u2 = 0; u2 < LW; ++u2) {
+                    const uint4 wq = b.wr[ii * LW + u2];
+                    acc[0][0] += __builtin_bit_cast(float, (wq.x ^ wq.y ^ wq.z ^ wq.w ^ av.x) & 0x3fffffffu);
+                }
+                continue;
+            }
+            csx = mfma16<BF16>(av, ones, csx);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint32_t bq[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if constexpr (E == 8) {
+                        bq[r] = and_or(pick(b.wr[ii], j) >> (r * BITS), pair_mask, magic);
+                    } else {
+                        bq[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8), pair_mask, magic);
+                    }
+                }
+                c[j] = mfma16<BF16>(av, make_uint4(bq[0], bq[1], bq[2], bq[3]), c[j]);
+            }
+            if (((it + 1) & fl_mask) == 0) {
+                const int fbl = (a.FL <= IPB) ? (((ii + 1) >> a.fl_log2) - 1) : 0;
+                const float4* mrow = (const float4*)(mtw + fbl * kTileN + cg * 4);
+                const float4 m01 = mrow[0], m23 = mrow[1];
+                const float sj[4] = {m01.x, m01.z, m23.x, m23.z};
+                const float zj[4] = {m01.y, m01.w, m23.y, m23.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int i = 0; i < RT; ++i)
+                        acc[j][i] = __builtin_fmaf(sj[j], c[j][i], __builtin_fmaf(zj[j], csx[i], acc[j][i]));
+                    c[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
+                csx = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+        __builtin_amdgcn_wave_barrier();  // the table is rewritten by the next batch
+    };
+
+    if constexpr (!LOOP) {
+        Batch b;
+        issue(0, b);
+        __builtin_amdgcn_sched_barrier(0);
+        process(0, b);
+    } else {
+        Batch nxt;
+        issue(0, nxt);
+        for (int ib = 0; ib < nit; ib += IPB) {
+            const Batch cur = nxt;
+            if (ib + IPB < nit) issue(ib + IPB, nxt);
+            __builtin_amdgcn_sched_barrier(0);
+            process(ib, cur);
+        }
+    }
+    GLA_STAMP(1);
+    wg_finish<RT, kWaves, RT>(a, acc, red, ticket, tile, split, m0, n0);
+}
+
+#ifdef GLA_TRACE
+long long* g_trace = nullptr;
+#endif
+
+int row_tile(int M) { return M > 4 ? 16 : (M >= 3 ? 4 : (M == 2 ? 2 : 1)); }
 
 struct Geometry {
-    int E, R, RW, S, tiles, MT, mchunks, Mp, gr, G, GW, FL;
+    int E, LW, KPS, T, R, RW, S, tiles, RT, mchunks, Mp, gr, G, GW, FL, waves, unit, nb, nfb;
+    bool direct;  // 4/8-bit codes at M <= 4: the variant without workgroup staging
     size_t smem;
 };
 
+// tile_config encoding: (waves per workgroup) * 1000 + (batches of kBatch loads per wave).
 bool geometry(const gla_matmul_args& p, Geometry& g) {
     g.E = 32 / p.W_nbits;
+    g.LW = g.E < 8 ? 8 / g.E : 1;
+    g.KPS = g.E * g.LW;
+    g.T = g.KPS / 8;
     g.R = p.K / g.E;
     g.tiles = ceil_div(p.N, kTileN);
-    g.MT = row_tile(p.M);
-    g.mchunks = ceil_div(p.M, g.MT);
-    g.Mp = g.mchunks * g.MT;
+    g.RT = row_tile(p.M);
+    g.mchunks = ceil_div(p.M, g.RT);
+    g.Mp = g.mchunks * g.RT;
     const bool grouped = p.W_group_mode >= GLA_WGM_SCALE || (p.W_group_mode == GLA_WGM_SHIFT && !p.zero_is_scalar);
     const int gs = grouped ? p.group_size : p.K;
+    // every K-block of one MFMA step must lie in one group
+    const int k_per_iter = 4 * g.KPS;
+    if (gs % k_per_iter != 0) return false;
     g.gr = gs / g.E;
-    if (g.gr < 1) return false;
     g.G = p.K / gs;
-
-    int slabs = ceil_div(g.R, kSlabRows);
-    int per_wg;
-    if (p.tile_config > 0) {
-        per_wg = p.tile_config;
+    // one wave, one batch: 4 quarters x kBatch loads of word rows
+    g.unit = 4 * kBatch;
+    const int units = ceil_div(g.R, g.unit);  // wave-batches along K
+    const int max_waves = (g.RT == 16) ? 4 : 16;  // the cross-wave buffer is [waves][RT][64] floats
+    int waves, nb;
+    if (p.tile_config >= 1000) {
+        waves = p.tile_config / 1000;
+        nb = p.tile_config % 1000;
+        if (!(waves == 4 || waves == 8 || waves == 16) || waves > max_waves || nb < 1) return false;
     } else {
-        // enough workgroups to fill 256 CUs about four times over, then as few slabs as possible
-        int want = ceil_div(1024, g.tiles * g.mchunks);
-        if (want < 1) want = 1;
-        if (want > slabs) want = slabs;
-        per_wg = ceil_div(slabs, want);
+        // Slabs along K: enough workgroups to cover the CUs, and few enough wave-batches per
+        // workgroup that every load of the kernel is in flight at once (one batch per wave).
+        int s_min = ceil_div(200, g.tiles * g.mchunks);
+        if (s_min < 1) s_min = 1;
+        int want_s = ceil_div(units, max_waves);
+        if (want_s < s_min) want_s = s_min;
+        if (want_s > units) want_s = units;
+        int per_wg = ceil_div(units, want_s);  // wave-batches per workgroup
+        // prefer a slab count that divides K exactly into 4, 8 or 16 wave-batches (no ragged slab)
+        if (g.R % g.unit == 0) {
+            for (int s2 = want_s; s2 <= units && s2 <= 4 * want_s + 4; ++s2) {
+                const int q = units / s2;
+                if (units % s2 == 0 && (q == 4 || q == 8 || q == 16) && q <= max_waves) {
+                    per_wg = q;
+                    break;
+                }
+            }
+        }
+        waves = per_wg <= 4 ? 4 : (per_wg <= 8 && max_waves >= 8 ? 8 : max_waves);
+        nb = ceil_div(per_wg, waves);
     }
-    if (per_wg > slabs) per_wg = slabs;
-    // LDS budget: activation slab + row sums + (s, zz) table + wave partials
-    for (;; --per_wg) {
-        g.RW = per_wg * kSlabRows;
+    g.direct = (g.RT <= 4) && (p.W_nbits == 4 || p.W_nbits == 8);
+    if (g.direct && nb > 1 && waves != 4) {  // the looping direct variant runs 4 waves
+        nb *= waves / 4;
+        waves = 4;
+    }
+    const int it_per_group = gs / k_per_iter;
+    for (;;) {
+        g.waves = waves;
+        g.nb = nb;
+        g.RW = waves * nb * g.unit;
         g.GW = g.RW / g.gr + 2;
-        const size_t xw = (p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16) ? g.E : g.E / 2;
-        g.smem = (size_t)g.MT * g.RW * xw * 4 + (size_t)g.MT * g.RW * 4 + (size_t)g.GW * kTileN * 8 +
-                 (size_t)kWaves * g.MT * kTileN * 4;
+        // iterations per flush: whole groups, at most 1024 K-values between folds
+        const int nit = g.RW / g.LW / waves / 4;
+        int fl = 1;
+        while (fl * 2 * k_per_iter <= 1024 && it_per_group % (fl * 2) == 0 && nit % (fl * 2) == 0) fl *= 2;
+        g.FL = fl;
+        const int ipb = kBatch / g.LW;
+        g.nfb = fl >= ipb ? 1 : ipb / fl;
+        if (g.direct)
+            g.smem = (size_t)waves * g.nfb * kTileN * 8 + (size_t)waves * g.RT * kTileN * 4;
+        else
+            g.smem = (size_t)(g.RW / g.LW) * g.RT * g.T * 16 + (size_t)g.GW * kTileN * 8 +
+                     (size_t)waves * g.RT * kTileN * 4;
         if (g.smem <= 60 * 1024) break;
-        if (per_wg == 1) return false;
+        if (nb > 1) {
+            --nb;
+        } else if (waves > 4) {
+            waves /= 2;
+        } else {
+            return false;
+        }
     }
     g.S = ceil_div(g.R, g.RW);
-    if (g.S > 1 && (int64_t)g.tiles * g.mchunks * 4 > kCounterBytes) return false;
-    const int nl = g.RW / kWaves / 4;
-    int fl = 1;
-    if (g.gr >= 4 && g.gr % 4 == 0) {
-        const int flmax = g.gr / 4;
-        while (fl < 16 && flmax % (fl * 2) == 0 && nl % (fl * 2) == 0) fl *= 2;
+    if (g.direct && g.S * g.RW != g.R) {
+        // the direct variant has no zero-padded activation slab: a ragged last slab takes the staged kernel
+        g.direct = false;
+        g.smem = (size_t)(g.RW / g.LW) * g.RT * g.T * 16 + (size_t)g.GW * kTileN * 8 +
+                 (size_t)g.waves * g.RT * kTileN * 4;
+        if (g.smem > 60 * 1024) return false;
     }
-    g.FL = fl;
+    if (g.S > 1 && (int64_t)g.tiles * g.mchunks * 4 > kCounterBytes) return false;
     return true;
 }
 
-template <int BITS, bool BF16, int MT>
+template <int BITS, bool BF16, int RT>
 void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
     dim3 grid(g.tiles * g.S, g.mchunks);
-    constexpr bool F32 = (BITS == 8) && BF16;
-    hipLaunchKernelGGL((gemv_packed_kernel<BITS, BF16, MT, F32>), grid, dim3(kThreads), g.smem, stream, a);
+    if constexpr (RT <= 4 && (BITS == 4 || (BITS == 8 && !BF16))) {
+        if (g.direct) {
+            if (g.nb > 1)
+                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
+            else if (g.waves == 16)
+                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
+            else if (g.waves == 8)
+                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 8, false>), grid, dim3(512), g.smem, stream, a);
+            else
+                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, false>), grid, dim3(256), g.smem, stream, a);
+            return;
+        }
+    }
+    if constexpr (RT == 16) {
+        hipLaunchKernelGGL((gemv_packed_kernel<BITS, BF16, RT, 4>), grid, dim3(256), g.smem, stream, a);
+    } else {
+        if (g.waves == 16)
+            hipLaunchKernelGGL((gemv_packed_kernel<BITS, BF16, RT, 16>), grid, dim3(1024), g.smem, stream, a);
+        else if (g.waves == 8)
+            hipLaunchKernelGGL((gemv_packed_kernel<BITS, BF16, RT, 8>), grid, dim3(512), g.smem, stream, a);
+        else
+            hipLaunchKernelGGL((gemv_packed_kernel<BITS, BF16, RT, 4>), grid, dim3(256), g.smem, stream, a);
+    }
 }
 
 template <int BITS, bool BF16>
-void launch_mt(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
-    switch (g.MT) {
+void launch_rt(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
+    switch (g.RT) {
         case 1: launch_one<BITS, BF16, 1>(a, g, stream); break;
         case 2: launch_one<BITS, BF16, 2>(a, g, stream); break;
         case 4: launch_one<BITS, BF16, 4>(a, g, stream); break;
-        default: launch_one<BITS, BF16, 8>(a, g, stream); break;
+        default: launch_one<BITS, BF16, 16>(a, g, stream); break;
     }
 }
 
 template <bool BF16>
 void launch_bits(const GemvArgs& a, const Geometry& g, int bits, hipStream_t stream) {
     switch (bits) {
-        case 1: launch_mt<1, BF16>(a, g, stream); break;
-        case 2: launch_mt<2, BF16>(a, g, stream); break;
-        case 4: launch_mt<4, BF16>(a, g, stream); break;
-        default: launch_mt<8, BF16>(a, g, stream); break;
+        case 1: launch_rt<1, BF16>(a, g, stream); break;
+        case 2: launch_rt<2, BF16>(a, g, stream); break;
+        case 4: launch_rt<4, BF16>(a, g, stream); break;
+        default: launch_rt<8, BF16>(a, g, stream); break;
     }
 }
 
@@ -430,6 +855,7 @@ bool gemv_packed_eligible(const gla_matmul_args& p) {
     if (!(p.W_nbits == 1 || p.W_nbits == 2 || p.W_nbits == 4 || p.W_nbits == 8)) return false;
     if (p.elements_per_sample * p.W_nbits != 32) return false;
     if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16)) return false;
+    if (p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16) return false;  // 128 + q is not exact in bf16 for q > 127
     if (p.acc_dtype != GLA_DT_FP32) return false;
     if (p.W_group_mode < 0 || p.W_group_mode > GLA_WGM_FMA) return false;
     if (p.channel_scale_mode < 0 || p.channel_scale_mode > GLA_CSM_BOTH) return false;
@@ -439,14 +865,18 @@ bool gemv_packed_eligible(const gla_matmul_args& p) {
     if (p.x_stride_k != 1 || p.x_stride_m % 8 != 0 || p.out_stride_n != 1) return false;
     if (((uintptr_t)p.w & 15) || ((uintptr_t)p.x & 15)) return false;
     const int E = 32 / p.W_nbits;
-    if (p.K % E != 0) return false;
+    const int KPS = E < 8 ? 8 : E;
+    if (p.K % KPS != 0) return false;
     const bool uses_scales = p.W_group_mode >= GLA_WGM_SCALE;
     const bool uses_zeros = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
     if (uses_scales && (p.scales == nullptr || p.meta_stride_n != 1)) return false;
     if (uses_zeros && p.zeros == nullptr) return false;
     if (uses_zeros && !p.zero_is_scalar && p.meta_stride_n != 1) return false;
     const bool grouped = uses_scales || (uses_zeros && !p.zero_is_scalar);
-    if (grouped && (p.group_size < E || p.group_size % E != 0 || p.K % p.group_size != 0)) return false;
+    if (grouped && (p.group_size < E || p.K % p.group_size != 0)) return false;
+    if (grouped && (((uintptr_t)p.scales & 7) || (uses_zeros && !p.zero_is_scalar && ((uintptr_t)p.zeros & 7)) ||
+                    p.meta_stride_g % 4 != 0))
+        return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
     if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
     Geometry g;
@@ -458,7 +888,7 @@ int gemv_packed_default_config(const gla_matmul_args& p) {
     gla_matmul_args q = p;
     q.tile_config = -1;
     if (!geometry(q, g)) return -1;
-    return g.RW / kSlabRows;
+    return g.waves * 1000 + g.nb;
 }
 
 int64_t gemv_packed_workspace_bytes(const gla_matmul_args& p) {
@@ -471,10 +901,13 @@ int64_t gemv_packed_workspace_bytes(const gla_matmul_args& p) {
 int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
     Geometry g;
     if (!geometry(p, g)) {
-        set_error("gemv_packed: shape does not fit the kernel's LDS budget");
+        set_error("gemv_packed: shape does not fit the kernel's tiling or LDS budget");
         return GLA_ERR_MISALIGNED_SHAPE;
     }
     GemvArgs a;
+#ifdef GLA_TRACE
+    a.trace = g_trace;
+#endif
     a.w = (const uint32_t*)p.w; a.x = p.x; a.scales = p.scales; a.zeros = p.zeros; a.scales_x = p.scales_x;
     a.out = p.out; a.partials = nullptr; a.counters = nullptr;
     if (g.S > 1) {
@@ -488,7 +921,9 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
         a.partials = (float*)((char*)p.workspace + kCounterBytes);
     }
     a.M = p.M; a.N = p.N; a.K = p.K; a.R = g.R; a.RW = g.RW; a.S = g.S; a.tiles = g.tiles; a.Mp = g.Mp;
-    a.gr = g.gr; a.G = g.G; a.GW = g.GW; a.FL = g.FL;
+    a.gr = g.gr; a.G = g.G; a.GW = g.GW; a.FL = g.FL; a.waves = g.waves; a.nfb = g.nfb;
+    a.fl_log2 = 0;
+    while ((1 << a.fl_log2) < g.FL) ++a.fl_log2;
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.z_scalar = p.zero_is_scalar; a.out_dt = p.output_dtype; a.sx_dt = p.sx_dtype;
     a.wsk = p.w_stride_k; a.xsm = p.x_stride_m; a.osm = p.out_stride_m; a.msg = p.meta_stride_g;
