@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Headline benchmark: A16W4 group-128 decode GEMV (M = 1) on the Llama-3-8B MLP shapes.
+
+A "step" is one decode token through the two MLP linears of the benchmark configuration:
+x[1,4096] -> W_up[14336,4096] -> h[1,14336] -> W_down[4096,14336] -> y[1,4096], both
+A16W4 (HQQ asymmetric, group 128, 32-bit packing, fp16), launched through the C ABI
+(`gla_matmul`).  Consecutive steps use different weight copies (several GB in total) so that no
+cache level holds the weights between steps.  The metric is algorithmic bytes per step (every
+operand read once, the output written once) divided by the time per step.
+
+Prints ONE JSON line (see the `out` dict at the end).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import gemlite_amd  # noqa: E402
+from gemlite_amd import DType, GemLiteLinear, _ext  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+SHAPES = [(14336, 4096), (4096, 14336)]  # (N, K): up / down projection
+GROUP = 128
+
+
+def algorithmic_bytes(N, K, M=1, nbits=4, gs=GROUP):
+    """W_q + scales + zeros + x + out, each touched once (fp16 metadata and activations)."""
+    return N * K * nbits // 8 + 2 * (N * K // gs) * 2 + M * K * 2 + M * N * 2
+
+
+def make_layer(N, K, seed, device):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    W_q = torch.randint(0, 16, (N, K), generator=g, dtype=torch.int32).to(torch.uint8)
+    scales = (torch.randn((N * K // GROUP, 1), generator=g) * 0.02).abs().to(torch.float16)
+    zeros = (torch.rand((N * K // GROUP, 1), generator=g) * 3 + 6).to(torch.float16)
+    layer = GemLiteLinear(4, GROUP, K, N, DType.FP16, DType.FP16)
+    layer.pack(W_q.to(device), scales.to(device), zeros.to(device))
+    return layer, (W_q, scales, zeros)
+
+
+def clone_layer(layer):
+    c = GemLiteLinear()
+    c.load_state_dict({k: v.clone() for k, v in layer.state_dict().items()})
+    return c
+
+
+class Launch:
+    """A prepared `gla_matmul` call: argument struct built once, launched on the current stream."""
+
+    def __init__(self, lib, layer, x, out, device):
+        m = layer.get_meta_args()
+        self.lib = lib
+        self.args = _ext.build_matmul_args(
+            x, layer.W_q, layer.scales, layer.zeros, None, out,
+            W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5],
+            output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+            data_contiguous=m[11], matmul_type=gemlite_amd.GEMLITE_MATMUL_TYPES_MAPPING["GEMV_REVSPLITK"],
+        )
+        need = lib.gla_matmul_workspace_bytes(ctypes.byref(self.args))
+        if need < 0:
+            raise RuntimeError(lib.gla_last_error().decode())
+        if need > 0:
+            ws = _ext.get_workspace(device, need)
+            self.args.workspace = ws.data_ptr()
+            self.args.workspace_bytes = ws.numel()
+        self.keep = (layer, x, out)
+
+    def __call__(self):
+        rc = self.lib.gla_matmul(ctypes.byref(self.args), torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(self.lib.gla_last_error().decode())
+
+
+def cpu_baseline(host_tensors, x_host, y_gpu, threads):
+    """The reference's CPU path (HQQ dequantize + fp32 matmul) as restated in oracle/oracle_c.c,
+    timed on this box's host cores on whole steps of the same workload; also the parity check."""
+    import numpy as np
+
+    lib = ctypes.CDLL(os.path.join(ROOT, "oracle", "liboracle_c.so"))
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    i64 = ctypes.c_int64
+    arrs = []
+    for (W_q, scales, zeros) in host_tensors:
+        arrs.append((np.ascontiguousarray(W_q.numpy()), scales.float().numpy().reshape(-1).copy(),
+                     zeros.float().numpy().reshape(-1).copy()))
+    Wbuf = [np.empty(a[0].shape, dtype=np.float32) for a in arrs]
+
+    def step(x):
+        v = x
+        for (W_q, s, z), W in zip(arrs, Wbuf):
+            N, K = W_q.shape
+            lib.orc_hqq_dequantize(p(W_q), p(s), p(z), i64(N), i64(K), i64(GROUP), p(W), threads)
+            y = np.empty((1, N), dtype=np.float32)
+            lib.orc_matmul_nt_f32(p(v), p(W), i64(1), i64(N), i64(K), p(y), threads)
+            v = np.ascontiguousarray(y.astype(np.float16).astype(np.float32))  # fp16 hand-over like the GPU chain
+        return v
+
+    x32 = np.ascontiguousarray(x_host.float().numpy())
+    y_ref = step(x32)  # warm-up + reference output
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        step(x32)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or reps >= 20:
+            break
+    sec = dt / reps
+    err = float(np.linalg.norm(y_gpu.astype(np.float64) - y_ref) / np.linalg.norm(y_ref))
+    return sec, reps, err
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--rotate-gb", type=float, default=3.0, help="total bytes of distinct weight copies")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (the hot path has no cross-GPU work); use --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    lib = _ext.load_library()
+
+    step_bytes = sum(algorithmic_bytes(N, K) for N, K in SHAPES)
+    copies = max(2, int(a.rotate_gb * 1e9 // step_bytes) + 1)
+
+    # weights: one seeded set per shape, cloned `copies` times on the device
+    base, host = [], []
+    for i, (N, K) in enumerate(SHAPES):
+        layer, host_t = make_layer(N, K, seed=i, device=device)
+        base.append(layer)
+        host.append(host_t)
+    sets = [base] + [[clone_layer(l) for l in base] for _ in range(copies - 1)]
+
+    g = torch.Generator(device="cpu").manual_seed(1234)
+    x_host = torch.randn((1, SHAPES[0][1]), generator=g).to(torch.float16)
+    x = x_host.to(device)
+    h = torch.empty((1, SHAPES[0][0]), dtype=torch.float16, device=device)
+    y = torch.empty((1, SHAPES[1][0]), dtype=torch.float16, device=device)
+    launches = [(Launch(lib, s[0], x, h, device), Launch(lib, s[1], h, y, device)) for s in sets]
+
+    def run_steps(first, count):
+        for i in range(first, first + count):
+            up, down = launches[i % copies]
+            up()
+            down()
+
+    # ---- warm-up (eager), then graphs of the timed steps
+    run_steps(0, a.warmup)
+    torch.cuda.synchronize()
+
+    chunk = min(a.steps, 256)
+    full, rem = divmod(a.steps, chunk)
+    side = torch.cuda.Stream()
+    graphs = []
+    with torch.cuda.stream(side):
+        run_steps(0, 2)
+        torch.cuda.synchronize()
+        for n_steps in ([chunk] if full else []) + ([rem] if rem else []):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=side):
+                run_steps(0, n_steps)
+            graphs.append(gr)
+    torch.cuda.synchronize()
+    for gr in graphs:  # one untimed replay each
+        gr.replay()
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly a.steps steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    if full:
+        for _ in range(full):
+            graphs[0].replay()
+    if rem:
+        graphs[-1].replay()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / a.steps
+    value = step_bytes / (elapsed / a.steps) / 1e9
+
+    # ---- launch duration of the dominant kernel (the 4096 -> 14336 GEMV): HIP events on the
+    # launch stream around a timed region that holds only that kernel, one launch per weight copy
+    def kernel_avg_us(which, reps=8):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(gr, stream=side):
+                for i in range(copies):
+                    launches[i][which]()
+            gr.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            for _ in range(reps):
+                gr.replay()
+            e1.record(side)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * copies)
+
+    up_avg = kernel_avg_us(0)
+    down_avg = kernel_avg_us(1)
+    kbytes = algorithmic_bytes(*SHAPES[0])
+    achieved = kbytes / (up_avg * 1e-6) / 1e9
+
+    y_gpu = y.float().cpu().numpy()
+
+    out = {
+        "metric": "A16W4 gs128 GEMV GB/s (%HBM peak) @M=1",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16",
+        "data": "synthetic",
+        "config": {
+            "workload": "A16W4 HQQ gs=128 fp16 Llama-3-8B MLP decode, M=1: 4096->14336 then 14336->4096 per step",
+            "bytes_per_step": step_bytes,
+            "weight_copies": copies,
+            "launch": "HIP graph replay of prepared gla_matmul calls",
+            "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_direct_kernel<4-bit, fp16, M=1> on 4096->14336",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "bytes_per_launch": kbytes,
+            "avg_launch_us": round(up_avg, 3),
+            "traffic": None,
+        },
+        "extra": {
+            "down_proj_avg_launch_us": round(down_avg, 3),
+            "down_proj_GBps": round(algorithmic_bytes(*SHAPES[1]) / (down_avg * 1e-6) / 1e9, 1),
+        },
+    }
+
+    if not a.no_cpu:
+        threads = min(os.cpu_count() or 1, 16)
+        sec, reps, err = cpu_baseline(host, x_host, y_gpu, threads)
+        out["cpu_baseline"] = {
+            "value": round(step_bytes / sec / 1e9, 3),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{reps} whole steps (HQQ dequantize of both weight matrices + fp32 matmul), "
+                      f"{sec * 1e3:.1f} ms per step",
+        }
+        out["extra"]["gpu_vs_cpu_rel_frobenius_err"] = round(err, 6)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
