@@ -107,6 +107,15 @@ __device__ __forceinline__ void store_from_float(void* p, int dt, int64_t idx, f
     }
 }
 
+// Store with the element type fixed at compile time (DT is a GLA_DT_* id).
+template <int DT>
+__device__ __forceinline__ void store_typed(void* p, int64_t idx, float v) {
+    if constexpr (DT == GLA_DT_FP32) ((float*)p)[idx] = v;
+    else if constexpr (DT == GLA_DT_FP16) ((uint16_t*)p)[idx] = float_to_half_bits(v);
+    else if constexpr (DT == GLA_DT_BF16) ((uint16_t*)p)[idx] = float_to_bf16_bits(v);
+    else ((int32_t*)p)[idx] = (int32_t)v;
+}
+
 __host__ __device__ __forceinline__ int dtype_size(int dt) {
     switch (dt) {
         case GLA_DT_FP32: case GLA_DT_INT32: case 7: return 4;

@@ -4,11 +4,6 @@
 namespace gla {
 bool gemv_kmajor_eligible(const gla_matmul_args&) { return false; }
 int launch_gemv_kmajor(const gla_matmul_args&, hipStream_t) { return GLA_ERR_UNSUPPORTED_MODE; }
-bool gemm_wn_eligible(const gla_matmul_args&) { return false; }
-int64_t gemm_wn_workspace_bytes(const gla_matmul_args&) { return 0; }
-int launch_gemm_wn(const gla_matmul_args&, hipStream_t) { return GLA_ERR_UNSUPPORTED_MODE; }
-bool gemm_8bit_eligible(const gla_matmul_args&) { return false; }
-int launch_gemm_8bit(const gla_matmul_args&, hipStream_t) { return GLA_ERR_UNSUPPORTED_MODE; }
 bool gemm_mxfp4_eligible(const gla_matmul_args&) { return false; }
 int launch_gemm_mxfp4(const gla_matmul_args&, hipStream_t) { return GLA_ERR_UNSUPPORTED_MODE; }
 }
