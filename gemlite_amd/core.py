@@ -395,7 +395,9 @@ class GemLiteLinear(torch.nn.Module):
             scales_t = scales_t.to(torch.float8_e4m3fn)
         if mx:
             wgm, csm = 2, 0
-            scales_t = scales_t.T
+            # [N, K/gs] like the reference's view (gemlite/core.py:719), but materialised row-major
+            # so that the block scales of one output row are consecutive bytes for the MFMA kernel
+            scales_t = scales_t.T.contiguous()
 
         self.W_group_mode = wgm
         self.channel_scale_mode = csm
@@ -491,7 +493,10 @@ class GemLiteLinear(torch.nn.Module):
         self.device = device
         self._set_param("W_q", W_q)
         self._set_param("bias", sd.get("bias"))
-        self._set_param("scales", sd.get("scales"))
+        scales = sd.get("scales")
+        if scales is not None and is_mx_dtype(self.input_dtype) and scales.dim() == 2 and scales.stride(-1) != 1:
+            scales = scales.contiguous()  # checkpoints written by the reference hold the transposed view
+        self._set_param("scales", scales)
         self._set_param("zeros", sd.get("zeros"))
         self._set_param("metadata", torch.tensor(self.get_meta_args(), device=device, dtype=torch.int32))
         self._set_param(

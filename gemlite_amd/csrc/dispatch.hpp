@@ -28,7 +28,7 @@ int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream);
 bool gemm_8bit_eligible(const gla_matmul_args& p);
 int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream);
 
-// ---- block-scaled MXFP4 MFMA GEMM (gemm_mxfp4.hip) -------------------------
+// ---- block-scaled MXFP4 MFMA GEMM (gemm_8bit.hip) -------------------------
 bool gemm_mxfp4_eligible(const gla_matmul_args& p);
 int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream);
 

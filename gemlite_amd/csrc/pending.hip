@@ -4,6 +4,4 @@
 namespace gla {
 bool gemv_kmajor_eligible(const gla_matmul_args&) { return false; }
 int launch_gemv_kmajor(const gla_matmul_args&, hipStream_t) { return GLA_ERR_UNSUPPORTED_MODE; }
-bool gemm_mxfp4_eligible(const gla_matmul_args&) { return false; }
-int launch_gemm_mxfp4(const gla_matmul_args&, hipStream_t) { return GLA_ERR_UNSUPPORTED_MODE; }
 }

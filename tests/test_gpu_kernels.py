@@ -278,3 +278,40 @@ def test_a4w4_mxfp4(device, M):
     y = to_np(layer(x.to(device)))
     y_fp = to_np(x) @ to_np(W).T
     assert rel_frob(y, y_fp) < 0.2
+
+
+@pytest.mark.parametrize("M", [64, 300])
+def test_a4w4_mxfp4_wide(device, M):
+    # K a multiple of the full 256-value step, N across several column tiles with a ragged last one
+    N, K = 1352, 2048
+    W = gen_x(N, K, torch.float16, seed=8, std=0.02)
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.float16)
+    lin.weight.data = W
+    layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.float16).from_linear(lin.to(device))
+    assert layer.scales.stride() == (K // 32, 1)
+    check_layer(layer, gen_x(M, K, torch.float16, seed=M).to(device), torch.float16, types=["GEMM"])
+
+
+@pytest.mark.parametrize("K", [1056, 2240])
+def test_int8_ragged_k_bit_exact(device, K):
+    # K that is a multiple of 32 but not of the 128-byte pipeline step
+    N = 300
+    g = torch.Generator().manual_seed(K)
+    W = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    layer = GemLiteLinear(8, None, K, N, DType.INT8, DType.INT32).pack(W.to(device), None, None)
+    for M in (40, 130, 260):
+        x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+        ref = (x.long() @ W.long().t()).numpy()
+        y = layer.forward_manual(x.to(device), matmul_type="GEMM")
+        assert np.array_equal(y.cpu().numpy(), ref), M
+
+
+def test_fp8_ragged_k(device):
+    N, K = 520, 2112  # 16.5 pipeline steps
+    W = gen_x(N, K, torch.bfloat16, seed=11, std=0.02)
+    W_q, s = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn)
+    proc = helper.A8W8_FP8_dynamic(device=device)
+    proc.dtype = torch.bfloat16
+    layer = proc.from_weights(W_q, scales=s)
+    for M in (70, 200):
+        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM"])

@@ -106,7 +106,7 @@ def test_pack_mxfp4_layout():
     # bytes [N, K/2] (low nibble = even k) handed over as the [K/2, N] view; e8m0 scales as the [N, K/32] view
     assert l.W_q.shape == (K // 2, N) and l.W_q.stride() == (1, K // 2) and l.W_q.dtype == torch.uint8
     assert int(l.W_q[3, 5]) == int(codes[5, 6]) | (int(codes[5, 7]) << 4)
-    assert l.scales.shape == (N, K // 32) and l.scales.dtype == torch.uint8 and l.scales.stride() == (1, N)
+    assert l.scales.shape == (N, K // 32) and l.scales.dtype == torch.uint8 and l.scales.stride() == (K // 32, 1)
     assert (l.W_group_mode, l.channel_scale_mode, l.elements_per_sample) == (0, 4, 2)
     assert l.W_q.numel() == N * K // 2  # packed byte count (reference: tests/test_mxfp.py:96)
 
@@ -273,7 +273,7 @@ def test_operand_bounds_are_checked_on_the_host():
         _ext.build_matmul_args(x[:, : K // 2].contiguous(), W, s, s, None, out, **kw)  # x shorter than K
     with pytest.raises(ValueError, match="out"):
         _ext.build_matmul_args(x, W, s, s, None, out[:1].clone(), **kw)
-    # micro-scaled layers hand their scales over as the [N, K/32] view of a [K/32, N] buffer
+    # micro-scaled layers hand their scales over as a row-major [N, K/32] array
     codes = torch.randint(0, 16, (N, K)).to(torch.uint8)
     e8 = torch.randint(110, 130, (N, K // 32)).to(torch.uint8)
     l = gemlite_amd.helper.A4W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16).from_weights(codes, scales=e8)
@@ -283,4 +283,4 @@ def test_operand_bounds_are_checked_on_the_host():
         torch.zeros(M, N, dtype=torch.bfloat16), W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
         elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
         channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11])
-    assert (a.meta_stride_g, a.meta_stride_n) == (N, 1) and (a.w_stride_k, a.w_stride_n) == (1, K // 2)
+    assert (a.meta_stride_g, a.meta_stride_n) == (1, K // 32) and (a.w_stride_k, a.w_stride_n) == (1, K // 2)
