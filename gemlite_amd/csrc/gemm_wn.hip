@@ -1,23 +1,30 @@
 // MFMA GEMM for fp16/bf16 activations x 32-bit packed low-bit weights stored [K/e, N], N fastest:
 // out[M,N] = x[M,K] * dequant(W)[K,N], dequantisation fused into the B-operand path.  The prefill
-// path of A16W4 / A16W8 / A16W2 layers.
+// and mid-batch path of A16W4 / A16W8 / A16W2 layers.
 //
-// Takes the place of the reference's GPTQ-style GEMM and, for mid-size batches, of its split-K
-// GEMM (reference: gemlite/triton_kernels/gemm_kernels.py:285-496,
+// Takes the place of the reference's GPTQ-style GEMM and of its split-K GEMM (reference:
+// gemlite/triton_kernels/gemm_kernels.py:285-496,
 // gemlite/triton_kernels/gemm_splitK_kernels.py:300-523; dequant
 // gemlite/triton_kernels/utils.py:73-105).
 //
-//  * Workgroup tile BM x 256, K step 64; waves in a (BM/64) x 2 grid, wave tile 64 x 128 of
-//    v_mfma_f32_32x32x16 tiles, 128 accumulator registers per lane.
+//  * Workgroup tile BM x 256 with BM = 32, 64, 128 or 256, K step 64; waves in a WAVES_M x 2
+//    grid, wave tile (32 TI) x 128 of v_mfma_f32_32x32x16 tiles.
 //  * Weights never pass through LDS.  A lane's 128-bit load holds the words of 4 adjacent
 //    columns; word component j is the B operand of column tile j, so the wave's 128 columns are
 //    the interleaved set {4r + j}.  A word is unpacked with the pair trick of the GEMV kernel
 //    (codes OR-ed into the mantissa of 1024.0 / 128.0, two per VALU op), then (q - OFF) * s + z'
 //    is applied with packed fp16 math (fp32 for bf16 activations) once per wave and reused for
-//    both 32-row tiles.
-//  * Activations go global -> registers -> LDS (double-buffered, rows padded to 144 bytes); each
-//    16-byte chunk is reordered on the way in to the K-slot order the unpacking produces, so A
-//    fragments are plain 128-bit LDS reads.
+//    all of its 32-row tiles.  Weight words for the next PF K steps are in flight in registers,
+//    so a workgroup that streams its weights from HBM (small M) is not bound by load latency.
+//  * Activations are copied global -> LDS by the load unit (global_load_lds) into a ring of
+//    PF + 1 tiles with dense 128-byte rows whose 16-byte chunks are XOR-swizzled by (row >> 1) & 7;
+//    the reordering of each chunk to the K-slot order the unpacking produces happens when a
+//    fragment is read (v_perm).
+//  * Scales / zero points of the next quantisation group are fetched one group ahead.
+//  * When the output has too few tiles to fill the chip (small M), K is split over gridDim.y:
+//    every split writes an fp32 partial tile to the workspace and a second small kernel on the
+//    same stream sums the splits in order, applies the channel scales and stores the output
+//    (deterministic, no float atomics, output need not be zeroed).
 #include <type_traits>
 
 #include "common.hpp"
@@ -30,10 +37,11 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kBKw = 64;         // K per pipeline stage
-constexpr int kRowB = 144;       // padded LDS row (128 bytes of fp16 + 16)
+constexpr int kBKw = 64;    // K per pipeline stage
+constexpr int kRowW = 128;  // LDS row: 64 fp16/bf16 values
 constexpr int kWavesNw = 2;
 constexpr int kBNw = kWavesNw * 128;
+constexpr int64_t kWsReserved = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
 
 struct GemmWnArgs {
     const uint16_t* x;
@@ -43,10 +51,13 @@ struct GemmWnArgs {
     const void* scales_x;
     void* out;
     int M, N, K;
-    int gs;       // K-values per quantisation group (K when ungrouped)
+    int gs;  // K-values per quantisation group (K when ungrouped)
     int64_t xsm, wsk, osm, msg, sxm;
     int wgm, csm, meta_dt, z_dt, z_scalar, out_dt, sx_dt;
     int tiles_m, tiles_n;
+    int S;    // K splits (gridDim.y)
+    int sps;  // pipeline stages per split
+    float* partials;  // [S][M][N] when S > 1
 };
 
 __device__ __forceinline__ void tile_coords_wn(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -62,26 +73,18 @@ __device__ __forceinline__ void tile_coords_wn(int pid, int tiles_m, int tiles_n
     tn = (t % width) / gsize;
 }
 
-// Reorder one 16-byte chunk of activations (8 consecutive K-values) to the K-slot order of the
-// B operand: W4 pairs (j, j+4); W8 pairs (j, j+2) inside each half; W2 handled by the caller.
-template <int BITS>
-__device__ __forceinline__ u32x4 permute_chunk(u32x4 v) {
+// Interleave two runs of 4 consecutive 16-bit values (lo0:lo1 and hi0:hi1) so that register r
+// holds (lo[r], hi[r]): the K-slot order of the unpacked B operand.
+__device__ __forceinline__ u32x4 pair_order(uint32_t lo0, uint32_t lo1, uint32_t hi0, uint32_t hi1) {
     u32x4 o;
-    if constexpr (BITS == 4) {
-        o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
-        o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
-        o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
-        o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
-    } else {  // BITS == 8
-        o.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
-        o.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
-        o.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
-        o.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-    }
+    o.x = __builtin_amdgcn_perm(hi0, lo0, 0x05040100u);
+    o.y = __builtin_amdgcn_perm(hi0, lo0, 0x07060302u);
+    o.z = __builtin_amdgcn_perm(hi1, lo1, 0x05040100u);
+    o.w = __builtin_amdgcn_perm(hi1, lo1, 0x07060302u);
     return o;
 }
 
-// Per-column dequant constants of one quantisation group, prepared once per group.
+// Per-column dequant constants of one quantisation group.
 template <bool BF16>
 struct ColMeta;
 template <>
@@ -104,6 +107,15 @@ __device__ __forceinline__ ColMeta<BF16> make_meta(float s, float zp) {
         m.z = half2_t{(half_t)zp, (half_t)zp};
     }
     return m;
+}
+
+__device__ __forceinline__ float fold_zero(float s, float z, int wgm) {
+    switch (wgm) {
+        case GLA_WGM_SHIFT: return -z;
+        case GLA_WGM_SHIFT_SCALE: return -z * s;
+        case GLA_WGM_FMA: return z;
+        default: return 0.0f;
+    }
 }
 
 // pair register holding (OFF + q_lo, OFF + q_hi) -> dequantised pair in the activation type
@@ -130,18 +142,31 @@ __device__ __forceinline__ float16_t mfma32(const u32x4& a, const u32x4& b, floa
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
 }
 
-// BITS in {2, 4, 8}; WAVES_M in {1, 2, 4}
-template <int BITS, bool BF16, int WAVES_M>
-__global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWnArgs p) {
+// s_waitcnt vmcnt(N) only: vmcnt is bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "no wait"
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// BITS in {2, 4, 8}; WAVES_M in {1, 2, 4}; TI = 32-row MFMA tiles per wave (1 or 2)
+template <int BITS, bool BF16, int WAVES_M, int TI>
+__global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_wn_kernel(GemmWnArgs p) {
     constexpr int E = 32 / BITS;
-    constexpr int BM = WAVES_M * 64;
-    constexpr int NT = WAVES_M * kWavesNw * 64;
-    constexpr int TI = 2, TJ = 4;
-    constexpr int WL = (BITS == 8) ? 8 : 4;             // 128-bit weight loads per lane per stage
-    constexpr int A_CHUNKS = (BM * 8 + NT - 1) / NT;    // 16-byte chunks of A per thread per stage
-    constexpr int STAGE = BM * kRowB;
+    constexpr int WM = 32 * TI;
+    constexpr int BM = WAVES_M * WM;
+    constexpr int NW = WAVES_M * kWavesNw;   // waves
+    constexpr int TJ = 4;
+    constexpr int WL = (BITS == 8) ? 8 : 4;  // 128-bit weight loads per lane per stage
+    constexpr int PF = (BITS == 8) ? 2 : 3;  // stages in flight ahead of the one being multiplied
+    constexpr int RING = PF + 1;             // LDS tiles of A
+    constexpr int STAGE = BM * kRowW;
+    constexpr int A_INSTR = BM / 8;          // copy instructions per stage (8 rows each)
+    constexpr int A_PER_WAVE = (A_INSTR + NW - 1) / NW;
+    constexpr int LPS = A_PER_WAVE + WL;     // vector-memory loads per wave per stage
     constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
     constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
+    static_assert((PF - 1) * LPS < 64, "outstanding loads must fit the vmcnt counter");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -152,74 +177,72 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWn
     tile_coords_wn(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * kBNw;
 
-    // ---- A staging slots
-    int a_off[A_CHUNKS], a_off2[BITS == 2 ? A_CHUNKS : 1], a_dst[A_CHUNKS];
+    // ---- A copies: instruction q = wave + NW i moves rows 8q..8q+7; lane (row l/8, position l%8)
+    // fetches the chunk that belongs at that position of the swizzled row.  A wave with no
+    // instruction of its own (short tiles) repeats the last one: same data to the same place.
+    const uint16_t* a_src[A_PER_WAVE];
+    int a_dst[A_PER_WAVE];
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-        const int id = tid + i * NT, row = id >> 3, c = id & 7;
+    for (int i = 0; i < A_PER_WAVE; ++i) {
+        int q = wave + NW * i;
+        if (q > A_INSTR - 1) q = A_INSTR - 1;
+        const int row = q * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
         int gm = m0 + row;
         if (gm > p.M - 1) gm = p.M - 1;
-        a_off[i] = gm * (int)p.xsm + c * 8;  // element offset
-        // 2-bit words hold 16 K-values: K-slots (j, j+8) need chunk c and its partner c^1 of the block
-        if constexpr (BITS == 2) a_off2[i] = gm * (int)p.xsm + (c ^ 1) * 8;
-        a_dst[i] = row * kRowB + c * 16;
+        a_src[i] = p.x + (int64_t)gm * p.xsm + chunk * 8;
+        a_dst[i] = q * 8 * kRowW;
     }
-    u32x4 a_reg[A_CHUNKS];
-    u32x4 a_reg2[BITS == 2 ? A_CHUNKS : 1];  // partner chunk for the 2-bit slot order
 
     // ---- B stream: lane owns columns n0 + wn*128 + 4*r32 + {0..3}
     int coln = n0 + wn * 128 + r32 * 4;
     const bool col_ok = coln + 3 < p.N;  // N % 4 == 0 is required, so a lane is all-in or all-out
     if (coln > p.N - 4) coln = p.N - 4;
     const uint32_t* wcol = p.w + coln;
-    u32x4 w_reg[WL];
+    u32x4 w_ring[PF][WL];
 
-    auto issue_loads = [&](int k0) {
+    auto issue_a = [&](int kk, int slot) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) {
-            a_reg[i] = *(const u32x4*)(p.x + (size_t)(unsigned)(a_off[i] + k0));
-            if constexpr (BITS == 2) a_reg2[i] = *(const u32x4*)(p.x + (size_t)(unsigned)(a_off2[i] + k0));
-        }
-        const int wr0 = k0 / E;
+        for (int i = 0; i < A_PER_WAVE; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[i] + kk * kBKw),
+                                             (__attribute__((address_space(3))) void*)(smem + slot * STAGE + a_dst[i]),
+                                             16, 0, 0);
+    };
+    auto issue_w = [&](int kk, u32x4(&dst)[WL]) __attribute__((always_inline)) {
+        const int wr0 = kk * (kBKw / E);
 #pragma unroll
         for (int u = 0; u < WL; ++u) {
             int row;
-            if constexpr (BITS == 8) row = wr0 + 4 * (u / 2) + 2 * kb + (u % 2);   // step u/2: rows 4s + 2kb + {0,1}
-            else if constexpr (BITS == 4) row = wr0 + 2 * u + kb;                  // step u: row 2s + kb
-            else row = wr0 + u;                                                    // step u: row s (both K-halves read it)
-            w_reg[u] = *(const u32x4*)(wcol + (int64_t)row * p.wsk);
-        }
-    };
-    auto store_a = [&](int stage) {
-        unsigned char* base = smem + stage * STAGE;
-#pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) {
-            const int id = tid + i * NT;
-            if (A_CHUNKS * NT > BM * 8 && id >= BM * 8) continue;
-            u32x4 o;
-            if constexpr (BITS == 2) {
-                // chunk c of a 16-K block pairs with its partner: even chunk = K 0..7, odd = K 8..15.
-                // destination chunk (kb = c & 1) holds slots (j, j+8), j = 4*kb .. 4*kb+3
-                const bool odd = (id & 1) != 0;
-                const u32x4 lo = odd ? a_reg2[i] : a_reg[i];   // K 0..7 of the block
-                const u32x4 hi = odd ? a_reg[i] : a_reg2[i];   // K 8..15
-                const uint32_t l0 = odd ? lo.z : lo.x, l1 = odd ? lo.w : lo.y;
-                const uint32_t h0 = odd ? hi.z : hi.x, h1 = odd ? hi.w : hi.y;
-                o.x = __builtin_amdgcn_perm(h0, l0, 0x05040100u);
-                o.y = __builtin_amdgcn_perm(h0, l0, 0x07060302u);
-                o.z = __builtin_amdgcn_perm(h1, l1, 0x05040100u);
-                o.w = __builtin_amdgcn_perm(h1, l1, 0x07060302u);
-            } else {
-                o = permute_chunk<BITS>(a_reg[i]);
-            }
-            *(u32x4*)(base + a_dst[i]) = o;
+            if constexpr (BITS == 8) row = wr0 + 4 * (u / 2) + 2 * kb + (u % 2);  // step u/2: rows 4s + 2kb + {0,1}
+            else if constexpr (BITS == 4) row = wr0 + 2 * u + kb;                 // step u: row 2s + kb
+            else row = wr0 + u;                                                   // step u: row s (both K-halves read it)
+            dst[u] = *(const u32x4*)(wcol + (int64_t)row * p.wsk);
         }
     };
 
-    // ---- per-group dequant constants for the lane's 4 columns
-    ColMeta<BF16> meta[TJ];
+    // ---- per-group dequant constants for the lane's 4 columns, fetched one group ahead
     const bool grouped = p.wgm >= GLA_WGM_SCALE || (p.wgm == GLA_WGM_SHIFT && !p.z_scalar);
-    auto load_meta = [&](int g) {
+    const bool fast_meta = grouped && (p.meta_dt == GLA_DT_FP16 || p.meta_dt == GLA_DT_BF16) && !p.z_scalar &&
+                           p.z_dt == p.meta_dt && p.wgm >= GLA_WGM_SHIFT_SCALE;
+    const int n_groups = p.K / p.gs;
+    ColMeta<BF16> meta[TJ];
+    u32x2 raw_s = {0, 0}, raw_z = {0, 0};
+    auto fetch_meta = [&](int g) __attribute__((always_inline)) {  // fast path only: 4 adjacent 16-bit scales and zeros
+        if (g > n_groups - 1) g = n_groups - 1;
+        raw_s = *(const u32x2*)((const uint16_t*)p.scales + (int64_t)g * p.msg + coln);
+        raw_z = *(const u32x2*)((const uint16_t*)p.zeros + (int64_t)g * p.msg + coln);
+    };
+    auto convert_meta = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const uint16_t sv = (uint16_t)((j < 2 ? raw_s.x : raw_s.y) >> (16 * (j & 1)));
+            const uint16_t zv = (uint16_t)((j < 2 ? raw_z.x : raw_z.y) >> (16 * (j & 1)));
+            const float s = p.meta_dt == GLA_DT_BF16 ? bf16_bits_to_float(sv) : half_bits_to_float(sv);
+            const float z = p.meta_dt == GLA_DT_BF16 ? bf16_bits_to_float(zv) : half_bits_to_float(zv);
+            meta[j] = make_meta<BF16>(s, fold_zero(s, z, p.wgm));
+        }
+    };
+    auto load_meta_slow = [&](int g) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
             float s = 1.0f, z = 0.0f;
@@ -227,14 +250,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWn
             if (p.wgm >= GLA_WGM_SCALE) s = load_as_float(p.scales, p.meta_dt, idx);
             if (p.wgm == GLA_WGM_SHIFT || p.wgm >= GLA_WGM_SHIFT_SCALE)
                 z = p.z_scalar ? load_as_float(p.zeros, p.z_dt, 0) : load_as_float(p.zeros, p.z_dt, idx);
-            float zp;
-            switch (p.wgm) {
-                case GLA_WGM_SHIFT: zp = -z; break;
-                case GLA_WGM_SHIFT_SCALE: zp = -z * s; break;
-                case GLA_WGM_FMA: zp = z; break;
-                default: zp = 0.0f; break;
-            }
-            meta[j] = make_meta<BF16>(s, zp);
+            meta[j] = make_meta<BF16>(s, fold_zero(s, z, p.wgm));
         }
     };
 
@@ -249,28 +265,64 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWn
     uint32_t pair_mask = kPairMask, magic = kMagic;
     asm volatile("" : "+s"(pair_mask), "+v"(magic));  // registers, so that v_and_or_b32 is selected
 
-    const int a_row0 = (wm * 64 + r32) * kRowB;
-    const int steps = p.K / kBKw;
-    const int stages_per_group = p.gs / kBKw;  // >= 1, checked on the host
+    const int sw = (r32 >> 1) & 7;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
+    const int a_row0 = (wm * WM + r32) * kRowW;
+    const int total_steps = p.K / kBKw;
+    const int k_first = blockIdx.y * p.sps;  // first stage of this split
+    const int steps = (total_steps - k_first) < p.sps ? (total_steps - k_first) : p.sps;
+    const int spg = p.gs / kBKw;  // stages per group, >= 1 (checked on the host)
 
-    issue_loads(0);
-    load_meta(0);
-    store_a(0);
-    __syncthreads();
-
-#pragma unroll 1
-    for (int k = 0; k < steps; ++k) {
-        const int cur = k & 1;
-        u32x4 wc[WL];
+    // ---- prologue: PF stages in flight
 #pragma unroll
-        for (int u = 0; u < WL; ++u) wc[u] = w_reg[u];
-        if (k + 1 < steps) issue_loads((k + 1) * kBKw);
-        const unsigned char* base = smem + cur * STAGE;
+    for (int u = 0; u < PF; ++u) {
+        if (u < steps) {
+            issue_a(k_first + u, u);
+            issue_w(k_first + u, w_ring[u]);
+        }
+    }
+    if (fast_meta) {
+        fetch_meta(k_first / spg);
+        convert_meta();
+        fetch_meta(k_first / spg + 1);
+    } else {
+        load_meta_slow(grouped ? k_first / spg : 0);
+    }
+
+    // One pipeline step; U = k % PF is the register slot of the stage being multiplied.
+    auto step = [&](int k, auto u_tag) __attribute__((always_inline)) {
+        constexpr int U = decltype(u_tag)::value;
+        const int kk = k_first + k;
+        // Stage k has landed once at most the loads of the stages issued after it are outstanding
+        // (those of stages k+1 .. k+PF-1, fewer at the end of the split).
+        const int later = (steps - 1 - k) < (PF - 1) ? (steps - 1 - k) : (PF - 1);
+        if (later >= 2) wait_vmcnt<(PF >= 3 ? 2 : 0) * LPS>();
+        else if (later == 1) wait_vmcnt<LPS>();
+        else wait_vmcnt<0>();
+        __syncthreads();  // every wave's copies of stage k are in LDS, and every wave is done with stage k-1
+        if (k + PF < steps) issue_a(kk + PF, (k + PF) % RING);  // overwrites the tile of stage k-1
+        const unsigned char* base = smem + (k % RING) * STAGE;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {  // four MFMA K-steps of 16
             u32x4 af[TI];
 #pragma unroll
-            for (int i = 0; i < TI; ++i) af[i] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB + s * 32 + kb * 16);
+            for (int i = 0; i < TI; ++i) {
+                const unsigned char* row = base + a_row0 + i * 32 * kRowW;
+                if constexpr (BITS == 2) {
+                    // a word holds 16 K-values; half kb unpacks slots (j, j + 8), j = 4kb .. 4kb+3
+                    const u32x2 lo = *(const u32x2*)(row + (((2 * s) ^ sw) << 4) + 8 * kb);
+                    const u32x2 hi = *(const u32x2*)(row + (((2 * s + 1) ^ sw) << 4) + 8 * kb);
+                    af[i] = pair_order(lo.x, lo.y, hi.x, hi.y);
+                } else {
+                    const u32x4 v = *(const u32x4*)(row + (((2 * s + kb) ^ sw) << 4));
+                    if constexpr (BITS == 4) af[i] = pair_order(v.x, v.y, v.z, v.w);  // slots (j, j + 4)
+                    else {  // two words of 4 codes: slots (j, j + 2) inside each word
+                        af[i].x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
+                        af[i].y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
+                        af[i].z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
+                        af[i].w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
+                    }
+                }
+            }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
                 u32x4 bq;
@@ -278,14 +330,11 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWn
                 for (int r = 0; r < 4; ++r) {
                     uint32_t t;
                     if constexpr (BITS == 4) {
-                        const uint32_t w = wc[s][j];
-                        t = ((w >> (r * 4)) & pair_mask) | magic;
+                        t = ((w_ring[U][s][j] >> (r * 4)) & pair_mask) | magic;
                     } else if constexpr (BITS == 8) {
-                        const uint32_t w = wc[2 * s + r / 2][j];
-                        t = ((w >> ((r % 2) * 8)) & pair_mask) | magic;
+                        t = ((w_ring[U][2 * s + r / 2][j] >> ((r % 2) * 8)) & pair_mask) | magic;
                     } else {
-                        const uint32_t w = wc[s][j];
-                        t = ((w >> ((4 * kb + r) * 2)) & pair_mask) | magic;
+                        t = ((w_ring[U][s][j] >> ((4 * kb + r) * 2)) & pair_mask) | magic;
                     }
                     bq[r] = dequant_pair<BF16>(t, meta[j]);
                 }
@@ -294,27 +343,52 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWn
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the unpacking of later K-steps from being hoisted (register pressure)
         }
-        if (k + 1 < steps) {
-            store_a(cur ^ 1);
-            if (grouped && ((k + 1) % stages_per_group) == 0) load_meta((k + 1) / stages_per_group);
+        if (k + PF < steps) issue_w(kk + PF, w_ring[U]);
+        if (k + 1 < steps && grouped && ((kk + 1) % spg) == 0) {
+            if (fast_meta) {
+                convert_meta();
+                fetch_meta((kk + 1) / spg + 1);
+            } else {
+                load_meta_slow((kk + 1) / spg);
+            }
         }
-        __syncthreads();
+    };
+
+#pragma unroll 1
+    for (int k = 0; k < steps; k += PF) {
+        step(k, std::integral_constant<int, 0>{});
+        if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
+        if constexpr (PF >= 3) {
+            if (k + 2 < steps) step(k + 2, std::integral_constant<int, 2>{});
+        }
     }
 
     // ---- epilogue: lane holds column 4*r32 + j of tile j, rows 8*(e/4) + 4*kb + e%4 of tile i
     if (!col_ok) return;
+    if (p.S > 1) {  // partial tile; the reduction kernel finishes
+        float* part = p.partials + (size_t)blockIdx.y * p.M * p.N + coln;
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
+                if (m < p.M)
+                    *(float4_t*)(part + (size_t)m * p.N) = float4_t{acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
+            }
+        return;
+    }
     float sb[TJ];
 #pragma unroll
     for (int j = 0; j < TJ; ++j)
         sb[j] = (p.csm & 1) ? load_as_float(p.scales, p.meta_dt, coln + j) : 1.0f;
     const bool row_scale = (p.csm & 2) != 0;
-    auto emit = [&](auto dt_tag) {
+    auto emit = [&](auto dt_tag) __attribute__((always_inline)) {
         constexpr int DT = decltype(dt_tag)::value;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
+                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
                 if (m < p.M) {
                     const float sa = row_scale ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
                     const int64_t o = (int64_t)m * p.osm + coln;
@@ -329,27 +403,85 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) void gemm_wn_kernel(GemmWn
     else emit(std::integral_constant<int, GLA_DT_FP32>{});
 }
 
-template <int BITS, bool BF16, int WAVES_M>
+// Sum the K splits in order, apply the channel scales and store: one thread per 4 adjacent columns.
+__global__ __launch_bounds__(256) void splitk_finish_kernel(GemmWnArgs p) {
+    const int n4 = p.N / 4;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.M * n4) return;
+    const int m = (int)(idx / n4), n = (int)(idx % n4) * 4;
+    const size_t slab = (size_t)p.M * p.N;
+    const float* src = p.partials + (size_t)m * p.N + n;
+    float4_t v = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < p.S; ++s) v += *(const float4_t*)(src + s * slab);
+    const float sa = (p.csm & 2) ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float sb = (p.csm & 1) ? load_as_float(p.scales, p.meta_dt, n + j) : 1.0f;
+        store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n + j, v[j] * (sa * sb));
+    }
+}
+
+template <int BITS, bool BF16, int WAVES_M, int TI>
 int launch_wn(const GemmWnArgs& a, hipStream_t stream) {
-    constexpr int BM = WAVES_M * 64;
-    const size_t smem = 2 * (size_t)BM * kRowB;
+    constexpr int BM = WAVES_M * TI * 32;
+    constexpr int PF = (BITS == 8) ? 2 : 3;
+    const size_t smem = (size_t)(PF + 1) * BM * kRowW;
     static bool configured = false;
-    auto kern = gemm_wn_kernel<BITS, BF16, WAVES_M>;
+    auto kern = gemm_wn_kernel<BITS, BF16, WAVES_M, TI>;
     if (!configured && smem > 48 * 1024) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_wn: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
         configured = true;
     }
-    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n), dim3(WAVES_M * kWavesNw * 64), smem, stream, a);
-    return check_hip(hipGetLastError(), "gemm_wn launch");
+    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(WAVES_M * kWavesNw * 64), smem, stream, a);
+    int rc = check_hip(hipGetLastError(), "gemm_wn launch");
+    if (rc == GLA_OK && a.S > 1) {
+        const int64_t items = (int64_t)a.M * (a.N / 4);
+        hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, a);
+        rc = check_hip(hipGetLastError(), "gemm_wn split-K reduction launch");
+    }
+    return rc;
 }
 
 template <int BITS, bool BF16>
-int launch_wn_m(const GemmWnArgs& a, int waves_m, hipStream_t stream) {
-    if (waves_m == 4) return launch_wn<BITS, BF16, 4>(a, stream);
-    if (waves_m == 2) return launch_wn<BITS, BF16, 2>(a, stream);
-    return launch_wn<BITS, BF16, 1>(a, stream);
+int launch_wn_m(const GemmWnArgs& a, int bm, hipStream_t stream) {
+    if (bm == 256) return launch_wn<BITS, BF16, 4, 2>(a, stream);
+    if (bm == 128) return launch_wn<BITS, BF16, 2, 2>(a, stream);
+    if (bm == 64) return launch_wn<BITS, BF16, 1, 2>(a, stream);
+    return launch_wn<BITS, BF16, 1, 1>(a, stream);
+}
+
+// tile_config encoding: BM (32, 64, 128 or 256; other = chosen here) + 1000 * K splits (0 = chosen here)
+struct WnPlan {
+    int bm, tiles_m, tiles_n, S, sps;
+};
+
+WnPlan wn_plan(const gla_matmul_args& p) {
+    WnPlan g;
+    const int cfg = p.tile_config > 0 ? p.tile_config : 0;
+    g.bm = cfg % 1000;
+    if (!(g.bm == 32 || g.bm == 64 || g.bm == 128 || g.bm == 256))
+        g.bm = p.M > 128 ? 256 : (p.M > 64 ? 128 : (p.M > 32 ? 64 : 32));
+    g.tiles_m = ceil_div(p.M, g.bm);
+    g.tiles_n = ceil_div(p.N, kBNw);
+    const int total_steps = p.K / kBKw;
+    int want = cfg / 1000;
+    if (want <= 0) {
+        // enough workgroups for 256 CUs (two or more each while tiles are small), but no split
+        // shorter than 8 stages (512 K-values) and at most 32 splits
+        const int tiles = g.tiles_m * g.tiles_n;
+        const int target = g.bm >= 128 ? 256 : 512;
+        want = tiles * 2 > target ? 1 : ceil_div(target, tiles);
+        const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
+        if (want > max_s) want = max_s;
+        if (want > 32) want = 32;
+    }
+    if (want > total_steps) want = total_steps;
+    if (want < 1) want = 1;
+    g.sps = ceil_div(total_steps, want);
+    g.S = ceil_div(total_steps, g.sps);
+    return g;
 }
 
 }  // namespace
@@ -368,7 +500,6 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     if (p.x_stride_k != 1 || p.x_stride_m % 8 != 0 || p.out_stride_n != 1) return false;
     if (((uintptr_t)p.w & 15) || ((uintptr_t)p.x & 15)) return false;
     if (p.K % kBKw != 0) return false;
-    if ((int64_t)p.M * p.x_stride_m >= (1ll << 31)) return false;
     const bool uses_scales = p.W_group_mode >= GLA_WGM_SCALE;
     const bool uses_zeros = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
     if (uses_scales && (p.scales == nullptr || p.meta_stride_n != 1)) return false;
@@ -381,7 +512,10 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     return true;
 }
 
-int64_t gemm_wn_workspace_bytes(const gla_matmul_args&) { return 0; }
+int64_t gemm_wn_workspace_bytes(const gla_matmul_args& p) {
+    const WnPlan g = wn_plan(p);
+    return g.S > 1 ? kWsReserved + (int64_t)g.S * p.M * p.N * 4 : 0;
+}
 
 int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream) {
     GemmWnArgs a;
@@ -393,15 +527,23 @@ int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream) {
     a.xsm = p.x_stride_m; a.wsk = p.w_stride_k; a.osm = p.out_stride_m; a.msg = p.meta_stride_g; a.sxm = p.sx_stride_m;
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.z_scalar = p.zero_is_scalar; a.out_dt = p.output_dtype; a.sx_dt = p.sx_dtype;
-    int waves_m = p.tile_config > 0 ? p.tile_config : (p.M > 128 ? 4 : (p.M > 64 ? 2 : 1));
-    if (!(waves_m == 1 || waves_m == 2 || waves_m == 4)) waves_m = 4;
-    a.tiles_m = ceil_div(p.M, waves_m * 64);
-    a.tiles_n = ceil_div(p.N, kBNw);
+    const WnPlan g = wn_plan(p);
+    a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps;
+    a.partials = nullptr;
+    if (g.S > 1) {
+        const int64_t need = gemm_wn_workspace_bytes(p);
+        if (p.workspace == nullptr || (int64_t)p.workspace_bytes < need) {
+            set_error("gemm_wn: workspace of %lld bytes required, %llu given", (long long)need,
+                      (unsigned long long)p.workspace_bytes);
+            return GLA_ERR_WORKSPACE_TOO_SMALL;
+        }
+        a.partials = (float*)((char*)p.workspace + kWsReserved);
+    }
     const bool bf16 = p.input_dtype == GLA_DT_BF16;
     switch (p.W_nbits) {
-        case 2: return bf16 ? launch_wn_m<2, true>(a, waves_m, stream) : launch_wn_m<2, false>(a, waves_m, stream);
-        case 4: return bf16 ? launch_wn_m<4, true>(a, waves_m, stream) : launch_wn_m<4, false>(a, waves_m, stream);
-        default: return launch_wn_m<8, false>(a, waves_m, stream);
+        case 2: return bf16 ? launch_wn_m<2, true>(a, g.bm, stream) : launch_wn_m<2, false>(a, g.bm, stream);
+        case 4: return bf16 ? launch_wn_m<4, true>(a, g.bm, stream) : launch_wn_m<4, false>(a, g.bm, stream);
+        default: return launch_wn_m<8, false>(a, g.bm, stream);
     }
 }
 
