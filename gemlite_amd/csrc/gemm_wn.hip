@@ -20,7 +20,7 @@
 //    PF + 1 tiles with dense 128-byte rows whose 16-byte chunks are XOR-swizzled by (row >> 1) & 7;
 //    the reordering of each chunk to the K-slot order the unpacking produces happens when a
 //    fragment is read (v_perm).
-//  * Scales / zero points of the next quantisation group are fetched one group ahead.
+//  * Scales and zero points ride along with every stage (one dword copy per lane).
 //  * When the output has too few tiles to fill the chip (small M), K is split over gridDim.y:
 //    every split writes an fp32 partial tile to the workspace and a second small kernel on the
 //    same stream sums the splits in order, applies the channel scales and stores the output
@@ -149,6 +149,11 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// LDS ring of pipeline stages: as many as fit with two workgroups per CU where the tile is small.
+constexpr int ring_slots(int bm) { return bm >= 128 ? 3 : 4; }
+// One ring slot: A tile, weight words of both wave columns, scales and zeros of the 256 columns.
+constexpr int slot_bytes(int bits, int bm) { return bm * kRowW + 2 * (bits == 8 ? 8 : 4) * 1024 + 1024; }
+
 // BITS in {2, 4, 8}; WAVES_M in {1, 2, 4}; TI = 32-row MFMA tiles per wave (1 or 2)
 template <int BITS, bool BF16, int WAVES_M, int TI>
 __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_wn_kernel(GemmWnArgs p) {
@@ -158,15 +163,18 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
     constexpr int NW = WAVES_M * kWavesNw;   // waves
     constexpr int TJ = 4;
     constexpr int WL = (BITS == 8) ? 8 : 4;  // 128-bit weight loads per lane per stage
-    constexpr int PF = (BITS == 8) ? 2 : 3;  // stages in flight ahead of the one being multiplied
-    constexpr int RING = PF + 1;             // LDS tiles of A
-    constexpr int STAGE = BM * kRowW;
-    constexpr int A_INSTR = BM / 8;          // copy instructions per stage (8 rows each)
-    constexpr int A_PER_WAVE = (A_INSTR + NW - 1) / NW;
-    constexpr int LPS = A_PER_WAVE + WL;     // vector-memory loads per wave per stage
+    constexpr int RING = ring_slots(BM);
+    constexpr int PF = RING - 1;             // stages in flight ahead of the one being multiplied
+    constexpr int SLOT = slot_bytes(BITS, BM);
+    constexpr int W_OFF = BM * kRowW, S_OFF = W_OFF + 2 * WL * 1024, Z_OFF = S_OFF + 512;
+    constexpr int A_JOBS = BM / 8;           // 16-byte copy instructions for the A tile (8 rows each)
+    constexpr int JOBS16 = A_JOBS + 2 * WL;  // ... and for the weight words (one per load per wave column)
+    constexpr int J16 = (JOBS16 + NW - 1) / NW;  // per wave
+    constexpr int J4 = (4 + NW - 1) / NW;        // 4-byte copy instructions per wave: scales / zeros x 2 wave columns
+    constexpr int LPS = J16 + J4;                // copy instructions per wave per stage
     constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
     constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
-    static_assert((PF - 1) * LPS < 64, "outstanding loads must fit the vmcnt counter");
+    static_assert(PF * LPS < 64, "outstanding copies must fit the vmcnt counter");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -176,81 +184,112 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
     int tm, tn;
     tile_coords_wn(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * kBNw;
-
-    // ---- A copies: instruction q = wave + NW i moves rows 8q..8q+7; lane (row l/8, position l%8)
-    // fetches the chunk that belongs at that position of the swizzled row.  A wave with no
-    // instruction of its own (short tiles) repeats the last one: same data to the same place.
-    const uint16_t* a_src[A_PER_WAVE];
-    int a_dst[A_PER_WAVE];
-#pragma unroll
-    for (int i = 0; i < A_PER_WAVE; ++i) {
-        int q = wave + NW * i;
-        if (q > A_INSTR - 1) q = A_INSTR - 1;
-        const int row = q * 8 + (lane >> 3);
-        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-        int gm = m0 + row;
-        if (gm > p.M - 1) gm = p.M - 1;
-        a_src[i] = p.x + (int64_t)gm * p.xsm + chunk * 8;
-        a_dst[i] = q * 8 * kRowW;
-    }
-
-    // ---- B stream: lane owns columns n0 + wn*128 + 4*r32 + {0..3}
+    // the lane's output columns: n0 + wn*128 + 4*r32 + {0..3}
     int coln = n0 + wn * 128 + r32 * 4;
     const bool col_ok = coln + 3 < p.N;  // N % 4 == 0 is required, so a lane is all-in or all-out
     if (coln > p.N - 4) coln = p.N - 4;
-    const uint32_t* wcol = p.w + coln;
-    u32x4 w_ring[PF][WL];
 
-    auto issue_a = [&](int kk, int slot) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < A_PER_WAVE; ++i)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[i] + kk * kBKw),
-                                             (__attribute__((address_space(3))) void*)(smem + slot * STAGE + a_dst[i]),
-                                             16, 0, 0);
-    };
-    auto issue_w = [&](int kk, u32x4(&dst)[WL]) __attribute__((always_inline)) {
-        const int wr0 = kk * (kBKw / E);
-#pragma unroll
-        for (int u = 0; u < WL; ++u) {
-            int row;
-            if constexpr (BITS == 8) row = wr0 + 4 * (u / 2) + 2 * kb + (u % 2);  // step u/2: rows 4s + 2kb + {0,1}
-            else if constexpr (BITS == 4) row = wr0 + 2 * u + kb;                 // step u: row 2s + kb
-            else row = wr0 + u;                                                   // step u: row s (both K-halves read it)
-            dst[u] = *(const u32x4*)(wcol + (int64_t)row * p.wsk);
-        }
-    };
-
-    // ---- per-group dequant constants for the lane's 4 columns, fetched one group ahead
     const bool grouped = p.wgm >= GLA_WGM_SCALE || (p.wgm == GLA_WGM_SHIFT && !p.z_scalar);
-    const bool fast_meta = grouped && (p.meta_dt == GLA_DT_FP16 || p.meta_dt == GLA_DT_BF16) && !p.z_scalar &&
-                           p.z_dt == p.meta_dt && p.wgm >= GLA_WGM_SHIFT_SCALE;
-    const int n_groups = p.K / p.gs;
-    ColMeta<BF16> meta[TJ];
-    u32x2 raw_s = {0, 0}, raw_z = {0, 0};
-    auto fetch_meta = [&](int g) __attribute__((always_inline)) {  // fast path only: 4 adjacent 16-bit scales and zeros
-        if (g > n_groups - 1) g = n_groups - 1;
-        raw_s = *(const u32x2*)((const uint16_t*)p.scales + (int64_t)g * p.msg + coln);
-        raw_z = *(const u32x2*)((const uint16_t*)p.zeros + (int64_t)g * p.msg + coln);
-    };
-    auto convert_meta = [&]() __attribute__((always_inline)) {
+    const bool has_s = p.wgm >= GLA_WGM_SCALE;
+    const bool has_zt = (p.wgm == GLA_WGM_SHIFT || p.wgm >= GLA_WGM_SHIFT_SCALE) && !p.z_scalar;
+    const float z_const = ((p.wgm == GLA_WGM_SHIFT || p.wgm >= GLA_WGM_SHIFT_SCALE) && p.z_scalar)
+                              ? load_as_float(p.zeros, p.z_dt, 0) : 0.0f;
+
+    // ---- copy plan.  Every operand of a stage reaches LDS through global_load_lds: nothing in the
+    // K loop loads into registers from global memory, so the only waits on the vector-memory
+    // counter are the explicit ones below.  Job q = wave + NW i of a stage (wave-uniform):
+    //   q < A_JOBS          rows 8q..8q+7 of the A tile; lane (row l/8, position l%8) fetches the
+    //                       chunk that belongs at that position of the swizzled row;
+    //   otherwise           load u of wave column c: every lane fetches its own 16 bytes (4 adjacent
+    //                       columns of one word row) into a slot only it and its peers in the other
+    //                       wave rows read back.
+    // A source address is a wave-uniform base that advances per stage plus a 32-bit lane offset.
+    unsigned off16[J16];
+    int dst16[J16];
+    bool is_a16[J16];
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-            const uint16_t sv = (uint16_t)((j < 2 ? raw_s.x : raw_s.y) >> (16 * (j & 1)));
-            const uint16_t zv = (uint16_t)((j < 2 ? raw_z.x : raw_z.y) >> (16 * (j & 1)));
-            const float s = p.meta_dt == GLA_DT_BF16 ? bf16_bits_to_float(sv) : half_bits_to_float(sv);
-            const float z = p.meta_dt == GLA_DT_BF16 ? bf16_bits_to_float(zv) : half_bits_to_float(zv);
-            meta[j] = make_meta<BF16>(s, fold_zero(s, z, p.wgm));
+    for (int i = 0; i < J16; ++i) {
+        int q = wave + NW * i;
+        if (q > JOBS16 - 1) q = JOBS16 - 1;  // surplus jobs repeat the last one: same data, same place
+        is_a16[i] = q < A_JOBS;
+        if (is_a16[i]) {
+            const int row = q * 8 + (lane >> 3);
+            const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+            int gm = m0 + row;
+            if (gm > p.M - 1) gm = p.M - 1;
+            off16[i] = (unsigned)(gm * (int)p.xsm + chunk * 8) * 2u;
+            dst16[i] = q * 8 * kRowW;
+        } else {
+            const int c = (q - A_JOBS) / WL, u = (q - A_JOBS) % WL;
+            int col = n0 + c * 128 + r32 * 4;
+            if (col > p.N - 4) col = p.N - 4;
+            int row;
+            if constexpr (BITS == 8) row = 4 * (u / 2) + 2 * kb + (u % 2);  // K-step u/2: rows 4s + 2kb + {0,1}
+            else if constexpr (BITS == 4) row = 2 * u + kb;                 // K-step u: row 2s + kb
+            else row = u;                                                   // K-step u: row s (both K-halves read it)
+            off16[i] = (unsigned)(col + row * (int)p.wsk) * 4u;
+            dst16[i] = W_OFF + (c * WL + u) * 1024;
+        }
+    }
+    // scales / zeros: job (kind, c) copies the 128 values of wave column c, one dword (2 columns) per lane
+    unsigned off4[J4];
+    int dst4[J4];
+    bool is_z4[J4];
+#pragma unroll
+    for (int i = 0; i < J4; ++i) {
+        int q = wave + NW * i;
+        if (q > 3) q = 3;
+        is_z4[i] = q >= 2;
+        const int c = q & 1;
+        int col = n0 + c * 128 + 2 * lane;
+        if (col > p.N - 2) col = p.N - 2;
+        const bool present = is_z4[i] ? has_zt : has_s;
+        off4[i] = present ? (unsigned)col * 2u : 0u;  // absent: every lane reads the first dword of the weights
+        dst4[i] = (is_z4[i] ? Z_OFF : S_OFF) + c * 256;
+    }
+    const unsigned char* s_base = has_s ? (const unsigned char*)p.scales : (const unsigned char*)p.w;
+    const unsigned char* z_base = has_zt ? (const unsigned char*)p.zeros : (const unsigned char*)p.w;
+    const int64_t s_stride = has_s ? p.msg * 2 : 0, z_stride = has_zt ? p.msg * 2 : 0;  // bytes per group
+    const int64_t w_stage = (int64_t)(kBKw / E) * p.wsk * 4;                              // bytes per stage
+
+    auto issue = [&](int kk, int g, int slot) __attribute__((always_inline)) {
+        unsigned char* base = smem + slot * SLOT;
+        const unsigned char* xk = (const unsigned char*)p.x + (int64_t)kk * (kBKw * 2);
+        const unsigned char* wk = (const unsigned char*)p.w + kk * w_stage;
+#pragma unroll
+        for (int i = 0; i < J16; ++i) {
+            const unsigned char* src = (is_a16[i] ? xk : wk) + off16[i];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)(base + dst16[i]), 16, 0, 0);
+        }
+        const unsigned char* sk = s_base + g * s_stride;
+        const unsigned char* zk = z_base + g * z_stride;
+#pragma unroll
+        for (int i = 0; i < J4; ++i) {
+            const unsigned char* src = (is_z4[i] ? zk : sk) + off4[i];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                             (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
         }
     };
-    auto load_meta_slow = [&](int g) __attribute__((always_inline)) {
+
+    // ---- dequant constants: branch-free; absent scales / zeros are masked to 0 and replaced by
+    // constants, and the zero-point term of every dequant mode is z * (c1 + c2 * s)
+    const bool meta_bf16 = p.meta_dt == GLA_DT_BF16;
+    const uint32_t s_mask = has_s ? 0xffffu : 0u, z_mask = has_zt ? 0xffffu : 0u;
+    const float s_add = has_s ? 0.0f : 1.0f, z_add = has_zt ? 0.0f : z_const;
+    const float c1 = p.wgm == GLA_WGM_SHIFT ? -1.0f : (p.wgm == GLA_WGM_FMA ? 1.0f : 0.0f);
+    const float c2 = p.wgm == GLA_WGM_SHIFT_SCALE ? -1.0f : 0.0f;
+    ColMeta<BF16> meta[TJ];
+    auto convert_meta = [&](u32x2 raw_s, u32x2 raw_z) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-            float s = 1.0f, z = 0.0f;
-            const int64_t idx = (int64_t)g * p.msg + coln + j;
-            if (p.wgm >= GLA_WGM_SCALE) s = load_as_float(p.scales, p.meta_dt, idx);
-            if (p.wgm == GLA_WGM_SHIFT || p.wgm >= GLA_WGM_SHIFT_SCALE)
-                z = p.z_scalar ? load_as_float(p.zeros, p.z_dt, 0) : load_as_float(p.zeros, p.z_dt, idx);
-            meta[j] = make_meta<BF16>(s, fold_zero(s, z, p.wgm));
+            const uint32_t sv = ((j < 2 ? raw_s.x : raw_s.y) >> (16 * (j & 1))) & s_mask;
+            const uint32_t zv = ((j < 2 ? raw_z.x : raw_z.y) >> (16 * (j & 1))) & z_mask;
+            const float s_h = half_bits_to_float((uint16_t)sv), s_b = __builtin_bit_cast(float, sv << 16);
+            const float z_h = half_bits_to_float((uint16_t)zv), z_b = __builtin_bit_cast(float, zv << 16);
+            const float s = (meta_bf16 ? s_b : s_h) + s_add;
+            const float z = (meta_bf16 ? z_b : z_h) + z_add;
+            meta[j] = make_meta<BF16>(s, z * __builtin_fmaf(c2, s, c1));
         }
     };
 
@@ -267,40 +306,47 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
 
     const int sw = (r32 >> 1) & 7;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
     const int a_row0 = (wm * WM + r32) * kRowW;
+    const int w_lane = W_OFF + wn * WL * 1024 + lane * 16;
+    const int m_lane = wn * 256 + r32 * 8;
     const int total_steps = p.K / kBKw;
     const int k_first = blockIdx.y * p.sps;  // first stage of this split
     const int steps = (total_steps - k_first) < p.sps ? (total_steps - k_first) : p.sps;
+    const int kk_last = k_first + steps - 1;
     const int spg = p.gs / kBKw;  // stages per group, >= 1 (checked on the host)
+    const int g_last = grouped ? kk_last / spg : 0;
 
-    // ---- prologue: PF stages in flight
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-        if (u < steps) {
-            issue_a(k_first + u, u);
-            issue_w(k_first + u, w_ring[u]);
+    // stage to copy next and its quantisation group, advanced without a division; past the end of
+    // the split the last stage is copied again so that every step issues the same number of copies
+    int ik = k_first, ig = grouped ? k_first / spg : 0, ic = grouped ? k_first % spg : 0;
+    auto issue_next = [&](int slot) __attribute__((always_inline)) {
+        issue(ik < kk_last ? ik : kk_last, ig < g_last ? ig : g_last, slot);
+        ++ik;
+        ++ic;
+        if (ic == spg) {
+            ic = 0;
+            ++ig;
         }
-    }
-    if (fast_meta) {
-        fetch_meta(k_first / spg);
-        convert_meta();
-        fetch_meta(k_first / spg + 1);
-    } else {
-        load_meta_slow(grouped ? k_first / spg : 0);
-    }
+    };
 
-    // One pipeline step; U = k % PF is the register slot of the stage being multiplied.
-    auto step = [&](int k, auto u_tag) __attribute__((always_inline)) {
-        constexpr int U = decltype(u_tag)::value;
-        const int kk = k_first + k;
-        // Stage k has landed once at most the loads of the stages issued after it are outstanding
-        // (those of stages k+1 .. k+PF-1, fewer at the end of the split).
-        const int later = (steps - 1 - k) < (PF - 1) ? (steps - 1 - k) : (PF - 1);
-        if (later >= 2) wait_vmcnt<(PF >= 3 ? 2 : 0) * LPS>();
-        else if (later == 1) wait_vmcnt<LPS>();
-        else wait_vmcnt<0>();
-        __syncthreads();  // every wave's copies of stage k are in LDS, and every wave is done with stage k-1
-        if (k + PF < steps) issue_a(kk + PF, (k + PF) % RING);  // overwrites the tile of stage k-1
-        const unsigned char* base = smem + (k % RING) * STAGE;
+#pragma unroll
+    for (int u = 0; u < PF; ++u) issue_next(u);
+
+    int slot = 0;  // ring slot of the stage being multiplied
+#pragma unroll 1
+    for (int k = 0; k < steps; ++k) {
+        // copies complete in issue order: once at most those of PF - 1 stages are outstanding, stage k has landed
+        // A bare barrier on purpose: __syncthreads() carries a release fence, which for copies into
+        // LDS means draining the whole counter and with it the pipeline.  Each wave has waited for
+        // its own part of stage k; the barrier makes all parts visible and says that every wave is
+        // done reading stage k-1.  The empty asm statements keep the compiler from moving LDS
+        // accesses across it.
+        wait_vmcnt<(PF - 1) * LPS>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_next(slot == 0 ? RING - 1 : slot - 1);  // overwrites the slot of stage k-1
+        const unsigned char* base = smem + slot * SLOT;
+        convert_meta(*(const u32x2*)(base + S_OFF + m_lane), *(const u32x2*)(base + Z_OFF + m_lane));
 #pragma unroll
         for (int s = 0; s < 4; ++s) {  // four MFMA K-steps of 16
             u32x4 af[TI];
@@ -323,6 +369,13 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
                     }
                 }
             }
+            u32x4 wv[BITS == 8 ? 2 : 1];
+            if constexpr (BITS == 8) {
+                wv[0] = *(const u32x4*)(base + w_lane + (2 * s) * 1024);
+                wv[1] = *(const u32x4*)(base + w_lane + (2 * s + 1) * 1024);
+            } else {
+                wv[0] = *(const u32x4*)(base + w_lane + s * 1024);
+            }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
                 u32x4 bq;
@@ -330,11 +383,11 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
                 for (int r = 0; r < 4; ++r) {
                     uint32_t t;
                     if constexpr (BITS == 4) {
-                        t = ((w_ring[U][s][j] >> (r * 4)) & pair_mask) | magic;
+                        t = ((wv[0][j] >> (r * 4)) & pair_mask) | magic;
                     } else if constexpr (BITS == 8) {
-                        t = ((w_ring[U][2 * s + r / 2][j] >> ((r % 2) * 8)) & pair_mask) | magic;
+                        t = ((wv[r / 2][j] >> ((r % 2) * 8)) & pair_mask) | magic;
                     } else {
-                        t = ((w_ring[U][s][j] >> ((4 * kb + r) * 2)) & pair_mask) | magic;
+                        t = ((wv[0][j] >> ((4 * kb + r) * 2)) & pair_mask) | magic;
                     }
                     bq[r] = dequant_pair<BF16>(t, meta[j]);
                 }
@@ -343,24 +396,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the unpacking of later K-steps from being hoisted (register pressure)
         }
-        if (k + PF < steps) issue_w(kk + PF, w_ring[U]);
-        if (k + 1 < steps && grouped && ((kk + 1) % spg) == 0) {
-            if (fast_meta) {
-                convert_meta();
-                fetch_meta((kk + 1) / spg + 1);
-            } else {
-                load_meta_slow((kk + 1) / spg);
-            }
-        }
-    };
-
-#pragma unroll 1
-    for (int k = 0; k < steps; k += PF) {
-        step(k, std::integral_constant<int, 0>{});
-        if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
-        if constexpr (PF >= 3) {
-            if (k + 2 < steps) step(k + 2, std::integral_constant<int, 2>{});
-        }
+        slot = slot == RING - 1 ? 0 : slot + 1;
     }
 
     // ---- epilogue: lane holds column 4*r32 + j of tile j, rows 8*(e/4) + 4*kb + e%4 of tile i
@@ -424,8 +460,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmWnArgs p) {
 template <int BITS, bool BF16, int WAVES_M, int TI>
 int launch_wn(const GemmWnArgs& a, hipStream_t stream) {
     constexpr int BM = WAVES_M * TI * 32;
-    constexpr int PF = (BITS == 8) ? 2 : 3;
-    const size_t smem = (size_t)(PF + 1) * BM * kRowW;
+    const size_t smem = (size_t)ring_slots(BM) * slot_bytes(BITS, BM);
     static bool configured = false;
     auto kern = gemm_wn_kernel<BITS, BF16, WAVES_M, TI>;
     if (!configured && smem > 48 * 1024) {
@@ -500,6 +535,9 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     if (p.x_stride_k != 1 || p.x_stride_m % 8 != 0 || p.out_stride_n != 1) return false;
     if (((uintptr_t)p.w & 15) || ((uintptr_t)p.x & 15)) return false;
     if (p.K % kBKw != 0) return false;
+    // lane offsets inside the activation and weight arrays are 32-bit
+    if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)(p.K / p.elements_per_sample) * p.w_stride_k >= (1ll << 31))
+        return false;
     const bool uses_scales = p.W_group_mode >= GLA_WGM_SCALE;
     const bool uses_zeros = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
     if (uses_scales && (p.scales == nullptr || p.meta_stride_n != 1)) return false;
@@ -507,6 +545,12 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     if (uses_zeros && !p.zero_is_scalar && p.meta_stride_n != 1) return false;
     const bool grouped = uses_scales || (uses_zeros && !p.zero_is_scalar);
     if (grouped && (p.group_size % kBKw != 0 || p.K % p.group_size != 0)) return false;
+    // scales and tensor zeros are read as four adjacent 16-bit values per lane
+    const bool zeros_tensor = uses_zeros && !p.zero_is_scalar;
+    if ((uses_scales || zeros_tensor) && !(p.meta_dtype == GLA_DT_FP16 || p.meta_dtype == GLA_DT_BF16)) return false;
+    if (zeros_tensor && p.zeros_dtype != p.meta_dtype) return false;
+    if (uses_scales && (((uintptr_t)p.scales & 3) || p.meta_stride_g % 2 != 0)) return false;
+    if (zeros_tensor && (((uintptr_t)p.zeros & 3) || p.meta_stride_g % 2 != 0)) return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
     if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
     return true;
