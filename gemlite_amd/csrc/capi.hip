@@ -139,6 +139,7 @@ Family choose(const gla_matmul_args& p, int type) {
     if (want_gemv) {
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
+        if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // K-major 8-bit operands: the split-K MFMA kernel streams them
         return F_GENERIC;
     }
     if (gemm_wn_eligible(p)) return F_GEMM_WN;
@@ -180,6 +181,7 @@ int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
     switch (choose(*args, resolve_type(*args))) {
         case F_GEMV_PACKED: return gemv_packed_workspace_bytes(*args);
         case F_GEMM_WN: return gemm_wn_workspace_bytes(*args);
+        case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(*args);
         default: return 0;
     }
 }

@@ -27,6 +27,7 @@ int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream);
 // ---- MFMA GEMM on 8-bit operands, both K-contiguous (gemm_8bit.hip) --------
 bool gemm_8bit_eligible(const gla_matmul_args& p);
 int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream);
+int64_t gemm_8bit_workspace_bytes(const gla_matmul_args& p);  // also for the MXFP4 entry
 
 // ---- block-scaled MXFP4 MFMA GEMM (gemm_8bit.hip) -------------------------
 bool gemm_mxfp4_eligible(const gla_matmul_args& p);

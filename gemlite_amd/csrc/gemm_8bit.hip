@@ -10,14 +10,17 @@
 // micro-scaled formats (reference: gemlite/triton_kernels/gemm_kernels.py:285-496 and :509-737,
 // epilogue :471-488, tl.dot_scaled :696).
 //
-//  * Workgroup tile BM x 256, K step of 128 bytes per row (128 fp8/int8 values or 256 fp4
-//    values); 8 waves in a 2 x 4 grid, wave tile (BM/2) x 64 of 32x32 MFMA tiles; the
+//  * Workgroup tile BM x 256, pipeline stage of 64 bytes of K per row (64 fp8/int8 values or 128
+//    fp4 values); 8 waves in a 2 x 4 grid, wave tile (BM/2) x 64 of 32x32 MFMA tiles; the
 //    accumulators stay in registers for the whole K loop.
-//  * Operand tiles are copied global -> LDS by the load unit itself (global_load_lds, 16 bytes
-//    per lane), double-buffered: the copy of step k+1 runs while step k is multiplied, and no
-//    vector register is spent on staging.  The LDS image is dense; 16-byte chunk c of row r is
-//    placed at chunk position c ^ ((r >> 1) & 7), chosen on the global side of the copy, so that
-//    the 16 lanes of one LDS read phase hit 16 distinct bank groups.
+//  * Operand tiles (and the MXFP4 block scales) are copied global -> LDS by the load unit itself
+//    (global_load_lds) into a ring of 4 stages, all in flight: a stage's slot is refilled as soon as
+//    every wave has read its fragments into registers, which happens one step before they are
+//    multiplied (fragments are double-buffered in registers), so LDS latency and the barrier are
+//    hidden behind the MFMAs and the loop waits only for the oldest copy.  The LDS
+//    image is dense; 16-byte chunk c of row r is placed at chunk position c ^ ((r >> 2) & 3),
+//    chosen on the global side of the copy, so that the 16 lanes of one LDS read phase hit 16
+//    distinct bank groups.
 //  * Workgroups are renumbered so that each of the 8 XCDs (one L2 each) works on its own band
 //    of output tiles, and tiles inside a band are visited in groups that share operand panels.
 #include <type_traits>
@@ -34,7 +37,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2 };
 
-constexpr int kRowB8 = 128;  // bytes per LDS row = bytes of K per pipeline step
+constexpr int kRowB8 = 64;  // bytes per LDS row = bytes of K per pipeline stage
 constexpr int kBN = 256;
 constexpr int kWavesM = 2, kWavesN = 4;
 constexpr int kThreads8 = kWavesM * kWavesN * 64;
@@ -49,6 +52,9 @@ struct Gemm8Args {
     int64_t lda, ldb, osm, sxm, msn;
     int csm, meta_dt, sx_dt, out_dt;
     int tiles_m, tiles_n;
+    int S;     // K splits (gridDim.y)
+    int sps;   // pipeline stages per split
+    void* partials;  // [S][M][N] 32-bit accumulators when S > 1
 };
 
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -64,16 +70,34 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
     tn = (t % width) / gsize;
 }
 
+// s_waitcnt vmcnt(N) only: vmcnt is bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "no wait"
+template <int N>
+__device__ __forceinline__ void wait_vmcnt8() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
+constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 ? (bm + kBN) * 4 : 0); }
+
 template <int MODE, int BM>
 __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     constexpr int WM = BM / kWavesM;  // wave tile rows
     constexpr int TI = WM / 32;       // 32-row MFMA tiles per wave along M
     constexpr int TJ = 2;             // 64 columns per wave
-    constexpr int STAGE = (BM + kBN) * kRowB8;
-    constexpr int A_INSTR = BM / 8;        // copy instructions (8 rows each) for the A tile
-    constexpr int INSTR = (BM + kBN) / 8;  // ... for both tiles
-    constexpr int PER_WAVE = INSTR / 8;
     constexpr bool MX = MODE == kMXFP4;
+    constexpr int NW = kWavesM * kWavesN;
+    constexpr int RING = kRing8;
+    constexpr int SLOT = slot_bytes8(MODE, BM);
+    constexpr int B_OFF = BM * kRowB8, S_OFF = (BM + kBN) * kRowB8;
+    constexpr int A_JOBS = BM / 16;           // 16-byte copy instructions for the A tile (16 rows each)
+    constexpr int JOBS16 = A_JOBS + kBN / 16; // ... and the B tile
+    constexpr int J16 = (JOBS16 + NW - 1) / NW;
+    constexpr int JOBS4 = (BM + kBN) / 64;    // MXFP4: 4-byte copies of block scales, 64 rows each
+    constexpr int J4 = MX ? 1 : 0;
+    constexpr int LPS = J16 + J4;             // copy instructions per wave per stage
+    static_assert(RING * LPS < 64, "outstanding copies must fit the vmcnt counter");
+    static_assert(JOBS4 <= NW, "one scale copy per wave");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -83,41 +107,76 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * kBN;
 
-    // ---- global -> LDS copy plan: instruction q = wave + 8 i moves 8 rows of one tile; lane
-    // (row l/8, position l%8) fetches the chunk that belongs at that position of the swizzled row
-    const int crow = lane >> 3, cpos = lane & 7;
-    const uint8_t* g_src[PER_WAVE];
-    int l_off[PER_WAVE], chunk16[PER_WAVE];
+    // ---- copy plan.  Everything a stage needs reaches LDS through global_load_lds, so the K loop
+    // holds no loads into registers and the only waits on the vector-memory counter are the
+    // explicit ones below.  Job q = wave + NW i (wave-uniform) moves 16 rows x 64 bytes of one tile:
+    // lane (row l/4, position l%4) fetches the 16-byte chunk that belongs at that position of the
+    // swizzled row (chunk c of row r sits at position c ^ ((r >> 2) & 3)).  A source address is a
+    // wave-uniform base that advances per stage plus a 32-bit lane offset.
+    unsigned off16[J16];
+    int chunk16[J16], dst16[J16];
+    bool is_a16[J16];
 #pragma unroll
-    for (int i = 0; i < PER_WAVE; ++i) {
-        const int q = wave + 8 * i;  // wave-uniform
-        const bool is_a = q < A_INSTR;
-        const int row8 = (is_a ? q : q - A_INSTR) * 8;
-        const int row = row8 + crow;
-        const int chunk = cpos ^ ((row >> 1) & 7);
-        chunk16[i] = chunk * 16;
-        if (is_a) {
+    for (int i = 0; i < J16; ++i) {
+        int q = wave + NW * i;
+        if (q > JOBS16 - 1) q = JOBS16 - 1;  // surplus jobs repeat the last one: same data, same place
+        is_a16[i] = q < A_JOBS;
+        const int row = (is_a16[i] ? q : q - A_JOBS) * 16 + (lane >> 2);
+        chunk16[i] = ((lane & 3) ^ ((row >> 2) & 3)) * 16;
+        if (is_a16[i]) {
             int gm = m0 + row;
             if (gm > p.M - 1) gm = p.M - 1;
-            g_src[i] = p.a + (int64_t)gm * p.lda + chunk * 16;
-            l_off[i] = row8 * kRowB8;
+            off16[i] = (unsigned)(gm * (int)p.lda);
+            dst16[i] = q * 16 * kRowB8;
         } else {
             int gn = n0 + row;
             if (gn > p.N - 1) gn = p.N - 1;
-            g_src[i] = p.b + (int64_t)gn * p.ldb + chunk * 16;
-            l_off[i] = (BM + row8) * kRowB8;
+            off16[i] = (unsigned)(gn * (int)p.ldb);
+            dst16[i] = B_OFF + (q - A_JOBS) * 16 * kRowB8;
         }
     }
-    // a row's last step may hold fewer than 128 bytes: chunks past the end re-read chunk 0 of the
-    // step (always inside the row) and are never multiplied
-    auto copy_step = [&](int k0, int stage) {
-        const int limit = p.Kb - k0;
+    // MXFP4: job q copies the 4 scale bytes (4 blocks of 32 values) of 64 rows, one row per lane
+    unsigned off4 = 0;
+    int dst4 = 0;
+    bool is_a4 = false;
+    if constexpr (MX) {
+        int q = wave;
+        if (q > JOBS4 - 1) q = JOBS4 - 1;
+        is_a4 = q < BM / 64;
+        if (is_a4) {
+            int gm = m0 + q * 64 + lane;
+            if (gm > p.M - 1) gm = p.M - 1;
+            off4 = (unsigned)(gm * (int)p.sxm);
+        } else {
+            int gn = n0 + (q - BM / 64) * 64 + lane;
+            if (gn > p.N - 1) gn = p.N - 1;
+            off4 = (unsigned)(gn * (int)p.msn);
+        }
+        dst4 = S_OFF + q * 256;
+    }
+
+    const int total_steps = (p.Kb + kRowB8 - 1) / kRowB8;
+    const int k_first = blockIdx.y * p.sps;  // first stage of this split
+    const int steps = (total_steps - k_first) < p.sps ? (total_steps - k_first) : p.sps;
+    // A row's last stage may hold fewer than 64 bytes: chunks past the end re-read chunk 0 of the
+    // stage (always inside the row) and are never multiplied.  Stages past the end of K copy the
+    // last one again so that every step issues the same number of copies.
+    auto issue = [&](int k, int slot) __attribute__((always_inline)) {
+        const int kk = k_first + (k > steps - 1 ? steps - 1 : k);  // absolute stage
+        unsigned char* base = smem + slot * SLOT;
+        const int limit = p.Kb - kk * kRowB8;
+        const uint8_t* ak = p.a + kk * kRowB8;
+        const uint8_t* bk = p.b + kk * kRowB8;
 #pragma unroll
-        for (int i = 0; i < PER_WAVE; ++i) {
-            const uint8_t* src = g_src[i] + k0 - (chunk16[i] < limit ? 0 : chunk16[i]);
+        for (int i = 0; i < J16; ++i) {
+            const uint8_t* src = (is_a16[i] ? ak : bk) + (off16[i] + (unsigned)(chunk16[i] < limit ? chunk16[i] : 0));
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)(smem + stage * STAGE + l_off[i]),
-                                             16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(base + dst16[i]), 16, 0, 0);
+        }
+        if constexpr (MX) {
+            const uint8_t* sk = (is_a4 ? (const uint8_t*)p.scales_x : (const uint8_t*)p.scales) + kk * 4;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4),
+                                             (__attribute__((address_space(3))) void*)(base + dst4), 4, 0, 0);
         }
     };
 
@@ -132,125 +191,151 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
     const int r32 = lane & 31, kb = lane >> 5;
-    const int sw = (r32 >> 1) & 7;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
+    const int sw = (r32 >> 2) & 3;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
+    // the two 16-byte chunks of a 64-byte row this lane feeds to the MFMAs of a stage:
+    // fp8 (one K-step of 64 bytes): chunks 2kb, 2kb+1; int8 / fp4 (two K-steps of 32 bytes): chunks kb, 2+kb
+    const int c0 = ((MODE == kFP8 ? 2 * kb : kb) ^ sw) << 4;
+    const int c1 = ((MODE == kFP8 ? 2 * kb + 1 : 2 + kb) ^ sw) << 4;
     const int a_row0 = (wm * WM + r32) * kRowB8;
-    const int b_row0 = (BM + wn * 64 + r32) * kRowB8;
+    const int b_row0 = B_OFF + (wn * 64 + r32) * kRowB8;
+    const int sa_row0 = S_OFF + (wm * WM + r32) * 4;
+    const int sb_row0 = S_OFF + (BM + wn * 64 + r32) * 4;
 
-    // ---- MXFP4 block scales: 8 bytes (8 blocks of 32) per row per step, fetched one step ahead
-    u32x2 sa_next[MX ? TI : 1], sb_next[MX ? TJ : 1];
-    const uint8_t* sa_ptr[MX ? TI : 1];
-    const uint8_t* sb_ptr[MX ? TJ : 1];
-    if constexpr (MX) {
-#pragma unroll
-        for (int i = 0; i < TI; ++i) {
-            int gm = m0 + wm * WM + i * 32 + r32;
-            if (gm > p.M - 1) gm = p.M - 1;
-            sa_ptr[i] = (const uint8_t*)p.scales_x + (int64_t)gm * p.sxm;
-        }
+    // Operand fragments are double-buffered in registers: while the MFMAs of stage k run on one
+    // set, the LDS reads of stage k+1 fill the other, so neither LDS latency nor the barrier
+    // leaves the matrix pipe idle.
+    u32x4 fa[2][TI][2], fb[2][TJ][2];
+    unsigned fsa[2][MX ? TI : 1], fsb[2][MX ? TJ : 1];
+    auto load_frags = [&](int slot, auto buf_tag) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf_tag)::value;
+        const unsigned char* base = smem + slot * SLOT;
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-            int gn = n0 + wn * 64 + j * 32 + r32;
-            if (gn > p.N - 1) gn = p.N - 1;
-            sb_ptr[j] = (const uint8_t*)p.scales + (int64_t)gn * p.msn;
+            fb[B][j][0] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c0);
+            fb[B][j][1] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c1);
         }
-    }
-    auto load_scales = [&](int step) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            fa[B][i][0] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c0);
+            fa[B][i][1] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c1);
+        }
         if constexpr (MX) {
-            const bool upper = p.Kb - step * kRowB8 > 64;  // blocks 4..7 of the step exist
+            // half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2
 #pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                sa_next[i].x = *(const unsigned int*)(sa_ptr[i] + step * 8);
-                sa_next[i].y = upper ? *(const unsigned int*)(sa_ptr[i] + step * 8 + 4) : 0u;
-            }
+            for (int i = 0; i < TI; ++i) fsa[B][i] = *(const unsigned*)(base + sa_row0 + i * 128) >> (8 * kb);
 #pragma unroll
-            for (int j = 0; j < TJ; ++j) {
-                sb_next[j].x = *(const unsigned int*)(sb_ptr[j] + step * 8);
-                sb_next[j].y = upper ? *(const unsigned int*)(sb_ptr[j] + step * 8 + 4) : 0u;
-            }
+            for (int j = 0; j < TJ; ++j) fsb[B][j] = *(const unsigned*)(base + sb_row0 + j * 128) >> (8 * kb);
         }
     };
-
-    // ---- pipeline
-    const int steps = (p.Kb + kRowB8 - 1) / kRowB8;
-    copy_step(0, 0);
-    load_scales(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-#pragma unroll 1
-    for (int k = 0; k < steps; ++k) {
-        const int cur = k & 1;
-        u32x2 sa_cur[MX ? TI : 1], sb_cur[MX ? TJ : 1];
-        if constexpr (MX) {
-            // half-wave kb multiplies blocks kb, 2+kb, 4+kb, 6+kb: shift them into bytes 0 and 2
-#pragma unroll
-            for (int i = 0; i < TI; ++i) sa_cur[i] = u32x2{sa_next[i].x >> (8 * kb), sa_next[i].y >> (8 * kb)};
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) sb_cur[j] = u32x2{sb_next[j].x >> (8 * kb), sb_next[j].y >> (8 * kb)};
-        }
-        if (k + 1 < steps) {
-            copy_step((k + 1) * kRowB8, cur ^ 1);  // that buffer was last read in step k-1
-            load_scales(k + 1);
-        }
-        const unsigned char* base = smem + cur * STAGE;
-        const int limit = p.Kb - k * kRowB8;  // valid bytes of this step (>= 128 except in a ragged tail)
+    auto multiply = [&](int limit, auto buf_tag) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf_tag)::value;
         if constexpr (MODE == kFP8) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {  // two MFMA K-steps of 64 bytes: chunks 4h + 2kb and the next
-                if (h * 64 >= limit) break;
-                const int c0 = ((4 * h + 2 * kb) ^ sw) << 4, c1 = ((4 * h + 2 * kb + 1) ^ sw) << 4;
-                int8_t_v bf[TJ];
+            for (int i = 0; i < TI; ++i) {
+                const u32x4 lo = fa[B][i][0], hi = fa[B][i][1];
+                const int8_t_v af = int8_t_v{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
 #pragma unroll
                 for (int j = 0; j < TJ; ++j) {
-                    const u32x4 lo = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c0);
-                    const u32x4 hi = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c1);
-                    bf[j] = int8_t_v{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-                }
-#pragma unroll
-                for (int i = 0; i < TI; ++i) {
-                    const u32x4 lo = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c0);
-                    const u32x4 hi = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c1);
-                    const int8_t_v af = int8_t_v{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-#pragma unroll
-                    for (int j = 0; j < TJ; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af, bf[j], acc[i][j], 0, 0, 0, 127, 0, 127);
+                    const u32x4 bl = fb[B][j][0], bh = fb[B][j][1];
+                    const int8_t_v bf = int8_t_v{(int)bl.x, (int)bl.y, (int)bl.z, (int)bl.w, (int)bh.x, (int)bh.y, (int)bh.z, (int)bh.w};
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af, bf, acc[i][j], 0, 0, 0, 127, 0, 127);
                 }
             }
         } else {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {  // four MFMA K-steps of 32 bytes: chunk 2s + kb
+            for (int s = 0; s < 2; ++s) {  // two MFMA K-steps of 32 bytes
                 if (s * 32 >= limit) break;
-                const int c0 = ((2 * s + kb) ^ sw) << 4;
-                u32x4 bf[TJ];
-#pragma unroll
-                for (int j = 0; j < TJ; ++j) bf[j] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c0);
 #pragma unroll
                 for (int i = 0; i < TI; ++i) {
-                    const u32x4 af = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c0);
+                    const u32x4 af = fa[B][i][s];
 #pragma unroll
                     for (int j = 0; j < TJ; ++j) {
+                        const u32x4 bf = fb[B][j][s];
                         if constexpr (MODE == kINT8) {
                             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
                                 int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w},
-                                int4_t{(int)bf[j].x, (int)bf[j].y, (int)bf[j].z, (int)bf[j].w}, acc[i][j], 0, 0, 0);
+                                int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w}, acc[i][j], 0, 0, 0);
                         } else {
-                            const int8_t_v a8 = int8_t_v{(int)af.x, (int)af.y, (int)af.z, (int)af.w, 0, 0, 0, 0};
-                            const int8_t_v b8 = int8_t_v{(int)bf[j].x, (int)bf[j].y, (int)bf[j].z, (int)bf[j].w, 0, 0, 0, 0};
-                            const int sa = (int)((s < 2) ? sa_cur[i].x : sa_cur[i].y);
-                            const int sb = (int)((s < 2) ? sb_cur[j].x : sb_cur[j].y);
+                            // fp4 operands occupy the first four of the eight operand registers; the rest is not read
+                            const int4_t a4 = int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w};
+                            const int4_t b4 = int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w};
+                            const int8_t_v a8 = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
+                            const int8_t_v b8 = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
                             if (s & 1)
-                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 4, 4, 2, sa, 2, sb);
+                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 4, 4, 2, (int)fsa[B][i], 2, (int)fsb[B][j]);
                             else
-                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 4, 4, 0, sa, 0, sb);
+                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 4, 4, 0, (int)fsa[B][i], 0, (int)fsb[B][j]);
                         }
                     }
                 }
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's part of step k+1 has landed
-        __syncthreads();
+    };
+
+    // ---- pipeline.  Copies complete in issue order.  Barriers are bare on purpose (a __syncthreads()
+    // carries a release fence, which for copies into LDS means draining the counter and with it the
+    // pipeline); the empty asm statements pin LDS accesses to their side of a barrier.
+    // DB (fragments double-buffered): RING stages in flight; step k reads stage k+1 into registers
+    // and multiplies stage k, whose slot is refilled first.  Otherwise (MXFP4 with the 256-row tile,
+    // which has no registers to spare): RING - 1 stages in flight; step k reads and multiplies stage k
+    // and refills the slot of stage k-1.
+    constexpr bool DB = !(MX && BM == 256);
+    constexpr int AHEAD = DB ? RING : RING - 1;
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) issue(u, u);
+    if constexpr (DB) {
+        wait_vmcnt8<(RING - 1) * LPS>();  // stage 0 has landed (this wave's part)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();     // ... and everybody else's
+        asm volatile("" ::: "memory");
+        load_frags(0, std::integral_constant<int, 0>{});
+    }
+
+    int slot = 0;  // ring slot of the stage being multiplied
+    auto step = [&](int k, auto buf_tag) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf_tag)::value;
+        // the stage read in this step has landed once at most the copies of the RING - 2 stages issued
+        // after it are outstanding; after the barrier the slot refilled below is no longer read by anyone
+        wait_vmcnt8<(RING - 2) * LPS>();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if constexpr (DB) {
+            issue(k + RING, slot);
+            slot = slot == RING - 1 ? 0 : slot + 1;
+            load_frags(slot, std::integral_constant<int, B ^ 1>{});
+            multiply(p.Kb - (k_first + k) * kRowB8, buf_tag);
+        } else {
+            issue(k + RING - 1, slot == 0 ? RING - 1 : slot - 1);
+            load_frags(slot, std::integral_constant<int, 0>{});
+            multiply(p.Kb - (k_first + k) * kRowB8, std::integral_constant<int, 0>{});
+            slot = slot == RING - 1 ? 0 : slot + 1;
+        }
+    };
+#pragma unroll 1
+    for (int k = 0; k < steps; k += 2) {
+        step(k, std::integral_constant<int, 0>{});
+        if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue: lane holds column r32 of each 32-wide tile, rows 8*(e/4) + 4*kb + e%4
+    if (p.S > 1) {  // partial tile, raw 32-bit accumulators; the reduction kernel finishes
+        typedef typename std::conditional<MODE == kINT8, int32_t, float>::type raw_t;
+        raw_t* part = (raw_t*)p.partials + (size_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
+                if (m >= p.M) continue;
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) {
+                    const int n = n0 + wn * 64 + j * 32 + r32;
+                    if (n < p.N) part[(size_t)m * p.N + n] = acc[i][j][e];
+                }
+            }
+        return;
+    }
     float sb[TJ];
     bool n_ok[TJ];
     const bool col_scale = !MX && (p.csm & 1);
@@ -287,9 +372,32 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     else emit(std::integral_constant<int, GLA_DT_FP32>{});
 }
 
+// Sum the K splits in order (exactly, for integer accumulators), apply the channel scales and store.
+template <bool INT>
+__global__ __launch_bounds__(256) void splitk_finish8_kernel(Gemm8Args p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.M * p.N) return;
+    const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+    const size_t slab = (size_t)p.M * p.N;
+    const int64_t o = (int64_t)m * p.osm + n;
+    float scale = 1.0f;
+    if (p.csm & 1) scale *= load_as_float(p.scales, p.meta_dt, n);
+    if (p.csm & 2) scale *= load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm);
+    if constexpr (INT) {
+        int32_t v = 0;
+        for (int s = 0; s < p.S; ++s) v += ((const int32_t*)p.partials)[s * slab + idx];
+        if (p.out_dt == GLA_DT_INT32) ((int32_t*)p.out)[o] = v;
+        else store_from_float(p.out, p.out_dt, o, (float)v * scale);
+    } else {
+        float v = 0.0f;
+        for (int s = 0; s < p.S; ++s) v += ((const float*)p.partials)[s * slab + idx];
+        store_from_float(p.out, p.out_dt, o, v * scale);
+    }
+}
+
 template <int MODE, int BM>
 int launch_bm(const Gemm8Args& a, hipStream_t stream) {
-    const size_t smem = 2 * (size_t)(BM + kBN) * kRowB8;
+    const size_t smem = (size_t)kRing8 * slot_bytes8(MODE, BM);
     static bool configured = false;  // per instantiation; the attribute is sticky per function
     auto kern = gemm_8bit_kernel<MODE, BM>;
     if (!configured) {
@@ -298,8 +406,17 @@ int launch_bm(const Gemm8Args& a, hipStream_t stream) {
         if (rc != GLA_OK) return rc;
         configured = true;
     }
-    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n), dim3(kThreads8), smem, stream, a);
-    return check_hip(hipGetLastError(), "gemm_8bit launch");
+    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(kThreads8), smem, stream, a);
+    int rc = check_hip(hipGetLastError(), "gemm_8bit launch");
+    if (rc == GLA_OK && a.S > 1) {
+        const int64_t items = (int64_t)a.M * a.N;
+        Gemm8Args f = a;
+        if (MODE == kMXFP4) f.csm = 0;  // block scales were applied inside the MFMAs
+        hipLaunchKernelGGL((splitk_finish8_kernel<MODE == kINT8>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+                           stream, f);
+        rc = check_hip(hipGetLastError(), "gemm_8bit split-K reduction launch");
+    }
+    return rc;
 }
 
 template <int MODE>
@@ -309,10 +426,49 @@ int launch_mode(const Gemm8Args& a, int bm, hipStream_t stream) {
     return launch_bm<MODE, 64>(a, stream);
 }
 
-int pick_bm(int M, int tile_config) {
-    int bm = tile_config > 0 ? tile_config : (M > 128 ? 256 : (M > 64 ? 128 : 64));
-    if (bm != 64 && bm != 128 && bm != 256) bm = 256;
-    return bm;
+// tile_config encoding: BM (64, 128 or 256; other = chosen here) + 1000 * K splits (0 = chosen here)
+struct Plan8 {
+    int bm, tiles_m, tiles_n, S, sps;
+};
+
+constexpr int64_t kWsReserved8 = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
+
+Plan8 plan8(int M, int N, int Kb, int tile_config) {
+    Plan8 g;
+    const int cfg = tile_config > 0 ? tile_config : 0;
+    g.bm = cfg % 1000;
+    if (g.bm != 64 && g.bm != 128 && g.bm != 256) g.bm = M > 128 ? 256 : (M > 64 ? 128 : 64);
+    g.tiles_m = ceil_div(M, g.bm);
+    g.tiles_n = ceil_div(N, kBN);
+    const int total_steps = ceil_div(Kb, kRowB8);
+    int want = cfg / 1000;
+    if (want <= 0) {
+        // one workgroup per CU at least, but no split shorter than 16 stages and at most 16 splits
+        const int tiles = g.tiles_m * g.tiles_n;
+        want = tiles * 2 > 256 ? 1 : ceil_div(256, tiles);
+        const int max_s = total_steps / 16 > 0 ? total_steps / 16 : 1;
+        if (want > max_s) want = max_s;
+        if (want > 16) want = 16;
+    }
+    if (want > total_steps) want = total_steps;
+    if (want < 1) want = 1;
+    g.sps = ceil_div(total_steps, want);
+    g.S = ceil_div(total_steps, g.sps);
+    return g;
+}
+
+int attach_plan(const gla_matmul_args& p, const Plan8& g, Gemm8Args& a) {
+    a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps; a.partials = nullptr;
+    if (g.S > 1) {
+        const int64_t need = kWsReserved8 + (int64_t)g.S * p.M * p.N * 4;
+        if (p.workspace == nullptr || (int64_t)p.workspace_bytes < need) {
+            set_error("gemm_8bit: workspace of %lld bytes required, %llu given", (long long)need,
+                      (unsigned long long)p.workspace_bytes);
+            return GLA_ERR_WORKSPACE_TOO_SMALL;
+        }
+        a.partials = (char*)p.workspace + kWsReserved8;
+    }
+    return GLA_OK;
 }
 
 }  // namespace
@@ -327,6 +483,7 @@ bool gemm_8bit_eligible(const gla_matmul_args& p) {
     if (p.K % (fp8 ? 64 : 32) != 0 || p.x_stride_m % 16 != 0 || p.w_stride_n % 16 != 0) return false;
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
     if (i8 && p.acc_dtype != GLA_DT_INT32) return false;
+    if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
     if (p.output_dtype == GLA_DT_INT32 && !(i8 && p.channel_scale_mode == GLA_CSM_NONE)) return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
     if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
@@ -339,11 +496,17 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype;
-    const int bm = pick_bm(p.M, p.tile_config);
-    a.tiles_n = ceil_div(p.N, kBN);
-    a.tiles_m = ceil_div(p.M, bm);
-    if (p.input_dtype == GLA_DT_INT8) return launch_mode<kINT8>(a, bm, stream);
-    return launch_mode<kFP8>(a, bm, stream);
+    const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
+    const int rc = attach_plan(p, g, a);
+    if (rc != GLA_OK) return rc;
+    if (p.input_dtype == GLA_DT_INT8) return launch_mode<kINT8>(a, g.bm, stream);
+    return launch_mode<kFP8>(a, g.bm, stream);
+}
+
+int64_t gemm_8bit_workspace_bytes(const gla_matmul_args& p) {
+    const bool mx = p.input_dtype == GLA_DT_MXFP4;
+    const Plan8 g = plan8(p.M, p.N, mx ? p.K / 2 : p.K, p.tile_config);
+    return g.S > 1 ? kWsReserved8 + (int64_t)g.S * p.M * p.N * 4 : 0;
 }
 
 // MXFP4 x MXFP4: x is [M, K/2] bytes, w the [K/2, N] view of [N, K/2] bytes, and both e8m0
@@ -359,6 +522,8 @@ bool gemm_mxfp4_eligible(const gla_matmul_args& p) {
     if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15) || ((uintptr_t)p.scales & 3) || ((uintptr_t)p.scales_x & 3))
         return false;
     if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
+    if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
+    if ((int64_t)p.M * p.sx_stride_m >= (1ll << 31) || (int64_t)p.N * p.meta_stride_n >= (1ll << 31)) return false;
     return true;
 }
 
@@ -368,10 +533,10 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
     a.M = p.M; a.N = p.N; a.Kb = p.K / 2; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.csm = 0; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype;
-    const int bm = pick_bm(p.M, p.tile_config);
-    a.tiles_n = ceil_div(p.N, kBN);
-    a.tiles_m = ceil_div(p.M, bm);
-    return launch_mode<kMXFP4>(a, bm, stream);
+    const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
+    const int rc = attach_plan(p, g, a);
+    if (rc != GLA_OK) return rc;
+    return launch_mode<kMXFP4>(a, g.bm, stream);
 }
 
 }  // namespace gla
