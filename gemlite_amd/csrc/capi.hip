@@ -135,15 +135,16 @@ int validate(const gla_matmul_args* p) {
 
 Family choose(const gla_matmul_args& p, int type) {
     if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : F_GENERIC;
-    const bool want_gemv = type <= GLA_MATMUL_GEMV_SPLITK;
-    if (want_gemv) {
+    // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
+    const bool small = type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16;
+    if (small) {
+        // 2-bit codes at more than 4 rows: the streaming kernel's staged variant is slower than the GEMM
+        if (p.W_nbits == 2 && p.M > 4 && gemm_wn_eligible(p)) return F_GEMM_WN;
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
-        if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // K-major 8-bit operands: the split-K MFMA kernel streams them
-        return F_GENERIC;
     }
     if (gemm_wn_eligible(p)) return F_GEMM_WN;
-    if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;
+    if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // also streams K-major 8-bit operands at small M (split-K)
     return F_GENERIC;
 }
 

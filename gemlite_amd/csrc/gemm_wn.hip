@@ -93,7 +93,7 @@ struct ColMeta<false> {
 };
 template <>
 struct ColMeta<true> {
-    float s, z;
+    float s, z;  // s and z' - 128 s in fp32: the offset of the unpacking trick is folded into the constant
 };
 
 template <bool BF16>
@@ -101,7 +101,7 @@ __device__ __forceinline__ ColMeta<BF16> make_meta(float s, float zp) {
     ColMeta<BF16> m;
     if constexpr (BF16) {
         m.s = s;
-        m.z = zp;
+        m.z = __builtin_fmaf(-128.0f, s, zp);
     } else {
         m.s = half2_t{(half_t)s, (half_t)s};
         m.z = half2_t{(half_t)zp, (half_t)zp};
@@ -122,11 +122,13 @@ __device__ __forceinline__ float fold_zero(float s, float z, int wgm) {
 template <bool BF16>
 __device__ __forceinline__ uint32_t dequant_pair(uint32_t t, const ColMeta<BF16>& m) {
     if constexpr (BF16) {
-        // bf16 bits are the top half of an fp32: 128 + q is exact there too
-        const float lo = __builtin_bit_cast(float, t << 16) - 128.0f;
-        const float hi = __builtin_bit_cast(float, t & 0xffff0000u) - 128.0f;
-        const float wl = __builtin_fmaf(lo, m.s, m.z), wh = __builtin_fmaf(hi, m.s, m.z);
-        return (uint32_t)float_to_bf16_bits(wl) | ((uint32_t)float_to_bf16_bits(wh) << 16);
+        // bf16 bits are the top half of an fp32, where 128 + q is exact too; (128 + q) s + (z' - 128 s)
+        // in fp32, then one hardware round-to-nearest-even conversion of the pair
+        const float lo = __builtin_bit_cast(float, t << 16);
+        const float hi = __builtin_bit_cast(float, t & 0xffff0000u);
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        const f32x2 w = {__builtin_fmaf(lo, m.s, m.z), __builtin_fmaf(hi, m.s, m.z)};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2_t));
     } else {
         half2_t q = __builtin_bit_cast(half2_t, t) - half2_t{(half_t)1024.0f, (half_t)1024.0f};
         half2_t w = __builtin_elementwise_fma(q, m.s, m.z);

@@ -488,6 +488,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     using SH = Shape<BITS>;
     constexpr int E = SH::E, LW = SH::LW;
     static_assert(SH::T == 1, "direct variant handles one MFMA K-step per super row");
+    constexpr int RI = RT < 4 ? RT : 4;  // accumulator rows a lane folds
     constexpr int IPB = kBatch / LW;  // wave iterations per batch
     constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
     constexpr float OFF = Magic<BF16>::off;
@@ -515,7 +516,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     int col = n0 + cg * 4;
     if (col > a.N - 4) col = a.N - 4;  // clamped lanes are never stored
     const uint32_t* wbase = a.w + col;
-    int mrow = m0 + (cg & (RT - 1));  // rows >= RT of the A operand may hold anything
+    int mrow = m0 + (RT == 16 ? cg : (cg & (RT - 1)));  // rows >= RT of the A operand may hold anything
     if (mrow > a.M - 1) mrow = a.M - 1;
     const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)mrow * a.xsm;
     const bool fast_meta = (a.meta_dt == GLA_DT_FP16 || a.meta_dt == GLA_DT_BF16) && !a.z_scalar &&
@@ -566,13 +567,13 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
         }
     };
 
-    float acc[4][RT];
+    float acc[4][RI];
     float4_t c[4], csx;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         c[j] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < RT; ++i) acc[j][i] = 0.0f;
+        for (int i = 0; i < RI; ++i) acc[j][i] = 0.0f;
     }
     csx = float4_t{0.f, 0.f, 0.f, 0.f};
     const uint4 ones = make_uint4(Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones);
@@ -666,7 +667,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
 #pragma unroll
-                    for (int i = 0; i < RT; ++i)
+                    for (int i = 0; i < RI; ++i)
                         acc[j][i] = __builtin_fmaf(sj[j], c[j][i], __builtin_fmaf(zj[j], csx[i], acc[j][i]));
                     c[j] = float4_t{0.f, 0.f, 0.f, 0.f};
                 }
@@ -692,7 +693,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
         }
     }
     GLA_STAMP(1);
-    wg_finish<RT, kWaves, RT>(a, acc, red, ticket, tile, split, m0, n0);
+    wg_finish<RT, kWaves, RI>(a, acc, red, ticket, tile, split, m0, n0);
 }
 
 #ifdef GLA_TRACE
@@ -708,7 +709,7 @@ struct Geometry {
 };
 
 // tile_config encoding: (waves per workgroup) * 1000 + (batches of kBatch loads per wave).
-bool geometry(const gla_matmul_args& p, Geometry& g) {
+bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     g.E = 32 / p.W_nbits;
     g.LW = g.E < 8 ? 8 / g.E : 1;
     g.KPS = g.E * g.LW;
@@ -728,7 +729,9 @@ bool geometry(const gla_matmul_args& p, Geometry& g) {
     // one wave, one batch: 4 quarters x kBatch loads of word rows
     g.unit = 4 * kBatch;
     const int units = ceil_div(g.R, g.unit);  // wave-batches along K
-    const int max_waves = (g.RT == 16) ? 4 : 16;  // the cross-wave buffer is [waves][RT][64] floats
+    const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8);
+    // the cross-wave buffer is [waves][RT][64] floats; the staged 16-row kernel runs 4 waves
+    const int max_waves = (g.RT == 16) ? (can_direct ? 8 : 4) : 16;
     int waves, nb;
     if (p.tile_config >= 1000) {
         waves = p.tile_config / 1000;
@@ -756,7 +759,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g) {
         waves = per_wg <= 4 ? 4 : (per_wg <= 8 && max_waves >= 8 ? 8 : max_waves);
         nb = ceil_div(per_wg, waves);
     }
-    g.direct = (g.RT <= 4) && (p.W_nbits == 4 || p.W_nbits == 8);
+    g.direct = can_direct;
     if (g.direct && nb > 1 && waves != 4) {  // the looping direct variant runs 4 waves
         nb *= waves / 4;
         waves = 4;
@@ -791,6 +794,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g) {
     g.S = ceil_div(g.R, g.RW);
     if (g.direct && g.S * g.RW != g.R) {
         // the direct variant has no zero-padded activation slab: a ragged last slab takes the staged kernel
+        if (g.RT == 16 && g.waves > 4) return geometry(p, g, false);
         g.direct = false;
         g.smem = (size_t)(g.RW / g.LW) * g.RT * g.T * 16 + (size_t)g.GW * kTileN * 8 +
                  (size_t)g.waves * g.RT * kTileN * 4;
@@ -803,13 +807,14 @@ bool geometry(const gla_matmul_args& p, Geometry& g) {
 template <int BITS, bool BF16, int RT>
 void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
     dim3 grid(g.tiles * g.S, g.mchunks);
-    if constexpr (RT <= 4 && (BITS == 4 || (BITS == 8 && !BF16))) {
+    if constexpr (BITS == 4 || (BITS == 8 && !BF16)) {
         if (g.direct) {
             if (g.nb > 1)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
-            else if (g.waves == 16)
-                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
-            else if (g.waves == 8)
+            else if (g.waves == 16) {
+                if constexpr (RT <= 4)
+                    hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
+            } else if (g.waves == 8)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 8, false>), grid, dim3(512), g.smem, stream, a);
             else
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, false>), grid, dim3(256), g.smem, stream, a);
