@@ -79,6 +79,95 @@ class Launch:
             raise RuntimeError(self.lib.gla_last_error().decode())
 
 
+def time_us(fn, reps, warm=3):
+    """Average microseconds per call of `fn` on the current stream (events on that stream)."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def extra_points(lib, device):
+    """The other points of the benchmark table, measured briefly (synthetic data, same C ABI):
+    GEMM TFLOP/s at M=4096 for each operand format, activation quantisers, the 4096^2 decode GEMV."""
+    from gemlite_amd import helper
+    out = {}
+    g = torch.Generator(device="cpu").manual_seed(7)
+
+    def prepared(layer, x, scales_x, y):
+        m = layer.get_meta_args()
+        args = _ext.build_matmul_args(
+            x, layer.W_q, layer.scales, layer.zeros, scales_x, y,
+            W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5],
+            output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+            data_contiguous=m[11])
+        need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))
+        if need > 0:
+            ws = _ext.get_workspace(device, need)
+            args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+
+        def run():
+            if lib.gla_matmul(ctypes.byref(args), torch.cuda.current_stream().cuda_stream) != 0:
+                raise RuntimeError(lib.gla_last_error().decode())
+        return run
+
+    def point(name, M, N, K, us, peak_tf):
+        tf = 2.0 * M * N * K / us / 1e6
+        out[name] = {"M": M, "N": N, "K": K, "us": round(us, 1), "TFLOP/s": round(tf, 1),
+                     "frac_of_peak": round(tf / peak_tf, 4), "peak_TFLOP/s": peak_tf}
+
+    # A16W4 gs128 fp16, M = 4096 (fused-dequant MFMA GEMM)
+    M, N, K = 4096, 4096, 4096
+    layer, _ = make_layer(N, K, seed=11, device=device)
+    x = torch.randn((M, K), generator=g).to(torch.float16).to(device)
+    y = torch.empty((M, N), dtype=torch.float16, device=device)
+    point("gemm_a16w4_gs128_fp16", M, N, K, time_us(prepared(layer, x, None, y), 20), 2500.0)
+    del layer, x, y
+
+    # A8W8 fp8 / int8 dynamic, M = 4096, N = K = 8192: activation quantiser + GEMM
+    M, N, K = 4096, 8192, 8192
+    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
+        layer = proc(device=device).from_weights(W)
+        xq, sx = gemlite_amd.scale_activations_per_token(x, wdt)
+        point(f"gemm_a8w8_{name}", M, N, K, time_us(prepared(layer, xq, sx, y), 20), 5000.0)
+        us = time_us(lambda: gemlite_amd.scale_activations_per_token(x, wdt), 20)
+        out[f"actquant_per_token_{name}"] = {"M": M, "K": K, "us": round(us, 1),
+                                            "GB/s": round((M * K * 3 + M * 4) / us / 1e3, 1)}
+        del layer, xq, sx
+    del W, x, y
+
+    # A4W4 MXFP4 dynamic, M = 4096, N = K = 16384
+    M, N, K = 4096, 16384, 16384
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+    lin.weight.data = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
+    del lin
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    xq, sx = gemlite_amd.scale_activations_mxfp4(x)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    point("gemm_a4w4_mxfp4", M, N, K, time_us(prepared(layer, xq, sx, y), 10), 10100.0)
+    us = time_us(lambda: gemlite_amd.scale_activations_mxfp4(x), 20)
+    out["actquant_mxfp4"] = {"M": M, "K": K, "us": round(us, 1),
+                             "GB/s": round((M * K * 2 + M * K // 2 + M * K // 32) / us / 1e3, 1)}
+    # the same layer at M = 1: weight-streaming, HBM-bound
+    x1 = torch.randn((1, K), generator=g).to(torch.bfloat16).to(device)
+    xq1, sx1 = gemlite_amd.scale_activations_mxfp4(x1)
+    y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
+    us = time_us(prepared(layer, xq1, sx1, y1), 50)
+    out["gemv_a4w4_mxfp4_M1"] = {"N": N, "K": K, "us": round(us, 1),
+                                 "GB/s": round((N * K // 2 + N * K // 32 + K // 2 + N * 2) / us / 1e3, 1)}
+    return out
+
+
 def cpu_baseline(host_tensors, x_host, y_gpu, threads):
     """The reference's CPU path (HQQ dequantize + fp32 matmul) as restated in oracle/oracle_c.c,
     timed on this box's host cores on whole steps of the same workload; also the parity check."""
@@ -124,6 +213,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--rotate-gb", type=float, default=3.0, help="total bytes of distinct weight copies")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary benchmark points")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a 256 MiB device copy (a kernel of known traffic, to scale profiler byte counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (the hot path has no cross-GPU work); use --gpus 1")
@@ -216,6 +308,14 @@ def main():
 
     y_gpu = y.float().cpu().numpy()
 
+    if a.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     out = {
         "metric": "A16W4 gs128 GEMV GB/s (%HBM peak) @M=1",
         "value": round(value, 1),
@@ -252,6 +352,17 @@ def main():
             "down_proj_GBps": round(algorithmic_bytes(*SHAPES[1]) / (down_avg * 1e-6) / 1e9, 1),
         },
     }
+
+    # traffic per launch of the dominant kernel as read from the HBM byte counters, when a profile holds it
+    traffic_file = os.path.join(ROOT, "profiles", "gemv_direct_a16w4_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            out["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+
+    if not a.no_extra:
+        del launches, sets, base
+        torch.cuda.empty_cache()
+        out["extra"].update(extra_points(lib, device))
 
     if not a.no_cpu:
         threads = min(os.cpu_count() or 1, 16)
