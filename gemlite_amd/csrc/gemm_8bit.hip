@@ -39,8 +39,7 @@ enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2 };
 
 constexpr int kRowB8 = 64;  // bytes per LDS row = bytes of K per pipeline stage
 constexpr int kBN = 256;
-constexpr int kWavesM = 2, kWavesN = 4;
-constexpr int kThreads8 = kWavesM * kWavesN * 64;
+constexpr int kWavesM = 2;  // wave rows; wave columns WN (4 or 2) are a template parameter
 
 struct Gemm8Args {
     const uint8_t* a;      // [M, Kb] bytes
@@ -77,16 +76,34 @@ __device__ __forceinline__ void wait_vmcnt8() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// Scheduling hint for one pipeline step: spread NR LDS reads evenly between NM MFMAs.  Without it
+// the compiler issues all MFMAs first and all reads after; as the barrier keeps the waves of a
+// workgroup in phase, the matrix pipe and the LDS would then take turns instead of overlapping.
+template <int NM, int NR, int I = 0>
+__device__ __forceinline__ void interleave_mfma_with_lds_reads() {
+    if constexpr (I < NM) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        constexpr int n = NR / NM + (I < NR % NM ? 1 : 0);
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);  // n LDS reads
+        interleave_mfma_with_lds_reads<NM, NR, I + 1>();
+    }
+}
+
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
 constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 ? (bm + kBN) * 4 : 0); }
 
-template <int MODE, int BM>
-__global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
+// WN = wave columns.  4: 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
+// (LDS reads bound the 256-row tile: the LDS returns about 64 bytes per clock and CU to 128-bit reads,
+// and this wave tile reads 1.5 fragments per MFMA.  A 2-column variant with 128 x 128 wave tiles reads
+// a third less but needs the accumulators in AGPRs; the compiler's allocation for it spilled.)
+template <int MODE, int BM, int WN>
+__global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args p) {
     constexpr int WM = BM / kWavesM;  // wave tile rows
     constexpr int TI = WM / 32;       // 32-row MFMA tiles per wave along M
-    constexpr int TJ = 2;             // 64 columns per wave
+    constexpr int WNC = kBN / WN;     // wave tile columns
+    constexpr int TJ = WNC / 32;      // 32-column MFMA tiles per wave along N
     constexpr bool MX = MODE == kMXFP4;
-    constexpr int NW = kWavesM * kWavesN;
+    constexpr int NW = kWavesM * WN;
     constexpr int RING = kRing8;
     constexpr int SLOT = slot_bytes8(MODE, BM);
     constexpr int B_OFF = BM * kRowB8, S_OFF = (BM + kBN) * kRowB8;
@@ -94,15 +111,14 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     constexpr int JOBS16 = A_JOBS + kBN / 16; // ... and the B tile
     constexpr int J16 = (JOBS16 + NW - 1) / NW;
     constexpr int JOBS4 = (BM + kBN) / 64;    // MXFP4: 4-byte copies of block scales, 64 rows each
-    constexpr int J4 = MX ? 1 : 0;
+    constexpr int J4 = MX ? (JOBS4 + NW - 1) / NW : 0;
     constexpr int LPS = J16 + J4;             // copy instructions per wave per stage
     static_assert(RING * LPS < 64, "outstanding copies must fit the vmcnt counter");
-    static_assert(JOBS4 <= NW, "one scale copy per wave");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / kWavesN, wn = wave % kWavesN;
+    const int wm = wave / WN, wn = wave % WN;
     int tm, tn;
     tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * kBN;
@@ -136,23 +152,26 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
         }
     }
     // MXFP4: job q copies the 4 scale bytes (4 blocks of 32 values) of 64 rows, one row per lane
-    unsigned off4 = 0;
-    int dst4 = 0;
-    bool is_a4 = false;
+    unsigned off4[MX ? J4 : 1];
+    int dst4[MX ? J4 : 1];
+    bool is_a4[MX ? J4 : 1];
     if constexpr (MX) {
-        int q = wave;
-        if (q > JOBS4 - 1) q = JOBS4 - 1;
-        is_a4 = q < BM / 64;
-        if (is_a4) {
-            int gm = m0 + q * 64 + lane;
-            if (gm > p.M - 1) gm = p.M - 1;
-            off4 = (unsigned)(gm * (int)p.sxm);
-        } else {
-            int gn = n0 + (q - BM / 64) * 64 + lane;
-            if (gn > p.N - 1) gn = p.N - 1;
-            off4 = (unsigned)(gn * (int)p.msn);
+#pragma unroll
+        for (int i = 0; i < J4; ++i) {
+            int q = wave + NW * i;
+            if (q > JOBS4 - 1) q = JOBS4 - 1;
+            is_a4[i] = q < BM / 64;
+            if (is_a4[i]) {
+                int gm = m0 + q * 64 + lane;
+                if (gm > p.M - 1) gm = p.M - 1;
+                off4[i] = (unsigned)(gm * (int)p.sxm);
+            } else {
+                int gn = n0 + (q - BM / 64) * 64 + lane;
+                if (gn > p.N - 1) gn = p.N - 1;
+                off4[i] = (unsigned)(gn * (int)p.msn);
+            }
+            dst4[i] = S_OFF + q * 256;
         }
-        dst4 = S_OFF + q * 256;
     }
 
     const int total_steps = (p.Kb + kRowB8 - 1) / kRowB8;
@@ -174,9 +193,12 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
                                              (__attribute__((address_space(3))) void*)(base + dst16[i]), 16, 0, 0);
         }
         if constexpr (MX) {
-            const uint8_t* sk = (is_a4 ? (const uint8_t*)p.scales_x : (const uint8_t*)p.scales) + kk * 4;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4),
-                                             (__attribute__((address_space(3))) void*)(base + dst4), 4, 0, 0);
+#pragma unroll
+            for (int i = 0; i < J4; ++i) {
+                const uint8_t* sk = (is_a4[i] ? (const uint8_t*)p.scales_x : (const uint8_t*)p.scales) + kk * 4;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
+                                                 (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
+            }
         }
     };
 
@@ -197,27 +219,32 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     const int c0 = ((MODE == kFP8 ? 2 * kb : kb) ^ sw) << 4;
     const int c1 = ((MODE == kFP8 ? 2 * kb + 1 : 2 + kb) ^ sw) << 4;
     const int a_row0 = (wm * WM + r32) * kRowB8;
-    const int b_row0 = B_OFF + (wn * 64 + r32) * kRowB8;
+    const int b_row0 = B_OFF + (wn * WNC + r32) * kRowB8;
     const int sa_row0 = S_OFF + (wm * WM + r32) * 4;
-    const int sb_row0 = S_OFF + (BM + wn * 64 + r32) * 4;
+    const int sb_row0 = S_OFF + (BM + wn * WNC + r32) * 4;
 
     // Operand fragments are double-buffered in registers: while the MFMAs of stage k run on one
     // set, the LDS reads of stage k+1 fill the other, so neither LDS latency nor the barrier
     // leaves the matrix pipe idle.
-    u32x4 fa[2][TI][2], fb[2][TJ][2];
+    // fp8: the two chunks form the eight-register operand of one MFMA; int8 / fp4: one chunk per K-step
+    typedef union {
+        int8_t_v v8;
+        u32x4 c[2];
+    } frag_t;
+    frag_t fa[2][TI], fb[2][TJ];
     unsigned fsa[2][MX ? TI : 1], fsb[2][MX ? TJ : 1];
     auto load_frags = [&](int slot, auto buf_tag) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
         const unsigned char* base = smem + slot * SLOT;
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-            fb[B][j][0] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c0);
-            fb[B][j][1] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c1);
+            fb[B][j].c[0] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c0);
+            fb[B][j].c[1] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c1);
         }
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
-            fa[B][i][0] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c0);
-            fa[B][i][1] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c1);
+            fa[B][i].c[0] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c0);
+            fa[B][i].c[1] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c1);
         }
         if constexpr (MX) {
             // half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2
@@ -231,26 +258,23 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
         constexpr int B = decltype(buf_tag)::value;
         if constexpr (MODE == kFP8) {
 #pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                const u32x4 lo = fa[B][i][0], hi = fa[B][i][1];
-                const int8_t_v af = int8_t_v{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+            for (int i = 0; i < TI; ++i)
 #pragma unroll
-                for (int j = 0; j < TJ; ++j) {
-                    const u32x4 bl = fb[B][j][0], bh = fb[B][j][1];
-                    const int8_t_v bf = int8_t_v{(int)bl.x, (int)bl.y, (int)bl.z, (int)bl.w, (int)bh.x, (int)bh.y, (int)bh.z, (int)bh.w};
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af, bf, acc[i][j], 0, 0, 0, 127, 0, 127);
-                }
-            }
+                for (int j = 0; j < TJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[B][i].v8, fb[B][j].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
         } else {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {  // two MFMA K-steps of 32 bytes
-                if (s * 32 >= limit) break;
+                // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
+                // must not live across control flow)
+                const bool valid = MODE != kINT8 || s * 32 < limit;
 #pragma unroll
                 for (int i = 0; i < TI; ++i) {
-                    const u32x4 af = fa[B][i][s];
+                    u32x4 af = fa[B][i].c[s];
+                    if (!valid) af = u32x4{0, 0, 0, 0};
 #pragma unroll
                     for (int j = 0; j < TJ; ++j) {
-                        const u32x4 bf = fb[B][j][s];
+                        const u32x4 bf = fb[B][j].c[s];
                         if constexpr (MODE == kINT8) {
                             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
                                 int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w},
@@ -279,7 +303,7 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     // and multiplies stage k, whose slot is refilled first.  Otherwise (MXFP4 with the 256-row tile,
     // which has no registers to spare): RING - 1 stages in flight; step k reads and multiplies stage k
     // and refills the slot of stage k-1.
-    constexpr bool DB = !(MX && BM == 256);
+    constexpr bool DB = !(MX && BM == 256 && WN == 4);
     constexpr int AHEAD = DB ? RING : RING - 1;
 #pragma unroll
     for (int u = 0; u < AHEAD; ++u) issue(u, u);
@@ -305,6 +329,7 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
             slot = slot == RING - 1 ? 0 : slot + 1;
             load_frags(slot, std::integral_constant<int, B ^ 1>{});
             multiply(p.Kb - (k_first + k) * kRowB8, buf_tag);
+            interleave_mfma_with_lds_reads<TI * TJ * (MODE == kFP8 ? 1 : 2), (TI + TJ) * (MX ? 3 : 2)>();
         } else {
             issue(k + RING - 1, slot == 0 ? RING - 1 : slot - 1);
             load_frags(slot, std::integral_constant<int, 0>{});
@@ -330,7 +355,7 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
                 if (m >= p.M) continue;
 #pragma unroll
                 for (int j = 0; j < TJ; ++j) {
-                    const int n = n0 + wn * 64 + j * 32 + r32;
+                    const int n = n0 + wn * WNC + j * 32 + r32;
                     if (n < p.N) part[(size_t)m * p.N + n] = acc[i][j][e];
                 }
             }
@@ -342,7 +367,7 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
     const bool row_scale = !MX && (p.csm & 2);
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
-        const int n = n0 + wn * 64 + j * 32 + r32;
+        const int n = n0 + wn * WNC + j * 32 + r32;
         n_ok[j] = n < p.N;
         sb[j] = (col_scale && n_ok[j]) ? load_as_float(p.scales, p.meta_dt, n) : 1.0f;
     }
@@ -355,7 +380,7 @@ __global__ __launch_bounds__(kThreads8) void gemm_8bit_kernel(Gemm8Args p) {
                 const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
                 if (m < p.M) {
                     const float sa = row_scale ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
-                    const int64_t o = (int64_t)m * p.osm + n0 + wn * 64 + r32;
+                    const int64_t o = (int64_t)m * p.osm + n0 + wn * WNC + r32;
 #pragma unroll
                     for (int j = 0; j < TJ; ++j) {
                         if (!n_ok[j]) continue;
@@ -395,18 +420,18 @@ __global__ __launch_bounds__(256) void splitk_finish8_kernel(Gemm8Args p) {
     }
 }
 
-template <int MODE, int BM>
+template <int MODE, int BM, int WN>
 int launch_bm(const Gemm8Args& a, hipStream_t stream) {
     const size_t smem = (size_t)kRing8 * slot_bytes8(MODE, BM);
     static bool configured = false;  // per instantiation; the attribute is sticky per function
-    auto kern = gemm_8bit_kernel<MODE, BM>;
+    auto kern = gemm_8bit_kernel<MODE, BM, WN>;
     if (!configured) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_8bit: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
         configured = true;
     }
-    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(kThreads8), smem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(kWavesM * WN * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "gemm_8bit launch");
     if (rc == GLA_OK && a.S > 1) {
         const int64_t items = (int64_t)a.M * a.N;
@@ -421,9 +446,9 @@ int launch_bm(const Gemm8Args& a, hipStream_t stream) {
 
 template <int MODE>
 int launch_mode(const Gemm8Args& a, int bm, hipStream_t stream) {
-    if (bm == 256) return launch_bm<MODE, 256>(a, stream);
-    if (bm == 128) return launch_bm<MODE, 128>(a, stream);
-    return launch_bm<MODE, 64>(a, stream);
+    if (bm == 256) return launch_bm<MODE, 256, 4>(a, stream);
+    if (bm == 128) return launch_bm<MODE, 128, 4>(a, stream);
+    return launch_bm<MODE, 64, 4>(a, stream);
 }
 
 // tile_config encoding: BM (64, 128 or 256; other = chosen here) + 1000 * K splits (0 = chosen here)
