@@ -20,6 +20,7 @@ from .core import (
     GemLiteLinearTriton,
     config_key,
     forward_functional,
+    forward_functional_op,
     get_closest_m,
     get_default_gemv,
     get_matmul_type,

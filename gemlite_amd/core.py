@@ -200,6 +200,29 @@ def forward_functional(
     return out
 
 
+# The same function as a torch custom op with a fake (meta) implementation, so that graphs traced
+# by torch.compile can hold it as one opaque node (reference: gemlite/core.py:193-200, :276-285).
+# The module's forward calls the plain function: eager decode steps do not pay the op dispatch.
+def _make_custom_op():
+    try:
+        @torch.library.custom_op("gemlite::forward_functional", mutates_args=())
+        def forward_functional_op(x: Tensor, bias: Optional[Tensor], tensor_args: List[Tensor], meta_args: List[int],
+                                  matmul_type: int = -1) -> Tensor:
+            return forward_functional(x, bias, tensor_args, meta_args, matmul_type)
+
+        @forward_functional_op.register_fake
+        def _(x, bias, tensor_args, meta_args, matmul_type=-1):
+            out_features = tensor_args[0].shape[1]
+            return torch.empty(x.shape[:-1] + (out_features,), device=x.device, dtype=DTYPE_TO_TORCH[int(meta_args[6])])
+
+        return forward_functional_op
+    except Exception:  # the name is taken (the reference package is loaded in this process) or torch is too old
+        return None
+
+
+forward_functional_op = _make_custom_op()
+
+
 # ---------------------------------------------------------------------------
 # module
 # ---------------------------------------------------------------------------

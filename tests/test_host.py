@@ -284,3 +284,20 @@ def test_operand_bounds_are_checked_on_the_host():
         elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
         channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11])
     assert (a.meta_stride_g, a.meta_stride_n) == (1, K // 32) and (a.w_stride_k, a.w_stride_n) == (1, K // 2)
+
+
+def test_custom_op_is_registered_with_a_fake():
+    # the functional forward is also a torch custom op, traceable without running a kernel
+    # (reference: gemlite/core.py:193-200, :276-285)
+    import gemlite_amd
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    op = gemlite_amd.forward_functional_op
+    assert op is not None and hasattr(torch.ops.gemlite, "forward_functional")
+    N, K, M = 64, 128, 3
+    l = GemLiteLinear(4, 64, K, N, DType.FP16, DType.BF16)
+    l.pack(torch.randint(0, 16, (N, K)).to(torch.uint8), torch.ones(N * K // 64, 1).half(), torch.ones(N * K // 64, 1).half())
+    with FakeTensorMode():
+        x = torch.empty((2, M, K), dtype=torch.float16, device="cuda")
+        tensors = [torch.empty(t.shape, dtype=t.dtype, device="cuda") for t in l.get_tensor_args()]
+        y = torch.ops.gemlite.forward_functional(x, None, tensors, l.get_meta_args(), -1)
+        assert y.shape == (2, M, N) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
