@@ -94,8 +94,9 @@ constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode
 
 // WN = wave columns.  4: 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
 // (LDS reads bound the 256-row tile: the LDS returns about 64 bytes per clock and CU to 128-bit reads,
-// and this wave tile reads 1.5 fragments per MFMA.  A 2-column variant with 128 x 128 wave tiles reads
-// a third less but needs the accumulators in AGPRs; the compiler's allocation for it spilled.)
+// and this wave tile reads 1.5 fragments per MFMA.  A 2-column variant (4 waves, 128 x 128 wave tiles,
+// accumulators in AGPRs) reads a third less but, with one wave per SIMD and fragments read in the
+// step that multiplies them, measured slower: 1255 against 1650-1800 TFLOP/s in fp8.)
 template <int MODE, int BM, int WN>
 __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args p) {
     constexpr int WM = BM / kWavesM;  // wave tile rows
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // and multiplies stage k, whose slot is refilled first.  Otherwise (MXFP4 with the 256-row tile,
     // which has no registers to spare): RING - 1 stages in flight; step k reads and multiplies stage k
     // and refills the slot of stage k-1.
-    constexpr bool DB = !(MX && BM == 256 && WN == 4);
+    constexpr bool DB = WN == 4 && !(MX && BM == 256);
     constexpr int AHEAD = DB ? RING : RING - 1;
 #pragma unroll
     for (int u = 0; u < AHEAD; ++u) issue(u, u);
@@ -337,10 +338,15 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             slot = slot == RING - 1 ? 0 : slot + 1;
         }
     };
+    if constexpr (DB) {
 #pragma unroll 1
-    for (int k = 0; k < steps; k += 2) {
-        step(k, std::integral_constant<int, 0>{});
-        if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
+        for (int k = 0; k < steps; k += 2) {  // two steps per trip: the fragment buffers alternate
+            step(k, std::integral_constant<int, 0>{});
+            if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
+        }
+    } else {
+#pragma unroll 1
+        for (int k = 0; k < steps; ++k) step(k, std::integral_constant<int, 0>{});
     }
 
     // ---- epilogue: lane holds column r32 of each 32-wide tile, rows 8*(e/4) + 4*kb + e%4
