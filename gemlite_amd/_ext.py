@@ -87,6 +87,7 @@ SYMBOLS = {
     "gla_get_matmul_type": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "gla_get_closest_m": (ctypes.c_int, [ctypes.c_int]),
     "gla_select_config": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
+    "gla_matmul_family": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),
     "gla_scale_activations_per_token": (
@@ -300,6 +301,17 @@ def matmul(args: MatmulArgs, device: torch.device):
         args.workspace = ws.data_ptr()
         args.workspace_bytes = ws.numel()
     _check(lib.gla_matmul(ctypes.byref(args), _stream_ptr(device)), "gla_matmul")
+
+
+FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4"]
+
+
+def matmul_family(args: MatmulArgs) -> str:
+    """Name of the kernel family ``gla_matmul`` would run for ``args`` (host logic only)."""
+    f = load_library().gla_matmul_family(ctypes.byref(args))
+    if f < 0:
+        _check(f, "gla_matmul_family")
+    return FAMILIES[f]
 
 
 def select_config(args: MatmulArgs) -> int:

@@ -175,6 +175,12 @@ int gla_select_config(const gla_matmul_args* args) {
     return 0;
 }
 
+int gla_matmul_family(const gla_matmul_args* args) {
+    const int rc = validate(args);
+    if (rc != GLA_OK) return rc;
+    return (int)choose(*args, resolve_type(*args));
+}
+
 int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
     const int rc = validate(args);
     if (rc != GLA_OK) return rc;

@@ -96,12 +96,13 @@ struct ColMeta<true> {
     float s, z;  // s and z' - 128 s in fp32: the offset of the unpacking trick is folded into the constant
 };
 
-template <bool BF16>
+// OFF: the offset the unpacking leaves on the codes in the fp32 path (128, or 0 for byte codes)
+template <bool BF16, int OFF = 128>
 __device__ __forceinline__ ColMeta<BF16> make_meta(float s, float zp) {
     ColMeta<BF16> m;
     if constexpr (BF16) {
         m.s = s;
-        m.z = __builtin_fmaf(-128.0f, s, zp);
+        m.z = __builtin_fmaf(-(float)OFF, s, zp);
     } else {
         m.s = half2_t{(half_t)s, (half_t)s};
         m.z = half2_t{(half_t)zp, (half_t)zp};
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
             const float z_h = half_bits_to_float((uint16_t)zv), z_b = __builtin_bit_cast(float, zv << 16);
             const float s = (meta_bf16 ? s_b : s_h) + s_add;
             const float z = (meta_bf16 ? z_b : z_h) + z_add;
-            meta[j] = make_meta<BF16>(s, z * __builtin_fmaf(c2, s, c1));
+            meta[j] = make_meta<BF16, (BITS == 8 ? 0 : 128)>(s, z * __builtin_fmaf(c2, s, c1));
         }
     };
 
@@ -386,6 +387,15 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
                     uint32_t t;
                     if constexpr (BITS == 4) {
                         t = ((wv[0][j] >> (r * 4)) & pair_mask) | magic;
+                    } else if constexpr (BITS == 8 && BF16) {
+                        // 128 + q is not exact in bf16 above 127: convert the two bytes (slots r%2 and
+                        // r%2 + 2 of the word) to fp32 directly, scale there and pack once
+                        const uint32_t w = wv[r / 2][j];
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        const f32x2 f = {__builtin_fmaf((float)((w >> ((r % 2) * 8)) & 0xffu), meta[j].s, meta[j].z),
+                                         __builtin_fmaf((float)((w >> ((r % 2) * 8 + 16)) & 0xffu), meta[j].s, meta[j].z)};
+                        bq[r] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+                        continue;
                     } else if constexpr (BITS == 8) {
                         t = ((wv[r / 2][j] >> ((r % 2) * 8)) & pair_mask) | magic;
                     } else {
@@ -528,7 +538,6 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     if (!(p.W_nbits == 2 || p.W_nbits == 4 || p.W_nbits == 8)) return false;
     if (p.elements_per_sample * p.W_nbits != 32) return false;
     if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16)) return false;
-    if (p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16) return false;  // 128 + q is not exact in bf16 for q > 127
     if (p.acc_dtype != GLA_DT_FP32) return false;
     if (p.W_group_mode < 0 || p.W_group_mode > GLA_WGM_FMA) return false;
     if (p.channel_scale_mode < 0 || p.channel_scale_mode > GLA_CSM_BOTH) return false;
@@ -551,8 +560,9 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     const bool zeros_tensor = uses_zeros && !p.zero_is_scalar;
     if ((uses_scales || zeros_tensor) && !(p.meta_dtype == GLA_DT_FP16 || p.meta_dtype == GLA_DT_BF16)) return false;
     if (zeros_tensor && p.zeros_dtype != p.meta_dtype) return false;
-    if (uses_scales && (((uintptr_t)p.scales & 3) || p.meta_stride_g % 2 != 0)) return false;
-    if (zeros_tensor && (((uintptr_t)p.zeros & 3) || p.meta_stride_g % 2 != 0)) return false;
+    const bool one_group = !grouped || p.group_size == p.K;  // then the stride between groups is never used
+    if (uses_scales && (((uintptr_t)p.scales & 3) || (!one_group && p.meta_stride_g % 2 != 0))) return false;
+    if (zeros_tensor && (((uintptr_t)p.zeros & 3) || (!one_group && p.meta_stride_g % 2 != 0))) return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
     if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
     return true;
@@ -589,7 +599,7 @@ int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream) {
     switch (p.W_nbits) {
         case 2: return bf16 ? launch_wn_m<2, true>(a, g.bm, stream) : launch_wn_m<2, false>(a, g.bm, stream);
         case 4: return bf16 ? launch_wn_m<4, true>(a, g.bm, stream) : launch_wn_m<4, false>(a, g.bm, stream);
-        default: return launch_wn_m<8, false>(a, g.bm, stream);
+        default: return bf16 ? launch_wn_m<8, true>(a, g.bm, stream) : launch_wn_m<8, false>(a, g.bm, stream);
     }
 }
 

@@ -490,8 +490,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     static_assert(SH::T == 1, "direct variant handles one MFMA K-step per super row");
     constexpr int RI = RT < 4 ? RT : 4;  // accumulator rows a lane folds
     constexpr int IPB = kBatch / LW;  // wave iterations per batch
-    constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
-    constexpr float OFF = Magic<BF16>::off;
+    // 8-bit codes with bf16 activations: 128 + q is exact in bf16 only up to q = 127, so a code is fed as
+    // two nibbles, q = lo + 16 hi: one MFMA multiplies x by 128 + lo, a second 16 x by 128 + hi, both into
+    // the same accumulator, which then holds sum x q + 128 * 17 * sum x.
+    constexpr bool SPLIT8 = BITS == 8 && BF16;
+    constexpr uint32_t kPairMask = SPLIT8 ? 0x000F000Fu : ((1u << BITS) - 1u) * 0x00010001u;
+    constexpr float OFF = SPLIT8 ? Magic<BF16>::off * 17.0f : Magic<BF16>::off;
 
     extern __shared__ __align__(16) unsigned char smem[];
     const int nfb = a.nfb;                                        // flush blocks per batch
@@ -645,18 +649,31 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
                 continue;
             }
             csx = mfma16<BF16>(av, ones, csx);
+            uint4 av16 = av;
+            if constexpr (SPLIT8) {
+                // 16 x: add 4 to the exponent of every non-zero bf16 half (zeros and denormals stay)
+                auto times16 = [](uint32_t v) {
+                    const uint32_t lo_nz = (v & 0x00007f80u) ? 0x00000200u : 0u;
+                    const uint32_t hi_nz = (v & 0x7f800000u) ? 0x02000000u : 0u;
+                    return v + (lo_nz | hi_nz);
+                };
+                av16 = make_uint4(times16(av.x), times16(av.y), times16(av.z), times16(av.w));
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                uint32_t bq[4];
+                uint32_t bq[4], bh[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     if constexpr (E == 8) {
                         bq[r] = and_or(pick(b.wr[ii], j) >> (r * BITS), pair_mask, magic);
                     } else {
                         bq[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8), pair_mask, magic);
+                        if constexpr (SPLIT8)
+                            bh[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8 + 4), pair_mask, magic);
                     }
                 }
                 c[j] = mfma16<BF16>(av, make_uint4(bq[0], bq[1], bq[2], bq[3]), c[j]);
+                if constexpr (SPLIT8) c[j] = mfma16<BF16>(av16, make_uint4(bh[0], bh[1], bh[2], bh[3]), c[j]);
             }
             if (((it + 1) & fl_mask) == 0) {
                 const int fbl = (a.FL <= IPB) ? (((ii + 1) >> a.fl_log2) - 1) : 0;
@@ -792,6 +809,9 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
         }
     }
     g.S = ceil_div(g.R, g.RW);
+    // 8-bit codes with bf16 activations exist only in the direct variant (nibble-split MFMAs)
+    const bool split8 = p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16;
+    if (split8 && !(g.direct && g.S * g.RW == g.R)) return false;
     if (g.direct && g.S * g.RW != g.R) {
         // the direct variant has no zero-padded activation slab: a ragged last slab takes the staged kernel
         if (g.RT == 16 && g.waves > 4) return geometry(p, g, false);
@@ -807,7 +827,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
 template <int BITS, bool BF16, int RT>
 void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
     dim3 grid(g.tiles * g.S, g.mchunks);
-    if constexpr (BITS == 4 || (BITS == 8 && !BF16)) {
+    if constexpr (BITS == 4 || BITS == 8) {
         if (g.direct) {
             if (g.nb > 1)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
@@ -860,7 +880,6 @@ bool gemv_packed_eligible(const gla_matmul_args& p) {
     if (!(p.W_nbits == 1 || p.W_nbits == 2 || p.W_nbits == 4 || p.W_nbits == 8)) return false;
     if (p.elements_per_sample * p.W_nbits != 32) return false;
     if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16)) return false;
-    if (p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16) return false;  // 128 + q is not exact in bf16 for q > 127
     if (p.acc_dtype != GLA_DT_FP32) return false;
     if (p.W_group_mode < 0 || p.W_group_mode > GLA_WGM_FMA) return false;
     if (p.channel_scale_mode < 0 || p.channel_scale_mode > GLA_CSM_BOTH) return false;
@@ -879,8 +898,10 @@ bool gemv_packed_eligible(const gla_matmul_args& p) {
     if (uses_zeros && !p.zero_is_scalar && p.meta_stride_n != 1) return false;
     const bool grouped = uses_scales || (uses_zeros && !p.zero_is_scalar);
     if (grouped && (p.group_size < E || p.K % p.group_size != 0)) return false;
-    if (grouped && (((uintptr_t)p.scales & 7) || (uses_zeros && !p.zero_is_scalar && ((uintptr_t)p.zeros & 7)) ||
-                    p.meta_stride_g % 4 != 0))
+    const bool one_group = !grouped || p.group_size == p.K;  // then the stride between groups is never used
+    if (grouped && ((uses_scales && ((uintptr_t)p.scales & 7)) ||
+                    (uses_zeros && !p.zero_is_scalar && ((uintptr_t)p.zeros & 7)) ||
+                    (!one_group && p.meta_stride_g % 4 != 0)))
         return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
     if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;

@@ -144,6 +144,17 @@ int gla_get_closest_m(int M);
  * reference: gemlite/triton_kernels/gemm_kernels.py:31-145). */
 int gla_select_config(const gla_matmul_args* args);
 
+/* Which kernel family gla_matmul would run for a problem: one of GLA_FAMILY_*, or a negative
+ * status.  No counterpart in the reference (its registry maps a matmul type to one Triton class,
+ * gemlite/core.py:57-67); here several families serve one type, and tests and tuners ask which. */
+#define GLA_FAMILY_GENERIC 0      /* layout-agnostic kernel, any mode and stride */
+#define GLA_FAMILY_GEMV_PACKED 1  /* streaming kernels for 32-bit packed codes, up to 16 rows */
+#define GLA_FAMILY_GEMV_KMAJOR 2
+#define GLA_FAMILY_GEMM_WN 3      /* fused-dequant MFMA GEMM for packed 2/4/8-bit codes */
+#define GLA_FAMILY_GEMM_8BIT 4    /* fp8 / int8 MFMA GEMM on K-major operands */
+#define GLA_FAMILY_GEMM_MXFP4 5   /* block-scaled FP4 MFMA GEMM */
+int gla_matmul_family(const gla_matmul_args* args);
+
 /* Scratch bytes gla_matmul needs for these arguments (0 if none).  The scratch
  * must be zero-filled once when it is allocated; the library leaves it zeroed
  * where it needs zeros.  (Plays the role of the reference's pre-zeroed output

@@ -301,3 +301,54 @@ def test_custom_op_is_registered_with_a_fake():
         tensors = [torch.empty(t.shape, dtype=t.dtype, device="cuda") for t in l.get_tensor_args()]
         y = torch.ops.gemlite.forward_functional(x, None, tensors, l.get_meta_args(), -1)
         assert y.shape == (2, M, N) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
+
+
+def _family(layer, M, x_dtype, scales_x=None, x=None):
+    m = layer.get_meta_args()
+    K = layer.in_features
+    if x is None:
+        x = torch.zeros(M, K, dtype=x_dtype)
+    out = torch.zeros(M, layer.out_features, dtype=gemlite_amd.DTYPE_TO_TORCH[m[6]])
+    a = _ext.build_matmul_args(
+        x, layer.W_q, layer.scales, layer.zeros, scales_x, out, W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+        elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
+        channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11])
+    return _ext.matmul_family(a)
+
+
+def test_benchmark_configurations_take_a_tuned_kernel_family():
+    # host logic only: which family gla_matmul would launch (the layout-agnostic kernel is correct but slow,
+    # so none of the benchmark configurations may fall to it)
+    g = torch.Generator().manual_seed(0)
+    N, K = 512, 1024
+    # A16W4 gs128 fp16 (decode and prefill)
+    W_q = torch.randint(0, 16, (N, K), generator=g).to(torch.uint8)
+    s, z = torch.rand(N * K // 128, 1).half(), torch.rand(N * K // 128, 1).half()
+    l = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q, s, z)
+    assert [_family(l, M, torch.float16) for M in (1, 2, 4, 8, 16, 64, 4096)] == ["GEMV_PACKED"] * 5 + ["GEMM_WN"] * 2
+    # A16W8 channel-wise and A16W2 gs64, bf16
+    W8 = torch.randint(0, 256, (N, K), generator=g).to(torch.uint8)
+    l8 = GemLiteLinear(8, K, K, N, DType.BF16, DType.BF16).pack(W8, torch.rand(N, 1).bfloat16(), torch.rand(N, 1).bfloat16())
+    assert (l8.W_group_mode, l8.channel_scale_mode) == (1, 1)
+    assert [_family(l8, M, torch.bfloat16) for M in (1, 16, 64, 512)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN", "GEMM_WN"]
+    l8h = GemLiteLinear(8, K, K, N, DType.FP16, DType.FP16).pack(W8, torch.rand(N, 1).half(), torch.rand(N, 1).half())
+    assert [_family(l8h, M, torch.float16) for M in (1, 16, 64)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN"]
+    W2 = torch.randint(0, 4, (N, K), generator=g).to(torch.uint8)
+    l2 = GemLiteLinear(2, 64, K, N, DType.BF16, DType.BF16).pack(
+        W2, torch.rand(N * K // 64, 1).bfloat16(), torch.rand(N * K // 64, 1).bfloat16())
+    assert [_family(l2, M, torch.bfloat16) for M in (1, 16, 64, 512)] == ["GEMV_PACKED", "GEMM_WN", "GEMM_WN", "GEMM_WN"]
+    # A8W8 fp8 / int8 dynamic and INT8 x INT8 -> INT32
+    Wb = torch.randn(N, K, generator=g).bfloat16() * 0.02
+    for proc, dt in ((gemlite_amd.helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), (gemlite_amd.helper.A8W8_INT8_dynamic, torch.int8)):
+        la = proc(device="cpu").from_weights(Wb)
+        for M in (1, 4096):
+            xq = torch.zeros(M, K, dtype=dt)
+            assert _family(la, M, None, scales_x=torch.ones(M, 1), x=xq) == "GEMM_8BIT"
+    # MXFP4
+    codes = torch.randint(0, 16, (N, K), generator=g).to(torch.uint8)
+    e8 = torch.randint(110, 130, (N, K // 32), generator=g).to(torch.uint8)
+    lm = gemlite_amd.helper.A4W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16).from_weights(codes, scales=e8)
+    for M in (1, 32, 1024):
+        xq = torch.zeros(M, K // 2, dtype=torch.uint8)
+        sx = torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
+        assert _family(lm, M, None, scales_x=sx, x=xq) == "GEMM_MXFP4"
