@@ -227,8 +227,12 @@ __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, 
 
     if (!active) return;
     uint32_t packed = 0;
+    // s is a power of two, so v / s is an exact exponent shift: ldexp gives the same value (signed zeros
+    // and denormal results included) in one instruction instead of a division sequence
+    const int down = 127 - (int)e;
+    (void)s;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) packed |= e2m1_code(v[j] / s) << (4 * j);
+    for (int j = 0; j < 8; ++j) packed |= e2m1_code(__builtin_ldexpf(v[j], down)) << (4 * j);
     *(uint32_t*)(y + (int64_t)row * (K / 2) + k / 2) = packed;
     if ((lane & 3) == 0) scales[(int64_t)row * groups + g] = (uint8_t)e;
 }
