@@ -62,7 +62,7 @@ class Launch:
             x, layer.W_q, layer.scales, layer.zeros, None, out,
             W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5],
             output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
-            data_contiguous=m[11], matmul_type=gemlite_amd.GEMLITE_MATMUL_TYPES_MAPPING["GEMV_REVSPLITK"],
+            data_contiguous=m[11],  # matmul type left to the dispatcher (RevSplit-K up to 4 rows, Split-K GEMM above)
         )
         need = lib.gla_matmul_workspace_bytes(ctypes.byref(self.args))
         if need < 0:
@@ -303,6 +303,38 @@ def main():
 
     up_avg = kernel_avg_us(0)
     down_avg = kernel_avg_us(1)
+
+    # the other batch sizes of the decode configuration (same weights, same rotation, graph replay)
+    def batch_avg_us(M, which, reps=4):
+        N, K = SHAPES[which]
+        xm = torch.randn((M, K), generator=g).to(torch.float16).to(device)
+        om = torch.empty((M, N), dtype=torch.float16, device=device)
+        ls = [Launch(lib, s[which], xm, om, device) for s in sets]
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            for l in ls[:2]:
+                l()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(gr, stream=side):
+                for l in ls:
+                    l()
+            gr.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            for _ in range(reps):
+                gr.replay()
+            e1.record(side)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * copies)
+
+    batch_points = {}
+    if not a.no_extra:
+        for M in (2, 4, 8, 16):
+            for which, name in ((0, "up"), (1, "down")):
+                us = batch_avg_us(M, which)
+                batch_points[f"gemv_mlp_{name}_M{M}"] = {
+                    "us": round(us, 2), "GB/s": round(algorithmic_bytes(*SHAPES[which], M=M) / us / 1e3, 1)}
     kbytes = algorithmic_bytes(*SHAPES[0])
     achieved = kbytes / (up_avg * 1e-6) / 1e9
 
@@ -350,6 +382,7 @@ def main():
         "extra": {
             "down_proj_avg_launch_us": round(down_avg, 3),
             "down_proj_GBps": round(algorithmic_bytes(*SHAPES[1]) / (down_avg * 1e-6) / 1e9, 1),
+            **batch_points,
         },
     }
 
