@@ -138,8 +138,6 @@ Family choose(const gla_matmul_args& p, int type) {
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
     const bool small = type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16;
     if (small) {
-        // 2-bit codes at more than 4 rows: the streaming kernel's staged variant is slower than the GEMM
-        if (p.W_nbits == 2 && p.M > 4 && gemm_wn_eligible(p)) return F_GEMM_WN;
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
     }

@@ -486,8 +486,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
 template <int BITS, bool BF16, int RT, int kWaves, bool LOOP>
 __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     using SH = Shape<BITS>;
-    constexpr int E = SH::E, LW = SH::LW;
-    static_assert(SH::T == 1, "direct variant handles one MFMA K-step per super row");
+    constexpr int E = SH::E, LW = SH::LW, T = SH::T;  // T MFMA K-steps per super row (2 for 2-bit codes)
+    static_assert(BITS == 2 || BITS == 4 || BITS == 8, "direct variant: 2-, 4- and 8-bit codes");
     constexpr int RI = RT < 4 ? RT : 4;  // accumulator rows a lane folds
     constexpr int IPB = kBatch / LW;  // wave iterations per batch
     // 8-bit codes with bf16 activations: 128 + q is exact in bf16 only up to q = 127, so a code is fed as
@@ -528,7 +528,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
 
     struct Batch {
         uint2 sr[2], zr[2];
-        uint4 xr[IPB];
+        uint4 xr[IPB * T];
         uint4 wr[kBatch];
     };
 
@@ -560,8 +560,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
         for (int u = 0; u < IPB; ++u) {
             int row = r0 + (lsr0 + 4 * (ib + u)) * LW;
             if (row > a.R - LW) row = a.R - LW;
-            if (GLA_EXP & 1) b.xr[u] = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);
-            else b.xr[u] = *(const uint4*)(xbase + (int64_t)row * E);
+#pragma unroll
+            for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xbase + (int64_t)row * E + 8 * t);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
@@ -626,54 +626,57 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
 #pragma unroll
         for (int ii = 0; ii < IPB; ++ii) {
             const int it = ib + ii;
-            // activation chunk -> the pair order of the code extraction
-            const uint4 xr = b.xr[ii];
-            uint4 av;
-            if constexpr (E == 8) {  // pairs (j, j + 4)
-                av.x = __builtin_amdgcn_perm(xr.z, xr.x, 0x05040100u);
-                av.y = __builtin_amdgcn_perm(xr.z, xr.x, 0x07060302u);
-                av.z = __builtin_amdgcn_perm(xr.w, xr.y, 0x05040100u);
-                av.w = __builtin_amdgcn_perm(xr.w, xr.y, 0x07060302u);
-            } else {  // two words of 4 codes: pairs (j, j + 2) inside each word
-                av.x = __builtin_amdgcn_perm(xr.y, xr.x, 0x05040100u);
-                av.y = __builtin_amdgcn_perm(xr.y, xr.x, 0x07060302u);
-                av.z = __builtin_amdgcn_perm(xr.w, xr.z, 0x05040100u);
-                av.w = __builtin_amdgcn_perm(xr.w, xr.z, 0x07060302u);
-            }
-            if (GLA_EXP & 2) {
 #pragma unroll
-                for (int u2 = 0; u2 < LW; ++u2) {
-                    const uint4 wq = b.wr[ii * LW + u2];
-                    acc[0][0] += __builtin_bit_cast(float, (wq.x ^ wq.y ^ wq.z ^ wq.w ^ av.x) & 0x3fffffffu);
+            for (int t = 0; t < T; ++t) {
+                // activation chunk -> the pair order of the code extraction
+                uint4 av;
+                if constexpr (E == 16) {  // 16 codes per word: K-step t pairs (4t + r, 4t + r + 8)
+                    const uint4 lo = b.xr[ii * T], hi = b.xr[ii * T + 1];
+                    const uint32_t l0 = t ? lo.z : lo.x, l1 = t ? lo.w : lo.y, h0 = t ? hi.z : hi.x, h1 = t ? hi.w : hi.y;
+                    av.x = __builtin_amdgcn_perm(h0, l0, 0x05040100u);
+                    av.y = __builtin_amdgcn_perm(h0, l0, 0x07060302u);
+                    av.z = __builtin_amdgcn_perm(h1, l1, 0x05040100u);
+                    av.w = __builtin_amdgcn_perm(h1, l1, 0x07060302u);
+                } else if constexpr (E == 8) {  // pairs (j, j + 4)
+                    const uint4 xr = b.xr[ii];
+                    av.x = __builtin_amdgcn_perm(xr.z, xr.x, 0x05040100u);
+                    av.y = __builtin_amdgcn_perm(xr.z, xr.x, 0x07060302u);
+                    av.z = __builtin_amdgcn_perm(xr.w, xr.y, 0x05040100u);
+                    av.w = __builtin_amdgcn_perm(xr.w, xr.y, 0x07060302u);
+                } else {  // two words of 4 codes: pairs (j, j + 2) inside each word
+                    const uint4 xr = b.xr[ii];
+                    av.x = __builtin_amdgcn_perm(xr.y, xr.x, 0x05040100u);
+                    av.y = __builtin_amdgcn_perm(xr.y, xr.x, 0x07060302u);
+                    av.z = __builtin_amdgcn_perm(xr.w, xr.z, 0x05040100u);
+                    av.w = __builtin_amdgcn_perm(xr.w, xr.z, 0x07060302u);
                 }
-                continue;
-            }
-            csx = mfma16<BF16>(av, ones, csx);
-            uint4 av16 = av;
-            if constexpr (SPLIT8) {
-                // 16 x: add 4 to the exponent of every non-zero bf16 half (zeros and denormals stay)
-                auto times16 = [](uint32_t v) {
-                    const uint32_t lo_nz = (v & 0x00007f80u) ? 0x00000200u : 0u;
-                    const uint32_t hi_nz = (v & 0x7f800000u) ? 0x02000000u : 0u;
-                    return v + (lo_nz | hi_nz);
-                };
-                av16 = make_uint4(times16(av.x), times16(av.y), times16(av.z), times16(av.w));
-            }
+                csx = mfma16<BF16>(av, ones, csx);
+                uint4 av16 = av;
+                if constexpr (SPLIT8) {
+                    // 16 x: add 4 to the exponent of every non-zero bf16 half (zeros and denormals stay)
+                    auto times16 = [](uint32_t v) {
+                        const uint32_t lo_nz = (v & 0x00007f80u) ? 0x00000200u : 0u;
+                        const uint32_t hi_nz = (v & 0x7f800000u) ? 0x02000000u : 0u;
+                        return v + (lo_nz | hi_nz);
+                    };
+                    av16 = make_uint4(times16(av.x), times16(av.y), times16(av.z), times16(av.w));
+                }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint32_t bq[4], bh[4];
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t bq[4], bh[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if constexpr (E == 8) {
-                        bq[r] = and_or(pick(b.wr[ii], j) >> (r * BITS), pair_mask, magic);
-                    } else {
-                        bq[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8), pair_mask, magic);
-                        if constexpr (SPLIT8)
-                            bh[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8 + 4), pair_mask, magic);
+                    for (int r = 0; r < 4; ++r) {
+                        if constexpr (E >= 8) {
+                            bq[r] = and_or(pick(b.wr[ii], j) >> ((4 * t + r) * BITS), pair_mask, magic);
+                        } else {
+                            bq[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8), pair_mask, magic);
+                            if constexpr (SPLIT8)
+                                bh[r] = and_or(pick(b.wr[ii * LW + r / 2], j) >> ((r % 2) * 8 + 4), pair_mask, magic);
+                        }
                     }
+                    c[j] = mfma16<BF16>(av, make_uint4(bq[0], bq[1], bq[2], bq[3]), c[j]);
+                    if constexpr (SPLIT8) c[j] = mfma16<BF16>(av16, make_uint4(bh[0], bh[1], bh[2], bh[3]), c[j]);
                 }
-                c[j] = mfma16<BF16>(av, make_uint4(bq[0], bq[1], bq[2], bq[3]), c[j]);
-                if constexpr (SPLIT8) c[j] = mfma16<BF16>(av16, make_uint4(bh[0], bh[1], bh[2], bh[3]), c[j]);
             }
             if (((it + 1) & fl_mask) == 0) {
                 const int fbl = (a.FL <= IPB) ? (((ii + 1) >> a.fl_log2) - 1) : 0;
@@ -746,7 +749,8 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     // one wave, one batch: 4 quarters x kBatch loads of word rows
     g.unit = 4 * kBatch;
     const int units = ceil_div(g.R, g.unit);  // wave-batches along K
-    const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8);
+    // 2-bit codes: direct only for the 16-row tile (up to 4 rows the staged kernel measured a little faster)
+    const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8 || (p.W_nbits == 2 && g.RT == 16));
     // the cross-wave buffer is [waves][RT][64] floats; the staged 16-row kernel runs 4 waves
     const int max_waves = (g.RT == 16) ? (can_direct ? 8 : 4) : 16;
     int waves, nb;
@@ -827,7 +831,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
 template <int BITS, bool BF16, int RT>
 void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
     dim3 grid(g.tiles * g.S, g.mchunks);
-    if constexpr (BITS == 4 || BITS == 8) {
+    if constexpr (BITS == 2 || BITS == 4 || BITS == 8) {
         if (g.direct) {
             if (g.nb > 1)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);

@@ -333,10 +333,11 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
     assert [_family(l8, M, torch.bfloat16) for M in (1, 16, 64, 512)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN", "GEMM_WN"]
     l8h = GemLiteLinear(8, K, K, N, DType.FP16, DType.FP16).pack(W8, torch.rand(N, 1).half(), torch.rand(N, 1).half())
     assert [_family(l8h, M, torch.float16) for M in (1, 16, 64)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN"]
-    W2 = torch.randint(0, 4, (N, K), generator=g).to(torch.uint8)
-    l2 = GemLiteLinear(2, 64, K, N, DType.BF16, DType.BF16).pack(
-        W2, torch.rand(N * K // 64, 1).bfloat16(), torch.rand(N * K // 64, 1).bfloat16())
-    assert [_family(l2, M, torch.bfloat16) for M in (1, 16, 64, 512)] == ["GEMV_PACKED", "GEMM_WN", "GEMM_WN", "GEMM_WN"]
+    K2 = 4096
+    W2 = torch.randint(0, 4, (N, K2), generator=g).to(torch.uint8)
+    l2 = GemLiteLinear(2, 64, K2, N, DType.BF16, DType.BF16).pack(
+        W2, torch.rand(N * K2 // 64, 1).bfloat16(), torch.rand(N * K2 // 64, 1).bfloat16())
+    assert [_family(l2, M, torch.bfloat16) for M in (1, 16, 64, 512)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN", "GEMM_WN"]
     # A8W8 fp8 / int8 dynamic and INT8 x INT8 -> INT32
     Wb = torch.randn(N, K, generator=g).bfloat16() * 0.02
     for proc, dt in ((gemlite_amd.helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), (gemlite_amd.helper.A8W8_INT8_dynamic, torch.int8)):
