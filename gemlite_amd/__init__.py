@@ -39,3 +39,4 @@ from .quant_utils import (
 load_config = GemLiteLinear.load_config
 cache_config = GemLiteLinear.cache_config
 reset_config = GemLiteLinear.reset_config
+from . import tune  # noqa: E402,F401  (offline tile tuner)

@@ -353,3 +353,21 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
         xq = torch.zeros(M, K // 2, dtype=torch.uint8)
         sx = torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
         assert _family(lm, M, None, scales_x=sx, x=xq) == "GEMM_MXFP4"
+
+
+def test_tuner_candidates_and_cache_file_round_trip(tmp_path):
+    from gemlite_amd import tune
+    assert tune.candidate_configs("GEMV_PACKED", 1, 4096)[0] == -1
+    c = tune.candidate_configs("GEMM_WN", 64, 8192)
+    assert c[0] == -1 and 64 + 1000 * 8 in c and all(v == -1 or v % 1000 in (32, 64, 128, 256) for v in c)
+    assert tune.candidate_configs("GENERIC", 1, 64) == [-1]
+    # entries the tuner writes survive cache_config / load_config in the reference's file layout
+    GemLiteLinear.reset_config()
+    key = gemlite_amd.core.config_key(64, 4096, 4096, 128, 8, gemlite_amd.core.get_type_id(1, 4))
+    gemlite_amd.GEMLITE_CONFIG_CACHE.setdefault("GEMM", {})[key] = {"tile_config": 8064, "us": 12.5}
+    f = str(tmp_path / "cfg.json")
+    GemLiteLinear.cache_config(f)
+    GemLiteLinear.reset_config()
+    GemLiteLinear.load_config(f)
+    assert gemlite_amd.core._cached_tile_config("GEMM", key) == 8064
+    GemLiteLinear.reset_config()
