@@ -530,6 +530,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
         uint2 sr[2], zr[2];
         uint4 xr[IPB * T];
         uint4 wr[kBatch];
+        unsigned xvalid;  // bit u: iteration u of the batch lies inside K (a ragged last slab runs past it)
     };
 
     // group (relative to g0w) whose fold closes flush block `fbl` of the batch starting at iteration ib
@@ -556,10 +557,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
                 }
             }
         }
+        b.xvalid = 0;
 #pragma unroll
         for (int u = 0; u < IPB; ++u) {
             int row = r0 + (lsr0 + 4 * (ib + u)) * LW;
-            if (row > a.R - LW) row = a.R - LW;
+            if (row <= a.R - LW) b.xvalid |= 1u << u;
+            else row = a.R - LW;  // loads stay in bounds; the activations are zeroed when they are used
 #pragma unroll
             for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xbase + (int64_t)row * E + 8 * t);
         }
@@ -630,21 +633,23 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
             for (int t = 0; t < T; ++t) {
                 // activation chunk -> the pair order of the code extraction
                 uint4 av;
+                const bool xok = (b.xvalid >> ii) & 1u;
+                const uint4 zero4 = make_uint4(0, 0, 0, 0);
                 if constexpr (E == 16) {  // 16 codes per word: K-step t pairs (4t + r, 4t + r + 8)
-                    const uint4 lo = b.xr[ii * T], hi = b.xr[ii * T + 1];
+                    const uint4 lo = xok ? b.xr[ii * T] : zero4, hi = xok ? b.xr[ii * T + 1] : zero4;
                     const uint32_t l0 = t ? lo.z : lo.x, l1 = t ? lo.w : lo.y, h0 = t ? hi.z : hi.x, h1 = t ? hi.w : hi.y;
                     av.x = __builtin_amdgcn_perm(h0, l0, 0x05040100u);
                     av.y = __builtin_amdgcn_perm(h0, l0, 0x07060302u);
                     av.z = __builtin_amdgcn_perm(h1, l1, 0x05040100u);
                     av.w = __builtin_amdgcn_perm(h1, l1, 0x07060302u);
                 } else if constexpr (E == 8) {  // pairs (j, j + 4)
-                    const uint4 xr = b.xr[ii];
+                    const uint4 xr = xok ? b.xr[ii] : zero4;
                     av.x = __builtin_amdgcn_perm(xr.z, xr.x, 0x05040100u);
                     av.y = __builtin_amdgcn_perm(xr.z, xr.x, 0x07060302u);
                     av.z = __builtin_amdgcn_perm(xr.w, xr.y, 0x05040100u);
                     av.w = __builtin_amdgcn_perm(xr.w, xr.y, 0x07060302u);
                 } else {  // two words of 4 codes: pairs (j, j + 2) inside each word
-                    const uint4 xr = b.xr[ii];
+                    const uint4 xr = xok ? b.xr[ii] : zero4;
                     av.x = __builtin_amdgcn_perm(xr.y, xr.x, 0x05040100u);
                     av.y = __builtin_amdgcn_perm(xr.y, xr.x, 0x07060302u);
                     av.z = __builtin_amdgcn_perm(xr.w, xr.z, 0x05040100u);
@@ -761,22 +766,12 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     } else {
         // Slabs along K: enough workgroups to cover the CUs, and few enough wave-batches per
         // workgroup that every load of the kernel is in flight at once (one batch per wave).
-        int s_min = ceil_div(200, g.tiles * g.mchunks);
+        int s_min = ceil_div(128, g.tiles * g.mchunks);
         if (s_min < 1) s_min = 1;
         int want_s = ceil_div(units, max_waves);
         if (want_s < s_min) want_s = s_min;
         if (want_s > units) want_s = units;
         int per_wg = ceil_div(units, want_s);  // wave-batches per workgroup
-        // prefer a slab count that divides K exactly into 4, 8 or 16 wave-batches (no ragged slab)
-        if (g.R % g.unit == 0) {
-            for (int s2 = want_s; s2 <= units && s2 <= 4 * want_s + 4; ++s2) {
-                const int q = units / s2;
-                if (units % s2 == 0 && (q == 4 || q == 8 || q == 16) && q <= max_waves) {
-                    per_wg = q;
-                    break;
-                }
-            }
-        }
         waves = per_wg <= 4 ? 4 : (per_wg <= 8 && max_waves >= 8 ? 8 : max_waves);
         nb = ceil_div(per_wg, waves);
     }
@@ -815,15 +810,8 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     g.S = ceil_div(g.R, g.RW);
     // 8-bit codes with bf16 activations exist only in the direct variant (nibble-split MFMAs)
     const bool split8 = p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16;
-    if (split8 && !(g.direct && g.S * g.RW == g.R)) return false;
-    if (g.direct && g.S * g.RW != g.R) {
-        // the direct variant has no zero-padded activation slab: a ragged last slab takes the staged kernel
-        if (g.RT == 16 && g.waves > 4) return geometry(p, g, false);
-        g.direct = false;
-        g.smem = (size_t)(g.RW / g.LW) * g.RT * g.T * 16 + (size_t)g.GW * kTileN * 8 +
-                 (size_t)g.waves * g.RT * kTileN * 4;
-        if (g.smem > 60 * 1024) return false;
-    }
+    if (split8 && !g.direct) return false;
+    // a ragged last slab is fine in either variant: rows past K multiply zeroed activations
     if (g.S > 1 && (int64_t)g.tiles * g.mchunks * 4 > kCounterBytes) return false;
     return true;
 }
