@@ -79,7 +79,7 @@ class Launch:
             raise RuntimeError(self.lib.gla_last_error().decode())
 
 
-def time_us(fn, reps, warm=3):
+def time_us(fn, reps, warm=25):
     """Average microseconds per call of `fn` on the current stream (events on that stream)."""
     for _ in range(warm):
         fn()
@@ -127,7 +127,7 @@ def extra_points(lib, device):
     layer, _ = make_layer(N, K, seed=11, device=device)
     x = torch.randn((M, K), generator=g).to(torch.float16).to(device)
     y = torch.empty((M, N), dtype=torch.float16, device=device)
-    point("gemm_a16w4_gs128_fp16", M, N, K, time_us(prepared(layer, x, None, y), 20), 2500.0)
+    point("gemm_a16w4_gs128_fp16", M, N, K, time_us(prepared(layer, x, None, y), 50), 2500.0)
     del layer, x, y
 
     # A8W8 fp8 / int8 dynamic, M = 4096, N = K = 8192: activation quantiser + GEMM
@@ -138,7 +138,7 @@ def extra_points(lib, device):
     for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
         layer = proc(device=device).from_weights(W)
         xq, sx = gemlite_amd.scale_activations_per_token(x, wdt)
-        point(f"gemm_a8w8_{name}", M, N, K, time_us(prepared(layer, xq, sx, y), 20), 5000.0)
+        point(f"gemm_a8w8_{name}", M, N, K, time_us(prepared(layer, xq, sx, y), 50), 5000.0)
         us = time_us(lambda: gemlite_amd.scale_activations_per_token(x, wdt), 20)
         out[f"actquant_per_token_{name}"] = {"M": M, "K": K, "us": round(us, 1),
                                             "GB/s": round((M * K * 3 + M * 4) / us / 1e3, 1)}
@@ -154,7 +154,7 @@ def extra_points(lib, device):
     x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
     xq, sx = gemlite_amd.scale_activations_mxfp4(x)
     y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    point("gemm_a4w4_mxfp4", M, N, K, time_us(prepared(layer, xq, sx, y), 10), 10100.0)
+    point("gemm_a4w4_mxfp4", M, N, K, time_us(prepared(layer, xq, sx, y), 30), 10100.0)
     us = time_us(lambda: gemlite_amd.scale_activations_mxfp4(x), 20)
     out["actquant_mxfp4"] = {"M": M, "K": K, "us": round(us, 1),
                              "GB/s": round((M * K * 2 + M * K // 2 + M * K // 32) / us / 1e3, 1)}

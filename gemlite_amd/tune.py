@@ -81,7 +81,8 @@ def tune_layer(layer: GemLiteLinear, batch_sizes: Iterable[int], reps: int = 20,
                 data_contiguous=m[11], matmul_type=GEMLITE_MATMUL_TYPES_MAPPING[matmul_type], tile_config=tile)
 
         family = _ext.matmul_family(build(-1))
-        timings = []
+        stream = torch.cuda.current_stream(device).cuda_stream
+        runnable = []
         for tile in candidate_configs(family, M, layer.in_features):
             args = build(tile)
             need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))
@@ -90,19 +91,25 @@ def tune_layer(layer: GemLiteLinear, batch_sizes: Iterable[int], reps: int = 20,
             if need > 0:
                 ws = _ext.get_workspace(device, need)
                 args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
-            stream = torch.cuda.current_stream(device).cuda_stream
             if lib.gla_matmul(ctypes.byref(args), stream) != 0:
                 continue
-            torch.cuda.synchronize(device)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(reps):
-                lib.gla_matmul(ctypes.byref(args), stream)
-            e1.record()
-            torch.cuda.synchronize(device)
-            timings.append((e0.elapsed_time(e1) * 1e3 / reps, tile))
-            if verbose:
-                print(f"  M={M} {family} tile={tile}: {timings[-1][0]:.1f} us")
+            runnable.append((tile, args))
+        torch.cuda.synchronize(device)
+        best_of = {}
+        for _ in range(2):  # two rounds over all candidates, best of both: the first timings of a run are slower
+            for tile, args in runnable:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _r in range(reps):
+                    lib.gla_matmul(ctypes.byref(args), stream)
+                e1.record()
+                torch.cuda.synchronize(device)
+                us = e0.elapsed_time(e1) * 1e3 / reps
+                best_of[tile] = min(us, best_of.get(tile, us))
+        timings = [(us, tile) for tile, us in best_of.items()]
+        if verbose:
+            for us, tile in timings:
+                print(f"  M={M} {family} tile={tile}: {us:.1f} us")
         if not timings:
             continue
         base = next((t for t, tile in timings if tile == -1), None)
