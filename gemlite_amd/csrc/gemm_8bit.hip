@@ -76,19 +76,6 @@ __device__ __forceinline__ void wait_vmcnt8() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-// Scheduling hint for one pipeline step: spread NR LDS reads evenly between NM MFMAs.  Without it
-// the compiler issues all MFMAs first and all reads after; as the barrier keeps the waves of a
-// workgroup in phase, the matrix pipe and the LDS would then take turns instead of overlapping.
-template <int NM, int NR, int I = 0>
-__device__ __forceinline__ void interleave_mfma_with_lds_reads() {
-    if constexpr (I < NM) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-        constexpr int n = NR / NM + (I < NR % NM ? 1 : 0);
-        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);  // n LDS reads
-        interleave_mfma_with_lds_reads<NM, NR, I + 1>();
-    }
-}
-
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
 constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 ? (bm + kBN) * 4 : 0); }
 
@@ -181,26 +168,25 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // A row's last stage may hold fewer than 64 bytes: chunks past the end re-read chunk 0 of the
     // stage (always inside the row) and are never multiplied.  Stages past the end of K copy the
     // last one again so that every step issues the same number of copies.
-    auto issue = [&](int k, int slot) __attribute__((always_inline)) {
+    // copy c (0 <= c < LPS) of stage k into ring slot `slot`
+    auto issue_one = [&](int k, int slot, int c) __attribute__((always_inline)) {
         const int kk = k_first + (k > steps - 1 ? steps - 1 : k);  // absolute stage
         unsigned char* base = smem + slot * SLOT;
-        const int limit = p.Kb - kk * kRowB8;
-        const uint8_t* ak = p.a + kk * kRowB8;
-        const uint8_t* bk = p.b + kk * kRowB8;
-#pragma unroll
-        for (int i = 0; i < J16; ++i) {
-            const uint8_t* src = (is_a16[i] ? ak : bk) + (off16[i] + (unsigned)(chunk16[i] < limit ? chunk16[i] : 0));
+        if (c < J16) {
+            const int limit = p.Kb - kk * kRowB8;
+            const uint8_t* src = (is_a16[c] ? p.a : p.b) + kk * kRowB8 + (off16[c] + (unsigned)(chunk16[c] < limit ? chunk16[c] : 0));
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)(base + dst16[i]), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(base + dst16[c]), 16, 0, 0);
+        } else if constexpr (MX) {
+            const int i = c - J16;
+            const uint8_t* sk = (is_a4[i] ? (const uint8_t*)p.scales_x : (const uint8_t*)p.scales) + kk * 4;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
+                                             (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
         }
-        if constexpr (MX) {
+    };
+    auto issue = [&](int k, int slot) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < J4; ++i) {
-                const uint8_t* sk = (is_a4[i] ? (const uint8_t*)p.scales_x : (const uint8_t*)p.scales) + kk * 4;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
-                                                 (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
-            }
-        }
+        for (int c = 0; c < LPS; ++c) issue_one(k, slot, c);
     };
 
     // ---- accumulators
@@ -234,65 +220,55 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     } frag_t;
     frag_t fa[2][TI], fb[2][TJ];
     unsigned fsa[2][MX ? TI : 1], fsb[2][MX ? TJ : 1];
-    auto load_frags = [&](int slot, auto buf_tag) __attribute__((always_inline)) {
+    // LDS read r of a stage's NRD: chunk reads of the weight tiles, then of the activation tiles,
+    // then (MXFP4) the scale words
+    constexpr int NRD = (TI + TJ) * (MX ? 3 : 2);
+    auto load_one = [&](int slot, auto buf_tag, int r) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
         const unsigned char* base = smem + slot * SLOT;
-#pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-            fb[B][j].c[0] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c0);
-            fb[B][j].c[1] = *(const u32x4*)(base + b_row0 + j * 32 * kRowB8 + c1);
-        }
-#pragma unroll
-        for (int i = 0; i < TI; ++i) {
-            fa[B][i].c[0] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c0);
-            fa[B][i].c[1] = *(const u32x4*)(base + a_row0 + i * 32 * kRowB8 + c1);
-        }
-        if constexpr (MX) {
+        if (r < 2 * TJ) {
+            fb[B][r / 2].c[r % 2] = *(const u32x4*)(base + b_row0 + (r / 2) * 32 * kRowB8 + (r % 2 ? c1 : c0));
+        } else if (r < 2 * (TI + TJ)) {
+            const int q = r - 2 * TJ;
+            fa[B][q / 2].c[q % 2] = *(const u32x4*)(base + a_row0 + (q / 2) * 32 * kRowB8 + (q % 2 ? c1 : c0));
+        } else if constexpr (MX) {
             // half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2
-#pragma unroll
-            for (int i = 0; i < TI; ++i) fsa[B][i] = *(const unsigned*)(base + sa_row0 + i * 128) >> (8 * kb);
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) fsb[B][j] = *(const unsigned*)(base + sb_row0 + j * 128) >> (8 * kb);
+            const int q = r - 2 * (TI + TJ);
+            if (q < TI) fsa[B][q] = *(const unsigned*)(base + sa_row0 + q * 128) >> (8 * kb);
+            else fsb[B][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> (8 * kb);
         }
     };
-    auto multiply = [&](int limit, auto buf_tag) __attribute__((always_inline)) {
+    auto load_frags = [&](int slot, auto buf_tag) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < NRD; ++r) load_one(slot, buf_tag, r);
+    };
+    // MFMA q of a stage's NM.  fp8: one K-step of 64 bytes per tile pair; int8 / fp4: two K-steps of 32
+    constexpr int NM = TI * TJ * (MODE == kFP8 ? 1 : 2);
+    auto multiply_one = [&](int limit, auto buf_tag, int q) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
+        const int s2 = q / (TI * TJ), i = (q % (TI * TJ)) / TJ, j = q % TJ;
         if constexpr (MODE == kFP8) {
-#pragma unroll
-            for (int i = 0; i < TI; ++i)
-#pragma unroll
-                for (int j = 0; j < TJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[B][i].v8, fb[B][j].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
         } else {
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {  // two MFMA K-steps of 32 bytes
-                // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
-                // must not live across control flow)
-                const bool valid = MODE != kINT8 || s * 32 < limit;
-#pragma unroll
-                for (int i = 0; i < TI; ++i) {
-                    u32x4 af = fa[B][i].c[s];
-                    if (!valid) af = u32x4{0, 0, 0, 0};
-#pragma unroll
-                    for (int j = 0; j < TJ; ++j) {
-                        const u32x4 bf = fb[B][j].c[s];
-                        if constexpr (MODE == kINT8) {
-                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                                int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w},
-                                int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w}, acc[i][j], 0, 0, 0);
-                        } else {
-                            // fp4 operands occupy the first four of the eight operand registers; the rest is not read
-                            const int4_t a4 = int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w};
-                            const int4_t b4 = int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w};
-                            const int8_t_v a8 = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
-                            const int8_t_v b8 = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
-                            if (s & 1)
-                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 4, 4, 2, (int)fsa[B][i], 2, (int)fsb[B][j]);
-                            else
-                                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 4, 4, 0, (int)fsa[B][i], 0, (int)fsb[B][j]);
-                        }
-                    }
-                }
+            // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
+            // must not live across control flow)
+            const bool valid = MODE != kINT8 || s2 * 32 < limit;
+            u32x4 af = fa[B][i].c[s2];
+            if (!valid) af = u32x4{0, 0, 0, 0};
+            const u32x4 bf = fb[B][j].c[s2];
+            if constexpr (MODE == kINT8) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w},
+                                                                  int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w}, acc[i][j], 0, 0, 0);
+            } else {
+                // fp4 operands occupy the first four of the eight operand registers; the rest is not read
+                const int4_t a4 = int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w};
+                const int4_t b4 = int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w};
+                const int8_t_v a8 = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
+                const int8_t_v b8 = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
+                if (s2 & 1)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 4, 4, 2, (int)fsb[B][j], 2, (int)fsa[B][i]);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 4, 4, 0, (int)fsb[B][j], 0, (int)fsa[B][i]);
             }
         }
     };
@@ -325,16 +301,35 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        // The step is cut into NM slices of one MFMA, a share of the copies and a share of
+        // the LDS reads, with the scheduler fenced between slices.  Left alone, the compiler issues the
+        // copies in one burst right after the barrier, where every wave of the workgroup queues at
+        // the one address unit of the CU (16 clocks per 16-byte-per-lane instruction) before its first
+        // MFMA, and the matrix pipe idles for that long in every step.
+        const int limit = p.Kb - (k_first + k) * kRowB8;
         if constexpr (DB) {
-            issue(k + RING, slot);
+            const int refill = slot;
             slot = slot == RING - 1 ? 0 : slot + 1;
-            load_frags(slot, std::integral_constant<int, B ^ 1>{});
-            multiply(p.Kb - (k_first + k) * kRowB8, buf_tag);
-            interleave_mfma_with_lds_reads<TI * TJ * (MODE == kFP8 ? 1 : 2), (TI + TJ) * (MX ? 3 : 2)>();
+#pragma unroll
+            for (int q = 0; q < NM; ++q) {
+                multiply_one(limit, buf_tag, q);
+#pragma unroll
+                for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING, refill, c);
+#pragma unroll
+                for (int r = q * NRD / NM; r < (q + 1) * NRD / NM; ++r) load_one(slot, std::integral_constant<int, B ^ 1>{}, r);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         } else {
-            issue(k + RING - 1, slot == 0 ? RING - 1 : slot - 1);
+            const int refill = slot == 0 ? RING - 1 : slot - 1;
             load_frags(slot, std::integral_constant<int, 0>{});
-            multiply(p.Kb - (k_first + k) * kRowB8, std::integral_constant<int, 0>{});
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < NM; ++q) {
+                multiply_one(limit, std::integral_constant<int, 0>{}, q);
+#pragma unroll
+                for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING - 1, refill, c);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             slot = slot == RING - 1 ? 0 : slot + 1;
         }
     };
@@ -349,52 +344,93 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         for (int k = 0; k < steps; ++k) step(k, std::integral_constant<int, 0>{});
     }
 
-    // ---- epilogue: lane holds column r32 of each 32-wide tile, rows 8*(e/4) + 4*kb + e%4
+    // ---- epilogue.  The weight fragment is the row operand of every MFMA, so a tile's accumulator is
+    // the transposed output tile: the lane holds output row r32 (of the tile) and, in elements
+    // 4g .. 4g+3, the four adjacent output columns 8g + 4kb .. + 3, which leave in one store.
+    const int n_wave = n0 + wn * WNC + 4 * kb;
     if (p.S > 1) {  // partial tile, raw 32-bit accumulators; the reduction kernel finishes
         typedef typename std::conditional<MODE == kINT8, int32_t, float>::type raw_t;
+        typedef raw_t raw4_t __attribute__((ext_vector_type(4)));
         raw_t* part = (raw_t*)p.partials + (size_t)blockIdx.y * p.M * p.N;
-#pragma unroll
-        for (int i = 0; i < TI; ++i)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
-                if (m >= p.M) continue;
-#pragma unroll
-                for (int j = 0; j < TJ; ++j) {
-                    const int n = n0 + wn * WNC + j * 32 + r32;
-                    if (n < p.N) part[(size_t)m * p.N + n] = acc[i][j][e];
-                }
-            }
-        return;
-    }
-    float sb[TJ];
-    bool n_ok[TJ];
-    const bool col_scale = !MX && (p.csm & 1);
-    const bool row_scale = !MX && (p.csm & 2);
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) {
-        const int n = n0 + wn * WNC + j * 32 + r32;
-        n_ok[j] = n < p.N;
-        sb[j] = (col_scale && n_ok[j]) ? load_as_float(p.scales, p.meta_dt, n) : 1.0f;
-    }
-    auto emit = [&](auto dt_tag) {
-        constexpr int DT = decltype(dt_tag)::value;
+        const bool wide = (p.N & 3) == 0;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
+            const int m = m0 + wm * WM + i * 32 + r32;
+            if (m >= p.M) continue;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
-                if (m < p.M) {
-                    const float sa = row_scale ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
-                    const int64_t o = (int64_t)m * p.osm + n0 + wn * WNC + r32;
+            for (int j = 0; j < TJ; ++j)
 #pragma unroll
-                    for (int j = 0; j < TJ; ++j) {
-                        if (!n_ok[j]) continue;
-                        if constexpr (DT == GLA_DT_INT32) ((int32_t*)p.out)[o + j * 32] = (int32_t)acc[i][j][e];
-                        else store_typed<DT>(p.out, o + j * 32, (float)acc[i][j][e] * (sa * sb[j]));
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n_wave + j * 32 + 8 * g;
+                    raw_t* dst = part + (size_t)m * p.N + n;
+                    if (wide && n + 3 < p.N) {
+                        *(raw4_t*)dst = raw4_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (n + t < p.N) dst[t] = acc[i][j][4 * g + t];
                     }
                 }
-            }
+        }
+        return;
+    }
+    const bool col_scale = !MX && (p.csm & 1);
+    const bool row_scale = !MX && (p.csm & 2);
+    float sb[TJ][16];
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int n = n_wave + j * 32 + 8 * (e / 4) + (e % 4);
+            sb[j][e] = (col_scale && n < p.N) ? load_as_float(p.scales, p.meta_dt, n) : 1.0f;
+        }
+    auto emit = [&](auto dt_tag) {
+        constexpr int DT = decltype(dt_tag)::value;
+        constexpr int ES = (DT == GLA_DT_FP16 || DT == GLA_DT_BF16) ? 2 : 4;
+        // four elements leave as one 8- or 16-byte store when every such group of the tensor is aligned
+        const bool wide = (p.osm & 3) == 0 && (((uintptr_t)p.out) & (4 * ES - 1)) == 0;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            const int m = m0 + wm * WM + i * 32 + r32;
+            if (m >= p.M) continue;
+            const float sa = row_scale ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n_wave + j * 32 + 8 * g;
+                    const int64_t o = (int64_t)m * p.osm + n;
+                    if (wide && n + 3 < p.N) {
+                        if constexpr (DT == GLA_DT_INT32) {
+                            *(int4_t*)((int32_t*)p.out + o) = int4_t{(int)acc[i][j][4 * g], (int)acc[i][j][4 * g + 1],
+                                                                     (int)acc[i][j][4 * g + 2], (int)acc[i][j][4 * g + 3]};
+                        } else {
+                            float v[4];
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) v[t] = (float)acc[i][j][4 * g + t] * (sa * sb[j][4 * g + t]);
+                            if constexpr (DT == GLA_DT_FP32) {
+                                *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
+                            } else {
+                                uint32_t lo, hi;
+                                if constexpr (DT == GLA_DT_FP16) {
+                                    lo = float_to_half_bits(v[0]) | ((uint32_t)float_to_half_bits(v[1]) << 16);
+                                    hi = float_to_half_bits(v[2]) | ((uint32_t)float_to_half_bits(v[3]) << 16);
+                                } else {
+                                    lo = float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+                                    hi = float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+                                }
+                                *(u32x2*)((uint16_t*)p.out + o) = u32x2{lo, hi};
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            if (n + t >= p.N) continue;
+                            if constexpr (DT == GLA_DT_INT32) ((int32_t*)p.out)[o + t] = (int32_t)acc[i][j][4 * g + t];
+                            else store_typed<DT>(p.out, o + t, (float)acc[i][j][4 * g + t] * (sa * sb[j][4 * g + t]));
+                        }
+                    }
+                }
         }
     };
     if (p.out_dt == GLA_DT_FP16) emit(std::integral_constant<int, GLA_DT_FP16>{});
