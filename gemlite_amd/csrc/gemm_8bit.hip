@@ -238,14 +238,30 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             else fsb[B][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> (8 * kb);
         }
     };
+    // The same for one K-step (h = 0, 1) of a stage, into fragment buffer 0: read r of TI + TJ chunk reads
+    // and, after them, of the TI + TJ scale words, which go to scale buffer SB
+    auto load_half = [&](int slot, int h, auto scale_tag, int r) __attribute__((always_inline)) {
+        constexpr int SB = decltype(scale_tag)::value;
+        const unsigned char* base = smem + slot * SLOT;
+        if (r < TJ) {
+            fb[0][r].c[h] = *(const u32x4*)(base + b_row0 + r * 32 * kRowB8 + (h ? c1 : c0));
+        } else if (r < TI + TJ) {
+            fa[0][r - TJ].c[h] = *(const u32x4*)(base + a_row0 + (r - TJ) * 32 * kRowB8 + (h ? c1 : c0));
+        } else if constexpr (MX) {
+            const int q = r - (TI + TJ);
+            if (q < TI) fsa[SB][q] = *(const unsigned*)(base + sa_row0 + q * 128) >> (8 * kb);
+            else fsb[SB][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> (8 * kb);
+        }
+    };
     auto load_frags = [&](int slot, auto buf_tag) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < NRD; ++r) load_one(slot, buf_tag, r);
     };
     // MFMA q of a stage's NM.  fp8: one K-step of 64 bytes per tile pair; int8 / fp4: two K-steps of 32
     constexpr int NM = TI * TJ * (MODE == kFP8 ? 1 : 2);
-    auto multiply_one = [&](int limit, auto buf_tag, int q) __attribute__((always_inline)) {
-        constexpr int B = decltype(buf_tag)::value;
+    auto multiply_one = [&](int limit, auto buf_tag, auto scale_tag, int q) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf_tag)::value;    // fragment buffer
+        constexpr int SB = decltype(scale_tag)::value; // scale buffer (MXFP4)
         const int s2 = q / (TI * TJ), i = (q % (TI * TJ)) / TJ, j = q % TJ;
         if constexpr (MODE == kFP8) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
@@ -266,9 +282,9 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                 const int8_t_v a8 = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
                 const int8_t_v b8 = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
                 if (s2 & 1)
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 4, 4, 2, (int)fsb[B][j], 2, (int)fsa[B][i]);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 4, 4, 2, (int)fsb[SB][j], 2, (int)fsa[SB][i]);
                 else
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 4, 4, 0, (int)fsb[B][j], 0, (int)fsa[B][i]);
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 4, 4, 0, (int)fsb[SB][j], 0, (int)fsa[SB][i]);
             }
         }
     };
@@ -276,28 +292,38 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // ---- pipeline.  Copies complete in issue order.  Barriers are bare on purpose (a __syncthreads()
     // carries a release fence, which for copies into LDS means draining the counter and with it the
     // pipeline); the empty asm statements pin LDS accesses to their side of a barrier.
-    // DB (fragments double-buffered): RING stages in flight; step k reads stage k+1 into registers
-    // and multiplies stage k, whose slot is refilled first.  Otherwise (MXFP4 with the 256-row tile,
-    // which has no registers to spare): RING - 1 stages in flight; step k reads and multiplies stage k
-    // and refills the slot of stage k-1.
-    constexpr bool DB = WN == 4 && !(MX && BM == 256);
-    constexpr int AHEAD = DB ? RING : RING - 1;
+    // Operand fragments are read one step ahead of the MFMAs that use them, so that LDS latency is
+    // hidden although the barrier keeps all waves of the workgroup in the same phase:
+    //  * whole stages (two register buffers): RING stages in flight; step k reads stage k+1 and
+    //    multiplies stage k, whose slot is refilled;
+    //  * HALF (MXFP4 with the 256-row tile, which has no registers for a second buffer): the two
+    //    K-steps of a stage are the two buffers.  RING - 1 stages in flight; step k multiplies K-step 0
+    //    of stage k while reading its K-step 1, then multiplies that while reading K-step 0 of stage
+    //    k+1, and refills the slot of stage k-1.  The scale words of a stage serve both K-steps and
+    //    alternate between two buffers.
+    constexpr bool HALF = MX && BM == 256;
+    constexpr int AHEAD = HALF ? RING - 1 : RING;
+    typedef std::integral_constant<int, 0> tag0;
 #pragma unroll
     for (int u = 0; u < AHEAD; ++u) issue(u, u);
-    if constexpr (DB) {
-        wait_vmcnt8<(RING - 1) * LPS>();  // stage 0 has landed (this wave's part)
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();     // ... and everybody else's
-        asm volatile("" ::: "memory");
-        load_frags(0, std::integral_constant<int, 0>{});
+    wait_vmcnt8<(AHEAD - 1) * LPS>();  // stage 0 has landed (this wave's part)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();      // ... and everybody else's
+    asm volatile("" ::: "memory");
+    if constexpr (HALF) {
+#pragma unroll
+        for (int r = 0; r < 2 * (TI + TJ); ++r) load_half(0, 0, tag0{}, r);
+    } else {
+        load_frags(0, tag0{});
     }
 
     int slot = 0;  // ring slot of the stage being multiplied
     auto step = [&](int k, auto buf_tag) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
-        // the stage read in this step has landed once at most the copies of the RING - 2 stages issued
-        // after it are outstanding; after the barrier the slot refilled below is no longer read by anyone
-        wait_vmcnt8<(RING - 2) * LPS>();
+        typedef std::integral_constant<int, B ^ 1> other;
+        // stage k+1, read in this step, has landed once at most the copies of the stages issued after
+        // it are outstanding; after the barrier the slot refilled below is no longer read by anyone
+        wait_vmcnt8<(AHEAD - 2) * LPS>();
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -307,41 +333,44 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         // the one address unit of the CU (16 clocks per 16-byte-per-lane instruction) before its first
         // MFMA, and the matrix pipe idles for that long in every step.
         const int limit = p.Kb - (k_first + k) * kRowB8;
-        if constexpr (DB) {
-            const int refill = slot;
-            slot = slot == RING - 1 ? 0 : slot + 1;
+        const int next = slot == RING - 1 ? 0 : slot + 1;
+        // (the reads go with the first slices only, so that the last of them has returned when the
+        // MFMAs that follow need it)
+        if constexpr (!HALF) {
+            constexpr int RS = NM > 2 ? NM * 3 / 4 : NM;  // slices that carry reads
 #pragma unroll
             for (int q = 0; q < NM; ++q) {
-                multiply_one(limit, buf_tag, q);
+                multiply_one(limit, buf_tag, buf_tag, q);
 #pragma unroll
-                for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING, refill, c);
+                for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING, slot, c);
 #pragma unroll
-                for (int r = q * NRD / NM; r < (q + 1) * NRD / NM; ++r) load_one(slot, std::integral_constant<int, B ^ 1>{}, r);
+                for (int r = q * NRD / RS; r < (q + 1) * NRD / RS && r < NRD; ++r) load_one(next, other{}, r);
                 __builtin_amdgcn_sched_barrier(0);
             }
         } else {
             const int refill = slot == 0 ? RING - 1 : slot - 1;
-            load_frags(slot, std::integral_constant<int, 0>{});
-            __builtin_amdgcn_sched_barrier(0);
+            constexpr int H = NM / 2, HS = H / 2, R1 = TI + TJ, R2 = 2 * (TI + TJ);
 #pragma unroll
             for (int q = 0; q < NM; ++q) {
-                multiply_one(limit, std::integral_constant<int, 0>{}, q);
+                multiply_one(limit, tag0{}, buf_tag, q);
 #pragma unroll
                 for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING - 1, refill, c);
+                if (q < H) {
+#pragma unroll
+                    for (int r = q * R1 / HS; r < (q + 1) * R1 / HS && r < R1; ++r) load_half(slot, 1, buf_tag, r);
+                } else {
+#pragma unroll
+                    for (int r = (q - H) * R2 / HS; r < (q - H + 1) * R2 / HS && r < R2; ++r) load_half(next, 0, other{}, r);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            slot = slot == RING - 1 ? 0 : slot + 1;
         }
+        slot = next;
     };
-    if constexpr (DB) {
 #pragma unroll 1
-        for (int k = 0; k < steps; k += 2) {  // two steps per trip: the fragment buffers alternate
-            step(k, std::integral_constant<int, 0>{});
-            if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
-        }
-    } else {
-#pragma unroll 1
-        for (int k = 0; k < steps; ++k) step(k, std::integral_constant<int, 0>{});
+    for (int k = 0; k < steps; k += 2) {  // two steps per trip: the register buffers alternate
+        step(k, std::integral_constant<int, 0>{});
+        if (k + 1 < steps) step(k + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue.  The weight fragment is the row operand of every MFMA, so a tile's accumulator is

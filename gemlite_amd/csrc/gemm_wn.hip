@@ -432,6 +432,9 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
     const bool row_scale = (p.csm & 2) != 0;
     auto emit = [&](auto dt_tag) __attribute__((always_inline)) {
         constexpr int DT = decltype(dt_tag)::value;
+        constexpr int ES = DT == GLA_DT_FP32 ? 4 : 2;
+        static_assert(TJ == 4, "a lane owns four adjacent columns");
+        const bool wide = (p.osm & 3) == 0 && (((uintptr_t)p.out) & (4 * ES - 1)) == 0;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
 #pragma unroll
@@ -440,8 +443,23 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
                 if (m < p.M) {
                     const float sa = row_scale ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
                     const int64_t o = (int64_t)m * p.osm + coln;
+                    if (wide) {  // the lane's four adjacent columns leave in one store
+                        float v[TJ];
 #pragma unroll
-                    for (int j = 0; j < TJ; ++j) store_typed<DT>(p.out, o + j, acc[i][j][e] * (sa * sb[j]));
+                        for (int j = 0; j < TJ; ++j) v[j] = acc[i][j][e] * (sa * sb[j]);
+                        if constexpr (DT == GLA_DT_FP32) {
+                            *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
+                        } else if constexpr (DT == GLA_DT_FP16) {
+                            *(u32x2*)((uint16_t*)p.out + o) = u32x2{float_to_half_bits(v[0]) | ((uint32_t)float_to_half_bits(v[1]) << 16),
+                                                                     float_to_half_bits(v[2]) | ((uint32_t)float_to_half_bits(v[3]) << 16)};
+                        } else {
+                            *(u32x2*)((uint16_t*)p.out + o) = u32x2{float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16),
+                                                                     float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16)};
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < TJ; ++j) store_typed<DT>(p.out, o + j, acc[i][j][e] * (sa * sb[j]));
+                    }
                 }
             }
         }
