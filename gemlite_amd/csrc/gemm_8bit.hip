@@ -49,6 +49,7 @@ struct Gemm8Args {
     void* out;
     int M, N, Kb;          // Kb = bytes of K per row
     int64_t lda, ldb, osm, sxm, msn;
+    int64_t sx_stage, sw_stage;  // MXFP4: bytes from one pipeline stage's scale word of a row to the next one's
     int csm, meta_dt, sx_dt, out_dt;
     int tiles_m, tiles_n;
     int S;     // K splits (gridDim.y)
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                                              (__attribute__((address_space(3))) void*)(base + dst16[c]), 16, 0, 0);
         } else if constexpr (MX) {
             const int i = c - J16;
-            const uint8_t* sk = (is_a4[i] ? (const uint8_t*)p.scales_x : (const uint8_t*)p.scales) + kk * 4;
+            const uint8_t* sk = is_a4[i] ? (const uint8_t*)p.scales_x + kk * p.sx_stage : (const uint8_t*)p.scales + kk * p.sw_stage;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
                                              (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
         }
@@ -527,6 +528,27 @@ struct Plan8 {
     int bm, tiles_m, tiles_n, S, sps;
 };
 
+// MXFP4 scales by pipeline stage.  In the caller's layout ([rows, K/32] bytes, K fastest) the four
+// scale bytes a row contributes to a stage lie one row stride apart from the next row's, so the
+// copy of a tile's scales touches one cache line per row and moves sixteen times the bytes it uses.
+// This kernel regroups them as dst[stage][row] (one 32-bit word each), which a tile copies as
+// consecutive words.  64 x 64 words per workgroup through LDS, both sides coalesced.
+__global__ __launch_bounds__(256) void mx_scales_by_stage_kernel(const uint8_t* src, int rows, int64_t row_stride, int stages, uint32_t* dst) {
+    __shared__ uint32_t tile[64][65];
+    const int r0 = blockIdx.x * 64, s0 = blockIdx.y * 64, t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = r0 + (t >> 6) + 4 * i, st = s0 + (t & 63);
+        if (r < rows && st < stages) tile[(t >> 6) + 4 * i][t & 63] = *(const uint32_t*)(src + (int64_t)r * row_stride + (int64_t)st * 4);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = r0 + (t & 63), st = s0 + (t >> 6) + 4 * i;
+        if (r < rows && st < stages) dst[(int64_t)st * rows + r] = tile[t & 63][(t >> 6) + 4 * i];
+    }
+}
+
 constexpr int64_t kWsReserved8 = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
 
 Plan8 plan8(int M, int N, int Kb, int tile_config) {
@@ -591,7 +613,7 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
-    a.out_dt = p.output_dtype;
+    a.out_dt = p.output_dtype; a.sx_stage = 0; a.sw_stage = 0;
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
@@ -599,10 +621,20 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     return launch_mode<kFP8>(a, g.bm, stream);
 }
 
+// MXFP4 scales regrouped by stage pay off once the GEMM itself takes much longer than regrouping
+// the weight scales (a pass over N x K/32 bytes): from the 128-row tile on.
+static bool mx_scales_staged(const gla_matmul_args& p, const Plan8& g) { return g.bm >= 128; }
+static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
 int64_t gemm_8bit_workspace_bytes(const gla_matmul_args& p) {
     const bool mx = p.input_dtype == GLA_DT_MXFP4;
     const Plan8 g = plan8(p.M, p.N, mx ? p.K / 2 : p.K, p.tile_config);
-    return g.S > 1 ? kWsReserved8 + (int64_t)g.S * p.M * p.N * 4 : 0;
+    int64_t need = g.S > 1 ? kWsReserved8 + align256((int64_t)g.S * p.M * p.N * 4) : 0;
+    if (mx && mx_scales_staged(p, g)) {
+        if (need == 0) need = kWsReserved8;
+        need += align256((int64_t)(p.K / 128) * p.M * 4) + align256((int64_t)(p.K / 128) * p.N * 4);
+    }
+    return need;
 }
 
 // MXFP4 x MXFP4: x is [M, K/2] bytes, w the [K/2, N] view of [N, K/2] bytes, and both e8m0
@@ -629,9 +661,23 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
     a.M = p.M; a.N = p.N; a.Kb = p.K / 2; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.csm = 0; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype;
+    a.sx_stage = 4; a.sw_stage = 4;
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
+    // with room in the workspace, both scale arrays are regrouped by stage first (same stream)
+    if (mx_scales_staged(p, g) && p.workspace != nullptr && (int64_t)p.workspace_bytes >= gemm_8bit_workspace_bytes(p)) {
+        const int stages = p.K / 128;
+        const int64_t part = g.S > 1 ? align256((int64_t)g.S * p.M * p.N * 4) : 0;
+        uint32_t* sx = (uint32_t*)((char*)p.workspace + kWsReserved8 + part);
+        uint32_t* sw = (uint32_t*)((char*)sx + align256((int64_t)stages * p.M * 4));
+        hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(ceil_div(p.M, 64), ceil_div(stages, 64)), dim3(256), 0, stream,
+                           (const uint8_t*)p.scales_x, p.M, (int64_t)p.sx_stride_m, stages, sx);
+        hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(ceil_div(p.N, 64), ceil_div(stages, 64)), dim3(256), 0, stream,
+                           (const uint8_t*)p.scales, p.N, (int64_t)p.meta_stride_n, stages, sw);
+        a.scales_x = sx; a.sxm = 4; a.sx_stage = (int64_t)p.M * 4;
+        a.scales = sw; a.msn = 4; a.sw_stage = (int64_t)p.N * 4;
+    }
     return launch_mode<kMXFP4>(a, g.bm, stream);
 }
 
