@@ -39,8 +39,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBKw = 64;    // K per pipeline stage
 constexpr int kRowW = 128;  // LDS row: 64 fp16/bf16 values
-constexpr int kWavesNw = 2;
-constexpr int kBNw = kWavesNw * 128;
+constexpr int kBNw = 256;   // workgroup tile columns: 256 / (32 TJ) wave columns of TJ 32-column MFMA tiles
 constexpr int64_t kWsReserved = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
 
 struct GemmWnArgs {
@@ -157,14 +156,18 @@ constexpr int ring_slots(int bm) { return bm >= 128 ? 3 : 4; }
 // One ring slot: A tile, weight words of both wave columns, scales and zeros of the 256 columns.
 constexpr int slot_bytes(int bits, int bm) { return bm * kRowW + 2 * (bits == 8 ? 8 : 4) * 1024 + 1024; }
 
-// BITS in {2, 4, 8}; WAVES_M in {1, 2, 4}; TI = 32-row MFMA tiles per wave (1 or 2)
-template <int BITS, bool BF16, int WAVES_M, int TI>
-__global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_wn_kernel(GemmWnArgs p) {
+// BITS in {2, 4, 8}; WAVES_M in {1, 2, 4}; TI = 32-row MFMA tiles per wave (1, 2 or 4); TJ = 32-column
+// tiles per wave (4 or 2).  Every wave dequantises the weights of its own columns, so the work of
+// unpacking is repeated WAVES_M times per workgroup: the 256-row tile uses 2 x 4 waves of 128 x 64
+// (TI 4, TJ 2) rather than 4 x 2 waves of 64 x 128, which halves the unpacking per MFMA.
+template <int BITS, bool BF16, int WAVES_M, int TI, int TJ>
+__global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_wn_kernel(GemmWnArgs p) {
+    static_assert(TJ == 4 || TJ == 2, "wave tile of 128 or 64 columns");
     constexpr int E = 32 / BITS;
     constexpr int WM = 32 * TI;
     constexpr int BM = WAVES_M * WM;
-    constexpr int NW = WAVES_M * kWavesNw;   // waves
-    constexpr int TJ = 4;
+    constexpr int WN = 8 / TJ;               // wave columns
+    constexpr int NW = WAVES_M * WN;         // waves
     constexpr int WL = (BITS == 8) ? 8 : 4;  // 128-bit weight loads per lane per stage
     constexpr int RING = ring_slots(BM);
     constexpr int PF = RING - 1;             // stages in flight ahead of the one being multiplied
@@ -182,15 +185,13 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
     extern __shared__ __align__(16) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / kWavesNw, wn = wave % kWavesNw;
+    const int wm = wave / WN, wn = wave % WN;
     const int r32 = lane & 31, kb = lane >> 5;
     int tm, tn;
     tile_coords_wn(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * kBNw;
-    // the lane's output columns: n0 + wn*128 + 4*r32 + {0..3}
-    int coln = n0 + wn * 128 + r32 * 4;
-    const bool col_ok = coln + 3 < p.N;  // N % 4 == 0 is required, so a lane is all-in or all-out
-    if (coln > p.N - 4) coln = p.N - 4;
+    // the wave's columns start at n_wave; as B operand of tile j the lane handles column n_wave + TJ r32 + j
+    const int n_wave = n0 + wn * 32 * TJ;
 
     const bool grouped = p.wgm >= GLA_WGM_SCALE || (p.wgm == GLA_WGM_SHIFT && !p.z_scalar);
     const bool has_s = p.wgm >= GLA_WGM_SCALE;
@@ -283,11 +284,18 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
     const float c1 = p.wgm == GLA_WGM_SHIFT ? -1.0f : (p.wgm == GLA_WGM_FMA ? 1.0f : 0.0f);
     const float c2 = p.wgm == GLA_WGM_SHIFT_SCALE ? -1.0f : 0.0f;
     ColMeta<BF16> meta[TJ];
-    auto convert_meta = [&](u32x2 raw_s, u32x2 raw_z) __attribute__((always_inline)) {
+    auto convert_meta = [&](const unsigned char* sp, const unsigned char* zp) __attribute__((always_inline)) {
+        uint32_t raw_s[TJ / 2], raw_z[TJ / 2];
+        if constexpr (TJ == 4) {
+            const u32x2 a = *(const u32x2*)sp, b = *(const u32x2*)zp;
+            raw_s[0] = a.x; raw_s[1] = a.y; raw_z[0] = b.x; raw_z[1] = b.y;
+        } else {
+            raw_s[0] = *(const uint32_t*)sp; raw_z[0] = *(const uint32_t*)zp;
+        }
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-            const uint32_t sv = ((j < 2 ? raw_s.x : raw_s.y) >> (16 * (j & 1))) & s_mask;
-            const uint32_t zv = ((j < 2 ? raw_z.x : raw_z.y) >> (16 * (j & 1))) & z_mask;
+            const uint32_t sv = (raw_s[j / 2] >> (16 * (j & 1))) & s_mask;
+            const uint32_t zv = (raw_z[j / 2] >> (16 * (j & 1))) & z_mask;
             const float s_h = half_bits_to_float((uint16_t)sv), s_b = __builtin_bit_cast(float, sv << 16);
             const float z_h = half_bits_to_float((uint16_t)zv), z_b = __builtin_bit_cast(float, zv << 16);
             const float s = (meta_bf16 ? s_b : s_h) + s_add;
@@ -309,8 +317,10 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
 
     const int sw = (r32 >> 1) & 7;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
     const int a_row0 = (wm * WM + r32) * kRowW;
-    const int w_lane = W_OFF + wn * WL * 1024 + lane * 16;
-    const int m_lane = wn * 256 + r32 * 8;
+    // weight words: a copy job holds 128 columns x the word rows of both K-halves, 16 bytes (4 columns) per copying lane
+    const int w_lane = TJ == 4 ? W_OFF + wn * WL * 1024 + lane * 16
+                               : W_OFF + (wn >> 1) * WL * 1024 + (kb * 32 + (wn & 1) * 16 + (r32 >> 1)) * 16 + (r32 & 1) * 8;
+    const int m_lane = wn * 64 * TJ + r32 * 2 * TJ;
     const int total_steps = p.K / kBKw;
     const int k_first = blockIdx.y * p.sps;  // first stage of this split
     const int steps = (total_steps - k_first) < p.sps ? (total_steps - k_first) : p.sps;
@@ -349,7 +359,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
         asm volatile("" ::: "memory");
         issue_next(slot == 0 ? RING - 1 : slot - 1);  // overwrites the slot of stage k-1
         const unsigned char* base = smem + slot * SLOT;
-        convert_meta(*(const u32x2*)(base + S_OFF + m_lane), *(const u32x2*)(base + Z_OFF + m_lane));
+        convert_meta(base + S_OFF + m_lane, base + Z_OFF + m_lane);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {  // four MFMA K-steps of 16
             u32x4 af[TI];
@@ -372,12 +382,21 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
                     }
                 }
             }
-            u32x4 wv[BITS == 8 ? 2 : 1];
+            uint32_t wv[BITS == 8 ? 2 : 1][TJ];
+            auto load_words = [&](int v, int u) __attribute__((always_inline)) {
+                if constexpr (TJ == 4) {
+                    const u32x4 t = *(const u32x4*)(base + w_lane + u * 1024);
+                    wv[v][0] = t.x; wv[v][1] = t.y; wv[v][2] = t.z; wv[v][3] = t.w;
+                } else {
+                    const u32x2 t = *(const u32x2*)(base + w_lane + u * 1024);
+                    wv[v][0] = t.x; wv[v][1] = t.y;
+                }
+            };
             if constexpr (BITS == 8) {
-                wv[0] = *(const u32x4*)(base + w_lane + (2 * s) * 1024);
-                wv[1] = *(const u32x4*)(base + w_lane + (2 * s + 1) * 1024);
+                load_words(0, 2 * s);
+                load_words(1, 2 * s + 1);
             } else {
-                wv[0] = *(const u32x4*)(base + w_lane + s * 1024);
+                load_words(0, s);
             }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
@@ -404,61 +423,85 @@ __global__ __launch_bounds__(WAVES_M * kWavesNw * 64) __attribute__((amdgpu_wave
                     bq[r] = dequant_pair<BF16>(t, meta[j]);
                 }
 #pragma unroll
-                for (int i = 0; i < TI; ++i) acc[i][j] = mfma32<BF16>(af[i], bq, acc[i][j]);
+                for (int i = 0; i < TI; ++i) acc[i][j] = mfma32<BF16>(bq, af[i], acc[i][j]);  // weights are the row operand
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the unpacking of later K-steps from being hoisted (register pressure)
         }
         slot = slot == RING - 1 ? 0 : slot + 1;
     }
 
-    // ---- epilogue: lane holds column 4*r32 + j of tile j, rows 8*(e/4) + 4*kb + e%4 of tile i
-    if (!col_ok) return;
+    // ---- epilogue.  With the weights as row operand an accumulator is the transposed output tile:
+    // the lane holds output row r32 of tile i and, in elements 4g .. 4g+3 of tile j, the columns
+    // n_wave + TJ (8g + 4kb + t) + j, t = 0..3.  Over t and j these are 4 TJ adjacent columns.
+    constexpr int RUN = 4 * TJ;
     if (p.S > 1) {  // partial tile; the reduction kernel finishes
-        float* part = p.partials + (size_t)blockIdx.y * p.M * p.N + coln;
+        float* part = p.partials + (size_t)blockIdx.y * p.M * p.N;
 #pragma unroll
-        for (int i = 0; i < TI; ++i)
+        for (int i = 0; i < TI; ++i) {
+            const int m = m0 + wm * WM + i * 32 + r32;
+            if (m >= p.M) continue;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
-                if (m < p.M)
-                    *(float4_t*)(part + (size_t)m * p.N) = float4_t{acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
+            for (int g = 0; g < 4; ++g) {
+                const int col = n_wave + TJ * (8 * g + 4 * kb);
+#pragma unroll
+                for (int c = 0; c < RUN; c += 4) {  // N % 4 == 0: a group of four columns is all-in or all-out
+                    if (col + c + 3 >= p.N) continue;
+                    float v[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) v[q] = acc[i][(c + q) % TJ][4 * g + (c + q) / TJ];
+                    *(float4_t*)(part + (size_t)m * p.N + col + c) = float4_t{v[0], v[1], v[2], v[3]};
+                }
             }
+        }
         return;
     }
-    float sb[TJ];
-#pragma unroll
-    for (int j = 0; j < TJ; ++j)
-        sb[j] = (p.csm & 1) ? load_as_float(p.scales, p.meta_dt, coln + j) : 1.0f;
     const bool row_scale = (p.csm & 2) != 0;
     auto emit = [&](auto dt_tag) __attribute__((always_inline)) {
         constexpr int DT = decltype(dt_tag)::value;
         constexpr int ES = DT == GLA_DT_FP32 ? 4 : 2;
-        static_assert(TJ == 4, "a lane owns four adjacent columns");
-        const bool wide = (p.osm & 3) == 0 && (((uintptr_t)p.out) & (4 * ES - 1)) == 0;
+        // 16-byte stores when every group of 16 / ES elements of the tensor that starts at a multiple of that is aligned
+        const bool wide = (((uintptr_t)p.out) & 15) == 0 && ((p.osm * ES) & 15) == 0;
+        float sa[TI];
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
+            const int m = m0 + wm * WM + i * 32 + r32;
+            sa[i] = (row_scale && m < p.M) ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
+        }
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * WM + i * 32 + 8 * (e / 4) + 4 * kb + (e % 4);
-                if (m < p.M) {
-                    const float sa = row_scale ? load_as_float(p.scales_x, p.sx_dt, (int64_t)m * p.sxm) : 1.0f;
-                    const int64_t o = (int64_t)m * p.osm + coln;
-                    if (wide) {  // the lane's four adjacent columns leave in one store
-                        float v[TJ];
+        for (int g = 0; g < 4; ++g) {
+            const int col = n_wave + TJ * (8 * g + 4 * kb);
+            float sb[RUN];
 #pragma unroll
-                        for (int j = 0; j < TJ; ++j) v[j] = acc[i][j][e] * (sa * sb[j]);
+            for (int c = 0; c < RUN; ++c) sb[c] = ((p.csm & 1) && col + c < p.N) ? load_as_float(p.scales, p.meta_dt, col + c) : 1.0f;
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                const int m = m0 + wm * WM + i * 32 + r32;
+                if (m >= p.M) continue;
+                float v[RUN];
+#pragma unroll
+                for (int c = 0; c < RUN; ++c) v[c] = acc[i][c % TJ][4 * g + c / TJ] * (sa[i] * sb[c]);
+                const int64_t o = (int64_t)m * p.osm + col;
+                constexpr int PER = 16 / ES;  // elements per 16-byte store
+#pragma unroll
+                for (int c = 0; c < RUN; c += PER) {
+                    if (wide && col + c + PER - 1 < p.N) {
                         if constexpr (DT == GLA_DT_FP32) {
-                            *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
-                        } else if constexpr (DT == GLA_DT_FP16) {
-                            *(u32x2*)((uint16_t*)p.out + o) = u32x2{float_to_half_bits(v[0]) | ((uint32_t)float_to_half_bits(v[1]) << 16),
-                                                                     float_to_half_bits(v[2]) | ((uint32_t)float_to_half_bits(v[3]) << 16)};
+                            *(float4_t*)((float*)p.out + o + c) = float4_t{v[c], v[c + 1], v[c + 2], v[c + 3]};
                         } else {
-                            *(u32x2*)((uint16_t*)p.out + o) = u32x2{float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16),
-                                                                     float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16)};
+                            u32x4 w;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                if constexpr (DT == GLA_DT_FP16)
+                                    w[q] = float_to_half_bits(v[c + 2 * q]) | ((uint32_t)float_to_half_bits(v[c + 2 * q + 1]) << 16);
+                                else
+                                    w[q] = float_to_bf16_bits(v[c + 2 * q]) | ((uint32_t)float_to_bf16_bits(v[c + 2 * q + 1]) << 16);
+                            }
+                            *(u32x4*)((uint16_t*)p.out + o + c) = w;
                         }
                     } else {
 #pragma unroll
-                        for (int j = 0; j < TJ; ++j) store_typed<DT>(p.out, o + j, acc[i][j][e] * (sa * sb[j]));
+                        for (int q = 0; q < PER; ++q)
+                            if (col + c + q < p.N) store_typed<DT>(p.out, o + c + q, v[c + q]);
                     }
                 }
             }
@@ -487,19 +530,19 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmWnArgs p) {
     }
 }
 
-template <int BITS, bool BF16, int WAVES_M, int TI>
+template <int BITS, bool BF16, int WAVES_M, int TI, int TJ>
 int launch_wn(const GemmWnArgs& a, hipStream_t stream) {
     constexpr int BM = WAVES_M * TI * 32;
     const size_t smem = (size_t)ring_slots(BM) * slot_bytes(BITS, BM);
     static bool configured = false;
-    auto kern = gemm_wn_kernel<BITS, BF16, WAVES_M, TI>;
+    auto kern = gemm_wn_kernel<BITS, BF16, WAVES_M, TI, TJ>;
     if (!configured && smem > 48 * 1024) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_wn: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
         configured = true;
     }
-    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(WAVES_M * kWavesNw * 64), smem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(WAVES_M * (8 / TJ) * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "gemm_wn launch");
     if (rc == GLA_OK && a.S > 1) {
         const int64_t items = (int64_t)a.M * (a.N / 4);
@@ -511,10 +554,10 @@ int launch_wn(const GemmWnArgs& a, hipStream_t stream) {
 
 template <int BITS, bool BF16>
 int launch_wn_m(const GemmWnArgs& a, int bm, hipStream_t stream) {
-    if (bm == 256) return launch_wn<BITS, BF16, 4, 2>(a, stream);
-    if (bm == 128) return launch_wn<BITS, BF16, 2, 2>(a, stream);
-    if (bm == 64) return launch_wn<BITS, BF16, 1, 2>(a, stream);
-    return launch_wn<BITS, BF16, 1, 1>(a, stream);
+    if (bm == 256) return launch_wn<BITS, BF16, 2, 4, 2>(a, stream);
+    if (bm == 128) return launch_wn<BITS, BF16, 2, 2, 4>(a, stream);
+    if (bm == 64) return launch_wn<BITS, BF16, 1, 2, 4>(a, stream);
+    return launch_wn<BITS, BF16, 1, 1, 4>(a, stream);
 }
 
 // tile_config encoding: BM (32, 64, 128 or 256; other = chosen here) + 1000 * K splits (0 = chosen here)
