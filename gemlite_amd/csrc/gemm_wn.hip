@@ -120,7 +120,7 @@ __device__ __forceinline__ float fold_zero(float s, float z, int wgm) {
 
 // pair register holding (OFF + q_lo, OFF + q_hi) -> dequantised pair in the activation type
 template <bool BF16>
-__device__ __forceinline__ uint32_t dequant_pair(uint32_t t, const ColMeta<BF16>& m) {
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t t, const ColMeta<BF16>& m, float off_lo = 1024.0f, float off_hi = 1024.0f) {
     if constexpr (BF16) {
         // bf16 bits are the top half of an fp32, where 128 + q is exact too; (128 + q) s + (z' - 128 s)
         // in fp32, then one hardware round-to-nearest-even conversion of the pair
@@ -130,7 +130,7 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t t, const ColMeta<BF16>
         const f32x2 w = {__builtin_fmaf(lo, m.s, m.z), __builtin_fmaf(hi, m.s, m.z)};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2_t));
     } else {
-        half2_t q = __builtin_bit_cast(half2_t, t) - half2_t{(half_t)1024.0f, (half_t)1024.0f};
+        half2_t q = __builtin_bit_cast(half2_t, t) - half2_t{(half_t)off_lo, (half_t)off_hi};
         half2_t w = __builtin_elementwise_fma(q, m.s, m.z);
         return __builtin_bit_cast(uint32_t, w);
     }
@@ -180,6 +180,10 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
     constexpr int LPS = J16 + J4;                // copy instructions per wave per stage
     constexpr uint32_t kPairMask = ((1u << BITS) - 1u) * 0x00010001u;
     constexpr uint32_t kMagic = BF16 ? 0x43004300u : 0x64006400u;
+    // fp16 (and bf16 with byte codes) unpack adjacent codes into adjacent K-slots, so the activation
+    // chunks are used as they lie; the other bf16 cases pair code j with j + 4 (j + 8) and reorder
+    // the activation chunk to match
+    constexpr bool NATURAL = !BF16 || BITS == 8;
     static_assert(PF * LPS < 64, "outstanding copies must fit the vmcnt counter");
 
     extern __shared__ __align__(16) unsigned char smem[];
@@ -314,6 +318,12 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
 
     uint32_t pair_mask = kPairMask, magic = kMagic;
     asm volatile("" : "+s"(pair_mask), "+v"(magic));  // registers, so that v_and_or_b32 is selected
+    // natural-order unpacking (fp16): mask and magic of a code pair that shares a byte
+    uint32_t nat_mask0 = BITS == 4 ? 0x00F0000Fu : 0x000C0003u, nat_magic0 = BITS == 4 ? 0x54006400u : 0x5C006400u;
+    uint32_t nat_mask1 = 0x00C00030u, nat_magic1 = 0x4C005400u;
+    asm volatile("" : "+s"(nat_mask0), "+v"(nat_magic0), "+s"(nat_mask1), "+v"(nat_magic1));
+    // 2-bit: the lane's eight codes are bytes 2kb and 2kb + 1 of the word
+    const uint32_t sel2_lo = 0x0c000c00u | ((2 * kb) << 16) | (2 * kb), sel2_hi = 0x0c000c00u | ((2 * kb + 1) << 16) | (2 * kb + 1);
 
     const int sw = (r32 >> 1) & 7;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
     const int a_row0 = (wm * WM + r32) * kRowW;
@@ -360,36 +370,37 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
         issue_next(slot == 0 ? RING - 1 : slot - 1);  // overwrites the slot of stage k-1
         const unsigned char* base = smem + slot * SLOT;
         convert_meta(base + S_OFF + m_lane, base + Z_OFF + m_lane);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {  // four MFMA K-steps of 16
-            u32x4 af[TI];
+        // Four MFMA K-steps of 16, software-pipelined: while the MFMAs of K-step s run, the LDS reads
+        // of K-step s+1 return and its operands are unpacked, one MFMA to every few VALU
+        // instructions.  (Left to itself the compiler unpacks, then multiplies; the waves of a
+        // workgroup run in phase, so matrix pipe and VALU would take turns.)
+        struct Raw {
+            u32x4 a[TI];                       // activation chunk(s) of the lane's row in each row tile
+            uint32_t w[BITS == 8 ? 2 : 1][TJ]; // weight words of the lane's column in each column tile
+        };
+        struct Ops {
+            u32x4 af[TI], bq[TJ];
+        };
+        auto read_raw = [&](int s, Raw& r) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < TI; ++i) {
                 const unsigned char* row = base + a_row0 + i * 32 * kRowW;
-                if constexpr (BITS == 2) {
+                if constexpr (BITS == 2 && !NATURAL) {
                     // a word holds 16 K-values; half kb unpacks slots (j, j + 8), j = 4kb .. 4kb+3
                     const u32x2 lo = *(const u32x2*)(row + (((2 * s) ^ sw) << 4) + 8 * kb);
                     const u32x2 hi = *(const u32x2*)(row + (((2 * s + 1) ^ sw) << 4) + 8 * kb);
-                    af[i] = pair_order(lo.x, lo.y, hi.x, hi.y);
+                    r.a[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
                 } else {
-                    const u32x4 v = *(const u32x4*)(row + (((2 * s + kb) ^ sw) << 4));
-                    if constexpr (BITS == 4) af[i] = pair_order(v.x, v.y, v.z, v.w);  // slots (j, j + 4)
-                    else {  // two words of 4 codes: slots (j, j + 2) inside each word
-                        af[i].x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);
-                        af[i].y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);
-                        af[i].z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);
-                        af[i].w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);
-                    }
+                    r.a[i] = *(const u32x4*)(row + (((2 * s + kb) ^ sw) << 4));
                 }
             }
-            uint32_t wv[BITS == 8 ? 2 : 1][TJ];
             auto load_words = [&](int v, int u) __attribute__((always_inline)) {
                 if constexpr (TJ == 4) {
                     const u32x4 t = *(const u32x4*)(base + w_lane + u * 1024);
-                    wv[v][0] = t.x; wv[v][1] = t.y; wv[v][2] = t.z; wv[v][3] = t.w;
+                    r.w[v][0] = t.x; r.w[v][1] = t.y; r.w[v][2] = t.z; r.w[v][3] = t.w;
                 } else {
                     const u32x2 t = *(const u32x2*)(base + w_lane + u * 1024);
-                    wv[v][0] = t.x; wv[v][1] = t.y;
+                    r.w[v][0] = t.x; r.w[v][1] = t.y;
                 }
             };
             if constexpr (BITS == 8) {
@@ -398,34 +409,82 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
             } else {
                 load_words(0, s);
             }
+        };
+        auto unpack = [&](const Raw& r, Ops& o) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                const u32x4 v = r.a[i];
+                if constexpr (NATURAL) o.af[i] = v;
+                else o.af[i] = pair_order(v.x, v.y, v.z, v.w);  // slots (j, j + 4), or (j, j + 8) for 2-bit codes
+            }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                u32x4 bq;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
+                for (int q = 0; q < 4; ++q) {
                     uint32_t t;
-                    if constexpr (BITS == 4) {
-                        t = ((wv[0][j] >> (r * 4)) & pair_mask) | magic;
-                    } else if constexpr (BITS == 8 && BF16) {
-                        // 128 + q is not exact in bf16 above 127: convert the two bytes (slots r%2 and
-                        // r%2 + 2 of the word) to fp32 directly, scale there and pack once
-                        const uint32_t w = wv[r / 2][j];
+                    if constexpr (BITS == 8 && BF16) {
+                        // 128 + q is not exact in bf16 above 127: convert bytes 2(q%2) and 2(q%2) + 1 of the
+                        // word to fp32 directly, scale there and pack once
+                        const uint32_t w = r.w[q / 2][j];
                         typedef float f32x2 __attribute__((ext_vector_type(2)));
-                        const f32x2 f = {__builtin_fmaf((float)((w >> ((r % 2) * 8)) & 0xffu), meta[j].s, meta[j].z),
-                                         __builtin_fmaf((float)((w >> ((r % 2) * 8 + 16)) & 0xffu), meta[j].s, meta[j].z)};
-                        bq[r] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-                        continue;
-                    } else if constexpr (BITS == 8) {
-                        t = ((wv[r / 2][j] >> ((r % 2) * 8)) & pair_mask) | magic;
+                        const f32x2 f = {__builtin_fmaf((float)((w >> ((q % 2) * 16)) & 0xffu), meta[j].s, meta[j].z),
+                                         __builtin_fmaf((float)((w >> ((q % 2) * 16 + 8)) & 0xffu), meta[j].s, meta[j].z)};
+                        o.bq[j][q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+                    } else if constexpr (NATURAL) {
+                        // fp16: register q gets the adjacent codes 2q and 2q+1 of the lane's eight, which
+                        // share a byte (4-, 2-bit) or are adjacent bytes: one v_perm puts that byte (those
+                        // bytes) into both halves, the mask keeps one code per half where it lies, and each
+                        // half's magic exponent is the one whose unit in the last place matches the code's
+                        // position: 1024 + q for bits 0.., 256 + q for bits 2.., 64 + q for bits 4.., 16 + q for bits 6..
+                        if constexpr (BITS == 8) {
+                            const uint32_t u = __builtin_amdgcn_perm(r.w[q / 2][j], r.w[q / 2][j], q % 2 ? 0x0c030c02u : 0x0c010c00u);
+                            t = u | 0x64006400u;
+                            o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
+                        } else if constexpr (BITS == 4) {
+                            const uint32_t u = __builtin_amdgcn_perm(r.w[0][j], r.w[0][j], 0x0c000c00u | (q << 16) | q);
+                            t = (u & nat_mask0) | nat_magic0;
+                            o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 1024.0f, 64.0f);
+                        } else {
+                            const uint32_t u = __builtin_amdgcn_perm(r.w[0][j], r.w[0][j], q / 2 ? sel2_hi : sel2_lo);
+                            if (q % 2 == 0) {
+                                t = (u & nat_mask0) | nat_magic0;
+                                o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 1024.0f, 256.0f);
+                            } else {
+                                t = (u & nat_mask1) | nat_magic1;
+                                o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 64.0f, 16.0f);
+                            }
+                        }
                     } else {
-                        t = ((wv[0][j] >> ((4 * kb + r) * 2)) & pair_mask) | magic;
+                        if constexpr (BITS == 4) t = ((r.w[0][j] >> (q * 4)) & pair_mask) | magic;
+                        else t = ((r.w[0][j] >> ((4 * kb + q) * 2)) & pair_mask) | magic;
+                        o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
                     }
-                    bq[r] = dequant_pair<BF16>(t, meta[j]);
                 }
-#pragma unroll
-                for (int i = 0; i < TI; ++i) acc[i][j] = mfma32<BF16>(bq, af[i], acc[i][j]);  // weights are the row operand
             }
-            __builtin_amdgcn_sched_barrier(0);  // keep the unpacking of later K-steps from being hoisted (register pressure)
+        };
+        Raw raw;
+        Ops ops[2];
+        read_raw(0, raw);
+        unpack(raw, ops[0]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            if (s < 3) read_raw(s + 1, raw);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+#pragma unroll
+                for (int i = 0; i < TI; ++i) acc[i][j] = mfma32<BF16>(ops[s & 1].bq[j], ops[s & 1].af[i], acc[i][j]);  // weights are the row operand
+            if (s < 3) {
+                unpack(raw, ops[(s + 1) & 1]);
+                constexpr int NMF = TI * TJ, NVA = 4 * TI + 16 * TJ;  // MFMAs and (at least) VALU instructions of the region
+                __builtin_amdgcn_sched_group_barrier(0x100, TI + (BITS == 8 ? 2 : 1), 0);  // the LDS reads first
+#pragma unroll
+                for (int q = 0; q < NMF; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, (NVA + NMF - 1) / NMF, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         slot = slot == RING - 1 ? 0 : slot + 1;
     }
