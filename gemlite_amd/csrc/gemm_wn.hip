@@ -170,7 +170,6 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
     constexpr int NW = WAVES_M * WN;         // waves
     constexpr int WL = (BITS == 8) ? 8 : 4;  // 128-bit weight loads per lane per stage
     constexpr int RING = ring_slots(BM);
-    constexpr int PF = RING - 1;             // stages in flight ahead of the one being multiplied
     constexpr int SLOT = slot_bytes(BITS, BM);
     constexpr int W_OFF = BM * kRowW, S_OFF = W_OFF + 2 * WL * 1024, Z_OFF = S_OFF + 512;
     constexpr int A_JOBS = BM / 8;           // 16-byte copy instructions for the A tile (8 rows each)
@@ -184,7 +183,7 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
     // chunks are used as they lie; the other bf16 cases pair code j with j + 4 (j + 8) and reorder
     // the activation chunk to match
     constexpr bool NATURAL = !BF16 || BITS == 8;
-    static_assert(PF * LPS < 64, "outstanding copies must fit the vmcnt counter");
+    static_assert(RING * LPS < 64, "outstanding copies must fit the vmcnt counter");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -351,142 +350,160 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
         }
     };
 
+    // ---- pipeline.  RING stages are in flight.  The loop is software-pipelined twice over:
+    //  * inside a stage, while the MFMAs of K-step s run, the LDS reads of K-step s+1 return and its
+    //    operands are unpacked, one MFMA to every few VALU instructions (left to itself the compiler
+    //    unpacks, then multiplies; the waves of a workgroup run in phase, so matrix pipe and VALU
+    //    would take turns);
+    //  * across stages, the barrier that publishes stage k+1 stands before the last K-step of
+    //    stage k, whose MFMAs then cover the conversion of stage k+1's scales and zeros and the
+    //    unpacking of its first K-step.  By then every wave has read all it needs of stage k, so
+    //    the copies of stage k+RING go to that slot right after the barrier.
+    // Copies complete in issue order.  The barrier is bare on purpose: __syncthreads() carries a
+    // release fence, which for copies into LDS means draining the whole counter and with it the
+    // pipeline.  The empty asm statements keep the compiler from moving LDS accesses across it.
+    struct Raw {
+        u32x4 a[TI];                       // activation chunk(s) of the lane's row in each row tile
+        uint32_t w[BITS == 8 ? 2 : 1][TJ]; // weight words of the lane's column in each column tile
+    };
+    struct Ops {
+        u32x4 af[TI], bq[TJ];
+    };
+    auto read_raw = [&](const unsigned char* base, int s, Raw& r) __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < PF; ++u) issue_next(u);
+        for (int i = 0; i < TI; ++i) {
+            const unsigned char* row = base + a_row0 + i * 32 * kRowW;
+            if constexpr (BITS == 2 && !NATURAL) {
+                // a word holds 16 K-values; half kb unpacks slots (j, j + 8), j = 4kb .. 4kb+3
+                const u32x2 lo = *(const u32x2*)(row + (((2 * s) ^ sw) << 4) + 8 * kb);
+                const u32x2 hi = *(const u32x2*)(row + (((2 * s + 1) ^ sw) << 4) + 8 * kb);
+                r.a[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
+            } else {
+                r.a[i] = *(const u32x4*)(row + (((2 * s + kb) ^ sw) << 4));
+            }
+        }
+        auto load_words = [&](int v, int u) __attribute__((always_inline)) {
+            if constexpr (TJ == 4) {
+                const u32x4 t = *(const u32x4*)(base + w_lane + u * 1024);
+                r.w[v][0] = t.x; r.w[v][1] = t.y; r.w[v][2] = t.z; r.w[v][3] = t.w;
+            } else {
+                const u32x2 t = *(const u32x2*)(base + w_lane + u * 1024);
+                r.w[v][0] = t.x; r.w[v][1] = t.y;
+            }
+        };
+        if constexpr (BITS == 8) {
+            load_words(0, 2 * s);
+            load_words(1, 2 * s + 1);
+        } else {
+            load_words(0, s);
+        }
+    };
+    auto unpack = [&](const Raw& r, Ops& o) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            const u32x4 v = r.a[i];
+            if constexpr (NATURAL) o.af[i] = v;
+            else o.af[i] = pair_order(v.x, v.y, v.z, v.w);  // slots (j, j + 4), or (j, j + 8) for 2-bit codes
+        }
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t t;
+                if constexpr (BITS == 8 && BF16) {
+                    // 128 + q is not exact in bf16 above 127: convert bytes 2(q%2) and 2(q%2) + 1 of the
+                    // word to fp32 directly, scale there and pack once
+                    const uint32_t w = r.w[q / 2][j];
+                    typedef float f32x2 __attribute__((ext_vector_type(2)));
+                    const f32x2 f = {__builtin_fmaf((float)((w >> ((q % 2) * 16)) & 0xffu), meta[j].s, meta[j].z),
+                                     __builtin_fmaf((float)((w >> ((q % 2) * 16 + 8)) & 0xffu), meta[j].s, meta[j].z)};
+                    o.bq[j][q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+                } else if constexpr (NATURAL) {
+                    // fp16: register q gets the adjacent codes 2q and 2q+1 of the lane's eight, which
+                    // share a byte (4-, 2-bit) or are adjacent bytes: one v_perm puts that byte (those
+                    // bytes) into both halves, the mask keeps one code per half where it lies, and each
+                    // half's magic exponent is the one whose unit in the last place matches the code's
+                    // position: 1024 + q for bits 0.., 256 + q for bits 2.., 64 + q for bits 4.., 16 + q for bits 6..
+                    if constexpr (BITS == 8) {
+                        const uint32_t u = __builtin_amdgcn_perm(r.w[q / 2][j], r.w[q / 2][j], q % 2 ? 0x0c030c02u : 0x0c010c00u);
+                        t = u | 0x64006400u;
+                        o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
+                    } else if constexpr (BITS == 4) {
+                        const uint32_t u = __builtin_amdgcn_perm(r.w[0][j], r.w[0][j], 0x0c000c00u | (q << 16) | q);
+                        t = (u & nat_mask0) | nat_magic0;
+                        o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 1024.0f, 64.0f);
+                    } else {
+                        const uint32_t u = __builtin_amdgcn_perm(r.w[0][j], r.w[0][j], q / 2 ? sel2_hi : sel2_lo);
+                        if (q % 2 == 0) {
+                            t = (u & nat_mask0) | nat_magic0;
+                            o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 1024.0f, 256.0f);
+                        } else {
+                            t = (u & nat_mask1) | nat_magic1;
+                            o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 64.0f, 16.0f);
+                        }
+                    }
+                } else {
+                    if constexpr (BITS == 4) t = ((r.w[0][j] >> (q * 4)) & pair_mask) | magic;
+                    else t = ((r.w[0][j] >> ((4 * kb + q) * 2)) & pair_mask) | magic;
+                    o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
+                }
+            }
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < RING; ++u) issue_next(u);
+    Raw raw;
+    Ops ops[2];
+    wait_vmcnt<(RING - 1) * LPS>();  // stage 0 has landed (this wave's part)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();    // ... and everybody else's
+    asm volatile("" ::: "memory");
+    convert_meta(smem + S_OFF + m_lane, smem + Z_OFF + m_lane);
+    read_raw(smem, 0, raw);
+    unpack(raw, ops[0]);
 
+    constexpr int NMF = TI * TJ;                                     // MFMAs of a K-step
+    constexpr int NVA = (NATURAL ? 0 : 4 * TI) + 16 * TJ;            // VALU instructions of an unpacking, roughly
+    constexpr int NRD = TI * (BITS == 2 && !NATURAL ? 2 : 1) + (BITS == 8 ? 2 : 1);  // LDS reads of a K-step
     int slot = 0;  // ring slot of the stage being multiplied
 #pragma unroll 1
     for (int k = 0; k < steps; ++k) {
-        // copies complete in issue order: once at most those of PF - 1 stages are outstanding, stage k has landed
-        // A bare barrier on purpose: __syncthreads() carries a release fence, which for copies into
-        // LDS means draining the whole counter and with it the pipeline.  Each wave has waited for
-        // its own part of stage k; the barrier makes all parts visible and says that every wave is
-        // done reading stage k-1.  The empty asm statements keep the compiler from moving LDS
-        // accesses across it.
-        wait_vmcnt<(PF - 1) * LPS>();
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue_next(slot == 0 ? RING - 1 : slot - 1);  // overwrites the slot of stage k-1
         const unsigned char* base = smem + slot * SLOT;
-        convert_meta(base + S_OFF + m_lane, base + Z_OFF + m_lane);
-        // Four MFMA K-steps of 16, software-pipelined: while the MFMAs of K-step s run, the LDS reads
-        // of K-step s+1 return and its operands are unpacked, one MFMA to every few VALU
-        // instructions.  (Left to itself the compiler unpacks, then multiplies; the waves of a
-        // workgroup run in phase, so matrix pipe and VALU would take turns.)
-        struct Raw {
-            u32x4 a[TI];                       // activation chunk(s) of the lane's row in each row tile
-            uint32_t w[BITS == 8 ? 2 : 1][TJ]; // weight words of the lane's column in each column tile
-        };
-        struct Ops {
-            u32x4 af[TI], bq[TJ];
-        };
-        auto read_raw = [&](int s, Raw& r) __attribute__((always_inline)) {
-#pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                const unsigned char* row = base + a_row0 + i * 32 * kRowW;
-                if constexpr (BITS == 2 && !NATURAL) {
-                    // a word holds 16 K-values; half kb unpacks slots (j, j + 8), j = 4kb .. 4kb+3
-                    const u32x2 lo = *(const u32x2*)(row + (((2 * s) ^ sw) << 4) + 8 * kb);
-                    const u32x2 hi = *(const u32x2*)(row + (((2 * s + 1) ^ sw) << 4) + 8 * kb);
-                    r.a[i] = u32x4{lo.x, lo.y, hi.x, hi.y};
-                } else {
-                    r.a[i] = *(const u32x4*)(row + (((2 * s + kb) ^ sw) << 4));
-                }
-            }
-            auto load_words = [&](int v, int u) __attribute__((always_inline)) {
-                if constexpr (TJ == 4) {
-                    const u32x4 t = *(const u32x4*)(base + w_lane + u * 1024);
-                    r.w[v][0] = t.x; r.w[v][1] = t.y; r.w[v][2] = t.z; r.w[v][3] = t.w;
-                } else {
-                    const u32x2 t = *(const u32x2*)(base + w_lane + u * 1024);
-                    r.w[v][0] = t.x; r.w[v][1] = t.y;
-                }
-            };
-            if constexpr (BITS == 8) {
-                load_words(0, 2 * s);
-                load_words(1, 2 * s + 1);
+        const int next = slot == RING - 1 ? 0 : slot + 1;
+        const unsigned char* nbase = smem + next * SLOT;
+        auto kstep = [&](auto s_tag) __attribute__((always_inline)) {
+            constexpr int s = decltype(s_tag)::value;
+            if constexpr (s == 3) {
+                // stage k+1 has landed once at most the copies of the RING - 2 stages after it are outstanding
+                wait_vmcnt<(RING - 2) * LPS>();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                issue_next(slot);  // stage k + RING
+                __builtin_amdgcn_sched_barrier(0);
+                read_raw(nbase, 0, raw);
             } else {
-                load_words(0, s);
+                read_raw(base, s + 1, raw);
             }
-        };
-        auto unpack = [&](const Raw& r, Ops& o) __attribute__((always_inline)) {
-#pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                const u32x4 v = r.a[i];
-                if constexpr (NATURAL) o.af[i] = v;
-                else o.af[i] = pair_order(v.x, v.y, v.z, v.w);  // slots (j, j + 4), or (j, j + 8) for 2-bit codes
-            }
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    uint32_t t;
-                    if constexpr (BITS == 8 && BF16) {
-                        // 128 + q is not exact in bf16 above 127: convert bytes 2(q%2) and 2(q%2) + 1 of the
-                        // word to fp32 directly, scale there and pack once
-                        const uint32_t w = r.w[q / 2][j];
-                        typedef float f32x2 __attribute__((ext_vector_type(2)));
-                        const f32x2 f = {__builtin_fmaf((float)((w >> ((q % 2) * 16)) & 0xffu), meta[j].s, meta[j].z),
-                                         __builtin_fmaf((float)((w >> ((q % 2) * 16 + 8)) & 0xffu), meta[j].s, meta[j].z)};
-                        o.bq[j][q] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-                    } else if constexpr (NATURAL) {
-                        // fp16: register q gets the adjacent codes 2q and 2q+1 of the lane's eight, which
-                        // share a byte (4-, 2-bit) or are adjacent bytes: one v_perm puts that byte (those
-                        // bytes) into both halves, the mask keeps one code per half where it lies, and each
-                        // half's magic exponent is the one whose unit in the last place matches the code's
-                        // position: 1024 + q for bits 0.., 256 + q for bits 2.., 64 + q for bits 4.., 16 + q for bits 6..
-                        if constexpr (BITS == 8) {
-                            const uint32_t u = __builtin_amdgcn_perm(r.w[q / 2][j], r.w[q / 2][j], q % 2 ? 0x0c030c02u : 0x0c010c00u);
-                            t = u | 0x64006400u;
-                            o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
-                        } else if constexpr (BITS == 4) {
-                            const uint32_t u = __builtin_amdgcn_perm(r.w[0][j], r.w[0][j], 0x0c000c00u | (q << 16) | q);
-                            t = (u & nat_mask0) | nat_magic0;
-                            o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 1024.0f, 64.0f);
-                        } else {
-                            const uint32_t u = __builtin_amdgcn_perm(r.w[0][j], r.w[0][j], q / 2 ? sel2_hi : sel2_lo);
-                            if (q % 2 == 0) {
-                                t = (u & nat_mask0) | nat_magic0;
-                                o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 1024.0f, 256.0f);
-                            } else {
-                                t = (u & nat_mask1) | nat_magic1;
-                                o.bq[j][q] = dequant_pair<BF16>(t, meta[j], 64.0f, 16.0f);
-                            }
-                        }
-                    } else {
-                        if constexpr (BITS == 4) t = ((r.w[0][j] >> (q * 4)) & pair_mask) | magic;
-                        else t = ((r.w[0][j] >> ((4 * kb + q) * 2)) & pair_mask) | magic;
-                        o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
-                    }
-                }
-            }
-        };
-        Raw raw;
-        Ops ops[2];
-        read_raw(0, raw);
-        unpack(raw, ops[0]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            if (s < 3) read_raw(s + 1, raw);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
 #pragma unroll
                 for (int i = 0; i < TI; ++i) acc[i][j] = mfma32<BF16>(ops[s & 1].bq[j], ops[s & 1].af[i], acc[i][j]);  // weights are the row operand
-            if (s < 3) {
-                unpack(raw, ops[(s + 1) & 1]);
-                constexpr int NMF = TI * TJ, NVA = 4 * TI + 16 * TJ;  // MFMAs and (at least) VALU instructions of the region
-                __builtin_amdgcn_sched_group_barrier(0x100, TI + (BITS == 8 ? 2 : 1), 0);  // the LDS reads first
+            if constexpr (s == 3) convert_meta(nbase + S_OFF + m_lane, nbase + Z_OFF + m_lane);
+            unpack(raw, ops[(s + 1) & 1]);
+            __builtin_amdgcn_sched_group_barrier(0x100, NRD + (s == 3 ? 2 : 0), 0);  // the LDS reads first
 #pragma unroll
-                for (int q = 0; q < NMF; ++q) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, (NVA + NMF - 1) / NMF, 0);
-                }
+            for (int q = 0; q < NMF; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, (NVA + (s == 3 ? 16 * TJ : 0) + NMF - 1) / NMF, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
-        }
-        slot = slot == RING - 1 ? 0 : slot + 1;
+        };
+        kstep(std::integral_constant<int, 0>{});
+        kstep(std::integral_constant<int, 1>{});
+        kstep(std::integral_constant<int, 2>{});
+        kstep(std::integral_constant<int, 3>{});
+        slot = next;
     }
 
     // ---- epilogue.  With the weights as row operand an accumulator is the transposed output tile:
