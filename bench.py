@@ -117,17 +117,38 @@ def extra_points(lib, device):
                 raise RuntimeError(lib.gla_last_error().decode())
         return run
 
-    def point(name, M, N, K, us, peak_tf):
+    # Sustained matrix rate of this board: a register-only MFMA loop (no memory traffic) with zero and
+    # with random operand bits.  With random bits the power limit lowers the clock; that rate, not the
+    # datasheet one, is what a GEMM on real data can at most reach here.
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+    probe = {}
+    for name, dt in (("fp16", 1), ("bf16", 2), ("fp8", 3), ("int8", 4), ("mxfp4", 17)):
+        rates = {}
+        for label, rnd in (("zero_operands", 0), ("random_operands", 1)):
+            flops = ctypes.c_double(0.0)
+
+            def run():
+                if lib.gla_probe_mfma(dt, rnd, 60000, sink.data_ptr(), ctypes.byref(flops),
+                                      torch.cuda.current_stream().cuda_stream) != 0:
+                    raise RuntimeError(lib.gla_last_error().decode())
+            us = time_us(run, 3, warm=1)
+            rates[label + "_TFLOP/s"] = round(flops.value / us / 1e6, 1)
+        probe[name] = rates
+    out["mfma_probe"] = probe
+
+    def point(name, M, N, K, us, peak_tf, kind):
         tf = 2.0 * M * N * K / us / 1e6
+        sustained = probe[kind]["random_operands_TFLOP/s"]
         out[name] = {"M": M, "N": N, "K": K, "us": round(us, 1), "TFLOP/s": round(tf, 1),
-                     "frac_of_peak": round(tf / peak_tf, 4), "peak_TFLOP/s": peak_tf}
+                     "frac_of_peak": round(tf / peak_tf, 4), "peak_TFLOP/s": peak_tf,
+                     "frac_of_sustained_mfma": round(tf / sustained, 4)}
 
     # A16W4 gs128 fp16, M = 4096 (fused-dequant MFMA GEMM)
     M, N, K = 4096, 4096, 4096
     layer, _ = make_layer(N, K, seed=11, device=device)
     x = torch.randn((M, K), generator=g).to(torch.float16).to(device)
     y = torch.empty((M, N), dtype=torch.float16, device=device)
-    point("gemm_a16w4_gs128_fp16", M, N, K, time_us(prepared(layer, x, None, y), 50), 2500.0)
+    point("gemm_a16w4_gs128_fp16", M, N, K, time_us(prepared(layer, x, None, y), 50), 2500.0, "fp16")
     del layer, x, y
 
     # A8W8 fp8 / int8 dynamic, M = 4096, N = K = 8192: activation quantiser + GEMM
@@ -138,7 +159,7 @@ def extra_points(lib, device):
     for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
         layer = proc(device=device).from_weights(W)
         xq, sx = gemlite_amd.scale_activations_per_token(x, wdt)
-        point(f"gemm_a8w8_{name}", M, N, K, time_us(prepared(layer, xq, sx, y), 50), 5000.0)
+        point(f"gemm_a8w8_{name}", M, N, K, time_us(prepared(layer, xq, sx, y), 50), 5000.0, name)
         us = time_us(lambda: gemlite_amd.scale_activations_per_token(x, wdt), 20)
         out[f"actquant_per_token_{name}"] = {"M": M, "K": K, "us": round(us, 1),
                                             "GB/s": round((M * K * 3 + M * 4) / us / 1e3, 1)}
@@ -154,7 +175,7 @@ def extra_points(lib, device):
     x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
     xq, sx = gemlite_amd.scale_activations_mxfp4(x)
     y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    point("gemm_a4w4_mxfp4", M, N, K, time_us(prepared(layer, xq, sx, y), 30), 10100.0)
+    point("gemm_a4w4_mxfp4", M, N, K, time_us(prepared(layer, xq, sx, y), 30), 10100.0, "mxfp4")
     us = time_us(lambda: gemlite_amd.scale_activations_mxfp4(x), 20)
     out["actquant_mxfp4"] = {"M": M, "K": K, "us": round(us, 1),
                              "GB/s": round((M * K * 2 + M * K // 2 + M * K // 32) / us / 1e3, 1)}

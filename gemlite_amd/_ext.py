@@ -88,6 +88,8 @@ SYMBOLS = {
     "gla_get_closest_m": (ctypes.c_int, [ctypes.c_int]),
     "gla_select_config": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul_family": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
+    "gla_probe_mfma": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                      ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]),
     "gla_matmul_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),
     "gla_scale_activations_per_token": (

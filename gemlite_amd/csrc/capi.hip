@@ -173,6 +173,10 @@ int gla_select_config(const gla_matmul_args* args) {
     return 0;
 }
 
+int gla_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, void* stream) {
+    return gla::launch_probe_mfma(dtype, random_operands, iters, sink, flops, (hipStream_t)stream);
+}
+
 int gla_matmul_family(const gla_matmul_args* args) {
     const int rc = validate(args);
     if (rc != GLA_OK) return rc;

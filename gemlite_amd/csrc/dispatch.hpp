@@ -43,4 +43,7 @@ int launch_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t
 int launch_unpack_over_cols(const void* packed, uint8_t* out, int64_t rows, int64_t pcols, int nbits, int width,
                             hipStream_t stream);
 
+// ---- diagnostic: sustained matrix rate (probe.hip) ---------------------------
+int launch_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, hipStream_t stream);
+
 }  // namespace gla

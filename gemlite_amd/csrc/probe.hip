@@ -1,0 +1,106 @@
+// Diagnostic: the matrix rate the device sustains.  A register-only loop of independent MFMAs on
+// every SIMD, no memory traffic.  With zero operands this reaches the datasheet rate; with random
+// operand bits the same loop runs into the board's power limit and the clock drops, which is the
+// ceiling any GEMM on real data sees.  Timed by the caller (events around the launch).
+// No counterpart in the reference.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace gla {
+
+namespace {
+
+typedef _Float16 half8_p __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_p __attribute__((ext_vector_type(8)));
+typedef int int8_p __attribute__((ext_vector_type(8)));
+typedef int int16_p __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t mix(uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+    return x;
+}
+
+// DT: GLA_DT_FP16, GLA_DT_BF16, GLA_DT_FP8, GLA_DT_INT8 or GLA_DT_MXFP4
+template <int DT>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, int random_operands, float* sink) {
+    constexpr int NACC = 8, NOP = 4;
+    float16_t acc[NACC];
+    int16_p iacc[NACC];
+    for (int a = 0; a < NACC; ++a)
+        for (int e = 0; e < 16; ++e) { acc[a][e] = 0.0f; iacc[a][e] = 0; }
+    int8_p a8[NOP], b8[NOP];
+    const uint32_t seed = (blockIdx.x * 256u + threadIdx.x) * 977u;
+    for (int o = 0; o < NOP; ++o)
+        for (int e = 0; e < 8; ++e) {
+            uint32_t ra = random_operands ? mix(seed + o * 64 + e) : 0u, rb = random_operands ? mix(seed + o * 64 + e + 32) : 0u;
+            if (DT == GLA_DT_FP8) { ra &= 0xbfbfbfbfu; rb &= 0xbfbfbfbfu; }                       // finite, |x| < 2
+            if (DT == GLA_DT_FP16 || DT == GLA_DT_BF16) { ra &= 0xbfffbfffu; rb &= 0xbfffbfffu; }   // finite, |x| < 2
+            a8[o][e] = (int)ra; b8[o][e] = (int)rb;
+        }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int a = 0; a < NACC; ++a) {
+            const int8_p x = a8[a % NOP], y = b8[(a / 2) % NOP];
+            const int4_t x4 = {x[0], x[1], x[2], x[3]}, y4 = {y[0], y[1], y[2], y[3]};
+            if constexpr (DT == GLA_DT_FP16)
+                acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_p, x4), __builtin_bit_cast(half8_p, y4), acc[a], 0, 0, 0);
+            else if constexpr (DT == GLA_DT_BF16)
+                acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_p, x4), __builtin_bit_cast(bf16x8_p, y4), acc[a], 0, 0, 0);
+            else if constexpr (DT == GLA_DT_FP8)
+                acc[a] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc[a], 0, 0, 0, 127, 0, 127);
+            else if constexpr (DT == GLA_DT_INT8)
+                iacc[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(x4, y4, iacc[a], 0, 0, 0);
+            else
+                acc[a] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc[a], 4, 4, 0, 127, 0, 127);
+        }
+    }
+    float s = 0.0f;
+    for (int a = 0; a < NACC; ++a)
+        for (int e = 0; e < 16; ++e) s += acc[a][e] + (float)iacc[a][e];
+    if (s == 123.456f) sink[0] = s;  // keeps the loop alive; never true for these operands in practice
+}
+
+}  // namespace
+
+int launch_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, hipStream_t stream) {
+    if (iters < 1 || sink == nullptr) {
+        set_error("gla_probe_mfma: iters >= 1 and a 4-byte device buffer are required");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    int dev = 0, cus = 0;
+    int rc = check_hip(hipGetDevice(&dev), "gla_probe_mfma: hipGetDevice");
+    if (rc != GLA_OK) return rc;
+    rc = check_hip(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev), "gla_probe_mfma: CU count");
+    if (rc != GLA_OK) return rc;
+    const int grid = cus * 2;  // two waves per SIMD
+    double per_mfma;
+    switch (dtype) {
+        case GLA_DT_FP16:
+            per_mfma = 2.0 * 32 * 32 * 16;
+            hipLaunchKernelGGL(probe_mfma_kernel<GLA_DT_FP16>, dim3(grid), dim3(256), 0, stream, iters, random_operands, (float*)sink);
+            break;
+        case GLA_DT_BF16:
+            per_mfma = 2.0 * 32 * 32 * 16;
+            hipLaunchKernelGGL(probe_mfma_kernel<GLA_DT_BF16>, dim3(grid), dim3(256), 0, stream, iters, random_operands, (float*)sink);
+            break;
+        case GLA_DT_FP8:
+            per_mfma = 2.0 * 32 * 32 * 64;
+            hipLaunchKernelGGL(probe_mfma_kernel<GLA_DT_FP8>, dim3(grid), dim3(256), 0, stream, iters, random_operands, (float*)sink);
+            break;
+        case GLA_DT_INT8:
+            per_mfma = 2.0 * 32 * 32 * 32;
+            hipLaunchKernelGGL(probe_mfma_kernel<GLA_DT_INT8>, dim3(grid), dim3(256), 0, stream, iters, random_operands, (float*)sink);
+            break;
+        case GLA_DT_MXFP4:
+            per_mfma = 2.0 * 32 * 32 * 64;
+            hipLaunchKernelGGL(probe_mfma_kernel<GLA_DT_MXFP4>, dim3(grid), dim3(256), 0, stream, iters, random_operands, (float*)sink);
+            break;
+        default:
+            set_error("gla_probe_mfma: dtype %d has no matrix instruction here", dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (flops != nullptr) *flops = (double)grid * 4 * (double)iters * 8 * per_mfma;
+    return check_hip(hipGetLastError(), "gla_probe_mfma launch");
+}
+
+}  // namespace gla

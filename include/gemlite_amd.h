@@ -155,6 +155,16 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_MXFP4 5   /* block-scaled FP4 MFMA GEMM */
 int gla_matmul_family(const gla_matmul_args* args);
 
+/* Diagnostic, no counterpart in the reference: launches a register-only loop of
+ * 8 * iters independent MFMAs per wave, two waves on every SIMD, no memory
+ * traffic, and stores the flops of the launch in *flops (may be NULL).  The
+ * caller times it (events on `stream`).  dtype: GLA_DT_FP16, GLA_DT_BF16,
+ * GLA_DT_FP8, GLA_DT_INT8 or GLA_DT_MXFP4.  With random_operands = 0 the loop
+ * reaches the datasheet rate; with 1 the operands are random bits and the
+ * board's power limit sets the clock, which is the rate a GEMM on real data can
+ * at most sustain.  sink: 4 bytes of device memory (never written in practice). */
+int gla_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, void* stream);
+
 /* Scratch bytes gla_matmul needs for these arguments (0 if none).  The scratch
  * must be zero-filled once when it is allocated; the library leaves it zeroed
  * where it needs zeros.  (Plays the role of the reference's pre-zeroed output

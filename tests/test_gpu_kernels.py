@@ -328,3 +328,25 @@ def test_tuner_fills_the_config_cache_and_results_stay_correct(device):
     for M in (1, 64):  # whatever tile won is now used by forward(), and the output is still right
         check_layer(layer, gen_x(M, K, torch.float16, seed=M).to(device), torch.float16, types=[])
     GemLiteLinear.reset_config()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype_id,flop_per_mfma", [(1, 2 * 32 * 32 * 16), (2, 2 * 32 * 32 * 16), (3, 2 * 32 * 32 * 64),
+                                                   (4, 2 * 32 * 32 * 32), (17, 2 * 32 * 32 * 64)])
+def test_mfma_probe_runs_and_reports_its_flops(device, dtype_id, flop_per_mfma):
+    """The diagnostic MFMA loop launches for every matrix format, reports the flops of the launch
+    (2 workgroups of 4 waves per CU, 8 MFMAs per iteration) and leaves its sink untouched."""
+    import ctypes
+    from gemlite_amd import _ext
+    lib = _ext.load_library()
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+    flops = ctypes.c_double(0.0)
+    for rnd in (0, 1):
+        rc = lib.gla_probe_mfma(dtype_id, rnd, 50, sink.data_ptr(), ctypes.byref(flops), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.gla_last_error().decode()
+    torch.cuda.synchronize()
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    assert flops.value == cus * 2 * 4 * 50 * 8 * flop_per_mfma
+    assert sink.item() == 0.0
+    assert lib.gla_probe_mfma(0, 0, 50, sink.data_ptr(), None, None) == -2   # fp32: no such loop
+    assert lib.gla_probe_mfma(1, 0, 0, sink.data_ptr(), None, None) == -1
