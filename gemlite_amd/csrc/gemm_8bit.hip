@@ -23,6 +23,11 @@
 //    distinct bank groups.
 //  * Workgroups are renumbered so that each of the 8 XCDs (one L2 each) works on its own band
 //    of output tiles, and tiles inside a band are visited in groups that share operand panels.
+//  * The weights are the row operand of every MFMA: an accumulator is the transposed output tile,
+//    so a lane holds four adjacent output columns of one row and stores them at once.
+//  * MXFP4 with tiles of 128 rows or more: a small kernel first regroups both scale arrays by
+//    pipeline stage in the workspace (dst[stage][row], one 32-bit word each), so that a tile's
+//    scales are one contiguous run per stage instead of one cache line per row.
 #include <type_traits>
 
 #include "common.hpp"
@@ -80,11 +85,12 @@ __device__ __forceinline__ void wait_vmcnt8() {
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
 constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 ? (bm + kBN) * 4 : 0); }
 
-// WN = wave columns.  4: 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
-// (LDS reads bound the 256-row tile: the LDS returns about 64 bytes per clock and CU to 128-bit reads,
-// and this wave tile reads 1.5 fragments per MFMA.  A 2-column variant (4 waves, 128 x 128 wave tiles,
-// accumulators in AGPRs) reads a third less but, with one wave per SIMD and fragments read in the
-// step that multiplies them, measured slower: 1255 against 1650-1800 TFLOP/s in fp8.)
+// WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
+// (A 2-column variant with 4 waves of 128 x 128 and accumulators in AGPRs reads a third less from
+// LDS per MFMA but, with one wave per SIMD and fragments read in the step that multiplies them,
+// measured slower.  LDS bandwidth is not what limits these loops: 128-bit reads sustain well over
+// 200 bytes per clock and CU, the loop needs about 35.  With random operands the board's power
+// limit is: the clock falls to about 1.55 GHz under these kernels.)
 template <int MODE, int BM, int WN>
 __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args p) {
     constexpr int WM = BM / kWavesM;  // wave tile rows

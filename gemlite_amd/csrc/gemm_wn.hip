@@ -7,20 +7,26 @@
 // gemlite/triton_kernels/gemm_splitK_kernels.py:300-523; dequant
 // gemlite/triton_kernels/utils.py:73-105).
 //
-//  * Workgroup tile BM x 256 with BM = 32, 64, 128 or 256, K step 64; waves in a WAVES_M x 2
-//    grid, wave tile (32 TI) x 128 of v_mfma_f32_32x32x16 tiles.
-//  * Weights never pass through LDS.  A lane's 128-bit load holds the words of 4 adjacent
-//    columns; word component j is the B operand of column tile j, so the wave's 128 columns are
-//    the interleaved set {4r + j}.  A word is unpacked with the pair trick of the GEMV kernel
-//    (codes OR-ed into the mantissa of 1024.0 / 128.0, two per VALU op), then (q - OFF) * s + z'
-//    is applied with packed fp16 math (fp32 for bf16 activations) once per wave and reused for
-//    all of its 32-row tiles.  Weight words for the next PF K steps are in flight in registers,
-//    so a workgroup that streams its weights from HBM (small M) is not bound by load latency.
-//  * Activations are copied global -> LDS by the load unit (global_load_lds) into a ring of
-//    PF + 1 tiles with dense 128-byte rows whose 16-byte chunks are XOR-swizzled by (row >> 1) & 7;
-//    the reordering of each chunk to the K-slot order the unpacking produces happens when a
-//    fragment is read (v_perm).
-//  * Scales and zero points ride along with every stage (one dword copy per lane).
+//  * Workgroup tile BM x 256 with BM = 32, 64, 128 or 256, K step 64, v_mfma_f32_32x32x16 tiles.
+//    BM <= 128: waves in a WAVES_M x 2 grid, wave tile (32 TI) x 128.  BM = 256: 2 x 4 waves of
+//    128 x 64, because every wave unpacks the weights of its own columns and the 4 x 2 arrangement
+//    would repeat that work four times per workgroup instead of twice.
+//  * Every operand of a stage (activation tile, packed weight words, scales, zeros) is copied
+//    global -> LDS by the load unit (global_load_lds) into a ring of 3 or 4 stages; the K loop
+//    loads nothing into registers from global memory and waits on the vector-memory counter only
+//    where it says so.  Activation rows are dense 128-byte rows whose 16-byte chunks are
+//    XOR-swizzled by (row >> 1) & 7.  A weight copy job moves 128 columns x both K-halves' word
+//    rows, 16 bytes (4 adjacent columns) per lane; with column tiles interleaved ({TJ r + j}) a
+//    lane reads the words of all its column tiles in one LDS access.
+//  * Unpacking: one v_perm replicates the byte (pair of bytes) that holds two adjacent codes into
+//    both 16-bit halves, a masked OR puts each code into the mantissa of a power of two whose
+//    last-place unit matches the code's bit position (1024 + q, 256 + q, 64 + q, 16 + q), and
+//    (t - offset) * s + z' runs in packed fp16.  Adjacent codes land in adjacent K-slots, so
+//    the activation fragment is used as it lies in memory.  bf16 activations: codes paired (j, j+4)
+//    in the mantissa of 128.0, fp32 fma, one packed round-to-nearest-even conversion (byte codes:
+//    direct byte-to-float conversion); the activation fragment is reordered to match (v_perm).
+//  * The weights are the row operand of the MFMA: an accumulator is the transposed output tile and
+//    a lane holds 4 TJ adjacent output columns of one row, stored 16 bytes at a time.
 //  * When the output has too few tiles to fill the chip (small M), K is split over gridDim.y:
 //    every split writes an fp32 partial tile to the workspace and a second small kernel on the
 //    same stream sums the splits in order, applies the channel scales and stores the output
@@ -652,10 +658,10 @@ WnPlan wn_plan(const gla_matmul_args& p) {
     const int total_steps = p.K / kBKw;
     int want = cfg / 1000;
     if (want <= 0) {
-        // enough workgroups for 256 CUs (two or more each while tiles are small), but no split
-        // shorter than 8 stages (512 K-values) and at most 32 splits
+        // enough workgroups for 256 CUs, but no split shorter than 8 stages (512 K-values) and at
+        // most 32 splits
         const int tiles = g.tiles_m * g.tiles_n;
-        const int target = g.bm >= 128 ? 256 : 512;
+        const int target = 256;
         want = tiles * 2 > target ? 1 : ceil_div(target, tiles);
         const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
         if (want > max_s) want = max_s;
