@@ -1,8 +1,10 @@
 """Processors: recipes that turn weights into packed ``GemLiteLinear`` layers.
 
-Only the recipes the hot path is measured on are provided; each mirrors the
-mode overrides of the reference class of the same name.
+Class names, constructor arguments and mode overrides follow the reference class of the same name
+(reference: gemlite/helper.py).
 """
+import gc
+
 import torch
 
 from .core import GemLiteLinear
@@ -10,10 +12,106 @@ from .dtypes import DType, TORCH_TO_DTYPE
 from .quant_utils import WeightQuantizerMXFP, quantize_weights_per_channel
 
 
+def cleanup_linear(linear_layer, del_orig=True):
+    """Drop the tensors of a replaced layer (reference: gemlite/helper.py:26-32)."""
+    if del_orig:
+        for attr in ("weight", "bias", "weight_scale", "W_q", "meta"):
+            val = getattr(linear_layer, attr, None)
+            if val is not None and hasattr(val, "__len__") and len(val) > 0:
+                setattr(linear_layer, attr, None)
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+
+
+def patch_model(model, device, processor, skip_modules=("lm_head", "vision", "visual"), group_size=64):
+    """Replace every ``torch.nn.Linear`` of ``model`` (outside ``skip_modules``) by
+    ``processor.from_linear(layer)`` (reference: gemlite/helper.py:35-87).  Processors that start
+    from an HQQ layer (``from_hqqlinear``) need the ``hqq`` package to quantize; without it they are
+    refused here, as the reference does."""
+    if hasattr(processor, "from_hqqlinear") and not hasattr(processor, "from_linear"):
+        raise ImportError("This processor requires the `hqq` package to quantize nn.Linear layers; "
+                          "quantize first and use from_weights().")
+    for name, module in model.named_modules():
+        module.name = name
+
+    def patch(parent):
+        for child_name, layer in parent.named_children():
+            if isinstance(layer, torch.nn.Linear):
+                layer = layer.to(device=device)
+                if not any(s in layer.name for s in skip_modules):
+                    layer = processor.from_linear(layer)
+                setattr(parent, child_name, layer)
+            else:
+                patch(layer)
+
+    patch(model)
+    model = model.to(device=device)
+    gc.collect()
+    return model
+
+
+class A16W8:
+    """fp16/bf16 activations x int8 or fp8 weights, one scale per output channel, weights kept as
+    unpacked bytes (reference: gemlite/helper.py:89-171).  ``post_scale``: multiply by the channel
+    scale after the K sum (W_group_mode 0, channel_scale_mode 1) instead of dequantising the weights
+    (W_group_mode 2, channel_scale_mode 0)."""
+
+    def __init__(self, device="cuda:0", dtype=None, fp8=None, fp32_scale=True, post_scale=False):
+        self.device = device
+        self.dtype = dtype
+        self.fp8 = fp8
+        self.fp32_scale = fp32_scale
+        self.post_scale = post_scale
+
+    def from_weights(self, weight, bias=None, scales=None):
+        if isinstance(weight, torch.nn.Parameter):
+            weight = weight.data
+        if isinstance(bias, torch.nn.Parameter):
+            bias = bias.data
+        out_features, in_features = weight.shape
+        if scales is None:
+            w_dtype = self.fp8 if self.fp8 else torch.int8
+            dtype = weight.dtype if self.dtype is None else self.dtype
+            assert dtype in (torch.float16, torch.bfloat16, torch.float32), \
+                f"Invalid weight dtype, should be floating point, got {dtype}"
+            W_q, scales = quantize_weights_per_channel(weight.to(self.device), w_dtype)
+        else:
+            assert weight.dtype.itemsize == 1, f"Invalid weight.dtype, should be 8-bit (INT8 or FP8), got {weight.dtype}"
+            dtype = self.dtype or (scales.dtype if scales.dtype in (torch.float16, torch.bfloat16) else torch.float16)
+            W_q, scales = weight.to(self.device), scales.to(self.device)
+        bias = bias.to(device=self.device, dtype=dtype) if bias is not None else None
+        layer = GemLiteLinear(
+            8, group_size=in_features, in_features=in_features, out_features=out_features,
+            input_dtype=TORCH_TO_DTYPE[dtype], output_dtype=TORCH_TO_DTYPE[dtype],
+        )
+        layer.pack(W_q, scales, zeros=None, bias=bias)
+        if self.post_scale:
+            layer.W_group_mode, layer.channel_scale_mode = 0, 1
+        else:
+            layer.W_group_mode, layer.channel_scale_mode = 2, 0
+        return layer
+
+    def from_linear(self, linear_layer, del_orig=True):
+        out_layer = self.from_weights(weight=linear_layer.weight, bias=linear_layer.bias)
+        cleanup_linear(linear_layer, del_orig)
+        return out_layer
+
+
+class A16W8_INT8(A16W8):
+    def __init__(self, device="cuda:0", dtype=None, fp32_scale=True, post_scale=False):
+        super().__init__(device=device, dtype=dtype, fp8=None, fp32_scale=fp32_scale, post_scale=post_scale)
+
+
+class A16W8_FP8(A16W8):
+    def __init__(self, device="cuda:0", dtype=None, fp8=torch.float8_e4m3fn, fp32_scale=True, post_scale=False):
+        super().__init__(device=device, dtype=dtype, fp8=fp8, fp32_scale=fp32_scale, post_scale=post_scale)
+
+
 class A16Wn:
     """fp16/bf16 activations x grouped 8/4/2/1-bit integer weights
-    (reference: gemlite/helper.py:174-272).  ``post_scale`` defaults to True, the
-    reference's default on AMD GPUs (reference: gemlite/helper.py:14-22)."""
+    (reference: gemlite/helper.py:174-302; the MXFP weight-only variants of that class are not
+    built).  ``post_scale`` defaults to True, the reference's default on AMD GPUs
+    (reference: gemlite/helper.py:14-22)."""
 
     def __init__(self, device="cuda:0", dtype=None, packing_bitwidth=None, post_scale=True):
         self.device = device
@@ -21,10 +119,25 @@ class A16Wn:
         self.packing_bitwidth = packing_bitwidth
         self.post_scale = post_scale
 
-    def from_weights(self, W_q, scales, zeros, W_nbits, group_size, bias=None):
+    def from_packed_weights(self, W_q, scales, zeros, W_nbits, group_size, bias=None, quant_type="INT"):
+        """Load pre-packed weights (already nibble/byte-packed)."""
+        return self.from_weights_(W_q, scales, zeros, W_nbits, group_size, bias, quant_type, packed=True)
+
+    def from_weights(self, W_q, scales, zeros, W_nbits, group_size, bias=None, quant_type="INT"):
+        return self.from_weights_(W_q, scales, zeros, W_nbits, group_size, bias, quant_type)
+
+    def from_weights_(self, W_q, scales, zeros, W_nbits, group_size, bias=None, quant_type="INT", packed=False):
+        if quant_type != "INT":
+            raise NotImplementedError(f"quant_type {quant_type}: only the grouped-integer recipe is built")
+        if isinstance(W_q, torch.nn.Parameter):
+            W_q = W_q.data
+        if isinstance(bias, torch.nn.Parameter):
+            bias = bias.data
         dtype = scales.dtype if self.dtype is None else self.dtype
         assert dtype in (torch.float16, torch.bfloat16, torch.float32), "Invalid scales.dtype, should floating point."
         out_features, in_features = W_q.shape
+        if packed:
+            in_features = in_features * 8 // W_nbits
         W_q = W_q.to(self.device)
         scales = scales.to(device=self.device, dtype=dtype)
         zeros = zeros.to(device=self.device, dtype=dtype) if isinstance(zeros, torch.Tensor) else zeros
@@ -33,7 +146,7 @@ class A16Wn:
             W_nbits, group_size=group_size, in_features=in_features, out_features=out_features,
             input_dtype=TORCH_TO_DTYPE[dtype], output_dtype=TORCH_TO_DTYPE[dtype], scaled_activations=False,
         )
-        layer.pack(W_q, scales, zeros, bias=bias, packing_bitwidth=self.packing_bitwidth)
+        layer.pack(W_q, scales, zeros, bias=bias, packing_bitwidth=self.packing_bitwidth, packed=packed)
         if group_size == in_features:  # channel-wise: scale after or before the K sum
             if self.post_scale:
                 layer.W_group_mode, layer.channel_scale_mode = 1, 1
@@ -41,23 +154,59 @@ class A16Wn:
                 layer.W_group_mode, layer.channel_scale_mode = 3, 0
         return layer
 
+    def from_hqqlinear(self, hqq_layer, del_orig=True):
+        """From an HQQ layer object: what it exposes (``unpack()``, ``meta['scale'|'zero'|'nbits'|
+        'group_size'|'shape'|'axis']``, ``bias``) is all that is used (reference: gemlite/helper.py:274-302)."""
+        assert hqq_layer.meta["axis"] == 1, "Only axis==1 is supported."
+        self.device = hqq_layer.W_q.device
+        W_nbits = hqq_layer.meta["nbits"]
+        group_size = hqq_layer.meta["group_size"]
+        if group_size is None:
+            group_size = hqq_layer.in_features
+        W_q = hqq_layer.unpack(dtype=torch.uint8).view(hqq_layer.meta["shape"])
+        scales, zeros = hqq_layer.meta["scale"].clone(), hqq_layer.meta["zero"].clone()
+        bias = hqq_layer.bias.clone() if hqq_layer.bias is not None else None
+        cleanup_linear(hqq_layer, del_orig)
+        return self.from_weights_(W_q=W_q, scales=scales, zeros=zeros, W_nbits=W_nbits, group_size=group_size,
+                                  bias=bias, quant_type="INT")
 
-class A16W8(A16Wn):
-    def from_weights(self, W_q, scales, zeros, group_size, bias=None):
-        return super().from_weights(W_q, scales, zeros, 8, group_size, bias)
+
+class A16Wn_HQQ_INT(A16Wn):
+    """The grouped-integer recipe with the bit width fixed; the group size follows from the shapes
+    (reference: gemlite/helper.py:344-381)."""
+
+    def __init__(self, device="cuda:0", dtype=None, W_nbits=None):
+        super().__init__(device=device, dtype=dtype)
+        self.W_nbits = W_nbits
+
+    def from_packed_weights(self, W_q_packed, scales, zeros, bias=None):
+        group_size = W_q_packed.numel() * (8 // self.W_nbits) // scales.numel()
+        return super().from_packed_weights(W_q_packed, scales, zeros, self.W_nbits, group_size, bias=bias)
+
+    def from_weights(self, W_q, scales, zeros, bias=None):
+        group_size = W_q.numel() // scales.numel()
+        return super().from_weights(W_q=W_q, scales=scales, zeros=zeros, W_nbits=self.W_nbits,
+                                    group_size=group_size, bias=bias, quant_type="INT")
 
 
-class A16W4(A16Wn):
-    def from_weights(self, W_q, scales, zeros, group_size, bias=None):
-        return super().from_weights(W_q, scales, zeros, 4, group_size, bias)
+class A16W8_HQQ_INT(A16Wn_HQQ_INT):
+    def __init__(self, device="cuda:0", dtype=None):
+        super().__init__(device=device, dtype=dtype, W_nbits=8)
 
 
-class A16W2(A16Wn):
-    def from_weights(self, W_q, scales, zeros, group_size, bias=None):
-        return super().from_weights(W_q, scales, zeros, 2, group_size, bias)
+class A16W4_HQQ_INT(A16Wn_HQQ_INT):
+    def __init__(self, device="cuda:0", dtype=None):
+        super().__init__(device=device, dtype=dtype, W_nbits=4)
 
 
-A16W8_HQQ_INT, A16W4_HQQ_INT, A16W2_HQQ_INT = A16W8, A16W4, A16W2
+class A16W2_HQQ_INT(A16Wn_HQQ_INT):
+    def __init__(self, device="cuda:0", dtype=None):
+        super().__init__(device=device, dtype=dtype, W_nbits=2)
+
+
+class A16W1_HQQ_INT(A16Wn_HQQ_INT):
+    def __init__(self, device="cuda:0", dtype=None):
+        super().__init__(device=device, dtype=dtype, W_nbits=1)
 
 
 class A8W8_dynamic:

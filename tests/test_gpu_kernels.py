@@ -350,3 +350,69 @@ def test_mfma_probe_runs_and_reports_its_flops(device, dtype_id, flop_per_mfma):
     assert sink.item() == 0.0
     assert lib.gla_probe_mfma(0, 0, 50, sink.data_ptr(), None, None) == -2   # fp32: no such loop
     assert lib.gla_probe_mfma(1, 0, 0, sink.data_ptr(), None, None) == -1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("post_scale", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("K", [2080, 2112])   # 2112 = 33 x 64: the matrix-core variant (3..16 rows); 2080: the vector one
+def test_a16w8_weight_only_unpacked_bytes(device, fp8, post_scale, dtype, K):
+    """fp16/bf16 activations x int8 / fp8 weights kept as bytes, one scale per channel
+    (reference processor: gemlite/helper.py:89-171, 336-342).  Up to 16 rows the K-major streaming
+    kernel runs; the codes are the oracle's."""
+    from gemlite_amd import _ext
+    N = 1028                              # K % 32 == 0 as the module requires; neither a multiple of the kernels' tiles
+    W = gen_x(N, K, dtype, seed=21, std=0.02)
+    proc = (helper.A16W8_FP8 if fp8 else helper.A16W8_INT8)(device=device, post_scale=post_scale)
+    # weights are quantised once on the host (CPU torch), then handed over pre-quantised
+    W_q_cpu, s_cpu = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+    proc.dtype = dtype
+    layer = proc.from_weights(W_q_cpu, scales=s_cpu)
+    assert (layer.W_group_mode, layer.channel_scale_mode) == ((0, 1) if post_scale else (2, 0))
+    assert layer.W_q.stride() == (1, K) and layer.W_q.dtype == (torch.float8_e4m3fn if fp8 else torch.int8)
+    q_ref, s_ref = orc.quantize_per_channel(to_np(W), not fp8)
+    got = layer.W_q.t().contiguous()
+    got = got.view(torch.uint8).cpu().numpy() if fp8 else got.cpu().numpy()
+    assert np.array_equal(got, q_ref)
+    for M in (1, 2, 3, 8, 16):
+        x = gen_x(M, K, dtype, seed=M).to(device)
+        out = torch.empty((M, N), dtype=dtype, device=device)
+        m = layer.get_meta_args()
+        args = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                      unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                      acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                      data_contiguous=m[11])
+        assert _ext.matmul_family(args) == "GEMV_KMAJOR"
+        check_layer(layer, x, dtype)
+    check_layer(layer, gen_x(40, K, dtype, seed=40).to(device), dtype)   # above 16 rows: the generic kernel
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("zeros_kind", ["tensor_fma", "tensor_shift_scale", "scalar"])
+def test_int8_bytes_with_zero_point_channelwise(device, dtype, zeros_kind):
+    """Unpacked int8 codes with a per-channel scale and a zero point: the K-major streaming kernels
+    fold the zero point into s (D - z X) / s D + z' X after the K sum."""
+    from gemlite_amd import _ext
+    N, K = 520, 2112
+    g = torch.Generator().manual_seed(3)
+    W_q = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    scales = (torch.rand((N, 1), generator=g) * 0.02 + 0.005).to(dtype)
+    if zeros_kind == "scalar":
+        zeros, fma = 3, True
+    else:
+        zeros, fma = (torch.rand((N, 1), generator=g) * 8 - 4).to(dtype).to(device), zeros_kind == "tensor_fma"
+    dt = DType.FP16 if dtype == torch.float16 else DType.BF16
+    layer = GemLiteLinear(8, K, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros, fma_mode=fma)
+    assert layer.W_q.dtype == torch.int8 and layer.W_q.stride() == (1, K)
+    for M in (1, 2, 5, 16):
+        x = gen_x(M, K, dtype, seed=M).to(device)
+        out = torch.empty((M, N), dtype=dtype, device=device)
+        m = layer.get_meta_args()
+        args = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                      unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                      acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                      data_contiguous=m[11])
+        assert _ext.matmul_family(args) == "GEMV_KMAJOR", (layer.W_group_mode, layer.channel_scale_mode)
+        check_layer(layer, x, dtype)
