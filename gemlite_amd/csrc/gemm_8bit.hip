@@ -539,9 +539,17 @@ struct Plan8 {
 // copy of a tile's scales touches one cache line per row and moves sixteen times the bytes it uses.
 // This kernel regroups them as dst[stage][row] (one 32-bit word each), which a tile copies as
 // consecutive words.  64 x 64 words per workgroup through LDS, both sides coalesced.
-__global__ __launch_bounds__(256) void mx_scales_by_stage_kernel(const uint8_t* src, int rows, int64_t row_stride, int stages, uint32_t* dst) {
+// blockIdx.z picks the array (0: activations, 1: weights), so that one launch regroups both.
+__global__ __launch_bounds__(256) void mx_scales_by_stage_kernel(const uint8_t* src_x, int rows_x, int64_t row_stride_x, uint32_t* dst_x,
+                                                                 const uint8_t* src_w, int rows_w, int64_t row_stride_w, uint32_t* dst_w,
+                                                                 int stages) {
     __shared__ uint32_t tile[64][65];
+    const uint8_t* src = blockIdx.z ? src_w : src_x;
+    const int rows = blockIdx.z ? rows_w : rows_x;
+    const int64_t row_stride = blockIdx.z ? row_stride_w : row_stride_x;
+    uint32_t* dst = blockIdx.z ? dst_w : dst_x;
     const int r0 = blockIdx.x * 64, s0 = blockIdx.y * 64, t = threadIdx.x;
+    if (r0 >= rows) return;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int r = r0 + (t >> 6) + 4 * i, st = s0 + (t & 63);
@@ -677,10 +685,10 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
         const int64_t part = g.S > 1 ? align256((int64_t)g.S * p.M * p.N * 4) : 0;
         uint32_t* sx = (uint32_t*)((char*)p.workspace + kWsReserved8 + part);
         uint32_t* sw = (uint32_t*)((char*)sx + align256((int64_t)stages * p.M * 4));
-        hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(ceil_div(p.M, 64), ceil_div(stages, 64)), dim3(256), 0, stream,
-                           (const uint8_t*)p.scales_x, p.M, (int64_t)p.sx_stride_m, stages, sx);
-        hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(ceil_div(p.N, 64), ceil_div(stages, 64)), dim3(256), 0, stream,
-                           (const uint8_t*)p.scales, p.N, (int64_t)p.meta_stride_n, stages, sw);
+        const int row_blocks = ceil_div(p.M > p.N ? p.M : p.N, 64);
+        hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(row_blocks, ceil_div(stages, 64), 2), dim3(256), 0, stream,
+                           (const uint8_t*)p.scales_x, p.M, (int64_t)p.sx_stride_m, sx,
+                           (const uint8_t*)p.scales, p.N, (int64_t)p.meta_stride_n, sw, stages);
         a.scales_x = sx; a.sxm = 4; a.sx_stage = (int64_t)p.M * 4;
         a.scales = sw; a.msn = 4; a.sw_stage = (int64_t)p.N * 4;
     }
