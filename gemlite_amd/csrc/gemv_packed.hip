@@ -725,7 +725,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
 long long* g_trace = nullptr;
 #endif
 
-int row_tile(int M) { return M > 4 ? 16 : (M >= 3 ? 4 : (M == 2 ? 2 : 1)); }
+int row_tile(int M) { return M >= 3 ? 16 : (M == 2 ? 2 : 1); }
 
 struct Geometry {
     int E, LW, KPS, T, R, RW, S, tiles, RT, mchunks, Mp, gr, G, GW, FL, waves, unit, nb, nfb;
@@ -757,7 +757,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     // 2-bit codes: direct only for the 16-row tile (up to 4 rows the staged kernel measured a little faster)
     const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8 || (p.W_nbits == 2 && g.RT == 16));
     // the cross-wave buffer is [waves][RT][64] floats; the staged 16-row kernel runs 4 waves
-    const int max_waves = (g.RT == 16) ? (can_direct ? 8 : 4) : 16;
+    const int max_waves = (g.RT == 16) ? (can_direct ? 16 : 4) : 16;
     int waves, nb;
     if (p.tile_config >= 1000) {
         waves = p.tile_config / 1000;
@@ -798,7 +798,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
         else
             g.smem = (size_t)(g.RW / g.LW) * g.RT * g.T * 16 + (size_t)g.GW * kTileN * 8 +
                      (size_t)waves * g.RT * kTileN * 4;
-        if (g.smem <= 60 * 1024) break;
+        if (g.smem <= (g.direct && g.RT == 16 ? 100 : 60) * 1024) break;
         if (nb > 1) {
             --nb;
         } else if (waves > 4) {
@@ -824,8 +824,15 @@ void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
             if (g.nb > 1)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
             else if (g.waves == 16) {
-                if constexpr (RT <= 4)
-                    hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
+                if constexpr (RT == 16) {  // its cross-wave buffer alone is 64 KiB
+                    static bool configured = false;
+                    if (!configured) {
+                        (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 16, false>,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
+                        configured = true;
+                    }
+                }
+                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
             } else if (g.waves == 8)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 8, false>), grid, dim3(512), g.smem, stream, a);
             else
