@@ -136,19 +136,32 @@ def extra_points(lib, device):
         probe[name] = rates
     out["mfma_probe"] = probe
 
-    def point(name, M, N, K, us, peak_tf, kind):
+    def point(name, M, N, K, us, peak_tf, kind, us_zero=None):
         tf = 2.0 * M * N * K / us / 1e6
         sustained = probe[kind]["random_operands_TFLOP/s"]
         out[name] = {"M": M, "N": N, "K": K, "us": round(us, 1), "TFLOP/s": round(tf, 1),
                      "frac_of_peak": round(tf / peak_tf, 4), "peak_TFLOP/s": peak_tf,
                      "frac_of_sustained_mfma": round(tf / sustained, 4)}
+        if us_zero is not None:
+            # the same launch on all-zero operands: same instructions and memory traffic, but far less
+            # switching power, so the clock stays up; the gap to `us` is the board's power limit
+            out[name]["us_zero_operands"] = round(us_zero, 1)
+            out[name]["frac_of_peak_zero_operands"] = round(2.0 * M * N * K / us_zero / 1e6 / peak_tf, 4)
+
+    def zeroed(run, *tensors):
+        """Time `run` again with the given operand tensors zero-filled (they are scratch copies)."""
+        for t in tensors:
+            t.view(torch.uint8).zero_()
+        return time_us(run, 30)
 
     # A16W4 gs128 fp16, M = 4096 (fused-dequant MFMA GEMM)
     M, N, K = 4096, 4096, 4096
     layer, _ = make_layer(N, K, seed=11, device=device)
     x = torch.randn((M, K), generator=g).to(torch.float16).to(device)
     y = torch.empty((M, N), dtype=torch.float16, device=device)
-    point("gemm_a16w4_gs128_fp16", M, N, K, time_us(prepared(layer, x, None, y), 50), 2500.0, "fp16")
+    run = prepared(layer, x, None, y)
+    us = time_us(run, 50)
+    point("gemm_a16w4_gs128_fp16", M, N, K, us, 2500.0, "fp16", zeroed(run, x, layer.W_q.data))
     del layer, x, y
 
     # A8W8 fp8 / int8 dynamic, M = 4096, N = K = 8192: activation quantiser + GEMM
@@ -159,7 +172,9 @@ def extra_points(lib, device):
     for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
         layer = proc(device=device).from_weights(W)
         xq, sx = gemlite_amd.scale_activations_per_token(x, wdt)
-        point(f"gemm_a8w8_{name}", M, N, K, time_us(prepared(layer, xq, sx, y), 50), 5000.0, name)
+        run = prepared(layer, xq, sx, y)
+        us = time_us(run, 50)
+        point(f"gemm_a8w8_{name}", M, N, K, us, 5000.0, name, zeroed(run, xq, layer.W_q.data))
         us = time_us(lambda: gemlite_amd.scale_activations_per_token(x, wdt), 20)
         out[f"actquant_per_token_{name}"] = {"M": M, "K": K, "us": round(us, 1),
                                             "GB/s": round((M * K * 3 + M * 4) / us / 1e3, 1)}
@@ -175,7 +190,12 @@ def extra_points(lib, device):
     x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
     xq, sx = gemlite_amd.scale_activations_mxfp4(x)
     y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    point("gemm_a4w4_mxfp4", M, N, K, time_us(prepared(layer, xq, sx, y), 30), 10100.0, "mxfp4")
+    run = prepared(layer, xq, sx, y)
+    us = time_us(run, 30)
+    w_saved = layer.W_q.data.clone()
+    point("gemm_a4w4_mxfp4", M, N, K, us, 10100.0, "mxfp4", zeroed(run, xq, layer.W_q.data))
+    layer.W_q.data.copy_(w_saved)
+    del w_saved
     us = time_us(lambda: gemlite_amd.scale_activations_mxfp4(x), 20)
     out["actquant_mxfp4"] = {"M": M, "K": K, "us": round(us, 1),
                              "GB/s": round((M * K * 2 + M * K // 2 + M * K // 32) / us / 1e3, 1)}
