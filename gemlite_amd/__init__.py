@@ -16,6 +16,7 @@ from .core import (
     GEMLITE_CONFIG_CACHE,
     GEMLITE_MATMUL_TYPES,
     GEMLITE_MATMUL_TYPES_MAPPING,
+    GEMLITE_TRITON_MAPPING,
     GemLiteLinear,
     GemLiteLinearTriton,
     config_key,

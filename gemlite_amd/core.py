@@ -179,25 +179,57 @@ def forward_functional(
     else:
         matmul_type_str = get_matmul_type(M, W_nbits, mx)
 
-    out = torch.empty((M, out_features), dtype=DTYPE_TO_TORCH[output_dtype], device=x.device)
-    if M > 0:
-        K = W_q.shape[0] * elements_per_sample
-        key = config_key(M, out_features, K, group_size, elements_per_sample, get_type_id(input_dtype, W_nbits))
-        args = _ext.build_matmul_args(
-            x2d, W_q, scales, zeros, scales_x, out,
-            W_nbits=W_nbits, group_size=group_size, unpack_mask=unpack_mask,
-            elements_per_sample=elements_per_sample, input_dtype=kernel_input_dtype, output_dtype=output_dtype,
-            acc_dtype=acc_dtype, meta_dtype=meta_dtype, channel_scale_mode=channel_scale_mode,
-            W_group_mode=W_group_mode, data_contiguous=data_contiguous,
-            matmul_type=GEMLITE_MATMUL_TYPES_MAPPING[matmul_type_str],
-            tile_config=_cached_tile_config(matmul_type_str, key),
-        )
-        _ext.matmul(args, x.device)
+    out = GEMLITE_TRITON_MAPPING[matmul_type_str].forward(
+        x2d, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
+        kernel_input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
+        data_contiguous, get_type_id(input_dtype, W_nbits),
+    )
 
     out = out.view(out_shape)
     if bias is not None:
         out += bias
     return out
+
+
+# ---------------------------------------------------------------------------
+# kernel plug-in level: one class per matmul type with the reference's interface
+# (reference: gemlite/core.py:57-67; gemlite/triton_kernels/gemm_kernels.py:741-799 and the
+# matching classes of the GEMV / split-K files).  All five run gla_matmul; the type is a hint the
+# library's dispatcher may override (up to 16 rows the streaming kernels run whatever was asked for).
+# ---------------------------------------------------------------------------
+def _kernel_forward(matmul_type_str):
+    def forward(x, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
+                input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
+                data_contiguous, type_id, meta_scale=0.0):
+        M, K, N = x.shape[0], W_q.shape[0] * elements_per_sample, W_q.shape[1]
+        out = torch.empty((M, N), dtype=DTYPE_TO_TORCH[int(output_dtype)], device=x.device)
+        if M > 0:
+            key = config_key(M, N, K, group_size, elements_per_sample, type_id)
+            args = _ext.build_matmul_args(
+                x, W_q, scales, zeros, scales_x, out,
+                W_nbits=W_nbits, group_size=group_size, unpack_mask=unpack_mask,
+                elements_per_sample=elements_per_sample, input_dtype=input_dtype, output_dtype=output_dtype,
+                acc_dtype=acc_dtype, meta_dtype=meta_dtype, channel_scale_mode=channel_scale_mode,
+                W_group_mode=W_group_mode, data_contiguous=data_contiguous,
+                matmul_type=GEMLITE_MATMUL_TYPES_MAPPING[matmul_type_str],
+                tile_config=_cached_tile_config(matmul_type_str, key),
+            )
+            _ext.matmul(args, x.device)
+        return out
+    return forward
+
+
+def _kernel_class(matmul_type_str):
+    return type(matmul_type_str.lower(), (), {
+        "kernel": ["gla_matmul"],
+        "matmul_type": matmul_type_str,
+        "forward": staticmethod(_kernel_forward(matmul_type_str)),
+        "__doc__": f"Kernel plug-in for matmul type {matmul_type_str}: forward(x, W_q, scales, zeros, scales_x, "
+                   "W_nbits, ..., type_id) -> Tensor[M, N], backed by the C ABI.",
+    })
+
+
+GEMLITE_TRITON_MAPPING = {name: _kernel_class(name) for name in GEMLITE_MATMUL_TYPES}
 
 
 # The same function as a torch custom op with a fake (meta) implementation, so that graphs traced
@@ -609,5 +641,6 @@ __all__ = [
     "GEMLITE_ACC_DTYPE",
     "GEMLITE_MATMUL_TYPES",
     "GEMLITE_MATMUL_TYPES_MAPPING",
+    "GEMLITE_TRITON_MAPPING",
     "GEMLITE_CONFIG_CACHE",
 ]

@@ -416,3 +416,18 @@ def test_int8_bytes_with_zero_point_channelwise(device, dtype, zeros_kind):
                                       data_contiguous=m[11])
         assert _ext.matmul_family(args) == "GEMV_KMAJOR", (layer.W_group_mode, layer.channel_scale_mode)
         check_layer(layer, x, dtype)
+
+
+@pytest.mark.gpu
+def test_kernel_plugin_classes_match_the_module(device):
+    """Calling a registry class's forward with the module's tensor / meta arguments gives what the
+    module gives (the seam a maintainer of the reference would plug the library into)."""
+    N, K = 512, 1024
+    W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16)
+    layer = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    W, s, z, _ = layer.get_tensor_args()
+    m = layer.get_meta_args()
+    for M, name in ((1, "GEMV_REVSPLITK"), (8, "GEMM_SPLITK"), (64, "GEMM")):
+        x = gen_x(M, K, torch.float16, seed=M).to(device)
+        y = gemlite_amd.GEMLITE_TRITON_MAPPING[name].forward(x, W, s, z, None, *m[1:], type_id=0)
+        assert torch.equal(y, layer.forward_manual(x, matmul_type=name))

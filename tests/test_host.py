@@ -371,3 +371,17 @@ def test_tuner_candidates_and_cache_file_round_trip(tmp_path):
     GemLiteLinear.load_config(f)
     assert gemlite_amd.core._cached_tile_config("GEMM", key) == 8064
     GemLiteLinear.reset_config()
+
+
+def test_kernel_plugin_registry_has_the_reference_interface():
+    """One class per matmul type with `kernel`, `matmul_type` and a static `forward` taking the
+    reference's argument list (reference: gemlite/core.py:57-67, triton_kernels/gemm_kernels.py:741-746)."""
+    import inspect
+    m = gemlite_amd.GEMLITE_TRITON_MAPPING
+    assert list(m) == gemlite_amd.GEMLITE_MATMUL_TYPES
+    want = ["x", "W_q", "scales", "zeros", "scales_x", "W_nbits", "group_size", "unpack_mask", "elements_per_sample",
+            "input_dtype", "output_dtype", "acc_dtype", "meta_dtype", "channel_scale_mode", "W_group_mode",
+            "data_contiguous", "type_id", "meta_scale"]
+    for name, cls in m.items():
+        assert cls.matmul_type == name and isinstance(cls.kernel, list)
+        assert list(inspect.signature(cls.forward).parameters) == want
