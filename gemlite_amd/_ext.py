@@ -305,7 +305,7 @@ def matmul(args: MatmulArgs, device: torch.device):
     _check(lib.gla_matmul(ctypes.byref(args), _stream_ptr(device)), "gla_matmul")
 
 
-FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4"]
+FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES"]
 
 
 def matmul_family(args: MatmulArgs) -> str:

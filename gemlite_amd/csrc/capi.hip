@@ -49,7 +49,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
     return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
 }
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4 };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES };
 
 int validate(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -143,6 +143,7 @@ Family choose(const gla_matmul_args& p, int type) {
     }
     if (gemm_wn_eligible(p)) return F_GEMM_WN;
     if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // also streams K-major 8-bit operands at small M (split-K)
+    if (gemm_kbytes_eligible(p)) return F_GEMM_KBYTES;
     return F_GENERIC;
 }
 
@@ -191,6 +192,7 @@ int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
         case F_GEMV_PACKED: return gemv_packed_workspace_bytes(*args);
         case F_GEMM_WN: return gemm_wn_workspace_bytes(*args);
         case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(*args);
+        case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(*args);
         default: return 0;
     }
 }
@@ -206,6 +208,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_GEMM_WN: return launch_gemm_wn(*args, s);
         case F_GEMM_8BIT: return launch_gemm_8bit(*args, s);
         case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
+        case F_GEMM_KBYTES: return launch_gemm_kbytes(*args, s);
         default: return launch_generic(*args, s);
     }
 }

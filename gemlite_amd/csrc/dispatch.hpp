@@ -43,6 +43,11 @@ int launch_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t
 int launch_unpack_over_cols(const void* packed, uint8_t* out, int64_t rows, int64_t pcols, int nbits, int width,
                             hipStream_t stream);
 
+// ---- MFMA GEMM for 16-bit activations x K-contiguous weight bytes (gemm_kbytes.hip)
+bool gemm_kbytes_eligible(const gla_matmul_args& p);
+int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream);
+int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p);
+
 // ---- diagnostic: sustained matrix rate (probe.hip) ---------------------------
 int launch_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, hipStream_t stream);
 

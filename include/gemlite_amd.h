@@ -153,6 +153,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_WN 3      /* fused-dequant MFMA GEMM for packed 2/4/8-bit codes */
 #define GLA_FAMILY_GEMM_8BIT 4    /* fp8 / int8 MFMA GEMM on K-major operands */
 #define GLA_FAMILY_GEMM_MXFP4 5   /* block-scaled FP4 MFMA GEMM */
+#define GLA_FAMILY_GEMM_KBYTES 6  /* MFMA GEMM for 16-bit activations x unpacked 8-bit weight bytes */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of

@@ -385,7 +385,17 @@ def test_a16w8_weight_only_unpacked_bytes(device, fp8, post_scale, dtype, K):
                                       data_contiguous=m[11])
         assert _ext.matmul_family(args) == "GEMV_KMAJOR"
         check_layer(layer, x, dtype)
-    check_layer(layer, gen_x(40, K, dtype, seed=40).to(device), dtype)   # above 16 rows: the generic kernel
+    # above 16 rows: the MFMA GEMM for weight bytes where K is a multiple of its 64-value stage, else the generic kernel
+    for M in (17, 40, 130, 300):
+        x = gen_x(M, K, dtype, seed=M).to(device)
+        out = torch.empty((M, N), dtype=dtype, device=device)
+        m = layer.get_meta_args()
+        args = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                      unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                      acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                      data_contiguous=m[11])
+        assert _ext.matmul_family(args) == ("GEMM_KBYTES" if K % 64 == 0 else "GENERIC")
+        check_layer(layer, x, dtype)
 
 
 @pytest.mark.gpu
