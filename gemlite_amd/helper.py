@@ -296,3 +296,28 @@ class A4W4_MXFP_dynamic:
         W_q, scales = self.quantizer_mx.quantize_mxfp4(W, index=True)
         bias = None if linear_layer.bias is None else linear_layer.bias.data.clone()
         return self.from_weights(W_q.view(N, K), scales=scales.view(N, K // 32), bias=bias)
+
+
+default_batch_sizes = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096]
+
+
+def warmup(processor, shapes, batch_sizes=default_batch_sizes, group_size=64, dtype=torch.float16):
+    """Build a layer of every ``(out_features, in_features)`` shape with ``processor`` and tune it at
+    every batch size, filling the config cache that ``GemLiteLinear.cache_config`` saves.  The
+    reference's function of the same name runs each shape once so that Triton autotunes it
+    (reference: gemlite/helper.py:1326-1376); here the offline tuner times the few tile alternatives
+    of the kernel family instead.  Processors that start from an HQQ layer need weights quantised
+    elsewhere and are refused."""
+    from .tune import tune_layer
+    if not hasattr(processor, "from_linear"):
+        raise ImportError("warmup() needs a processor with from_linear(); HQQ-based ones need the `hqq` package")
+    device = torch.device("cuda", torch.cuda.current_device())
+    results = {}
+    for out_features, in_features in shapes:
+        linear = torch.nn.Linear(in_features, out_features, bias=False, dtype=dtype, device=device)
+        layer = processor.from_linear(linear)
+        results[(out_features, in_features)] = tune_layer(layer, batch_sizes)
+        del layer, linear
+        torch.cuda.empty_cache()
+        gc.collect()
+    return results
