@@ -258,6 +258,71 @@ class A8W8_FP8_dynamic(A8W8_dynamic):
 A8W8_int8_dynamic, A8W8_fp8_dynamic = A8W8_INT8_dynamic, A8W8_FP8_dynamic
 
 
+class A8Wn_HQQ_INT_dynamic(A16Wn):
+    """fp8 activations quantised per token on the fly x grouped 8/4/2-bit integer weights
+    (reference: gemlite/helper.py:712-871).  Runs the layout-agnostic kernel (no tuned kernel for
+    fp8 activations against packed integer codes is built)."""
+
+    def __init__(self, device="cuda:0", packing_bitwidth=None, dtype=None, post_scale=True,
+                 fp8=torch.float8_e4m3fn, fp32_scale=False, W_nbits=None):
+        assert W_nbits is not None, "W_nbits argument should be either 8, 4 or 2, not None."
+        super().__init__(device=device, dtype=dtype, packing_bitwidth=packing_bitwidth, post_scale=post_scale)
+        self.fp8 = fp8
+        self.fp32_scale = fp32_scale
+        self.W_nbits = W_nbits
+
+    def from_packed_weights(self, W_q_packed, scales, zeros, bias=None):
+        group_size = W_q_packed.numel() * (8 // self.W_nbits) // scales.numel()
+        return self.from_weights_(W_q_packed, scales, zeros, self.W_nbits, group_size, bias=bias, packed=True)
+
+    def from_weights(self, W_q, scales, zeros, bias=None):
+        group_size = W_q.numel() // scales.numel()
+        return self.from_weights_(W_q, scales, zeros, self.W_nbits, group_size, bias=bias)
+
+    def from_weights_(self, W_q, scales, zeros, W_nbits, group_size, bias=None, quant_type="INT", packed=False):
+        if isinstance(W_q, torch.nn.Parameter):
+            W_q = W_q.data
+        if isinstance(bias, torch.nn.Parameter):
+            bias = bias.data
+        if self.dtype is None:
+            dtype = scales.dtype if scales.dtype in (torch.float16, torch.bfloat16) else torch.float16
+        else:
+            dtype = self.dtype
+        assert dtype in (torch.float16, torch.bfloat16, torch.float32), "Invalid scales.dtype, should be floating point."
+        out_features, in_features = W_q.shape
+        if packed:
+            in_features = in_features * 8 // W_nbits
+        W_q = W_q.to(self.device)
+        scales = scales.to(device=self.device, dtype=torch.float32 if self.fp32_scale else dtype) if scales is not None else None
+        zeros = zeros.to(device=self.device, dtype=dtype) if isinstance(zeros, torch.Tensor) else zeros
+        bias = bias.to(device=self.device, dtype=dtype) if bias is not None else None
+        layer = GemLiteLinear(
+            W_nbits, group_size=group_size, in_features=in_features, out_features=out_features,
+            input_dtype=TORCH_TO_DTYPE[self.fp8], output_dtype=TORCH_TO_DTYPE[dtype], scaled_activations=True,
+        )
+        layer.pack(W_q, scales, zeros, bias=bias, packing_bitwidth=self.packing_bitwidth, fma_mode=False, packed=packed)
+        if group_size == in_features:
+            if self.post_scale:
+                layer.W_group_mode, layer.channel_scale_mode = 1, 3
+            else:
+                layer.W_group_mode, layer.channel_scale_mode = 3, 2
+        return layer
+
+
+class A8W4_HQQ_INT_dynamic(A8Wn_HQQ_INT_dynamic):
+    def __init__(self, device="cuda:0", packing_bitwidth=None, dtype=None, post_scale=True,
+                 fp8=torch.float8_e4m3fn, fp32_scale=False):
+        super().__init__(device=device, packing_bitwidth=packing_bitwidth, dtype=dtype, post_scale=post_scale,
+                         fp8=fp8, fp32_scale=fp32_scale, W_nbits=4)
+
+
+class A8W2_HQQ_INT_dynamic(A8Wn_HQQ_INT_dynamic):
+    def __init__(self, device="cuda:0", packing_bitwidth=None, dtype=None, post_scale=True,
+                 fp8=torch.float8_e4m3fn, fp32_scale=False):
+        super().__init__(device=device, packing_bitwidth=packing_bitwidth, dtype=dtype, post_scale=post_scale,
+                         fp8=fp8, fp32_scale=fp32_scale, W_nbits=2)
+
+
 class A4W4_MXFP_dynamic:
     """MXFP4 activations (quantised on the fly) x MXFP4 weights
     (reference: gemlite/helper.py:1042-1114)."""

@@ -441,3 +441,21 @@ def test_kernel_plugin_classes_match_the_module(device):
         x = gen_x(M, K, torch.float16, seed=M).to(device)
         y = gemlite_amd.GEMLITE_TRITON_MAPPING[name].forward(x, W, s, z, None, *m[1:], type_id=0)
         assert torch.equal(y, layer.forward_manual(x, matmul_type=name))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("group_size", [128, None])
+def test_a8w4_hqq_int_dynamic_fp8_activations(device, group_size):
+    """fp8 activations quantised per token x 4-bit grouped weights (reference processor:
+    gemlite/helper.py:712-851; modes as tests/test_int.py:173-199 asserts them)."""
+    N, K = 256, 1024
+    gs = group_size or K
+    W_q, scales, zeros = gen_int_case(N, K, 4, gs, torch.float16)
+    layer = helper.A8W4_HQQ_INT_dynamic(device=device).from_weights(W_q, scales, zeros)
+    assert layer.scaled_activations and layer.input_dtype == DType.FP8
+    if group_size is None:
+        assert (layer.W_group_mode, layer.channel_scale_mode) == (1, 3)
+    else:
+        assert (layer.W_group_mode, layer.channel_scale_mode) == (3, 2)
+    for M in (1, 7, 40):
+        check_layer(layer, gen_x(M, K, torch.float16, seed=M).to(device), torch.bfloat16)
