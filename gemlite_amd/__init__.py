@@ -34,6 +34,7 @@ from .quant_utils import (
     WeightQuantizerMXFP,
     quantize_weights_per_channel,
     scale_activations_mxfp4,
+    scale_activations_mxfp8,
     scale_activations_per_token,
 )
 

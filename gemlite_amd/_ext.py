@@ -102,6 +102,11 @@ SYMBOLS = {
         [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
          ctypes.c_void_p],
     ),
+    "gla_scale_activations_mxfp8": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+         ctypes.c_void_p],
+    ),
     "gla_pack_over_cols": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p],
@@ -305,7 +310,7 @@ def matmul(args: MatmulArgs, device: torch.device):
     _check(lib.gla_matmul(ctypes.byref(args), _stream_ptr(device)), "gla_matmul")
 
 
-FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES"]
+FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8"]
 
 
 def matmul_family(args: MatmulArgs) -> str:
@@ -345,6 +350,18 @@ def scale_activations_mxfp4(x2d: torch.Tensor, y: torch.Tensor, scales: torch.Te
             x2d.data_ptr(), _dt(x2d), x2d.stride(0), M, K, y.data_ptr(), scales.data_ptr(), _stream_ptr(x2d.device)
         ),
         "gla_scale_activations_mxfp4",
+    )
+
+
+def scale_activations_mxfp8(x2d: torch.Tensor, y: torch.Tensor, scales: torch.Tensor):
+    _require_cuda(x2d, y, scales)
+    lib = load_library()
+    M, K = x2d.shape
+    _check(
+        lib.gla_scale_activations_mxfp8(
+            x2d.data_ptr(), _dt(x2d), x2d.stride(0), M, K, y.data_ptr(), scales.data_ptr(), _stream_ptr(x2d.device)
+        ),
+        "gla_scale_activations_mxfp8",
     )
 
 

@@ -24,7 +24,7 @@ from .dtypes import (
     TORCH_TO_DTYPE,
     is_mx_dtype,
 )
-from .quant_utils import scale_activations_mxfp4, scale_activations_per_token
+from .quant_utils import scale_activations_mxfp4, scale_activations_mxfp8, scale_activations_per_token
 
 logger = logging.getLogger(__name__)
 _FILE_LOCK = threading.Lock()
@@ -164,6 +164,10 @@ def forward_functional(
             x2d, scales_x = scale_activations_per_token(x2d, w_dtype=DTYPE_TO_TORCH[input_dtype])
         elif in_dt == DType.MXFP4 and channel_scale_mode == 4:
             x2d, scales_x = scale_activations_mxfp4(x2d)
+        elif in_dt == DType.MXFP8 and channel_scale_mode == 4:  # MXFP8 micro-scales on both sides
+            x2d, scales_x = scale_activations_mxfp8(x2d)
+        elif in_dt == DType.MXFP8 and channel_scale_mode == 2:  # MXFP8 weights, per-token post-scaled activations
+            x2d, scales_x = scale_activations_per_token(x2d, w_dtype=torch.float8_e4m3fn)
         else:
             raise NotImplementedError(
                 f"dynamic activation quantisation for input_dtype={in_dt}, channel_scale_mode={channel_scale_mode}"

@@ -188,7 +188,9 @@ __device__ __forceinline__ uint32_t e2m1_code(float v) {
 }
 
 // Four lanes share one 32-value group (8 values each): a wave covers 16 groups = 512 values.
-template <int XDT>
+// FP8OUT: MXFP8 (codes are e4m3fn bytes, y is [M, K]; the largest magnitude is 448) instead of MXFP4
+// (e2m1 nibbles, y is [M, K/2]; 6).
+template <int XDT, bool FP8OUT>
 __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, int64_t xsm, int M, int M_pad, int K,
                                                     uint8_t* __restrict__ y, uint8_t* __restrict__ scales) {
     const int groups = K / 32;
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, 
     amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
     amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
 
-    const uint32_t bits = __builtin_bit_cast(uint32_t, amax / 6.0f);
+    const uint32_t bits = __builtin_bit_cast(uint32_t, amax / (FP8OUT ? 448.0f : 6.0f));
     uint32_t e = (bits >> 23) & 0xffu;
     e += (bits & 0x7fffffu) ? 1u : 0u;
     e = e > 254u ? 254u : e;
@@ -231,6 +233,19 @@ __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, 
     // and denormal results included) in one instruction instead of a division sequence
     const int down = 127 - (int)e;
     (void)s;
+    if constexpr (FP8OUT) {
+        uint32_t w[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float q[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q[j] = fminf(fmaxf(__builtin_ldexpf(v[4 * h + j], down), -448.0f), 448.0f);
+            w[h] = f32_to_fp8_pair(q[0], q[1]) | (f32_to_fp8_pair(q[2], q[3]) << 16);
+        }
+        *(uint2*)(y + (int64_t)row * K + k) = make_uint2(w[0], w[1]);
+        if ((lane & 3) == 0) scales[(int64_t)row * groups + g] = (uint8_t)e;
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) packed |= e2m1_code(__builtin_ldexpf(v[j], down)) << (4 * j);
     *(uint32_t*)(y + (int64_t)row * (K / 2) + k / 2) = packed;
@@ -275,14 +290,27 @@ int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, 
     return check_hip(hipGetLastError(), "per-token activation quant launch");
 }
 
+static int launch_act_mx(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
+                         bool fp8, hipStream_t stream);
+
 int launch_act_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
                      hipStream_t stream) {
+    return launch_act_mx(x, x_dtype, x_stride_m, M, K, y, scales, false, stream);
+}
+
+int launch_act_mxfp8(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
+                     hipStream_t stream) {
+    return launch_act_mx(x, x_dtype, x_stride_m, M, K, y, scales, true, stream);
+}
+
+static int launch_act_mx(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
+                         bool fp8, hipStream_t stream) {
     if (x == nullptr || y == nullptr || scales == nullptr || M < 0 || K <= 0) {
-        set_error("scale_activations_mxfp4: null pointer or bad size");
+        set_error("scale_activations_mxfp: null pointer or bad size");
         return GLA_ERR_INVALID_ARGUMENT;
     }
-    if (K % 32 != 0 || x_stride_m % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)y & 3)) {
-        set_error("scale_activations_mxfp4: K must be a multiple of 32, the row stride of 8, x 16-byte aligned");
+    if (K % 32 != 0 || x_stride_m % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)y & (fp8 ? 7 : 3))) {
+        set_error("scale_activations_mxfp: K must be a multiple of 32, the row stride of 8, x 16-byte aligned");
         return GLA_ERR_MISALIGNED_SHAPE;
     }
     if (M == 0) return GLA_OK;
@@ -293,19 +321,22 @@ int launch_act_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int 
     dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     switch (x_dtype) {
         case GLA_DT_FP16:
-            hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP16>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            if (fp8) hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP16, true>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            else hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP16, false>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
             break;
         case GLA_DT_BF16:
-            hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_BF16>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            if (fp8) hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_BF16, true>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            else hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_BF16, false>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
             break;
         case GLA_DT_FP32:
-            hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP32>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            if (fp8) hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP32, true>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
+            else hipLaunchKernelGGL((mxfp4_kernel<GLA_DT_FP32, false>), grid, block, 0, stream, x, x_stride_m, M, M_pad, K, y, scales);
             break;
         default:
-            set_error("scale_activations_mxfp4: input type %d not supported", x_dtype);
+            set_error("scale_activations_mxfp: input type %d not supported", x_dtype);
             return GLA_ERR_UNSUPPORTED_DTYPE;
     }
-    return check_hip(hipGetLastError(), "MXFP4 activation quant launch");
+    return check_hip(hipGetLastError(), "MXFP activation quant launch");
 }
 
 }  // namespace gla

@@ -49,7 +49,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
     return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
 }
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8 };
 
 int validate(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -84,8 +84,16 @@ int validate(const gla_matmul_args* p) {
         }
         return GLA_OK;
     }
+    if (p->input_dtype == GLA_DT_MXFP8) {
+        if (!gemm_mxfp8_eligible(*p)) {
+            set_error("matmul: MXFP8 needs fp8 weight bytes with K-contiguous e8m0 scales per 32 values, K %% 128 == 0, "
+                      "16-byte aligned rows and channel_scale_mode 2 or 4 (K=%d, mode %d)", p->K, p->channel_scale_mode);
+            return GLA_ERR_UNSUPPORTED_MODE;
+        }
+        return GLA_OK;
+    }
     if (is_mx(p->input_dtype)) {
-        set_error("matmul: micro-scaled input type %d is not supported (MXFP4 x MXFP4 only)", p->input_dtype);
+        set_error("matmul: micro-scaled input type %d is not supported (MXFP4 and MXFP8 only)", p->input_dtype);
         return GLA_ERR_UNSUPPORTED_DTYPE;
     }
     switch (p->input_dtype) {
@@ -135,6 +143,7 @@ int validate(const gla_matmul_args* p) {
 
 Family choose(const gla_matmul_args& p, int type) {
     if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : F_GENERIC;
+    if (p.input_dtype == GLA_DT_MXFP8) return F_GEMM_MXFP8;  // validated as eligible; there is no other kernel for it
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
     const bool small = type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16;
     if (small) {
@@ -193,6 +202,7 @@ int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
         case F_GEMM_WN: return gemm_wn_workspace_bytes(*args);
         case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(*args);
         case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(*args);
+        case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(*args);
         default: return 0;
     }
 }
@@ -209,6 +219,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_GEMM_8BIT: return launch_gemm_8bit(*args, s);
         case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
         case F_GEMM_KBYTES: return launch_gemm_kbytes(*args, s);
+        case F_GEMM_MXFP8: return launch_gemm_mxfp8(*args, s);
         default: return launch_generic(*args, s);
     }
 }
@@ -221,6 +232,11 @@ int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride
 int gla_scale_activations_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y,
                                 uint8_t* scales, void* stream) {
     return launch_act_mxfp4(x, x_dtype, x_stride_m, M, K, y, scales, (hipStream_t)stream);
+}
+
+int gla_scale_activations_mxfp8(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y,
+                                uint8_t* scales, void* stream) {
+    return launch_act_mxfp8(x, x_dtype, x_stride_m, M, K, y, scales, (hipStream_t)stream);
 }
 
 int gla_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t cols, int W_nbits,

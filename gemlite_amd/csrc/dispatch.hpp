@@ -33,10 +33,17 @@ int64_t gemm_8bit_workspace_bytes(const gla_matmul_args& p);  // also for the MX
 bool gemm_mxfp4_eligible(const gla_matmul_args& p);
 int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream);
 
+// ---- MXFP8 weights x fp8 activations (per-token or block-scaled), MFMA GEMM (gemm_8bit.hip)
+bool gemm_mxfp8_eligible(const gla_matmul_args& p);
+int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream);
+int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p);
+
 // ---- activation quantisation (actquant.hip) and bit packing (bitpack.hip) --
 int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
                          float* scales, hipStream_t stream);
 int launch_act_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
+                     hipStream_t stream);
+int launch_act_mxfp8(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
                      hipStream_t stream);
 int launch_pack_over_cols(const uint8_t* codes, void* out, int64_t rows, int64_t cols, int nbits, int width,
                           hipStream_t stream);

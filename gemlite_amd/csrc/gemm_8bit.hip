@@ -40,7 +40,7 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2 };
+enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3 };
 
 constexpr int kRowB8 = 64;  // bytes per LDS row = bytes of K per pipeline stage
 constexpr int kBN = 256;
@@ -54,7 +54,10 @@ struct Gemm8Args {
     void* out;
     int M, N, Kb;          // Kb = bytes of K per row
     int64_t lda, ldb, osm, sxm, msn;
-    int64_t sx_stage, sw_stage;  // MXFP4: bytes from one pipeline stage's scale word of a row to the next one's
+    int64_t sx_stage, sw_stage;  // micro-scaled: bytes from one scale word of a row to the next one's
+    int a_unit;                  // MXFP8: the activations carry no block scales (per-token scale in the epilogue)
+    const void* ascales;         // micro-scaled: activation block scales (row stride asxm bytes); scales_x is the epilogue's
+    int64_t asxm;
     int csm, meta_dt, sx_dt, out_dt;
     int tiles_m, tiles_n;
     int S;     // K splits (gridDim.y)
@@ -83,7 +86,7 @@ __device__ __forceinline__ void wait_vmcnt8() {
 }
 
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
-constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 ? (bm + kBN) * 4 : 0); }
+constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 || mode == kMXFP8 ? (bm + kBN) * 4 : 0); }
 
 // WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
 // (A 2-column variant with 4 waves of 128 x 128 and accumulators in AGPRs reads a third less from
@@ -97,7 +100,9 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr int TI = WM / 32;       // 32-row MFMA tiles per wave along M
     constexpr int WNC = kBN / WN;     // wave tile columns
     constexpr int TJ = WNC / 32;      // 32-column MFMA tiles per wave along N
-    constexpr bool MX = MODE == kMXFP4;
+    constexpr bool MX = MODE == kMXFP4 || MODE == kMXFP8;  // block scales ride along with every stage
+    // MXFP8: a 32-bit scale word of a row covers 128 values = two stages; MXFP4: one stage
+    constexpr int SSH = MODE == kMXFP8 ? 1 : 0;
     constexpr int NW = kWavesM * WN;
     constexpr int RING = kRing8;
     constexpr int SLOT = slot_bytes8(MODE, BM);
@@ -159,7 +164,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             if (is_a4[i]) {
                 int gm = m0 + q * 64 + lane;
                 if (gm > p.M - 1) gm = p.M - 1;
-                off4[i] = (unsigned)(gm * (int)p.sxm);
+                off4[i] = (unsigned)(gm * (int)p.asxm);
             } else {
                 int gn = n0 + (q - BM / 64) * 64 + lane;
                 if (gn > p.N - 1) gn = p.N - 1;
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                                              (__attribute__((address_space(3))) void*)(base + dst16[c]), 16, 0, 0);
         } else if constexpr (MX) {
             const int i = c - J16;
-            const uint8_t* sk = is_a4[i] ? (const uint8_t*)p.scales_x + kk * p.sx_stage : (const uint8_t*)p.scales + kk * p.sw_stage;
+            const uint8_t* sk = is_a4[i] ? (const uint8_t*)p.ascales + (kk >> SSH) * p.sx_stage : (const uint8_t*)p.scales + (kk >> SSH) * p.sw_stage;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
                                              (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
         }
@@ -230,7 +235,8 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // LDS read r of a stage's NRD: chunk reads of the weight tiles, then of the activation tiles,
     // then (MXFP4) the scale words
     constexpr int NRD = (TI + TJ) * (MX ? 3 : 2);
-    auto load_one = [&](int slot, auto buf_tag, int r) __attribute__((always_inline)) {
+    // (`par`: parity of the absolute stage being read, which picks the half of an MXFP8 scale word)
+    auto load_one = [&](int slot, auto buf_tag, int r, int par) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
         const unsigned char* base = smem + slot * SLOT;
         if (r < 2 * TJ) {
@@ -239,10 +245,16 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             const int q = r - 2 * TJ;
             fa[B][q / 2].c[q % 2] = *(const u32x4*)(base + a_row0 + (q / 2) * 32 * kRowB8 + (q % 2 ? c1 : c0));
         } else if constexpr (MX) {
-            // half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2
+            // MXFP4: half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2.
+            // MXFP8: it multiplies with the scale of block kb of the stage, byte 2 par + kb of the word.
             const int q = r - 2 * (TI + TJ);
-            if (q < TI) fsa[B][q] = *(const unsigned*)(base + sa_row0 + q * 128) >> (8 * kb);
-            else fsb[B][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> (8 * kb);
+            const int sh = MODE == kMXFP8 ? 8 * (2 * par + kb) : 8 * kb;
+            if (q < TI) {
+                const unsigned v = *(const unsigned*)(base + sa_row0 + q * 128) >> sh;
+                fsa[B][q] = (MODE == kMXFP8 && p.a_unit) ? 127u : v;
+            } else {
+                fsb[B][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> sh;
+            }
         }
     };
     // The same for one K-step (h = 0, 1) of a stage, into fragment buffer 0: read r of TI + TJ chunk reads
@@ -260,18 +272,23 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             else fsb[SB][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> (8 * kb);
         }
     };
-    auto load_frags = [&](int slot, auto buf_tag) __attribute__((always_inline)) {
+    auto load_frags = [&](int slot, auto buf_tag, int par) __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < NRD; ++r) load_one(slot, buf_tag, r);
+        for (int r = 0; r < NRD; ++r) load_one(slot, buf_tag, r, par);
     };
     // MFMA q of a stage's NM.  fp8: one K-step of 64 bytes per tile pair; int8 / fp4: two K-steps of 32
-    constexpr int NM = TI * TJ * (MODE == kFP8 ? 1 : 2);
+    constexpr int NM = TI * TJ * (MODE == kFP8 || MODE == kMXFP8 ? 1 : 2);
     auto multiply_one = [&](int limit, auto buf_tag, auto scale_tag, int q) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;    // fragment buffer
         constexpr int SB = decltype(scale_tag)::value; // scale buffer (MXFP4)
         const int s2 = q / (TI * TJ), i = (q % (TI * TJ)) / TJ, j = q % TJ;
         if constexpr (MODE == kFP8) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
+        } else if constexpr (MODE == kMXFP8) {
+            // registers 0-3 of both half-waves are block 0 of the stage, registers 4-7 block 1, and the
+            // half-wave's scale is that of block kb: the chunk pair (kb, 2 + kb) as one operand
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0,
+                                                                        (int)fsb[SB][j], 0, (int)fsa[SB][i]);
         } else {
             // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
             // must not live across control flow)
@@ -308,7 +325,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     //    of stage k while reading its K-step 1, then multiplies that while reading K-step 0 of stage
     //    k+1, and refills the slot of stage k-1.  The scale words of a stage serve both K-steps and
     //    alternate between two buffers.
-    constexpr bool HALF = MX && BM == 256;
+    constexpr bool HALF = MODE == kMXFP4 && BM == 256;
     constexpr int AHEAD = HALF ? RING - 1 : RING;
     typedef std::integral_constant<int, 0> tag0;
 #pragma unroll
@@ -321,7 +338,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
 #pragma unroll
         for (int r = 0; r < 2 * (TI + TJ); ++r) load_half(0, 0, tag0{}, r);
     } else {
-        load_frags(0, tag0{});
+        load_frags(0, tag0{}, k_first & 1);
     }
 
     int slot = 0;  // ring slot of the stage being multiplied
@@ -351,7 +368,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
 #pragma unroll
                 for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING, slot, c);
 #pragma unroll
-                for (int r = q * NRD / RS; r < (q + 1) * NRD / RS && r < NRD; ++r) load_one(next, other{}, r);
+                for (int r = q * NRD / RS; r < (q + 1) * NRD / RS && r < NRD; ++r) load_one(next, other{}, r, (k_first + k + 1) & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         } else {
@@ -411,7 +428,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         return;
     }
     const bool col_scale = !MX && (p.csm & 1);
-    const bool row_scale = !MX && (p.csm & 2);
+    const bool row_scale = MODE != kMXFP4 && (p.csm & 2);
     float sb[TJ][16];
 #pragma unroll
     for (int j = 0; j < TJ; ++j)
@@ -627,7 +644,7 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
-    a.out_dt = p.output_dtype; a.sx_stage = 0; a.sw_stage = 0;
+    a.out_dt = p.output_dtype; a.sx_stage = 0; a.sw_stage = 0; a.a_unit = 0; a.ascales = nullptr; a.asxm = 0;
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
@@ -675,7 +692,7 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
     a.M = p.M; a.N = p.N; a.Kb = p.K / 2; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.csm = 0; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype;
-    a.sx_stage = 4; a.sw_stage = 4;
+    a.sx_stage = 4; a.sw_stage = 4; a.a_unit = 0; a.ascales = p.scales_x; a.asxm = p.sx_stride_m;
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
@@ -689,10 +706,84 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
         hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(row_blocks, ceil_div(stages, 64), 2), dim3(256), 0, stream,
                            (const uint8_t*)p.scales_x, p.M, (int64_t)p.sx_stride_m, sx,
                            (const uint8_t*)p.scales, p.N, (int64_t)p.meta_stride_n, sw, stages);
-        a.scales_x = sx; a.sxm = 4; a.sx_stage = (int64_t)p.M * 4;
+        a.ascales = sx; a.asxm = 4; a.sx_stage = (int64_t)p.M * 4;
         a.scales = sw; a.msn = 4; a.sw_stage = (int64_t)p.N * 4;
     }
     return launch_mode<kMXFP4>(a, g.bm, stream);
+}
+
+// MXFP8 weights (fp8-e4m3 codes, one e8m0 scale per 32 values, [N, K/32] with unit stride along K) x
+// fp8 activations that carry either the same kind of block scales (channel_scale_mode 4) or one fp32
+// scale per row applied after the K sum (channel_scale_mode 2, the reference processor's default:
+// gemlite/helper.py:876-923).
+bool gemm_mxfp8_eligible(const gla_matmul_args& p) {
+    if (p.input_dtype != GLA_DT_MXFP8) return false;
+    if (!(p.channel_scale_mode == GLA_CSM_MX || p.channel_scale_mode == GLA_CSM_ACTIVATION)) return false;
+    if (p.W_nbits != 8 || p.elements_per_sample != 1 || p.group_size != 32 || p.w_dtype != GLA_DT_FP8) return false;
+    if (p.scales == nullptr || p.scales_x == nullptr) return false;
+    if (p.w_stride_k != 1 || p.x_stride_k != 1 || p.out_stride_n != 1) return false;
+    if (p.meta_stride_g != 1 || p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3)) return false;
+    if (p.channel_scale_mode == GLA_CSM_MX && (p.sx_stride_g != 1 || p.sx_stride_m % 4 != 0 || ((uintptr_t)p.scales_x & 3)))
+        return false;
+    if (p.K % 128 != 0 || p.x_stride_m % 16 != 0 || p.w_stride_n % 16 != 0) return false;
+    if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
+    if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
+    if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
+    if ((int64_t)p.M * p.sx_stride_m >= (1ll << 31) || (int64_t)p.N * p.meta_stride_n >= (1ll << 31)) return false;
+    return true;
+}
+
+// the 256-row tile has no registers for the scale words next to two fragment buffers of 8-register operands
+static Plan8 plan_mxfp8(const gla_matmul_args& p) {
+    Plan8 g = plan8(p.M, p.N, p.K, p.tile_config);
+    if (g.bm == 256) {
+        const int cfg = (p.tile_config > 0 ? p.tile_config / 1000 : 0) * 1000 + 128;
+        g = plan8(p.M, p.N, p.K, cfg);
+    }
+    return g;
+}
+
+int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p) {
+    const Plan8 g = plan_mxfp8(p);
+    int64_t need = g.S > 1 ? kWsReserved8 + align256((int64_t)g.S * p.M * p.N * 4) : 0;
+    if (g.bm >= 128) {
+        if (need == 0) need = kWsReserved8;
+        need += align256((int64_t)(p.K / 128) * p.M * 4) + align256((int64_t)(p.K / 128) * p.N * 4);
+    }
+    return need;
+}
+
+int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
+    Gemm8Args a;
+    const bool act_blocks = p.channel_scale_mode == GLA_CSM_MX;
+    a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
+    a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
+    a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.sw_stage = 4;
+    a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
+    a.a_unit = act_blocks ? 0 : 1;
+    a.csm = act_blocks ? 0 : 2;  // per-token scale in the epilogue
+    // without activation block scales the copy jobs for them re-read the first weight scale word (never used)
+    a.ascales = act_blocks ? p.scales_x : p.scales;
+    a.asxm = act_blocks ? p.sx_stride_m : 0;
+    a.sx_stage = act_blocks ? 4 : 0;
+    const Plan8 g = plan_mxfp8(p);
+    const int rc = attach_plan(p, g, a);
+    if (rc != GLA_OK) return rc;
+    if (g.bm >= 128 && p.workspace != nullptr && (int64_t)p.workspace_bytes >= gemm_mxfp8_workspace_bytes(p)) {
+        const int words = p.K / 128;
+        const int64_t part = g.S > 1 ? align256((int64_t)g.S * p.M * p.N * 4) : 0;
+        uint32_t* sx = (uint32_t*)((char*)p.workspace + kWsReserved8 + part);
+        uint32_t* sw = (uint32_t*)((char*)sx + align256((int64_t)words * p.M * 4));
+        const int rows_x = act_blocks ? p.M : 0;
+        const int row_blocks = ceil_div(rows_x > p.N ? rows_x : p.N, 64);
+        hipLaunchKernelGGL(mx_scales_by_stage_kernel, dim3(row_blocks, ceil_div(words, 64), 2), dim3(256), 0, stream,
+                           (const uint8_t*)p.scales_x, rows_x, (int64_t)p.sx_stride_m, sx,
+                           (const uint8_t*)p.scales, p.N, (int64_t)p.meta_stride_n, sw, words);
+        a.scales = sw; a.msn = 4; a.sw_stage = (int64_t)p.N * 4;
+        if (act_blocks) { a.ascales = sx; a.asxm = 4; a.sx_stage = (int64_t)p.M * 4; }
+        else { a.ascales = sw; }
+    }
+    return launch_mode<kMXFP8>(a, g.bm, stream);
 }
 
 }  // namespace gla

@@ -323,6 +323,57 @@ class A8W2_HQQ_INT_dynamic(A8Wn_HQQ_INT_dynamic):
                          fp8=fp8, fp32_scale=fp32_scale, W_nbits=2)
 
 
+class A8W8_MXFP_dynamic:
+    """MXFP8 weights (fp8-e4m3 codes, one e8m0 scale per 32 values) x fp8 activations quantised on
+    the fly: per token with the scale applied after the K sum (``post_scale=True``, the default) or
+    with MXFP8 micro-scales (``post_scale=False``; not built here)
+    (reference: gemlite/helper.py:876-947)."""
+
+    def __init__(self, device="cuda:0", dtype=None, post_scale=True, fp8=torch.float8_e4m3fn):
+        self.device = device
+        self.dtype = dtype
+        self.mx_fp8_dtype = fp8
+        self.quantizer_mx = None
+        self.post_scale = post_scale
+        self.W_nbits = 8
+
+    def from_weights(self, weight, bias=None, scales=None):
+        if isinstance(weight, torch.nn.Parameter):
+            weight = weight.data
+        if isinstance(bias, torch.nn.Parameter):
+            bias = bias.data
+        out_features, in_features = weight.shape
+        assert scales is not None, "Scales parameter cannot be None. Use from_linear() call to pre-quantize the weights."
+        assert weight.is_floating_point() and weight.dtype.itemsize == 1, \
+            f"Invalid weight.dtype, should be an MXFP8 dtype, got {weight.dtype}."
+        assert scales.dtype in (torch.float8_e8m0fnu, torch.uint8), f"Invalid scales.dtype, got {scales.dtype}."
+        assert self.dtype is not None, "Input dtype should be either torch.float16 or torch.bfloat16, not None."
+        if scales.dtype == torch.uint8:
+            scales = scales.view(torch.float8_e8m0fnu)
+        bias = bias.to(device=self.device, dtype=self.dtype) if bias is not None else None
+        layer = GemLiteLinear(
+            self.W_nbits, group_size=32, in_features=in_features, out_features=out_features,
+            input_dtype=DType.MXFP8, output_dtype=TORCH_TO_DTYPE[self.dtype], scaled_activations=True,
+        )
+        layer.pack(weight.to(self.device), scales.to(self.device), zeros=None, bias=bias)
+        layer.W_group_mode = 0
+        layer.channel_scale_mode = 2 if self.post_scale else 4
+        return layer
+
+    def from_linear(self, linear_layer, del_orig=True):
+        if self.dtype is None:
+            self.dtype = linear_layer.weight.dtype
+        if self.quantizer_mx is None:
+            self.quantizer_mx = WeightQuantizerMXFP(device=self.device, compute_dtype=linear_layer.weight.dtype)
+        W = linear_layer.weight.data
+        bias = linear_layer.bias.clone() if linear_layer.bias is not None else None
+        N, K = W.shape
+        W_q, scales = self.quantizer_mx.quantize_mxfp8(W, index=True, mx_fp8_dtype=self.mx_fp8_dtype)
+        W_q, scales = W_q.view(N, K), scales.view(N, K // 32)
+        cleanup_linear(linear_layer, del_orig)
+        return self.from_weights(weight=W_q, scales=scales, bias=bias)
+
+
 class A4W4_MXFP_dynamic:
     """MXFP4 activations (quantised on the fly) x MXFP4 weights
     (reference: gemlite/helper.py:1042-1114)."""

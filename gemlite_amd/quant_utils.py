@@ -46,6 +46,22 @@ def scale_activations_per_token(tensor: Tensor, w_dtype: torch.dtype, fp32_scale
     return y.view(x_shape), scales
 
 
+def scale_activations_mxfp8(tensor: Tensor, w_dtype: torch.dtype = torch.float8_e4m3fn) -> Tuple[Tensor, Tensor]:
+    """MXFP8 dynamic quantisation: ``([M, K] e4m3fn codes, [ceil32(M), K/32] uint8 e8m0)``
+    (reference: gemlite/quant_utils.py:1025-1127)."""
+    if w_dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f"MXFP8 activations as {w_dtype}: only float8_e4m3fn is built")
+    x2d = tensor.reshape(-1, tensor.shape[-1])
+    if x2d.stride(-1) != 1:
+        x2d = x2d.contiguous()
+    M, K = x2d.shape
+    M_pad = (M + 31) // 32 * 32
+    out = torch.empty((M, K), dtype=torch.uint8, device=tensor.device)
+    scales = torch.empty((M_pad, K // 32), dtype=torch.uint8, device=tensor.device)
+    _ext.scale_activations_mxfp8(x2d, out, scales)
+    return out.view(torch.float8_e4m3fn).view(tensor.shape), scales
+
+
 def scale_activations_mxfp4(tensor: Tensor) -> Tuple[Tensor, Tensor]:
     """MXFP4 dynamic quantisation: ``([M, K/2] uint8 codes, [ceil32(M), K/32] uint8 e8m0)``
     (reference: gemlite/quant_utils.py:2108-2135)."""
@@ -69,7 +85,6 @@ def _not_built(name):
 
 
 scale_activations_per_block = _not_built("scale_activations_per_block")
-scale_activations_mxfp8 = _not_built("scale_activations_mxfp8")
 scale_activations_nvfp4 = _not_built("scale_activations_nvfp4")
 
 
@@ -114,6 +129,18 @@ class WeightQuantizerMXFP:
         scales = scales.to(torch.float8_e8m0fnu)
         if index:
             W_q = self.to_index(W_q)
+        return W_q, scales
+
+    def quantize_mxfp8(self, W: Tensor, index: bool = False, mx_fp8_dtype: torch.dtype = torch.float8_e4m3fn) -> Tuple[Tensor, Tensor]:
+        """Blocks of 32 along the last axis: s = 2^ceil(log2(amax/qmax)) clamped to >= 2^-30, values
+        clamp(w/s) cast to fp8 (reference: gemlite/quant_utils.py:102-128)."""
+        max_val = torch.finfo(mx_fp8_dtype).max
+        W_flat = W.reshape(-1, 32).float()
+        ideal = W_flat.abs().amax(dim=1, keepdim=True) / max_val
+        scales = (2 ** torch.ceil(torch.log2(ideal))).clamp_(min=2.0 ** -30)
+        W_q = (W_flat / scales).clamp_(min=-max_val, max=max_val)
+        scales = scales.to(torch.float8_e8m0fnu)
+        W_q = W_q.to(mx_fp8_dtype) if index else W_q.to(mx_fp8_dtype).to(W_flat.dtype)
         return W_q, scales
 
     def dequantize(self, W_q, scales, shape=None, dtype=None, meta_scales=None):

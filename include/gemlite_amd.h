@@ -154,6 +154,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_8BIT 4    /* fp8 / int8 MFMA GEMM on K-major operands */
 #define GLA_FAMILY_GEMM_MXFP4 5   /* block-scaled FP4 MFMA GEMM */
 #define GLA_FAMILY_GEMM_KBYTES 6  /* MFMA GEMM for 16-bit activations x unpacked 8-bit weight bytes */
+#define GLA_FAMILY_GEMM_MXFP8 7   /* MXFP8 weights x fp8 activations, MFMA GEMM */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of
@@ -190,6 +191,14 @@ int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride
  * bytes with M_pad = M rounded up to 32; rows M..M_pad-1 are set to 127.
  * (reference: gemlite/quant_utils.py:2005-2135, exponent trick :697-705) */
 int gla_scale_activations_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K,
+                                uint8_t* y, uint8_t* scales, void* stream);
+
+/* MXFP8 dynamic activation quantisation: per 32 consecutive k one e8m0 scale
+ * 2^ceil(log2(amax/448)) (exponent clamped to [97, 254]) and 32 fp8-e4m3fn codes
+ * of clamp(x / scale, -448, 448), rounded to nearest even.  y: [M, K] bytes;
+ * scales: [M_pad, K/32] bytes with M_pad = M rounded up to 32; rows M..M_pad-1
+ * are set to 127.  (reference: gemlite/quant_utils.py:1025-1127, exponent trick :697-705) */
+int gla_scale_activations_mxfp8(const void* x, int x_dtype, int64_t x_stride_m, int M, int K,
                                 uint8_t* y, uint8_t* scales, void* stream);
 
 /* Pack rows x cols 8-bit codes into words of packing_bitwidth bits along the

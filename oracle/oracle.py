@@ -269,6 +269,25 @@ def scale_activations_mxfp4(x):
     return packed, scales
 
 
+def scale_activations_mxfp8(x):
+    """Per 32 values: e8m0 exponent from amax / 448, codes = e4m3fn(clamp(x * (1 / s), -448, 448)),
+    round to nearest even; scales padded to a multiple of 32 rows with 127
+    (reference: gemlite/quant_utils.py:1025-1127; 1 / s is an exact power of two).
+    Returns ([M, K] e4m3fn bytes, [M_pad, K/32] uint8)."""
+    x = np.asarray(x, dtype=np.float32)
+    M, K = x.shape
+    g = x.reshape(M, K // 32, 32)
+    amax = np.abs(g).max(axis=2)
+    exp = next_power_of_2_exponent((amax / np.float32(448.0)).astype(np.float32))
+    s = (exp.astype(np.uint32) << 23).view(np.float32)
+    y = np.clip((g * (np.float32(1.0) / s)[:, :, None]).astype(np.float32), np.float32(-448.0), np.float32(448.0))
+    codes = e4m3fn_encode(y.reshape(M, K))
+    M_pad = (M + 31) // 32 * 32
+    scales = np.full((M_pad, K // 32), 127, dtype=np.uint8)
+    scales[:M] = exp.astype(np.uint8)
+    return codes, scales
+
+
 # ---------------------------------------------------------------------------
 # weight quantisers
 # ---------------------------------------------------------------------------
@@ -291,6 +310,39 @@ def quantize_mxfp4_weights(W):
     # e8m0 byte of a power of two is its biased exponent
     e = (s.view(np.uint32) >> 23).astype(np.uint8)
     return codes.astype(np.uint8).reshape(N, K), e.reshape(N, K // 32)
+
+
+def quantize_mxfp8_weights(W):
+    """Blocks of 32: s = clamp(2^ceil(log2(amax/448)), 2^-30); codes = e4m3fn(clamp(w/s, -448, 448))
+    (reference: gemlite/quant_utils.py:102-128).  Returns ([N, K] e4m3fn bytes, [N, K/32] e8m0 bytes)."""
+    W = np.asarray(W, dtype=np.float32)
+    N, K = W.shape
+    flat = W.reshape(-1, 32)
+    ideal = np.abs(flat).max(axis=1, keepdims=True) / np.float32(448.0)
+    with np.errstate(divide="ignore"):
+        s = np.exp2(np.ceil(np.log2(ideal))).astype(np.float32)
+    s = np.maximum(s, np.float32(2.0 ** -30))
+    y = np.clip((flat / s).astype(np.float32), np.float32(-448.0), np.float32(448.0))
+    e = (s.view(np.uint32) >> 23).astype(np.uint8)
+    return e4m3fn_encode(y).reshape(N, K), e.reshape(N, K // 32)
+
+
+def matmul_mxfp8_weights(a, scales_x, b_codes, b_scales):
+    """fp8 activations a [M, K] (decoded values) with one fp32 scale per row applied after the K sum x
+    MXFP8 weights: out[m, n] = scales_x[m] * sum_k a[m, k] * e4m3(b[n, k]) * 2^(sb[n, k/32] - 127)
+    (reference: gemlite/triton_kernels/gemm_kernels.py:659-726 with channel_scale_mode 2; the block
+    products are exact in fp32, only the accumulation order is free)."""
+    A = np.asarray(a, dtype=np.float64)
+    B = e4m3fn_decode(b_codes).astype(np.float64) * np.repeat(e8m0_decode(b_scales), 32, axis=1)
+    return ((A @ B.T) * np.asarray(scales_x, dtype=np.float64).reshape(-1, 1)).astype(np.float32)
+
+
+def matmul_mxfp8(a_codes, a_scales, b_codes, b_scales):
+    """Block-scaled e4m3 x e4m3: sum over 32-blocks of 2^(sa-127) 2^(sb-127) sum_k a_k b_k
+    (reference: gemlite/triton_kernels/gemm_kernels.py:659-726, tl.dot_scaled)."""
+    A = e4m3fn_decode(a_codes).astype(np.float64) * np.repeat(e8m0_decode(a_scales), 32, axis=1)
+    B = e4m3fn_decode(b_codes).astype(np.float64) * np.repeat(e8m0_decode(b_scales), 32, axis=1)
+    return (A @ B.T).astype(np.float32)
 
 
 def quantize_per_channel(W, to_int8):

@@ -67,6 +67,17 @@ def oracle_forward(layer, x, matmul_x=None, scales_x=None):
         b_codes = orc.unpack_fp4_bytes(Wb)
         sb = layer.scales.detach().cpu().contiguous().numpy()        # [N, K/32]
         out = orc.matmul_mx(a_codes, scales_x[: a_codes.shape[0]], b_codes, sb)
+    elif in_dt == DType.MXFP8:
+        Wb = layer.W_q.detach().cpu().t().contiguous().view(torch.uint8).numpy()   # [N, K] e4m3fn bytes
+        sb = layer.scales.detach().cpu().contiguous().numpy()                        # [N, K/32] e8m0 bytes
+        if csm == 2:   # per-token activations, scale applied after the K sum
+            if matmul_x is None:
+                matmul_x, scales_x = orc.scale_activations_per_token(xin, False)
+            out = orc.matmul_mxfp8_weights(orc.e4m3fn_decode(matmul_x), scales_x, Wb, sb)
+        else:          # micro-scales on both sides
+            if matmul_x is None:
+                matmul_x, scales_x = orc.scale_activations_mxfp8(xin)
+            out = orc.matmul_mxfp8(matmul_x, scales_x[: matmul_x.shape[0]], Wb, sb)
     else:
         if layer.scaled_activations:
             if matmul_x is None:

@@ -459,3 +459,51 @@ def test_a8w4_hqq_int_dynamic_fp8_activations(device, group_size):
         assert (layer.W_group_mode, layer.channel_scale_mode) == (3, 2)
     for M in (1, 7, 40):
         check_layer(layer, gen_x(M, K, torch.float16, seed=M).to(device), torch.bfloat16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("K", [384, 1024])
+def test_a8w8_mxfp8_weights_per_token_activations(device, K):
+    """MXFP8 weights x fp8 activations quantised per token, scale applied after the K sum
+    (reference processor: gemlite/helper.py:876-923, its default post_scale=True)."""
+    from gemlite_amd import _ext
+    N = 520
+    W = gen_x(N, K, torch.bfloat16, seed=31, std=0.03)
+    W[7, 64:96] = 0.0
+    codes, e8 = orc.quantize_mxfp8_weights(to_np(W))
+    layer = helper.A8W8_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_weights(
+        torch.from_numpy(codes).view(torch.float8_e4m3fn), scales=torch.from_numpy(e8))
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 2)
+    for M in (1, 5, 33, 64, 100, 130, 300):
+        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M", [1, 31, 64, 100])
+def test_mxfp8_activation_quantizer_bit_exact(device, dtype, M):
+    K = 1024
+    x = gen_x(M, K, dtype, seed=M + 3)
+    x[0, 32:64] = 0.0
+    if M > 2:
+        x[2, 0] = 448.0
+        x[2, 1:32] = 0.25
+    codes, e8 = gemlite_amd.scale_activations_mxfp8(x.to(device))
+    want_codes, want_e8 = orc.scale_activations_mxfp8(to_np(x))
+    assert codes.dtype == torch.float8_e4m3fn and e8.shape == ((M + 31) // 32 * 32, K // 32)
+    assert np.array_equal(codes.view(torch.uint8).cpu().numpy(), want_codes)
+    assert np.array_equal(e8.cpu().numpy(), want_e8)
+
+
+@pytest.mark.gpu
+def test_a8w8_mxfp8_block_scaled_both_sides(device):
+    """MXFP8 x MXFP8 with micro-scales on the activations too (post_scale=False,
+    channel_scale_mode 4; reference: gemlite/helper.py:917-919)."""
+    N, K = 520, 1024
+    W = gen_x(N, K, torch.bfloat16, seed=41, std=0.03)
+    codes, e8 = orc.quantize_mxfp8_weights(to_np(W))
+    layer = helper.A8W8_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=False).from_weights(
+        torch.from_numpy(codes).view(torch.float8_e4m3fn), scales=torch.from_numpy(e8))
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 4)
+    for M in (1, 5, 33, 100, 130, 300):
+        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16)

@@ -385,3 +385,24 @@ def test_kernel_plugin_registry_has_the_reference_interface():
     for name, cls in m.items():
         assert cls.matmul_type == name and isinstance(cls.kernel, list)
         assert list(inspect.signature(cls.forward).parameters) == want
+
+
+def test_mxfp8_processor_packs_like_the_reference():
+    """A8W8_MXFP_dynamic: fp8 codes kept as the [K, N] view, e8m0 scales [N, K/32] K-contiguous,
+    W_group_mode 0 and channel_scale_mode 2 (post_scale) / 4 (reference: gemlite/helper.py:876-923);
+    the module's weight quantiser agrees with the oracle's."""
+    from oracle import oracle as orc
+    g = torch.Generator().manual_seed(2)
+    W = (torch.randn((64, 256), generator=g) * 0.03).to(torch.bfloat16)
+    q = gemlite_amd.quant_utils.WeightQuantizerMXFP(compute_dtype=torch.bfloat16, device="cpu")
+    codes, e8 = q.quantize_mxfp8(W, index=True)
+    want_codes, want_e8 = orc.quantize_mxfp8_weights(W.float().numpy())
+    assert np.array_equal(codes.view(torch.uint8).reshape(64, 256).numpy(), want_codes)
+    assert np.array_equal(e8.view(torch.uint8).reshape(64, 8).numpy(), want_e8)
+    for post_scale, csm in ((True, 2), (False, 4)):
+        proc = gemlite_amd.helper.A8W8_MXFP_dynamic(device="cpu", dtype=torch.bfloat16, post_scale=post_scale)
+        l = proc.from_weights(codes.view(64, 256), scales=e8.view(64, 8))
+        assert (l.W_group_mode, l.channel_scale_mode) == (0, csm)
+        assert l.input_dtype == gemlite_amd.DType.MXFP8 and l.scaled_activations and l.elements_per_sample == 1
+        assert l.W_q.shape == (256, 64) and l.W_q.stride() == (1, 256) and l.W_q.dtype == torch.float8_e4m3fn
+        assert l.scales.shape == (64, 8) and l.scales.stride() == (8, 1) and l.scales.dtype == torch.uint8

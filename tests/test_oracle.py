@@ -362,3 +362,85 @@ def test_select_modes_like_reference_tests():
     assert s(True, N, None, N, True) == (0, 3)                         # fp8 both scaled (tests/test_int.py:269-271)
     assert s(True, N, None, N, False) == (0, 1)                        # weight-only channelwise
     assert s(True, N * 132, None, N, True, mx=True) == (2, 0)          # micro-scaled formats
+
+
+# ------------------------------------------------------------------ MXFP8 weights
+def test_mxfp8_weight_quantizer_matches_torch_codecs_and_bounds():
+    """oracle.quantize_mxfp8_weights against torch's own e4m3fn / e8m0 casts of the same closed form,
+    plus what the format fixes: power-of-two scales, |w/s| <= 448, reconstruction within half an
+    e4m3 step of the block's top binade."""
+    g = torch.Generator().manual_seed(11)
+    W = (torch.randn((24, 256), generator=g) * 0.05).float()
+    W[3, 32:64] = 0.0                       # an all-zero block: scale clamps to 2^-30, codes 0
+    W[5, 0] = 3.0                           # an outlier sets its block's scale
+    codes, e8 = orc.quantize_mxfp8_weights(W.numpy())
+    flat = W.reshape(-1, 32)
+    ideal = flat.abs().amax(dim=1, keepdim=True) / 448.0
+    s = (2 ** torch.ceil(torch.log2(ideal))).clamp_(min=2.0 ** -30)
+    want_codes = (flat / s).clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).reshape(24, 256).numpy()
+    want_e8 = s.to(torch.float8_e8m0fnu).view(torch.uint8).reshape(24, 8).numpy()
+    assert np.array_equal(codes, want_codes) and np.array_equal(e8, want_e8)
+    assert e8[3, 1] == 127 - 30 and not codes[3, 32:64].any()
+    sc = orc.e8m0_decode(e8)
+    deq = orc.e4m3fn_decode(codes) * np.repeat(sc, 32, axis=1)
+    # every block's largest value lands in the top binade [256, 448] * s or below; the e4m3 step there is 32 s
+    assert np.all(np.abs(deq - W.numpy()) <= 16.0 * np.repeat(sc, 32, axis=1) + 1e-12)
+    amax = np.abs(W.numpy()).reshape(24, 8, 32).max(axis=2)
+    nz = amax > 0
+    assert np.all(amax[nz] / sc[nz] <= 448.0) and np.all(amax[nz] / sc[nz] > 224.0)
+
+
+def test_matmul_mxfp8_weights_closed_forms():
+    """Unit scales reduce it to a plain matmul of the decoded values; raising one block's scale byte by
+    one doubles exactly that block's contribution; the row scale multiplies the row."""
+    rng = np.random.default_rng(5)
+    M, N, K = 3, 4, 64
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b_codes = rng.integers(0, 0x77, size=(N, K), dtype=np.uint8)          # finite e4m3 codes
+    ones = np.full((N, K // 32), 127, dtype=np.uint8)
+    sx = np.ones((M, 1), dtype=np.float32)
+    base = orc.matmul_mxfp8_weights(a, sx, b_codes, ones)
+    B = orc.e4m3fn_decode(b_codes).astype(np.float64)
+    assert np.allclose(base, a.astype(np.float64) @ B.T, rtol=1e-6)
+    bumped = ones.copy(); bumped[2, 1] = 128
+    want = base.astype(np.float64).copy()
+    want[:, 2] += a[:, 32:].astype(np.float64) @ B[2, 32:]
+    assert np.allclose(orc.matmul_mxfp8_weights(a, sx, b_codes, bumped), want, rtol=1e-6)
+    sx2 = np.array([[1.0], [0.5], [3.0]], dtype=np.float32)
+    assert np.allclose(orc.matmul_mxfp8_weights(a, sx2, b_codes, ones), base * sx2, rtol=1e-6)
+
+
+def test_mxfp8_activation_quantizer_closed_forms():
+    """oracle.scale_activations_mxfp8 against torch's e4m3fn cast of the same scaled values, the
+    exponent rule on hand-picked maxima, padding rows, and the reconstruction bound of the format."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((5, 128), generator=g).to(torch.bfloat16).float()
+    x[1, 32:64] = 0.0
+    x[2, 0] = 448.0; x[2, 1:32] = 0.25          # amax / 448 == 1 exactly: exponent 127, no round-up
+    x[3, 0] = 449.0                             # just above: mantissa != 0 -> exponent 128
+    codes, e8 = orc.scale_activations_mxfp8(x.numpy())
+    assert codes.shape == (5, 128) and e8.shape == (32, 4) and np.all(e8[5:] == 127)
+    assert e8[1, 1] == 97 and not codes[1, 32:64].any()
+    assert e8[2, 0] == 127 and e8[3, 0] == 128
+    s = torch.from_numpy(orc.e8m0_decode(e8[:5])).repeat_interleave(32, dim=1)
+    want = (x / s).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(codes, want)
+    deq = orc.e4m3fn_decode(codes) * s.numpy()
+    # a value of magnitude v s with v <= 448 is off by at most half an e4m3 step at v: 2^(floor(log2 v) - 4)
+    assert np.all(np.abs(deq - x.numpy()) <= np.maximum(np.abs(x.numpy()) / 16.0, s.numpy() * 2.0 ** -10) + 1e-30)
+
+
+def test_matmul_mxfp8_block_scaled_closed_form():
+    rng = np.random.default_rng(8)
+    a = rng.integers(0, 0x77, size=(2, 64), dtype=np.uint8)
+    b = rng.integers(0, 0x77, size=(3, 64), dtype=np.uint8)
+    sa = np.array([[127, 130], [125, 127]], dtype=np.uint8)
+    sb = np.array([[127, 127], [126, 129], [127, 120]], dtype=np.uint8)
+    A, B = orc.e4m3fn_decode(a).astype(np.float64), orc.e4m3fn_decode(b).astype(np.float64)
+    want = np.zeros((2, 3))
+    for m in range(2):
+        for n in range(3):
+            for blk in range(2):
+                sl = slice(32 * blk, 32 * blk + 32)
+                want[m, n] += 2.0 ** (int(sa[m, blk]) - 127) * 2.0 ** (int(sb[n, blk]) - 127) * (A[m, sl] @ B[n, sl])
+    assert np.allclose(orc.matmul_mxfp8(a, sa, b, sb), want, rtol=1e-6)
