@@ -40,7 +40,9 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3 };
+enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4 };
+// kMXFP8T: MXFP8 weights whose activations carry no block scales (their per-token scale is applied in the
+// epilogue), so no registers are spent on activation scale words and the 256-row tile fits
 
 constexpr int kRowB8 = 64;  // bytes per LDS row = bytes of K per pipeline stage
 constexpr int kBN = 256;
@@ -55,7 +57,6 @@ struct Gemm8Args {
     int M, N, Kb;          // Kb = bytes of K per row
     int64_t lda, ldb, osm, sxm, msn;
     int64_t sx_stage, sw_stage;  // micro-scaled: bytes from one scale word of a row to the next one's
-    int a_unit;                  // MXFP8: the activations carry no block scales (per-token scale in the epilogue)
     const void* ascales;         // micro-scaled: activation block scales (row stride asxm bytes); scales_x is the epilogue's
     int64_t asxm;
     int csm, meta_dt, sx_dt, out_dt;
@@ -86,7 +87,7 @@ __device__ __forceinline__ void wait_vmcnt8() {
 }
 
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
-constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 || mode == kMXFP8 ? (bm + kBN) * 4 : 0); }
+constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 || mode == kMXFP8 || mode == kMXFP8T ? (bm + kBN) * 4 : 0); }
 
 // WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
 // (A 2-column variant with 4 waves of 128 x 128 and accumulators in AGPRs reads a third less from
@@ -100,9 +101,11 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr int TI = WM / 32;       // 32-row MFMA tiles per wave along M
     constexpr int WNC = kBN / WN;     // wave tile columns
     constexpr int TJ = WNC / 32;      // 32-column MFMA tiles per wave along N
-    constexpr bool MX = MODE == kMXFP4 || MODE == kMXFP8;  // block scales ride along with every stage
+    constexpr bool M8 = MODE == kMXFP8 || MODE == kMXFP8T;
+    constexpr bool TOKEN = MODE == kMXFP8T;                 // no activation block scales
+    constexpr bool MX = MODE == kMXFP4 || M8;               // block scales ride along with every stage
     // MXFP8: a 32-bit scale word of a row covers 128 values = two stages; MXFP4: one stage
-    constexpr int SSH = MODE == kMXFP8 ? 1 : 0;
+    constexpr int SSH = M8 ? 1 : 0;
     constexpr int NW = kWavesM * WN;
     constexpr int RING = kRing8;
     constexpr int SLOT = slot_bytes8(MODE, BM);
@@ -110,7 +113,8 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr int A_JOBS = BM / 16;           // 16-byte copy instructions for the A tile (16 rows each)
     constexpr int JOBS16 = A_JOBS + kBN / 16; // ... and the B tile
     constexpr int J16 = (JOBS16 + NW - 1) / NW;
-    constexpr int JOBS4 = (BM + kBN) / 64;    // MXFP4: 4-byte copies of block scales, 64 rows each
+    constexpr int A_JOBS4 = TOKEN ? 0 : BM / 64;
+    constexpr int JOBS4 = A_JOBS4 + kBN / 64; // micro-scaled: 4-byte copies of block scales, 64 rows each
     constexpr int J4 = MX ? (JOBS4 + NW - 1) / NW : 0;
     constexpr int LPS = J16 + J4;             // copy instructions per wave per stage
     static_assert(RING * LPS < 64, "outstanding copies must fit the vmcnt counter");
@@ -160,17 +164,18 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         for (int i = 0; i < J4; ++i) {
             int q = wave + NW * i;
             if (q > JOBS4 - 1) q = JOBS4 - 1;
-            is_a4[i] = q < BM / 64;
+            is_a4[i] = q < A_JOBS4;
             if (is_a4[i]) {
                 int gm = m0 + q * 64 + lane;
                 if (gm > p.M - 1) gm = p.M - 1;
                 off4[i] = (unsigned)(gm * (int)p.asxm);
             } else {
-                int gn = n0 + (q - BM / 64) * 64 + lane;
+                int gn = n0 + (q - A_JOBS4) * 64 + lane;
                 if (gn > p.N - 1) gn = p.N - 1;
                 off4[i] = (unsigned)(gn * (int)p.msn);
             }
-            dst4[i] = S_OFF + q * 256;
+            // the LDS image keeps room for the activation scales of BM rows whether they are copied or not
+            dst4[i] = S_OFF + (is_a4[i] ? q : q - A_JOBS4 + BM / 64) * 256;
         }
     }
 
@@ -231,10 +236,10 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         u32x4 c[2];
     } frag_t;
     frag_t fa[2][TI], fb[2][TJ];
-    unsigned fsa[2][MX ? TI : 1], fsb[2][MX ? TJ : 1];
+    unsigned fsa[2][MX && !TOKEN ? TI : 1], fsb[2][MX ? TJ : 1];
     // LDS read r of a stage's NRD: chunk reads of the weight tiles, then of the activation tiles,
     // then (MXFP4) the scale words
-    constexpr int NRD = (TI + TJ) * (MX ? 3 : 2);
+    constexpr int NRD = (TI + TJ) * 2 + (MX ? (TOKEN ? TJ : TI + TJ) : 0);
     // (`par`: parity of the absolute stage being read, which picks the half of an MXFP8 scale word)
     auto load_one = [&](int slot, auto buf_tag, int r, int par) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
@@ -247,11 +252,10 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         } else if constexpr (MX) {
             // MXFP4: half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2.
             // MXFP8: it multiplies with the scale of block kb of the stage, byte 2 par + kb of the word.
-            const int q = r - 2 * (TI + TJ);
-            const int sh = MODE == kMXFP8 ? 8 * (2 * par + kb) : 8 * kb;
+            const int q = r - 2 * (TI + TJ) + (TOKEN ? TI : 0);   // TOKEN: weight scale words only
+            const int sh = M8 ? 8 * (2 * par + kb) : 8 * kb;
             if (q < TI) {
-                const unsigned v = *(const unsigned*)(base + sa_row0 + q * 128) >> sh;
-                fsa[B][q] = (MODE == kMXFP8 && p.a_unit) ? 127u : v;
+                if constexpr (!TOKEN) fsa[B][q] = *(const unsigned*)(base + sa_row0 + q * 128) >> sh;
             } else {
                 fsb[B][q - TI] = *(const unsigned*)(base + sb_row0 + (q - TI) * 128) >> sh;
             }
@@ -277,13 +281,16 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         for (int r = 0; r < NRD; ++r) load_one(slot, buf_tag, r, par);
     };
     // MFMA q of a stage's NM.  fp8: one K-step of 64 bytes per tile pair; int8 / fp4: two K-steps of 32
-    constexpr int NM = TI * TJ * (MODE == kFP8 || MODE == kMXFP8 ? 1 : 2);
+    constexpr int NM = TI * TJ * (MODE == kFP8 || M8 ? 1 : 2);
     auto multiply_one = [&](int limit, auto buf_tag, auto scale_tag, int q) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;    // fragment buffer
         constexpr int SB = decltype(scale_tag)::value; // scale buffer (MXFP4)
         const int s2 = q / (TI * TJ), i = (q % (TI * TJ)) / TJ, j = q % TJ;
         if constexpr (MODE == kFP8) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
+        } else if constexpr (TOKEN) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0,
+                                                                        (int)fsb[SB][j], 0, 127);
         } else if constexpr (MODE == kMXFP8) {
             // registers 0-3 of both half-waves are block 0 of the stage, registers 4-7 block 1, and the
             // half-wave's scale is that of block kb: the chunk pair (kb, 2 + kb) as one operand
@@ -644,7 +651,7 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
-    a.out_dt = p.output_dtype; a.sx_stage = 0; a.sw_stage = 0; a.a_unit = 0; a.ascales = nullptr; a.asxm = 0;
+    a.out_dt = p.output_dtype; a.sx_stage = 0; a.sw_stage = 0; a.ascales = nullptr; a.asxm = 0;
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
@@ -692,7 +699,7 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
     a.M = p.M; a.N = p.N; a.Kb = p.K / 2; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.csm = 0; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype;
-    a.sx_stage = 4; a.sw_stage = 4; a.a_unit = 0; a.ascales = p.scales_x; a.asxm = p.sx_stride_m;
+    a.sx_stage = 4; a.sw_stage = 4; a.ascales = p.scales_x; a.asxm = p.sx_stride_m;
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
@@ -733,10 +740,11 @@ bool gemm_mxfp8_eligible(const gla_matmul_args& p) {
     return true;
 }
 
-// the 256-row tile has no registers for the scale words next to two fragment buffers of 8-register operands
+// with block scales on both sides the 256-row tile has no registers for the scale words next to two
+// fragment buffers of 8-register operands
 static Plan8 plan_mxfp8(const gla_matmul_args& p) {
     Plan8 g = plan8(p.M, p.N, p.K, p.tile_config);
-    if (g.bm == 256) {
+    if (g.bm == 256 && p.channel_scale_mode == GLA_CSM_MX) {
         const int cfg = (p.tile_config > 0 ? p.tile_config / 1000 : 0) * 1000 + 128;
         g = plan8(p.M, p.N, p.K, cfg);
     }
@@ -760,7 +768,6 @@ int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.sw_stage = 4;
     a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
-    a.a_unit = act_blocks ? 0 : 1;
     a.csm = act_blocks ? 0 : 2;  // per-token scale in the epilogue
     // without activation block scales the copy jobs for them re-read the first weight scale word (never used)
     a.ascales = act_blocks ? p.scales_x : p.scales;
@@ -783,7 +790,7 @@ int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
         if (act_blocks) { a.ascales = sx; a.asxm = 4; a.sx_stage = (int64_t)p.M * 4; }
         else { a.ascales = sw; }
     }
-    return launch_mode<kMXFP8>(a, g.bm, stream);
+    return act_blocks ? launch_mode<kMXFP8>(a, g.bm, stream) : launch_mode<kMXFP8T>(a, g.bm, stream);
 }
 
 }  // namespace gla
