@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/gemlite_amd.h"
 
 namespace gla {
@@ -26,6 +28,17 @@ constexpr int kWave = 64;
 // error reporting (host)
 // ---------------------------------------------------------------------------
 void set_error(const char* fmt, ...);
+
+// Function attributes (the dynamic LDS limit) are kept per device: true the first time a call site
+// runs on the current device.  `seen` is the call site's own table (one per kernel instantiation).
+struct DeviceOnce {
+    std::atomic<bool> seen[64];
+    bool first() {
+        int d = 0;
+        if (hipGetDevice(&d) != hipSuccess || d < 0 || d >= 64) return true;
+        return !seen[d].exchange(true);
+    }
+};
 int check_hip(hipError_t e, const char* what);
 
 // ---------------------------------------------------------------------------

@@ -525,13 +525,12 @@ __global__ __launch_bounds__(256) void splitk_finish8_kernel(Gemm8Args p) {
 template <int MODE, int BM, int WN>
 int launch_bm(const Gemm8Args& a, hipStream_t stream) {
     const size_t smem = (size_t)kRing8 * slot_bytes8(MODE, BM);
-    static bool configured = false;  // per instantiation; the attribute is sticky per function
+    static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
     auto kern = gemm_8bit_kernel<MODE, BM, WN>;
-    if (!configured) {
+    if (once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_8bit: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
-        configured = true;
     }
     hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(kWavesM * WN * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "gemm_8bit launch");

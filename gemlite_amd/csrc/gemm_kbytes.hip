@@ -388,13 +388,12 @@ template <int WDT, bool BF16, int TI>
 int launch_kb(const GemmKbArgs& a, hipStream_t stream) {
     constexpr int BM = kWavesMb * 32 * TI;
     const size_t smem = (size_t)ring_slots_kb(BM) * slot_bytes_kb(BM);
-    static bool configured = false;
+    static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
     auto kern = gemm_kbytes_kernel<WDT, BF16, TI>;
-    if (!configured) {
+    if (once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_kbytes: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
-        configured = true;
     }
     hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(kWavesMb * kWavesNb * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "gemm_kbytes launch");

@@ -616,13 +616,12 @@ template <int BITS, bool BF16, int WAVES_M, int TI, int TJ>
 int launch_wn(const GemmWnArgs& a, hipStream_t stream) {
     constexpr int BM = WAVES_M * TI * 32;
     const size_t smem = (size_t)ring_slots(BM) * slot_bytes(BITS, BM);
-    static bool configured = false;
+    static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
     auto kern = gemm_wn_kernel<BITS, BF16, WAVES_M, TI, TJ>;
-    if (!configured && smem > 48 * 1024) {
+    if (smem > 48 * 1024 && once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_wn: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
-        configured = true;
     }
     hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(WAVES_M * (8 / TJ) * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "gemm_wn launch");

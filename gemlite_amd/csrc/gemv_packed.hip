@@ -825,12 +825,10 @@ void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
             else if (g.waves == 16) {
                 if constexpr (RT == 16) {  // its cross-wave buffer alone is 64 KiB
-                    static bool configured = false;
-                    if (!configured) {
+                    static DeviceOnce once;
+                    if (once.first())
                         (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 16, false>,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
-                        configured = true;
-                    }
                 }
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
             } else if (g.waves == 8)
