@@ -181,6 +181,37 @@ def extra_points(lib, device):
         del layer, xq, sx
     del W, x, y
 
+    # A8W8 MXFP8 weights, fp8 activations quantised per token (the reference processor's default), M = 4096, N = K = 8192
+    M, N, K = 4096, 8192, 8192
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+    lin.weight.data = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    layer = helper.A8W8_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
+    del lin
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    run = prepared(layer, xq, sx, y)
+    us = time_us(run, 50)
+    point("gemm_a8w8_mxfp8", M, N, K, us, 5000.0, "fp8", zeroed(run, xq, layer.W_q.data))
+    del layer, x, xq, sx, y
+
+    # A16W8 weight-only int8 bytes (unpacked), bf16, N = K = 8192: M = 4096 (MFMA GEMM) and M = 1 (streaming)
+    M, N, K = 4096, 8192, 8192
+    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
+    layer = helper.A16W8_INT8(device=device, post_scale=True).from_weights(W)
+    del W
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+    run = prepared(layer, x, None, y)
+    us = time_us(run, 30)
+    point("gemm_a16w8_int8_bytes_bf16", M, N, K, us, 2500.0, "bf16")
+    x1 = x[:1].contiguous()
+    y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
+    us = time_us(prepared(layer, x1, None, y1), 50)
+    out["gemv_a16w8_int8_bytes_M1"] = {"N": N, "K": K, "us": round(us, 1), "GB/s": round((N * K + N * 4 + K * 2 + N * 2) / us / 1e3, 1),
+                                       "note": "64 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"}
+    del layer, x, y, x1, y1
+
     # A4W4 MXFP4 dynamic, M = 4096, N = K = 16384
     M, N, K = 4096, 16384, 16384
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
