@@ -1,0 +1,109 @@
+"""Parity at the full sizes of the benchmark configurations.  The whole output is too large for the
+CPU oracle, so the HIP result is checked on a seeded sample of output columns, for which the oracle
+computes every row exactly (float64 / int64 accumulation) from the same weights and activations."""
+import numpy as np
+import pytest
+import torch
+
+import gemlite_amd
+from gemlite_amd import DType, GemLiteLinear, helper
+from oracle import oracle as orc
+from parity import FROB_TOL, gen_int_case, gen_x, rel_frob, to_np
+
+pytestmark = pytest.mark.gpu
+TIGHT_BF16, TIGHT_FP16 = 6e-3, 1.5e-3
+
+
+def sample_cols(N, count=48, seed=0):
+    rng = np.random.default_rng(seed)
+    cols = np.unique(np.concatenate([rng.integers(0, N, size=count), [0, N - 1]]))
+    return cols
+
+
+@pytest.mark.parametrize("nbits,gs,M", [(8, 16384, 1), (8, 16384, 16), (8, 16384, 64), (8, 16384, 512),
+                                        (2, 64, 1), (2, 64, 16), (2, 64, 64), (2, 64, 512)])
+def test_a16wn_bf16_16384_square(device, nbits, gs, M):
+    """bf16 activations x 8-bit channel-wise / 2-bit group-64 weights, N = K = 16384."""
+    N = K = 16384
+    W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.bfloat16, seed=nbits, scale_std=0.01)
+    layer = helper.A16Wn(device=device, post_scale=True).from_weights(W_q, scales, zeros, nbits, gs)
+    x = gen_x(M, K, torch.bfloat16, seed=M)
+    y = to_np(layer(x.to(device)))
+    cols = sample_cols(N, seed=M + nbits)
+    gpn = K // gs   # groups per output row
+    idx = (cols[:, None] * gpn + np.arange(gpn)[None, :]).reshape(-1)
+    want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], gs)
+    err = rel_frob(y[:, cols], want)
+    assert err <= FROB_TOL and err <= TIGHT_BF16, err
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_a8w8_dynamic_4096x8192x8192(device, fp8):
+    """Per-token dynamic activations x per-channel 8-bit weights at M = 4096, N = K = 8192: the
+    activation codes and scales are the oracle's bit for bit; sampled output columns follow from exact
+    integer (float64) sums of those codes."""
+    M, N, K = 4096, 8192, 8192
+    W = gen_x(N, K, torch.bfloat16, seed=3, std=0.02)
+    wq, sw = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+    proc = (helper.A8W8_FP8_dynamic if fp8 else helper.A8W8_INT8_dynamic)(device=device)
+    proc.dtype = torch.bfloat16
+    layer = proc.from_weights(wq, scales=sw)
+    x = gen_x(M, K, torch.bfloat16, seed=4)
+    y = to_np(layer(x.to(device)))
+    xq, sx = gemlite_amd.scale_activations_per_token(x.to(device), torch.float8_e4m3fn if fp8 else torch.int8)
+    rows = np.arange(0, M, 61)   # the quantiser on a subset of rows, against the oracle
+    want_q, want_s = orc.scale_activations_per_token(to_np(x)[rows], not fp8)
+    got_q = xq.view(torch.uint8).cpu().numpy()[rows] if fp8 else xq.cpu().numpy()[rows]
+    assert np.array_equal(got_q, want_q) and np.array_equal(sx.cpu().numpy()[rows], want_s)
+    cols = sample_cols(N, seed=7)
+    a = orc.e4m3fn_decode(xq.view(torch.uint8).cpu().numpy()) if fp8 else xq.cpu().numpy()
+    wsub = wq.view(torch.uint8).numpy()[cols] if fp8 else wq.numpy()[cols]
+    b = orc.e4m3fn_decode(wsub) if fp8 else wsub
+    acc = a.astype(np.float64) @ b.astype(np.float64).T
+    want = acc * sx.cpu().numpy().astype(np.float64) * to_np(sw).astype(np.float64).reshape(-1)[cols][None, :]
+    assert rel_frob(y[:, cols], want.astype(np.float32)) <= TIGHT_BF16
+
+
+@pytest.mark.parametrize("M", [1, 32, 1024])
+def test_a4w4_mxfp4_16384_square(device, M):
+    N = K = 16384
+    W = gen_x(N, K, torch.bfloat16, seed=9, std=0.02)
+    codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+    layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_weights(
+        torch.from_numpy(codes), scales=torch.from_numpy(e8))
+    x = gen_x(M, K, torch.bfloat16, seed=M)
+    y = to_np(layer(x.to(device)))
+    a_packed, sa = orc.scale_activations_mxfp4(to_np(x))
+    cols = sample_cols(N, seed=M)
+    want = orc.matmul_mx(orc.unpack_fp4_bytes(a_packed), sa[:M], codes[cols], e8[cols])
+    assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+
+
+@pytest.mark.parametrize("M", [1, 1024])
+def test_a8w8_mxfp8_8192_square(device, M):
+    N = K = 8192
+    W = gen_x(N, K, torch.bfloat16, seed=10, std=0.02)
+    codes, e8 = orc.quantize_mxfp8_weights(to_np(W))
+    layer = helper.A8W8_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_weights(
+        torch.from_numpy(codes).view(torch.float8_e4m3fn), scales=torch.from_numpy(e8))
+    x = gen_x(M, K, torch.bfloat16, seed=M)
+    y = to_np(layer(x.to(device)))
+    aq, sx = orc.scale_activations_per_token(to_np(x), False)
+    cols = sample_cols(N, seed=M)
+    want = orc.matmul_mxfp8_weights(orc.e4m3fn_decode(aq), sx, codes[cols], e8[cols])
+    assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+
+
+def test_a16w4_prefill_4096_cubed(device):
+    """fp16 activations x 4-bit group-128 weights at M = N = K = 4096 (the GEMM point of the headline metric)."""
+    M = N = K = 4096
+    W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16, seed=12)
+    layer = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    x = gen_x(M, K, torch.float16, seed=13)
+    y = to_np(layer(x.to(device)))
+    cols = sample_cols(N, seed=14)
+    gpn = K // 128
+    idx = (cols[:, None] * gpn + np.arange(gpn)[None, :]).reshape(-1)
+    want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], 128)
+    err = rel_frob(y[:, cols], want)
+    assert err <= FROB_TOL and err <= TIGHT_FP16, err
