@@ -757,7 +757,13 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     // 2-bit codes: direct only for the 16-row tile (up to 4 rows the staged kernel measured a little faster)
     const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8 || (p.W_nbits == 2 && g.RT == 16));
     // the cross-wave buffer is [waves][RT][64] floats; the staged 16-row kernel runs 4 waves
-    const int max_waves = (g.RT == 16) ? (can_direct ? 16 : 4) : 16;
+    int max_waves = (g.RT == 16) ? (can_direct ? 16 : 4) : 16;
+    // Large layers: once 8-wave workgroups still give every CU two or more, they stream better than
+    // 16-wave ones (measured on 16384^2: 4-bit 27.9 against 32.2 us, 8-bit 44 against 53 us).
+    if (max_waves > 8 && (int64_t)g.tiles * ceil_div(p.M, g.RT) * ceil_div(units, 8) >= 512) max_waves = 8;
+    // ... and 2-bit codes at the 16-row tile better still with 4 (35.5 against 43.6 us)
+    if (p.W_nbits == 2 && g.RT == 16 && max_waves > 4 && (int64_t)g.tiles * ceil_div(p.M, g.RT) * ceil_div(units, 4) >= 512)
+        max_waves = 4;
     int waves, nb;
     if (p.tile_config >= 1000) {
         waves = p.tile_config / 1000;
