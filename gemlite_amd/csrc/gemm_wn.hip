@@ -8,9 +8,10 @@
 // gemlite/triton_kernels/utils.py:73-105).
 //
 //  * Workgroup tile BM x 256 with BM = 32, 64, 128 or 256, K step 64, v_mfma_f32_32x32x16 tiles.
-//    BM <= 128: waves in a WAVES_M x 2 grid, wave tile (32 TI) x 128.  BM = 256: 2 x 4 waves of
-//    128 x 64, because every wave unpacks the weights of its own columns and the 4 x 2 arrangement
-//    would repeat that work four times per workgroup instead of twice.
+//    Four wave columns of 64 at every height: BM <= 128 is one wave row of BM x 64 wave tiles
+//    (4 waves), BM = 256 two wave rows of 128 x 64 (8 waves).  Every wave unpacks the weights of
+//    its own columns, so wave rows repeat that work and wave columns divide it; the unpacking,
+//    not the MFMA, bounds the short tiles.
 //  * Every operand of a stage (activation tile, packed weight words, scales, zeros) is copied
 //    global -> LDS by the load unit (global_load_lds) into a ring of 3 or 4 stages; the K loop
 //    loads nothing into registers from global memory and waits on the vector-memory counter only
@@ -635,10 +636,11 @@ int launch_wn(const GemmWnArgs& a, hipStream_t stream) {
 
 template <int BITS, bool BF16>
 int launch_wn_m(const GemmWnArgs& a, int bm, hipStream_t stream) {
+    // four wave columns of 64 at every tile height: a wave unpacks only its own 64 columns
     if (bm == 256) return launch_wn<BITS, BF16, 2, 4, 2>(a, stream);
-    if (bm == 128) return launch_wn<BITS, BF16, 2, 2, 4>(a, stream);
-    if (bm == 64) return launch_wn<BITS, BF16, 1, 2, 4>(a, stream);
-    return launch_wn<BITS, BF16, 1, 1, 4>(a, stream);
+    if (bm == 128) return launch_wn<BITS, BF16, 1, 4, 2>(a, stream);
+    if (bm == 64) return launch_wn<BITS, BF16, 1, 2, 2>(a, stream);
+    return launch_wn<BITS, BF16, 1, 1, 2>(a, stream);
 }
 
 // tile_config encoding: BM (32, 64, 128 or 256; other = chosen here) + 1000 * K splits (0 = chosen here)
