@@ -164,9 +164,9 @@ constexpr int ring_slots(int bm) { return bm >= 128 ? 3 : 4; }
 constexpr int slot_bytes(int bits, int bm) { return bm * kRowW + 2 * (bits == 8 ? 8 : 4) * 1024 + 1024; }
 
 // BITS in {2, 4, 8}; WAVES_M in {1, 2, 4}; TI = 32-row MFMA tiles per wave (1, 2 or 4); TJ = 32-column
-// tiles per wave (4 or 2).  Every wave dequantises the weights of its own columns, so the work of
-// unpacking is repeated WAVES_M times per workgroup: the 256-row tile uses 2 x 4 waves of 128 x 64
-// (TI 4, TJ 2) rather than 4 x 2 waves of 64 x 128, which halves the unpacking per MFMA.
+// tiles per wave (4 or 2; the launcher uses 2 throughout).  Every wave dequantises the weights of
+// its own columns, so the work of unpacking is repeated WAVES_M times per workgroup and divided by
+// the number of wave columns.
 template <int BITS, bool BF16, int WAVES_M, int TI, int TJ>
 __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_wn_kernel(GemmWnArgs p) {
     static_assert(TJ == 4 || TJ == 2, "wave tile of 128 or 64 columns");
