@@ -7,8 +7,8 @@
 // gemlite/triton_kernels/gemm_kernels.py:285-496, gemlite/triton_kernels/gemm_splitK_kernels.py:300-523;
 // the processor that builds such layers: gemlite/helper.py:89-171).
 //
-//  * Workgroup tile BM x 256 with BM = 64, 128 or 256, K step 64; 2 x 4 waves, wave tile
-//    (BM/2) x 64 of v_mfma_f32_32x32x16_{f16,bf16} tiles.
+//  * Workgroup tile BM x 256 with BM = 64, 128 or 256, K step 64; four wave columns of 64 and
+//    two wave rows of BM/2 (one wave row of 64 at BM = 64), v_mfma_f32_32x32x16_{f16,bf16} tiles.
 //  * Both operand tiles of a stage are copied global -> LDS by the load unit (global_load_lds) into
 //    a ring of 3 or 4 stages, all in flight.  Activation rows are dense 128-byte rows with 16-byte
 //    chunks XOR-swizzled by (row >> 1) & 7; weight rows are dense 64-byte rows swizzled by
@@ -44,7 +44,7 @@ constexpr int kBKb = 64;     // K per pipeline stage
 constexpr int kRowAb = 128;  // LDS row of the activation tile: 64 fp16/bf16 values
 constexpr int kRowBb = 64;   // LDS row of the weight tile: 64 bytes
 constexpr int kBNb = 256;
-constexpr int kWavesMb = 2, kWavesNb = 4;
+constexpr int kWavesNb = 4;
 constexpr int64_t kWsReservedB = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
 
 struct GemmKbArgs {
@@ -130,12 +130,12 @@ constexpr int ring_slots_kb(int bm) { return bm >= 256 ? 3 : 4; }
 constexpr int slot_bytes_kb(int bm) { return bm * kRowAb + kBNb * kRowBb; }
 
 // WDT: GLA_DT_INT8, GLA_DT_UINT8 or GLA_DT_FP8; TI = 32-row MFMA tiles per wave (1, 2 or 4)
-template <int WDT, bool BF16, int TI>
-__global__ __launch_bounds__(kWavesMb * kWavesNb * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kbytes_kernel(GemmKbArgs p) {
+template <int WDT, bool BF16, int WAVES_M, int TI>
+__global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kbytes_kernel(GemmKbArgs p) {
     constexpr int TJ = 2;
     constexpr int WM = 32 * TI;
-    constexpr int BM = kWavesMb * WM;
-    constexpr int NW = kWavesMb * kWavesNb;
+    constexpr int BM = WAVES_M * WM;
+    constexpr int NW = WAVES_M * kWavesNb;
     constexpr int RING = ring_slots_kb(BM);
     constexpr int SLOT = slot_bytes_kb(BM);
     constexpr int B_OFF = BM * kRowAb;
@@ -384,18 +384,18 @@ __global__ __launch_bounds__(256) void splitk_finish_kb_kernel(GemmKbArgs p) {
     store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n, v * sc);
 }
 
-template <int WDT, bool BF16, int TI>
+template <int WDT, bool BF16, int WAVES_M, int TI>
 int launch_kb(const GemmKbArgs& a, hipStream_t stream) {
-    constexpr int BM = kWavesMb * 32 * TI;
+    constexpr int BM = WAVES_M * 32 * TI;
     const size_t smem = (size_t)ring_slots_kb(BM) * slot_bytes_kb(BM);
     static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
-    auto kern = gemm_kbytes_kernel<WDT, BF16, TI>;
+    auto kern = gemm_kbytes_kernel<WDT, BF16, WAVES_M, TI>;
     if (once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_kbytes: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
     }
-    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(kWavesMb * kWavesNb * 64), smem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n, a.S), dim3(WAVES_M * kWavesNb * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "gemm_kbytes launch");
     if (rc == GLA_OK && a.S > 1) {
         const int64_t items = (int64_t)a.M * a.N;
@@ -407,9 +407,12 @@ int launch_kb(const GemmKbArgs& a, hipStream_t stream) {
 
 template <int WDT, bool BF16>
 int launch_kb_m(const GemmKbArgs& a, int bm, hipStream_t stream) {
-    if (bm == 256) return launch_kb<WDT, BF16, 4>(a, stream);
-    if (bm == 128) return launch_kb<WDT, BF16, 2>(a, stream);
-    return launch_kb<WDT, BF16, 1>(a, stream);
+    // four wave columns of 64.  A second wave row repeats the byte -> fp16/bf16 conversion, which
+    // bounds the 64-row tile: one row of four waves there (measured: -17 % time at 16384^2, M <= 64;
+    // at 128 rows the two arrangements time the same)
+    if (bm == 256) return launch_kb<WDT, BF16, 2, 4>(a, stream);
+    if (bm == 128) return launch_kb<WDT, BF16, 2, 2>(a, stream);
+    return launch_kb<WDT, BF16, 1, 2>(a, stream);
 }
 
 // tile_config encoding: BM (64, 128 or 256; other = chosen here) + 1000 * K splits (0 = chosen here)
