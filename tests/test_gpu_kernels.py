@@ -150,7 +150,7 @@ def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
     W_q, scales, zeros = gen_int_case(N, K, nbits, gs, dtype, seed=nbits * 10 + gs)
     dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
     layer = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device))
-    for M in (1, 4, 7, 64):
+    for M in (1, 4, 7, 24, 64, 100, 200):   # above 16 rows: every tile height of the MFMA GEMM
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
 
 
@@ -386,7 +386,7 @@ def test_a16w8_weight_only_unpacked_bytes(device, fp8, post_scale, dtype, K):
         assert _ext.matmul_family(args) == "GEMV_KMAJOR"
         check_layer(layer, x, dtype)
     # above 16 rows: the MFMA GEMM for weight bytes where K is a multiple of its 64-value stage, else the generic kernel
-    for M in (17, 40, 130, 300):
+    for M in (17, 40, 100, 130, 300):
         x = gen_x(M, K, dtype, seed=M).to(device)
         out = torch.empty((M, N), dtype=dtype, device=device)
         m = layer.get_meta_args()
