@@ -326,7 +326,7 @@ class A8W2_HQQ_INT_dynamic(A8Wn_HQQ_INT_dynamic):
 class A8W8_MXFP_dynamic:
     """MXFP8 weights (fp8-e4m3 codes, one e8m0 scale per 32 values) x fp8 activations quantised on
     the fly: per token with the scale applied after the K sum (``post_scale=True``, the default) or
-    with MXFP8 micro-scales (``post_scale=False``; not built here)
+    with MXFP8 micro-scales on the activations as well (``post_scale=False``)
     (reference: gemlite/helper.py:876-947)."""
 
     def __init__(self, device="cuda:0", dtype=None, post_scale=True, fp8=torch.float8_e4m3fn):
