@@ -156,7 +156,11 @@ def _check(status: int, what: str):
 
 
 def _stream_ptr(device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on ``device`` (the capture stream inside torch.cuda.graph)."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
 
 
 def _require_cuda(*tensors):
@@ -182,13 +186,28 @@ def get_closest_m(M: int) -> int:
 # workspace: one zero-initialised scratch tensor per device, grown on demand
 # ---------------------------------------------------------------------------
 _workspaces = {}
+_retired_workspaces = []  # outgrown buffers stay allocated: a captured HIP graph may still point at them
 
 
 def get_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Scratch memory for split-K partials, ticket counters and regrouped block scales.
+
+    Growing replaces the buffer (at least doubling, so the outgrown ones add up to less than the
+    live one) and never frees the old one.  Growing while the stream is being captured into a graph
+    is refused: the fill that zeroes the new buffer would become a node of the graph.  Run the
+    layer once before capturing it.
+    """
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        size = max(int(nbytes), 8 << 20)
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                f"gemlite_amd: the workspace has to grow to {int(nbytes)} bytes while a graph is being captured; "
+                "run the layer once at this shape before capturing"
+            )
+        size = max(int(nbytes), 8 << 20, 0 if ws is None else 2 * ws.numel())
+        if ws is not None:
+            _retired_workspaces.append(ws)
         ws = torch.zeros(size, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
@@ -308,6 +327,30 @@ def matmul(args: MatmulArgs, device: torch.device):
         args.workspace = ws.data_ptr()
         args.workspace_bytes = ws.numel()
     _check(lib.gla_matmul(ctypes.byref(args), _stream_ptr(device)), "gla_matmul")
+
+
+def matmul_prepared(args: MatmulArgs, need: int, x_ptr: int, out_ptr: int, sx_ptr, device: torch.device):
+    """Launch a ``gla_matmul_args`` that ``build_matmul_args`` filled and checked before, for the
+    same shapes, strides and weight tensors: only the activation, output and activation-scale
+    addresses (and the workspace, which may have grown) are refreshed.  ``need`` is what
+    ``gla_matmul_workspace_bytes`` returned for it."""
+    args.x = x_ptr
+    args.out = out_ptr
+    args.scales_x = sx_ptr
+    if need > 0:
+        ws = get_workspace(device, need)
+        args.workspace = ws.data_ptr()
+        args.workspace_bytes = ws.numel()
+    status = load_library().gla_matmul(ctypes.byref(args), _stream_ptr(device))
+    if status != GLA_OK:
+        _check(status, "gla_matmul")
+
+
+def matmul_workspace_need(args: MatmulArgs) -> int:
+    need = load_library().gla_matmul_workspace_bytes(ctypes.byref(args))
+    if need < 0:
+        _check(int(need), "gla_matmul_workspace_bytes")
+    return int(need)
 
 
 FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8"]

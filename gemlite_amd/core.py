@@ -201,24 +201,57 @@ def forward_functional(
 # matching classes of the GEMV / split-K files).  All five run gla_matmul; the type is a hint the
 # library's dispatcher may override (up to 16 rows the streaming kernels run whatever was asked for).
 # ---------------------------------------------------------------------------
+# Prepared launches: filling and bounds-checking a gla_matmul_args costs more host time than a
+# decode-sized kernel runs, so a filled struct is kept per (weight tensor object, shapes, strides,
+# dtypes, modes, tile) and later calls only refresh the activation / output addresses.  An entry is
+# trusted only while the weight, scale and zero tensors still sit at the addresses it was built for.
+# Entries are per thread: the struct is rewritten in place on every call.
+_PREPARED = {}
+_PREPARED_LIMIT = 8192
+_thread_id = threading.get_ident
+
+
 def _kernel_forward(matmul_type_str):
+    matmul_type_id = GEMLITE_MATMUL_TYPES_MAPPING[matmul_type_str]
+
     def forward(x, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
                 input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
                 data_contiguous, type_id, meta_scale=0.0):
         M, K, N = x.shape[0], W_q.shape[0] * elements_per_sample, W_q.shape[1]
         out = torch.empty((M, N), dtype=DTYPE_TO_TORCH[int(output_dtype)], device=x.device)
-        if M > 0:
-            key = config_key(M, N, K, group_size, elements_per_sample, type_id)
-            args = _ext.build_matmul_args(
-                x, W_q, scales, zeros, scales_x, out,
-                W_nbits=W_nbits, group_size=group_size, unpack_mask=unpack_mask,
-                elements_per_sample=elements_per_sample, input_dtype=input_dtype, output_dtype=output_dtype,
-                acc_dtype=acc_dtype, meta_dtype=meta_dtype, channel_scale_mode=channel_scale_mode,
-                W_group_mode=W_group_mode, data_contiguous=data_contiguous,
-                matmul_type=GEMLITE_MATMUL_TYPES_MAPPING[matmul_type_str],
-                tile_config=_cached_tile_config(matmul_type_str, key),
-            )
-            _ext.matmul(args, x.device)
+        if M == 0:
+            return out
+        if GEMLITE_CONFIG_CACHE:
+            tile = _cached_tile_config(matmul_type_str, config_key(M, N, K, group_size, elements_per_sample, type_id))
+        else:
+            tile = -1
+        sx_key = None if scales_x is None else (scales_x.shape, scales_x.stride(), scales_x.dtype)
+        key = (id(W_q), W_q.shape, W_q.stride(), _thread_id(), matmul_type_id, x.shape, x.stride(), x.dtype, sx_key,
+               x.device.index, W_nbits, group_size,
+               unpack_mask, elements_per_sample, input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode,
+               W_group_mode, data_contiguous, tile)
+        hit = _PREPARED.get(key)
+        if hit is not None:
+            args, need, w_ptr, s_ptr, z_ptr = hit
+            if (W_q.data_ptr() == w_ptr and (scales is None or scales.data_ptr() == s_ptr)
+                    and (zeros is None or zeros.data_ptr() == z_ptr)):
+                _ext.matmul_prepared(args, need, x.data_ptr(), out.data_ptr(),
+                                     None if scales_x is None else scales_x.data_ptr(), x.device)
+                return out
+        args = _ext.build_matmul_args(
+            x, W_q, scales, zeros, scales_x, out,
+            W_nbits=W_nbits, group_size=group_size, unpack_mask=unpack_mask,
+            elements_per_sample=elements_per_sample, input_dtype=input_dtype, output_dtype=output_dtype,
+            acc_dtype=acc_dtype, meta_dtype=meta_dtype, channel_scale_mode=channel_scale_mode,
+            W_group_mode=W_group_mode, data_contiguous=data_contiguous,
+            matmul_type=matmul_type_id, tile_config=tile,
+        )
+        need = _ext.matmul_workspace_need(args)
+        _ext.matmul_prepared(args, need, args.x, args.out, args.scales_x, x.device)
+        if len(_PREPARED) >= _PREPARED_LIMIT:
+            _PREPARED.clear()
+        _PREPARED[key] = (args, need, W_q.data_ptr(), None if scales is None else scales.data_ptr(),
+                          None if zeros is None else zeros.data_ptr())
         return out
     return forward
 

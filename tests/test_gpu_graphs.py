@@ -1,0 +1,64 @@
+"""forward() under HIP graph capture: the launches of a layer (activation quantisation, the
+matmul, a split-K finish) are recorded once and replayed with new inputs.  Every replay must equal
+the eager result bit for bit - the kernels are deterministic, the ticket counters of the split-K
+GEMV reset themselves, and nothing in the path allocates or clears memory once the layer has run
+at that shape."""
+import pytest
+import torch
+
+import gemlite_amd
+from gemlite_amd import DType, GemLiteLinear, _ext, helper
+from parity import gen_int_case, gen_x
+
+pytestmark = pytest.mark.gpu
+
+
+def _layers(device):
+    W_q, s, z = gen_int_case(1024, 8192, 4, 128, torch.float16, seed=1)
+    yield "A16W4", GemLiteLinear(4, 128, 8192, 1024, DType.FP16, DType.FP16).pack(W_q.to(device), s.to(device), z.to(device)), \
+        torch.float16, (1, 5, 64)      # split-K GEMV with tickets; split-K MFMA GEMM with its finishing kernel
+    W = gen_x(1032, 2048, torch.bfloat16, seed=2, std=0.02)
+    W_q8, s8 = gemlite_amd.quantize_weights_per_channel(W, torch.int8)
+    proc = helper.A8W8_INT8_dynamic(device=device)
+    proc.dtype = torch.bfloat16
+    yield "A8W8", proc.from_weights(W_q8, scales=s8), torch.bfloat16, (3, 70)   # activation quantiser + GEMM
+    lin = torch.nn.Linear(2048, 1032, bias=True, dtype=torch.bfloat16)
+    lin.weight.data = W
+    yield "MXFP4", helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device)), \
+        torch.bfloat16, (40,)
+
+
+def test_forward_replays_from_a_graph(device):
+    for name, layer, dtype, row_counts in _layers(device):
+        K = layer.in_features
+        for M in row_counts:
+            print(f"case: {name} M={M}", flush=True)
+            x_static = gen_x(M, K, dtype, seed=99).to(device)
+            layer(x_static)  # first run at this shape: sizes the workspace
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                y_static = layer(x_static)
+            for rep in range(4):
+                x_new = gen_x(M, K, dtype, seed=rep).to(device)
+                x_static.copy_(x_new)
+                graph.replay()
+                torch.cuda.synchronize()
+                got = y_static.clone()
+                want = layer(x_new)  # eager work between the replays
+                torch.cuda.synchronize()
+                assert torch.equal(got, want), (name, M, rep)
+
+
+def test_workspace_growth_is_refused_during_capture_and_keeps_old_buffers(device, monkeypatch):
+    ws = _ext.get_workspace(device, 1)
+    bigger = ws.numel() + 1
+    # the stream reports a capture in progress (no real capture: a failed one would outlive the test)
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(RuntimeError, match="before capturing"):
+        _ext.get_workspace(device, bigger)
+    assert _ext.get_workspace(device, ws.numel()).data_ptr() == ws.data_ptr()  # large enough: no growth, no refusal
+    monkeypatch.undo()
+    grown = _ext.get_workspace(device, bigger)
+    assert grown.numel() >= 2 * ws.numel() and grown.data_ptr() != ws.data_ptr()
+    assert any(r.data_ptr() == ws.data_ptr() for r in _ext._retired_workspaces)
