@@ -653,7 +653,10 @@ WnPlan wn_plan(const gla_matmul_args& p) {
     const int cfg = p.tile_config > 0 ? p.tile_config : 0;
     g.bm = cfg % 1000;
     if (!(g.bm == 32 || g.bm == 64 || g.bm == 128 || g.bm == 256))
-        g.bm = p.M > 128 ? 256 : (p.M > 64 ? 128 : (p.M > 32 ? 64 : 32));
+        // Up to 256 rows the 128-row tile: against the 256-row one it halves the K splits, and with
+        // them the fp32 partials, at the same number of workgroups (8192^2 4-bit, M=256: 55-58
+        // against 61-64 us)
+        g.bm = p.M > 256 ? 256 : (p.M > 64 ? 128 : (p.M > 32 ? 64 : 32));
     g.tiles_m = ceil_div(p.M, g.bm);
     g.tiles_n = ceil_div(p.N, kBNw);
     const int total_steps = p.K / kBKw;
@@ -662,7 +665,9 @@ WnPlan wn_plan(const gla_matmul_args& p) {
         // enough workgroups for 256 CUs, but no split shorter than 8 stages (512 K-values) and at
         // most 32 splits
         const int tiles = g.tiles_m * g.tiles_n;
-        const int target = 256;
+        // 2-bit codes on short tiles are bound by unpacking on one wave per SIMD: two workgroups per CU
+        // (16384^2, M=64: 72 against 90 us)
+        const int target = (p.W_nbits == 2 && g.bm <= 64) ? 512 : 256;
         want = tiles * 2 > target ? 1 : ceil_div(target, tiles);
         const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
         if (want > max_s) want = max_s;
