@@ -175,6 +175,14 @@ def forward_functional(
     elif x2d.dtype in TORCH_TO_DTYPE and not is_mx_dtype(input_dtype):
         # the kernels read x as the element type it actually has
         kernel_input_dtype = TORCH_TO_DTYPE[x2d.dtype].value
+    elif input_dtype in (DType.MXFP16.value, DType.MXBF16.value):
+        # weight-only MX layer: the 16-bit activations go to the kernel as they are
+        if x2d.dtype == torch.float16:
+            kernel_input_dtype = DType.MXFP16.value
+        elif x2d.dtype == torch.bfloat16:
+            kernel_input_dtype = DType.MXBF16.value
+        else:
+            raise NotImplementedError(f"weight-only MX layers take fp16 or bf16 activations, got {x2d.dtype}")
 
     M = x2d.shape[0]
     mx = is_mx_dtype(input_dtype)

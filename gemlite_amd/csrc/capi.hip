@@ -49,7 +49,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
     return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
 }
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8 };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM };
 
 int validate(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -84,8 +84,17 @@ int validate(const gla_matmul_args* p) {
         }
         return GLA_OK;
     }
+    if (p->input_dtype == GLA_DT_MXFP16 || p->input_dtype == GLA_DT_MXBF16) {
+        if (!mx_stream_eligible(*p)) {
+            set_error("matmul: weight-only MX layers need K-contiguous fp8 bytes or e2m1 nibble pairs with one e8m0 scale "
+                      "per 32 values, K %% 32 == 0, 16-byte aligned rows and channel_scale_mode 0 (K=%d, mode %d)",
+                      p->K, p->channel_scale_mode);
+            return GLA_ERR_UNSUPPORTED_MODE;
+        }
+        return GLA_OK;
+    }
     if (p->input_dtype == GLA_DT_MXFP8) {
-        if (!gemm_mxfp8_eligible(*p)) {
+        if (!gemm_mxfp8_eligible(*p) && !mx_stream_eligible(*p)) {
             set_error("matmul: MXFP8 needs fp8 weight bytes with K-contiguous e8m0 scales per 32 values, K %% 128 == 0, "
                       "16-byte aligned rows and channel_scale_mode 2 or 4 (K=%d, mode %d)", p->K, p->channel_scale_mode);
             return GLA_ERR_UNSUPPORTED_MODE;
@@ -93,7 +102,7 @@ int validate(const gla_matmul_args* p) {
         return GLA_OK;
     }
     if (is_mx(p->input_dtype)) {
-        set_error("matmul: micro-scaled input type %d is not supported (MXFP4 and MXFP8 only)", p->input_dtype);
+        set_error("matmul: micro-scaled input type %d is not supported (MXFP16, MXBF16, MXFP8 and MXFP4 only)", p->input_dtype);
         return GLA_ERR_UNSUPPORTED_DTYPE;
     }
     switch (p->input_dtype) {
@@ -142,8 +151,9 @@ int validate(const gla_matmul_args* p) {
 }
 
 Family choose(const gla_matmul_args& p, int type) {
-    if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : F_GENERIC;
-    if (p.input_dtype == GLA_DT_MXFP8) return F_GEMM_MXFP8;  // validated as eligible; there is no other kernel for it
+    if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
+    if (p.input_dtype == GLA_DT_MXFP8) return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;  // validated: one of the two
+    if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16) return F_MX_STREAM;
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
     const bool small = type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16;
     if (small) {
@@ -220,6 +230,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
         case F_GEMM_KBYTES: return launch_gemm_kbytes(*args, s);
         case F_GEMM_MXFP8: return launch_gemm_mxfp8(*args, s);
+        case F_MX_STREAM: return launch_mx_stream(*args, s);
         default: return launch_generic(*args, s);
     }
 }

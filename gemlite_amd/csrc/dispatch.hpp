@@ -38,6 +38,11 @@ bool gemm_mxfp8_eligible(const gla_matmul_args& p);
 int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream);
 int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p);
 
+// ---- streaming kernel for K-contiguous micro-scaled operands (mx_stream.hip): weight-only MX
+// layers (fp16/bf16 x MXFP8/MXFP4 weights), MXFP8 activations x MXFP4 weights
+bool mx_stream_eligible(const gla_matmul_args& p);
+int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream);
+
 // ---- activation quantisation (actquant.hip) and bit packing (bitpack.hip) --
 int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
                          float* scales, hipStream_t stream);

@@ -1,0 +1,249 @@
+// Streaming kernel for the micro-scaled (MX) formats whose operands are both K-contiguous:
+//
+//   activations  fp16 | bf16 (weight-only layers) | fp8-e4m3 bytes | e2m1 nibble pairs
+//   weights      fp8-e4m3 bytes | e2m1 nibble pairs, one e8m0 scale per 32 values along K
+//   act scales   none | one fp32 per row applied after the K sum | one e8m0 per 32 values
+//
+//   out(m,n) = sum_blocks ( sum_{k in block} a(m,k) w(n,k) ) * 2^(sw(n,block)-127) * 2^(sa(m,block)-127)
+//
+// (reference: gemlite/triton_kernels/gemm_kernels.py:509-737 and gemm_splitK_kernels.py:536-770:
+//  `tl.dot_scaled(a, scales_a, a_dtype, b, scales_b, b_dtype, acc)` with a_dtype in
+//  {fp16, bf16, e4m3, e2m1}, b_dtype in {e4m3, e2m1}, unit activation scales unless
+//  channel_scale_mode is 4, and the per-row activation scale of channel_scale_mode 2 at :714-717.)
+//
+// One wave owns one output column n: lane l takes the 32-blocks l, l+64, ... of weight row n
+// (16 or 32 contiguous bytes per block, so a wave reads 1-2 KiB of consecutive weight bytes per
+// step) and multiplies them with the same blocks of up to four activation rows.  Codes become
+// fp16 (bf16 for bf16 activations) pairs with the conversion instructions of gfx950 — exact, both
+// code sets are subsets of either type — and pairs are multiplied and summed in fp32 by the packed
+// dot instruction; the block's partial sum is then scaled once by the product of its two block
+// scales, as the scaled matrix instruction does.  A shuffle tree sums the lanes.
+//
+// The combinations that have a matrix-core kernel (MXFP4 x MXFP4, fp8 x MXFP8) do not come here;
+// this kernel is the decode path of the weight-only MX layers and the path at any batch size for
+// MXFP8 activations x MXFP4 weights and for weight-only MX layers (not tuned above a few rows:
+// every group of four activation rows streams the weights again).
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace gla {
+
+namespace {
+
+enum { A_F16 = 0, A_BF16 = 1, A_FP8 = 2, A_FP4 = 3 };
+enum { B_FP8 = 0, B_FP4 = 1 };
+
+struct MxArgs {
+    const uint8_t* x;
+    const uint8_t* w;
+    const uint8_t* scales;
+    const void* scales_x;
+    void* out;
+    int M, N, KB;  // KB = K / 32
+    int64_t xsm_bytes, wsn_bytes, osm, osn, msg, msn, sxm, sxg;
+    int csm, out_dt;
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <bool BF>
+struct Pair {
+    using type = half2_t;
+};
+template <>
+struct Pair<true> {
+    using type = bf16x2_t;
+};
+
+template <bool BF>
+__device__ __forceinline__ float dot2(typename Pair<BF>::type a, typename Pair<BF>::type b, float c) {
+    if constexpr (BF) return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
+    else return __builtin_amdgcn_fdot2(a, b, c, false);
+}
+
+// The 32 values of one block as 16 pairs (k, k+1), from e2m1 nibbles (16 bytes) ...
+template <bool BF>
+__device__ __forceinline__ void block_from_fp4(const uint8_t* p, typename Pair<BF>::type (&v)[16]) {
+    const u32x4 q = *(const u32x4*)p;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        if constexpr (BF) {
+            v[4 * d + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[d], 1.0f, 0);
+            v[4 * d + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[d], 1.0f, 1);
+            v[4 * d + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[d], 1.0f, 2);
+            v[4 * d + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q[d], 1.0f, 3);
+        } else {
+            v[4 * d + 0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[d], 1.0f, 0);
+            v[4 * d + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[d], 1.0f, 1);
+            v[4 * d + 2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[d], 1.0f, 2);
+            v[4 * d + 3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[d], 1.0f, 3);
+        }
+    }
+}
+
+// ... from e4m3 bytes (32 bytes) ...
+template <bool BF>
+__device__ __forceinline__ void block_from_fp8(const uint8_t* p, typename Pair<BF>::type (&v)[16]) {
+    const u32x4 q0 = *(const u32x4*)p, q1 = *(const u32x4*)(p + 16);
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+        const uint32_t w = d < 4 ? q0[d & 3] : q1[d & 3];
+        if constexpr (BF) {
+            v[2 * d + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+            v[2 * d + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true);
+        } else {
+            v[2 * d + 0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+            v[2 * d + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+        }
+    }
+}
+
+// ... or taken as they lie (64 bytes of fp16 / bf16).
+template <bool BF>
+__device__ __forceinline__ void block_from_16bit(const uint8_t* p, typename Pair<BF>::type (&v)[16]) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const u32x4 q = *(const u32x4*)(p + 16 * d);
+        // element copies first: a bit cast applied to `q[j]` directly took element 0 for every j
+        const uint32_t q0 = q.x, q1 = q.y, q2 = q.z, q3 = q.w;
+        v[4 * d + 0] = __builtin_bit_cast(typename Pair<BF>::type, q0);
+        v[4 * d + 1] = __builtin_bit_cast(typename Pair<BF>::type, q1);
+        v[4 * d + 2] = __builtin_bit_cast(typename Pair<BF>::type, q2);
+        v[4 * d + 3] = __builtin_bit_cast(typename Pair<BF>::type, q3);
+    }
+}
+
+template <int AK, int BK, int RM>
+__global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
+    constexpr bool BF = (AK == A_BF16);
+    using pair_t = typename Pair<BF>::type;
+    constexpr int kABytes = AK == A_FP4 ? 16 : (AK == A_FP8 ? 32 : 64);
+    constexpr int kBBytes = BK == B_FP4 ? 16 : 32;
+
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int m0 = blockIdx.y * RM;
+    if (n >= a.N) return;  // whole waves leave; no barrier follows
+
+    const uint8_t* wrow = a.w + (int64_t)n * a.wsn_bytes;
+    float acc[RM];
+#pragma unroll
+    for (int r = 0; r < RM; ++r) acc[r] = 0.0f;
+
+    for (int blk = lane; blk < a.KB; blk += 64) {
+        pair_t wv[16];
+        if constexpr (BK == B_FP4) block_from_fp4<BF>(wrow + (int64_t)blk * kBBytes, wv);
+        else block_from_fp8<BF>(wrow + (int64_t)blk * kBBytes, wv);
+        const float sw = e8m0_to_float(a.scales[(int64_t)n * a.msn + (int64_t)blk * a.msg]);
+#pragma unroll
+        for (int r = 0; r < RM; ++r) {
+            const int m = m0 + r;
+            if (m < a.M) {
+                const uint8_t* xp = a.x + (int64_t)m * a.xsm_bytes + (int64_t)blk * kABytes;
+                pair_t xv[16];
+                if constexpr (AK == A_FP4) block_from_fp4<BF>(xp, xv);
+                else if constexpr (AK == A_FP8) block_from_fp8<BF>(xp, xv);
+                else block_from_16bit<BF>(xp, xv);
+                float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; j += 2) {
+                    p0 = dot2<BF>(xv[j], wv[j], p0);
+                    p1 = dot2<BF>(xv[j + 1], wv[j + 1], p1);
+                }
+                float s = sw;
+                if (a.csm == GLA_CSM_MX)
+                    s *= e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)blk * a.sxg]);
+                acc[r] = __builtin_fmaf(p0 + p1, s, acc[r]);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < RM; ++r) {
+        float v = acc[r];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) v += wave_xor(v, off);
+        const int m = m0 + r;
+        if (lane == 0 && m < a.M) {
+            if (a.csm == GLA_CSM_ACTIVATION) v *= ((const float*)a.scales_x)[(int64_t)m * a.sxm];
+            store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, v);
+        }
+    }
+}
+
+int a_kind(const gla_matmul_args& p) {
+    switch (p.input_dtype) {
+        case GLA_DT_MXFP16: return A_F16;
+        case GLA_DT_MXBF16: return A_BF16;
+        case GLA_DT_MXFP8: return A_FP8;
+        case GLA_DT_MXFP4: return A_FP4;
+        default: return -1;
+    }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+template <int AK, int BK>
+void launch_rows(const MxArgs& a, int rm, dim3 grid, hipStream_t s) {
+    if (rm == 1) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 1>), grid, dim3(256), 0, s, a);
+    else if (rm == 2) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 2>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 4>), grid, dim3(256), 0, s, a);
+}
+
+template <int AK>
+void launch_b(const MxArgs& a, int bk, int rm, dim3 grid, hipStream_t s) {
+    if (bk == B_FP4) launch_rows<AK, B_FP4>(a, rm, grid, s);
+    else launch_rows<AK, B_FP8>(a, rm, grid, s);
+}
+
+}  // namespace
+
+bool mx_stream_eligible(const gla_matmul_args& p) {
+    const int ak = a_kind(p);
+    if (ak < 0 || p.group_size != 32 || p.K % 32 != 0) return false;
+    if (p.elements_per_sample != 1 && p.elements_per_sample != 2) return false;
+    if (p.W_nbits != (p.elements_per_sample == 2 ? 4 : 8)) return false;
+    if (p.scales == nullptr || p.x_stride_k != 1 || p.w_stride_k != 1) return false;
+    // x_stride_m counts stored elements (bytes for the 8- and 4-bit kinds, 16-bit words otherwise)
+    const int64_t xsm_bytes = p.x_stride_m * (ak <= A_BF16 ? 2 : 1);
+    if (xsm_bytes % 16 != 0 || p.w_stride_n % 16 != 0 || !aligned16(p.x) || !aligned16(p.w)) return false;
+    switch (p.output_dtype) {
+        case GLA_DT_FP32: case GLA_DT_FP16: case GLA_DT_BF16: case GLA_DT_MXFP16: case GLA_DT_MXBF16: break;
+        default: return false;
+    }
+    const int csm = p.channel_scale_mode;
+    if (csm == GLA_CSM_MX) return p.scales_x != nullptr && ak >= A_FP8;
+    if (csm == GLA_CSM_ACTIVATION) return p.scales_x != nullptr && p.sx_dtype == GLA_DT_FP32;
+    return csm == GLA_CSM_NONE;
+}
+
+int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream) {
+    if (!mx_stream_eligible(p)) {
+        set_error("mx_stream: operands must be K-contiguous with 16-byte aligned rows, group_size 32, "
+                  "channel_scale_mode 0, 2 or 4");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    const int ak = a_kind(p);
+    MxArgs a;
+    a.x = (const uint8_t*)p.x; a.w = (const uint8_t*)p.w; a.scales = (const uint8_t*)p.scales;
+    a.scales_x = p.scales_x; a.out = p.out;
+    a.M = p.M; a.N = p.N; a.KB = p.K / 32;
+    a.xsm_bytes = p.x_stride_m * (ak <= A_BF16 ? 2 : 1);
+    a.wsn_bytes = p.w_stride_n;
+    a.osm = p.out_stride_m; a.osn = p.out_stride_n;
+    a.msg = p.meta_stride_g; a.msn = p.meta_stride_n; a.sxm = p.sx_stride_m; a.sxg = p.sx_stride_g;
+    a.csm = p.channel_scale_mode;
+    a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
+    const int rm = p.M >= 3 ? 4 : p.M;
+    const int bk = p.elements_per_sample == 2 ? B_FP4 : B_FP8;
+    dim3 grid(ceil_div(p.N, 4), ceil_div(p.M, rm));
+    switch (ak) {
+        case A_F16: launch_b<A_F16>(a, bk, rm, grid, stream); break;
+        case A_BF16: launch_b<A_BF16>(a, bk, rm, grid, stream); break;
+        case A_FP8: launch_b<A_FP8>(a, bk, rm, grid, stream); break;
+        default: launch_b<A_FP4>(a, bk, rm, grid, stream); break;
+    }
+    return check_hip(hipGetLastError(), "mx_stream launch");
+}
+
+}  // namespace gla

@@ -108,16 +108,18 @@ class A16W8_FP8(A16W8):
 
 
 class A16Wn:
-    """fp16/bf16 activations x grouped 8/4/2/1-bit integer weights
-    (reference: gemlite/helper.py:174-302; the MXFP weight-only variants of that class are not
-    built).  ``post_scale`` defaults to True, the reference's default on AMD GPUs
-    (reference: gemlite/helper.py:14-22)."""
+    """fp16/bf16 activations x grouped 8/4/2/1-bit integer weights (``quant_type="INT"``) or x
+    MXFP8 / MXFP4 weights with one e8m0 scale per 32 values (``quant_type="MXFP"``)
+    (reference: gemlite/helper.py:174-332).  ``post_scale`` defaults to True, the reference's
+    default on AMD GPUs (reference: gemlite/helper.py:14-22)."""
 
     def __init__(self, device="cuda:0", dtype=None, packing_bitwidth=None, post_scale=True):
         self.device = device
         self.dtype = dtype
         self.packing_bitwidth = packing_bitwidth
         self.post_scale = post_scale
+        self.quantizer_mx = None
+        self.mx_fp8_dtype = torch.float8_e4m3fn
 
     def from_packed_weights(self, W_q, scales, zeros, W_nbits, group_size, bias=None, quant_type="INT"):
         """Load pre-packed weights (already nibble/byte-packed)."""
@@ -127,12 +129,13 @@ class A16Wn:
         return self.from_weights_(W_q, scales, zeros, W_nbits, group_size, bias, quant_type)
 
     def from_weights_(self, W_q, scales, zeros, W_nbits, group_size, bias=None, quant_type="INT", packed=False):
-        if quant_type != "INT":
-            raise NotImplementedError(f"quant_type {quant_type}: only the grouped-integer recipe is built")
+        assert quant_type in ("INT", "MXFP"), f"Invalid quant_type. Got {quant_type}, valid values are INT, MXFP."
         if isinstance(W_q, torch.nn.Parameter):
             W_q = W_q.data
         if isinstance(bias, torch.nn.Parameter):
             bias = bias.data
+        if quant_type == "MXFP":
+            return self._from_mxfp_weights(W_q, scales, W_nbits, group_size, bias, packed)
         dtype = scales.dtype if self.dtype is None else self.dtype
         assert dtype in (torch.float16, torch.bfloat16, torch.float32), "Invalid scales.dtype, should floating point."
         out_features, in_features = W_q.shape
@@ -153,6 +156,54 @@ class A16Wn:
             else:
                 layer.W_group_mode, layer.channel_scale_mode = 3, 0
         return layer
+
+    def _from_mxfp_weights(self, W_q, scales, W_nbits, group_size, bias, packed):
+        """Weight-only MX layer: the activations stay fp16 / bf16, the layer's input and output
+        types are MXFP16 / MXBF16 (reference: gemlite/helper.py:199-202, 222-237)."""
+        assert W_nbits in (8, 4), "Unsupported W_nbit for MXFP quant_dtype."
+        assert group_size == 32, "group_size should 32 for MXFP."
+        if W_nbits == 8:
+            assert W_q.dtype == self.mx_fp8_dtype, f"Unsupported dtype of W_q. got {W_q.dtype}"
+        else:
+            assert W_q.dtype == torch.uint8, f"Unsupported dtype of W_q. got {W_q.dtype}"
+        dtype = torch.float16 if self.dtype is None else self.dtype
+        if dtype == torch.float16:
+            gemlite_dtype = DType.MXFP16
+        elif dtype == torch.bfloat16:
+            gemlite_dtype = DType.MXBF16
+        else:
+            raise Exception(f"Unsupported dtype for MXFP. Got {dtype}, supported [torch.float16, torch.bfloat16]")
+        self.post_scale = False
+        out_features, in_features = W_q.shape
+        if packed and W_nbits == 4:
+            in_features *= 2
+        if scales.dtype == torch.uint8:
+            scales = scales.view(torch.float8_e8m0fnu)
+        scales = scales.view(out_features, in_features // group_size)
+        bias = bias.to(device=self.device, dtype=dtype) if bias is not None else None
+        layer = GemLiteLinear(
+            W_nbits, group_size=group_size, in_features=in_features, out_features=out_features,
+            input_dtype=gemlite_dtype, output_dtype=gemlite_dtype, scaled_activations=False,
+        )
+        layer.pack(W_q.to(self.device), scales.to(self.device), None, bias=bias,
+                   packing_bitwidth=self.packing_bitwidth, packed=packed)
+        return layer
+
+    def mxfp_from_linear(self, linear_layer, W_nbits, del_orig=True):
+        """Quantise a float layer to MXFP8 / MXFP4 weights (reference: gemlite/helper.py:304-332)."""
+        if self.quantizer_mx is None:
+            self.quantizer_mx = WeightQuantizerMXFP(device=self.device, compute_dtype=linear_layer.weight.dtype)
+        W = linear_layer.weight.data
+        bias = linear_layer.bias.clone() if linear_layer.bias is not None else None
+        N, K = W.shape
+        if W_nbits == 8:
+            W_q, scales = self.quantizer_mx.quantize_mxfp8(W, index=True, mx_fp8_dtype=self.mx_fp8_dtype)
+        else:
+            W_q, scales = self.quantizer_mx.quantize_mxfp4(W, index=True)
+        W_q, scales = W_q.view(N, K), scales.view(N, K // 32)
+        cleanup_linear(linear_layer, del_orig)
+        return self.from_weights_(W_q=W_q, scales=scales, zeros=None, W_nbits=W_nbits, group_size=32, bias=bias,
+                                  quant_type="MXFP")
 
     def from_hqqlinear(self, hqq_layer, del_orig=True):
         """From an HQQ layer object: what it exposes (``unpack()``, ``meta['scale'|'zero'|'nbits'|
@@ -207,6 +258,38 @@ class A16W2_HQQ_INT(A16Wn_HQQ_INT):
 class A16W1_HQQ_INT(A16Wn_HQQ_INT):
     def __init__(self, device="cuda:0", dtype=None):
         super().__init__(device=device, dtype=dtype, W_nbits=1)
+
+
+class A16Wn_MXFP(A16Wn):
+    """Weight-only MXFP8 / MXFP4 with the bit width fixed (reference: gemlite/helper.py:384-412)."""
+
+    def __init__(self, device="cuda:0", dtype=None, W_nbits=None):
+        super().__init__(device=device, dtype=dtype)
+        self.W_nbits = W_nbits
+
+    def from_packed_weights(self, W_q_packed, scales, bias=None):
+        """Load pre-packed MXFP weights (nibble/byte-packed)."""
+        group_size = W_q_packed.numel() * (8 // self.W_nbits) // scales.numel()
+        return super().from_packed_weights(W_q_packed, scales, zeros=None, W_nbits=self.W_nbits,
+                                           group_size=group_size, bias=bias, quant_type="MXFP")
+
+    def from_weights(self, W_q, scales, bias=None):
+        group_size = W_q.numel() // scales.numel()
+        return super().from_weights(W_q=W_q, scales=scales, zeros=None, W_nbits=self.W_nbits,
+                                    group_size=group_size, bias=bias, quant_type="MXFP")
+
+    def from_linear(self, linear_layer, del_orig=True):
+        return super().mxfp_from_linear(linear_layer=linear_layer, W_nbits=self.W_nbits, del_orig=del_orig)
+
+
+class A16W8_MXFP(A16Wn_MXFP):
+    def __init__(self, device="cuda:0", dtype=None):
+        super().__init__(device=device, dtype=dtype, W_nbits=8)
+
+
+class A16W4_MXFP(A16Wn_MXFP):
+    def __init__(self, device="cuda:0", dtype=None):
+        super().__init__(device=device, dtype=dtype, W_nbits=4)
 
 
 class A8W8_dynamic:
@@ -323,29 +406,39 @@ class A8W2_HQQ_INT_dynamic(A8Wn_HQQ_INT_dynamic):
                          fp8=fp8, fp32_scale=fp32_scale, W_nbits=2)
 
 
-class A8W8_MXFP_dynamic:
-    """MXFP8 weights (fp8-e4m3 codes, one e8m0 scale per 32 values) x fp8 activations quantised on
-    the fly: per token with the scale applied after the K sum (``post_scale=True``, the default) or
-    with MXFP8 micro-scales on the activations as well (``post_scale=False``)
-    (reference: gemlite/helper.py:876-947)."""
+class A8Wn_MXFP_dynamic:
+    """MXFP8 or MXFP4 weights (fp8-e4m3 bytes / e2m1 codes, one e8m0 scale per 32 values) x fp8
+    activations quantised on the fly: per token with the scale applied after the K sum
+    (``post_scale=True``, the default) or with MXFP8 micro-scales on the activations as well
+    (``post_scale=False``) (reference: gemlite/helper.py:950-1032)."""
 
-    def __init__(self, device="cuda:0", dtype=None, post_scale=True, fp8=torch.float8_e4m3fn):
+    def __init__(self, device="cuda:0", dtype=None, post_scale=True, fp8=torch.float8_e4m3fn, W_nbits=None):
+        assert W_nbits is not None, "W_nbits argument should be either 8 or 4, not None."
         self.device = device
         self.dtype = dtype
         self.mx_fp8_dtype = fp8
         self.quantizer_mx = None
         self.post_scale = post_scale
-        self.W_nbits = 8
+        self.W_nbits = W_nbits
 
-    def from_weights(self, weight, bias=None, scales=None):
+    def from_packed_weights(self, weight_packed, bias=None, scales=None):
+        """Load pre-packed MXFP weights (nibble-packed [N, K//2] for 4-bit)."""
+        return self.from_weights(weight_packed, bias=bias, scales=scales, packed=True)
+
+    def from_weights(self, weight, bias=None, scales=None, packed=False):
         if isinstance(weight, torch.nn.Parameter):
             weight = weight.data
         if isinstance(bias, torch.nn.Parameter):
             bias = bias.data
         out_features, in_features = weight.shape
+        if packed and self.W_nbits == 4:
+            in_features *= 2
         assert scales is not None, "Scales parameter cannot be None. Use from_linear() call to pre-quantize the weights."
-        assert weight.is_floating_point() and weight.dtype.itemsize == 1, \
-            f"Invalid weight.dtype, should be an MXFP8 dtype, got {weight.dtype}."
+        if self.W_nbits == 8:
+            assert weight.is_floating_point() and weight.dtype.itemsize == 1, \
+                f"Invalid weight.dtype, should be an MXFP8 dtype, got {weight.dtype}."
+        if self.W_nbits == 4:
+            assert weight.dtype == torch.uint8, f"Invalid weight.dtype, should be uint8 codes, got {weight.dtype}."
         assert scales.dtype in (torch.float8_e8m0fnu, torch.uint8), f"Invalid scales.dtype, got {scales.dtype}."
         assert self.dtype is not None, "Input dtype should be either torch.float16 or torch.bfloat16, not None."
         if scales.dtype == torch.uint8:
@@ -355,7 +448,7 @@ class A8W8_MXFP_dynamic:
             self.W_nbits, group_size=32, in_features=in_features, out_features=out_features,
             input_dtype=DType.MXFP8, output_dtype=TORCH_TO_DTYPE[self.dtype], scaled_activations=True,
         )
-        layer.pack(weight.to(self.device), scales.to(self.device), zeros=None, bias=bias)
+        layer.pack(weight.to(self.device), scales.to(self.device), zeros=None, bias=bias, packed=packed)
         layer.W_group_mode = 0
         layer.channel_scale_mode = 2 if self.post_scale else 4
         return layer
@@ -368,10 +461,27 @@ class A8W8_MXFP_dynamic:
         W = linear_layer.weight.data
         bias = linear_layer.bias.clone() if linear_layer.bias is not None else None
         N, K = W.shape
-        W_q, scales = self.quantizer_mx.quantize_mxfp8(W, index=True, mx_fp8_dtype=self.mx_fp8_dtype)
+        if self.W_nbits == 8:
+            W_q, scales = self.quantizer_mx.quantize_mxfp8(W, index=True, mx_fp8_dtype=self.mx_fp8_dtype)
+        else:
+            W_q, scales = self.quantizer_mx.quantize_mxfp4(W, index=True)
         W_q, scales = W_q.view(N, K), scales.view(N, K // 32)
         cleanup_linear(linear_layer, del_orig)
         return self.from_weights(weight=W_q, scales=scales, bias=bias)
+
+
+class A8W8_MXFP_dynamic(A8Wn_MXFP_dynamic):
+    """(reference: gemlite/helper.py:1034-1036)"""
+
+    def __init__(self, device="cuda:0", dtype=None, post_scale=True, fp8=torch.float8_e4m3fn):
+        super().__init__(device=device, dtype=dtype, post_scale=post_scale, fp8=fp8, W_nbits=8)
+
+
+class A8W4_MXFP_dynamic(A8Wn_MXFP_dynamic):
+    """(reference: gemlite/helper.py:1038-1040)"""
+
+    def __init__(self, device="cuda:0", dtype=None, post_scale=True, fp8=torch.float8_e4m3fn):
+        super().__init__(device=device, dtype=dtype, post_scale=post_scale, fp8=fp8, W_nbits=4)
 
 
 class A4W4_MXFP_dynamic:

@@ -44,6 +44,8 @@ extern "C" {
 #define GLA_DT_INT32 6
 #define GLA_DT_INT16 9
 #define GLA_DT_INT64 11
+#define GLA_DT_MXFP16 14 /* fp16 activations x micro-scaled weights (weight-only) */
+#define GLA_DT_MXBF16 15 /* bf16 activations x micro-scaled weights (weight-only) */
 #define GLA_DT_MXFP8 16
 #define GLA_DT_MXFP4 17
 #define GLA_DT_E8M0 19
@@ -155,6 +157,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_MXFP4 5   /* block-scaled FP4 MFMA GEMM */
 #define GLA_FAMILY_GEMM_KBYTES 6  /* MFMA GEMM for 16-bit activations x unpacked 8-bit weight bytes */
 #define GLA_FAMILY_GEMM_MXFP8 7   /* MXFP8 weights x fp8 activations, MFMA GEMM */
+#define GLA_FAMILY_MX_STREAM 8    /* streaming kernel: weight-only MX layers, MXFP8 x MXFP4 */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of

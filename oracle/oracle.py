@@ -345,6 +345,31 @@ def matmul_mxfp8(a_codes, a_scales, b_codes, b_scales):
     return (A @ B.T).astype(np.float32)
 
 
+def matmul_mx_mixed(a, a_kind, a_scales, b_codes, b_kind, b_scales, scales_x=None):
+    """The general form of the reference's micro-scaled matmul: activations of kind `a_kind` in
+    {"float" (fp16/bf16/fp32 values as they are), "e4m3" (bytes), "e2m1" (nibble codes)} with
+    optional e8m0 block scales `a_scales` [M, K/32] (None = unit scales, what the reference passes
+    for weight-only layers and for channel_scale_mode 2), weights of kind `b_kind` in {"e4m3",
+    "e2m1"} [N, K] with e8m0 block scales [N, K/32], and an optional fp32 scale per activation row
+    applied after the K sum (channel_scale_mode 2)
+    (reference: gemlite/triton_kernels/gemm_kernels.py:563-581 operand kinds, :659-664 unit
+    activation scales, :696 tl.dot_scaled, :714-717 per-row scale)."""
+    def decode(v, kind):
+        if kind == "e4m3":
+            return e4m3fn_decode(v).astype(np.float64)
+        if kind == "e2m1":
+            return e2m1_decode(v).astype(np.float64)
+        return np.asarray(v, dtype=np.float64)
+    A = decode(a, a_kind)
+    if a_scales is not None:
+        A = A * np.repeat(e8m0_decode(a_scales), 32, axis=1)
+    B = decode(b_codes, b_kind) * np.repeat(e8m0_decode(b_scales), 32, axis=1)
+    out = A @ B.T
+    if scales_x is not None:
+        out = out * np.asarray(scales_x, dtype=np.float64).reshape(-1, 1)
+    return out.astype(np.float32)
+
+
 def quantize_per_channel(W, to_int8):
     """s = max(amax_row / qmax, 1e-6); W_q = clamp(W / s); int8 rounds half to even
     (torch.round_), fp8 casts (reference: gemlite/helper.py:635-657)."""

@@ -59,7 +59,25 @@ def oracle_forward(layer, x, matmul_x=None, scales_x=None):
     wgm, csm = layer.W_group_mode, layer.channel_scale_mode
     in_dt = layer.input_dtype
     xin = to_np(x).reshape(-1, x.shape[-1])
-    if in_dt == DType.MXFP4:
+    if in_dt in (DType.MXFP16, DType.MXBF16):   # weight-only MX: activations as they are, unit scales
+        sb = layer.scales.detach().cpu().contiguous().numpy()        # [N, K/32]
+        if layer.elements_per_sample == 2:
+            b, kind = orc.unpack_fp4_bytes(layer.W_q.detach().cpu().t().contiguous().numpy()), "e2m1"
+        else:
+            b, kind = layer.W_q.detach().cpu().t().contiguous().view(torch.uint8).numpy(), "e4m3"
+        out = orc.matmul_mx_mixed(xin, "float", None, b, kind, sb)
+    elif in_dt == DType.MXFP8 and layer.elements_per_sample == 2:   # fp8 activations x MXFP4 weights
+        b = orc.unpack_fp4_bytes(layer.W_q.detach().cpu().t().contiguous().numpy())
+        sb = layer.scales.detach().cpu().contiguous().numpy()
+        if csm == 2:
+            if matmul_x is None:
+                matmul_x, scales_x = orc.scale_activations_per_token(xin, False)
+            out = orc.matmul_mx_mixed(matmul_x, "e4m3", None, b, "e2m1", sb, scales_x=scales_x)
+        else:
+            if matmul_x is None:
+                matmul_x, scales_x = orc.scale_activations_mxfp8(xin)
+            out = orc.matmul_mx_mixed(matmul_x, "e4m3", scales_x[: matmul_x.shape[0]], b, "e2m1", sb)
+    elif in_dt == DType.MXFP4:
         if matmul_x is None:
             matmul_x, scales_x = orc.scale_activations_mxfp4(xin)
         a_codes = orc.unpack_fp4_bytes(matmul_x)

@@ -507,3 +507,59 @@ def test_a8w8_mxfp8_block_scaled_both_sides(device):
     assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 4)
     for M in (1, 5, 33, 100, 130, 300):
         check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("W_nbits", [8, 4])
+def test_weight_only_mxfp_layers(device, dtype, W_nbits):
+    """fp16 / bf16 activations x MXFP8 / MXFP4 weights (reference processors A16W8_MXFP / A16W4_MXFP,
+    gemlite/helper.py:384-420), on the reference tests' ragged shapes (N=2032, K=3968 = 124 blocks)."""
+    N, K = 2032, 3968
+    W = gen_x(N, K, torch.bfloat16, seed=51, std=0.03)
+    W[5, 32:64] = 0.0
+    lin = torch.nn.Linear(K, N, bias=True, dtype=dtype)
+    lin.weight.data = W.to(dtype)
+    lin.bias.data = gen_x(1, N, dtype, seed=52).reshape(-1)
+    cls = helper.A16W8_MXFP if W_nbits == 8 else helper.A16W4_MXFP
+    layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
+    want = orc.quantize_mxfp8_weights(to_np(W.to(dtype))) if W_nbits == 8 else orc.quantize_mxfp4_weights(to_np(W.to(dtype)))
+    assert np.array_equal(layer.scales.cpu().numpy(), want[1])
+    for M in (1, 2, 3, 7, 33):
+        check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=["GEMV", "GEMM_SPLITK", "GEMM"])
+    # a one-hot activation row picks out one dequantised weight column exactly
+    x = torch.zeros(1, K, dtype=dtype)
+    x[0, 37] = 1.0
+    layer.bias = None
+    y = layer(x.to(device))
+    torch.cuda.synchronize()
+    y_ref = oracle_forward(layer, x)
+    assert np.array_equal(to_np(y), round_like(y_ref, dtype))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("post_scale", [True, False])
+def test_a8w4_mxfp8_activations_mxfp4_weights(device, post_scale):
+    """MXFP8 activations (per token, or with micro-scales) x MXFP4 weights
+    (reference processor A8W4_MXFP_dynamic, gemlite/helper.py:950-1040)."""
+    N, K = 520, 1056   # 33 blocks: not a multiple of the 128 the matrix-core kernels want
+    W = gen_x(N, K, torch.bfloat16, seed=61, std=0.03)
+    codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+    layer = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=post_scale).from_weights(
+        torch.from_numpy(codes), scales=torch.from_numpy(e8))
+    assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 2 if post_scale else 4)
+    for M in (1, 5, 33, 70):
+        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
+
+
+@pytest.mark.gpu
+def test_mxfp4_with_k_not_a_multiple_of_128_streams(device):
+    """MXFP4 x MXFP4 at K = 96, 160: three and five 32-blocks (the matrix-core kernel needs K % 128 == 0)."""
+    for K in (96, 160):
+        N = 72
+        W = gen_x(N, K, torch.bfloat16, seed=K, std=0.03)
+        codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+        layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_weights(
+            torch.from_numpy(codes), scales=torch.from_numpy(e8))
+        for M in (1, 6, 40):
+            check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])

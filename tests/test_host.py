@@ -406,3 +406,58 @@ def test_mxfp8_processor_packs_like_the_reference():
         assert l.input_dtype == gemlite_amd.DType.MXFP8 and l.scaled_activations and l.elements_per_sample == 1
         assert l.W_q.shape == (256, 64) and l.W_q.stride() == (1, 256) and l.W_q.dtype == torch.float8_e4m3fn
         assert l.scales.shape == (64, 8) and l.scales.stride() == (8, 1) and l.scales.dtype == torch.uint8
+
+
+def test_weight_only_and_mixed_mx_processors():
+    """A16W8_MXFP / A16W4_MXFP keep fp16 / bf16 activations (input and output type MXFP16 / MXBF16,
+    W_group_mode 2, channel_scale_mode 0; reference: gemlite/helper.py:199-237, 384-420);
+    A8W4_MXFP_dynamic is MXFP8 activations x MXFP4 weights (reference: gemlite/helper.py:950-1040).
+    All of them run the streaming MX kernel."""
+    g = torch.Generator().manual_seed(5)
+    N, K = 64, 256
+    W = (torch.randn((N, K), generator=g) * 0.03).to(torch.bfloat16)
+    lin = torch.nn.Linear(K, N, bias=True, dtype=torch.bfloat16)
+    lin.weight.data = W.clone()
+    for cls, nbits, e, wdt in ((gemlite_amd.helper.A16W8_MXFP, 8, 1, torch.float8_e4m3fn),
+                               (gemlite_amd.helper.A16W4_MXFP, 4, 2, torch.uint8)):
+        for dtype, dt in ((torch.float16, DType.MXFP16), (torch.bfloat16, DType.MXBF16)):
+            l = cls(device="cpu", dtype=dtype).from_linear(lin, del_orig=False)
+            assert l.input_dtype == dt and l.output_dtype == dt and not l.scaled_activations
+            assert (l.W_nbits, l.group_size, l.elements_per_sample) == (nbits, 32, e)
+            assert (l.W_group_mode, l.channel_scale_mode) == (2, 0)
+            assert l.W_q.shape == (K // e, N) and l.W_q.stride() == (1, K // e) and l.W_q.dtype == wdt
+            assert l.scales.shape == (N, K // 32) and l.scales.dtype == torch.uint8 and l.scales.stride() == (K // 32, 1)
+            assert l.bias.dtype == dtype
+            assert gemlite_amd.DTYPE_TO_TORCH[l.get_meta_args()[6]] == dtype
+            for M in (1, 5, 100):
+                m = l.get_meta_args()
+                x = torch.zeros(M, K, dtype=dtype)
+                out = torch.zeros(M, N, dtype=dtype)
+                a = _ext.build_matmul_args(
+                    x, l.W_q, l.scales, l.zeros, None, out, W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+                    elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
+                    channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11])
+                assert _ext.matmul_family(a) == "MX_STREAM"
+    # from_weights of pre-quantised codes gives the same layer as from_linear
+    q = gemlite_amd.quant_utils.WeightQuantizerMXFP(compute_dtype=torch.bfloat16, device="cpu")
+    codes, e8 = q.quantize_mxfp4(W, index=True)
+    l4 = gemlite_amd.helper.A16W4_MXFP(device="cpu", dtype=torch.float16).from_weights(codes.view(N, K), e8.view(N, K // 32))
+    l4b = gemlite_amd.helper.A16W4_MXFP(device="cpu", dtype=torch.float16).from_linear(lin, del_orig=False)
+    assert torch.equal(l4.W_q, l4b.W_q) and torch.equal(l4.scales, l4b.scales)
+    # MXFP8 activations x MXFP4 weights
+    for post_scale, csm in ((True, 2), (False, 4)):
+        l = gemlite_amd.helper.A8W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16, post_scale=post_scale).from_linear(
+            lin, del_orig=False)
+        assert l.input_dtype == DType.MXFP8 and l.scaled_activations and (l.W_nbits, l.elements_per_sample) == (4, 2)
+        assert (l.W_group_mode, l.channel_scale_mode) == (0, csm)
+        for M in (1, 64):
+            xq = torch.zeros(M, K, dtype=torch.float8_e4m3fn)
+            sx = torch.ones(M, 1) if post_scale else torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
+            assert _family(l, M, None, scales_x=sx, x=xq) == "MX_STREAM"
+    # MXFP4 x MXFP4 whose K is a multiple of 32 but not of 128 streams too (the matrix-core kernel wants 128)
+    K2 = 96
+    codes = torch.randint(0, 16, (N, K2), generator=g).to(torch.uint8)
+    e8 = torch.randint(110, 130, (N, K2 // 32), generator=g).to(torch.uint8)
+    lm = gemlite_amd.helper.A4W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16).from_weights(codes, scales=e8)
+    assert _family(lm, 3, None, scales_x=torch.full((32, K2 // 32), 127, dtype=torch.uint8),
+                   x=torch.zeros(3, K2 // 2, dtype=torch.uint8)) == "MX_STREAM"

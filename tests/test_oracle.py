@@ -444,3 +444,33 @@ def test_matmul_mxfp8_block_scaled_closed_form():
                 sl = slice(32 * blk, 32 * blk + 32)
                 want[m, n] += 2.0 ** (int(sa[m, blk]) - 127) * 2.0 ** (int(sb[n, blk]) - 127) * (A[m, sl] @ B[n, sl])
     assert np.allclose(orc.matmul_mxfp8(a, sa, b, sb), want, rtol=1e-6)
+
+
+def test_matmul_mx_mixed_reduces_to_the_pinned_forms():
+    """The general micro-scaled matmul agrees with the e2m1 x e2m1 and e4m3 x e4m3 forms pinned above,
+    is a plain matmul for float activations and unit weight scales, scales one block's contribution
+    by two when that block's weight scale goes up by one, and its per-row scale is a row scaling."""
+    rng = np.random.default_rng(16)
+    M, N, K = 3, 5, 96
+    a4 = rng.integers(0, 16, size=(M, K), dtype=np.uint8)
+    b4 = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    sa = rng.integers(120, 131, size=(M, K // 32), dtype=np.uint8)
+    sb = rng.integers(120, 131, size=(N, K // 32), dtype=np.uint8)
+    assert np.array_equal(orc.matmul_mx_mixed(a4, "e2m1", sa, b4, "e2m1", sb), orc.matmul_mx(a4, sa, b4, sb))
+    a8 = rng.integers(0, 0x7F, size=(M, K), dtype=np.uint8)   # below the NaN code
+    b8 = rng.integers(0, 0x7F, size=(N, K), dtype=np.uint8)
+    assert np.array_equal(orc.matmul_mx_mixed(a8, "e4m3", sa, b8, "e4m3", sb), orc.matmul_mxfp8(a8, sa, b8, sb))
+    rows = rng.uniform(0.5, 2.0, size=(M, 1)).astype(np.float32)
+    assert np.array_equal(orc.matmul_mx_mixed(a8, "e4m3", None, b8, "e4m3", sb, scales_x=rows),
+                          orc.matmul_mxfp8_weights(orc.e4m3fn_decode(a8), rows, b8, sb))
+    # float activations, unit scales: a plain matmul against the decoded codes (small integers / halves: exact)
+    x = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    unit = np.full((N, K // 32), 127, dtype=np.uint8)
+    assert np.array_equal(orc.matmul_mx_mixed(x, "float", None, b4, "e2m1", unit),
+                          (x.astype(np.float64) @ orc.e2m1_decode(b4).astype(np.float64).T).astype(np.float32))
+    # mixed kinds: fp8 activations x fp4 weights; bumping block 1 of the weight scales doubles that block
+    base = orc.matmul_mx_mixed(a8, "e4m3", None, b4, "e2m1", unit).astype(np.float64)
+    up = unit.copy()
+    up[:, 1] = 128
+    blk = orc.e4m3fn_decode(a8[:, 32:64]).astype(np.float64) @ orc.e2m1_decode(b4[:, 32:64]).astype(np.float64).T
+    assert np.array_equal(orc.matmul_mx_mixed(a8, "e4m3", None, b4, "e2m1", up), (base + blk).astype(np.float32))
