@@ -11,9 +11,10 @@
 //  {fp16, bf16, e4m3, e2m1}, b_dtype in {e4m3, e2m1}, unit activation scales unless
 //  channel_scale_mode is 4, and the per-row activation scale of channel_scale_mode 2 at :714-717.)
 //
-// One wave owns one output column n: lane l takes the 32-blocks l, l+64, ... of weight row n
-// (16 or 32 contiguous bytes per block, so a wave reads 1-2 KiB of consecutive weight bytes per
-// step) and multiplies them with the same blocks of up to four activation rows.  Codes become
+// One wave owns four output columns: lane l takes the 32-blocks l, l+64, ... of their weight rows
+// (16 or 32 contiguous bytes per block and row, so a wave reads 1-2 KiB of consecutive bytes of
+// each row per step) and multiplies them with the same blocks of up to eight activation rows, an
+// activation block being loaded once for the four columns.  Codes become
 // fp16 (bf16 for bf16 activations) pairs with the conversion instructions of gfx950 — exact, both
 // code sets are subsets of either type — and pairs are multiplied and summed in fp32 by the packed
 // dot instruction; the block's partial sum is then scaled once by the product of its two block
@@ -22,7 +23,7 @@
 // The combinations that have a matrix-core kernel (MXFP4 x MXFP4, fp8 x MXFP8) do not come here;
 // this kernel is the decode path of the weight-only MX layers and the path at any batch size for
 // MXFP8 activations x MXFP4 weights and for weight-only MX layers (not tuned above a few rows:
-// every group of four activation rows streams the weights again).
+// every group of eight activation rows streams the weights again).
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -113,7 +114,8 @@ __device__ __forceinline__ void block_from_16bit(const uint8_t* p, typename Pair
     }
 }
 
-template <int AK, int BK, int RM>
+// NC output columns per wave, RM activation rows per workgroup row.
+template <int AK, int BK, int RM, int NC>
 __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
     constexpr bool BF = (AK == A_BF16);
     using pair_t = typename Pair<BF>::type;
@@ -121,20 +123,34 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
     constexpr int kBBytes = BK == B_FP4 ? 16 : 32;
 
     const int lane = threadIdx.x & 63;
-    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * NC;
     const int m0 = blockIdx.y * RM;
-    if (n >= a.N) return;  // whole waves leave; no barrier follows
+    if (n0 >= a.N) return;  // whole waves leave; no barrier follows
 
-    const uint8_t* wrow = a.w + (int64_t)n * a.wsn_bytes;
-    float acc[RM];
+    // columns past N repeat the last one (loaded, never stored)
+    const uint8_t* wrow[NC];
+    const uint8_t* srow[NC];
 #pragma unroll
-    for (int r = 0; r < RM; ++r) acc[r] = 0.0f;
+    for (int c = 0; c < NC; ++c) {
+        const int n = n0 + c < a.N ? n0 + c : a.N - 1;
+        wrow[c] = a.w + (int64_t)n * a.wsn_bytes;
+        srow[c] = a.scales + (int64_t)n * a.msn;
+    }
+    float acc[RM][NC];
+#pragma unroll
+    for (int r = 0; r < RM; ++r)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[r][c] = 0.0f;
 
     for (int blk = lane; blk < a.KB; blk += 64) {
-        pair_t wv[16];
-        if constexpr (BK == B_FP4) block_from_fp4<BF>(wrow + (int64_t)blk * kBBytes, wv);
-        else block_from_fp8<BF>(wrow + (int64_t)blk * kBBytes, wv);
-        const float sw = e8m0_to_float(a.scales[(int64_t)n * a.msn + (int64_t)blk * a.msg]);
+        pair_t wv[NC][16];
+        float sw[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            if constexpr (BK == B_FP4) block_from_fp4<BF>(wrow[c] + (int64_t)blk * kBBytes, wv[c]);
+            else block_from_fp8<BF>(wrow[c] + (int64_t)blk * kBBytes, wv[c]);
+            sw[c] = e8m0_to_float(srow[c][(int64_t)blk * a.msg]);
+        }
 #pragma unroll
         for (int r = 0; r < RM; ++r) {
             const int m = m0 + r;
@@ -144,29 +160,35 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
                 if constexpr (AK == A_FP4) block_from_fp4<BF>(xp, xv);
                 else if constexpr (AK == A_FP8) block_from_fp8<BF>(xp, xv);
                 else block_from_16bit<BF>(xp, xv);
-                float p0 = 0.0f, p1 = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; j += 2) {
-                    p0 = dot2<BF>(xv[j], wv[j], p0);
-                    p1 = dot2<BF>(xv[j + 1], wv[j + 1], p1);
-                }
-                float s = sw;
+                float sa = 1.0f;
                 if (a.csm == GLA_CSM_MX)
-                    s *= e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)blk * a.sxg]);
-                acc[r] = __builtin_fmaf(p0 + p1, s, acc[r]);
+                    sa = e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)blk * a.sxg]);
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    float p0 = 0.0f, p1 = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 16; j += 2) {
+                        p0 = dot2<BF>(xv[j], wv[c][j], p0);
+                        p1 = dot2<BF>(xv[j + 1], wv[c][j + 1], p1);
+                    }
+                    acc[r][c] = __builtin_fmaf(p0 + p1, sw[c] * sa, acc[r][c]);
+                }
             }
         }
     }
 
 #pragma unroll
     for (int r = 0; r < RM; ++r) {
-        float v = acc[r];
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) v += wave_xor(v, off);
         const int m = m0 + r;
-        if (lane == 0 && m < a.M) {
-            if (a.csm == GLA_CSM_ACTIVATION) v *= ((const float*)a.scales_x)[(int64_t)m * a.sxm];
-            store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, v);
+        float rs = 1.0f;
+        if (a.csm == GLA_CSM_ACTIVATION && m < a.M) rs = ((const float*)a.scales_x)[(int64_t)m * a.sxm];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            float v = acc[r][c];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += wave_xor(v, off);
+            if (lane == 0 && m < a.M && n0 + c < a.N)
+                store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)(n0 + c) * a.osn, v * rs);
         }
     }
 }
@@ -183,11 +205,14 @@ int a_kind(const gla_matmul_args& p) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+constexpr int kCols = 4;  // output columns per wave
+
 template <int AK, int BK>
 void launch_rows(const MxArgs& a, int rm, dim3 grid, hipStream_t s) {
-    if (rm == 1) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 1>), grid, dim3(256), 0, s, a);
-    else if (rm == 2) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 2>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 4>), grid, dim3(256), 0, s, a);
+    if (rm == 1) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 1, kCols>), grid, dim3(256), 0, s, a);
+    else if (rm == 2) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 2, kCols>), grid, dim3(256), 0, s, a);
+    else if (rm == 4) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 4, kCols>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 8, kCols>), grid, dim3(256), 0, s, a);
 }
 
 template <int AK>
@@ -234,9 +259,9 @@ int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream) {
     a.msg = p.meta_stride_g; a.msn = p.meta_stride_n; a.sxm = p.sx_stride_m; a.sxg = p.sx_stride_g;
     a.csm = p.channel_scale_mode;
     a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
-    const int rm = p.M >= 3 ? 4 : p.M;
+    const int rm = p.M >= 5 ? 8 : (p.M >= 3 ? 4 : p.M);
     const int bk = p.elements_per_sample == 2 ? B_FP4 : B_FP8;
-    dim3 grid(ceil_div(p.N, 4), ceil_div(p.M, rm));
+    dim3 grid(ceil_div(p.N, 4 * kCols), ceil_div(p.M, rm));
     switch (ak) {
         case A_F16: launch_b<A_F16>(a, bk, rm, grid, stream); break;
         case A_BF16: launch_b<A_BF16>(a, bk, rm, grid, stream); break;
