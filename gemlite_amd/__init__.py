@@ -35,6 +35,7 @@ from .quant_utils import (
     quantize_weights_per_channel,
     scale_activations_mxfp4,
     scale_activations_mxfp8,
+    scale_activations_per_block,
     scale_activations_per_token,
 )
 

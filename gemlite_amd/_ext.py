@@ -97,6 +97,11 @@ SYMBOLS = {
         [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
          ctypes.c_void_p, ctypes.c_void_p],
     ),
+    "gla_scale_activations_per_block": (
+        ctypes.c_int,
+        [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+         ctypes.c_void_p, ctypes.c_void_p],
+    ),
     "gla_scale_activations_mxfp4": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
@@ -302,6 +307,13 @@ def _check_operand_bounds(a, x, W_q, scales, zeros, scales_x, out, mx):
     check("out", out, need((M, a.out_stride_m), (N, a.out_stride_n)))
     wgm, csm = a.W_group_mode, a.channel_scale_mode
     groups = K // 32 if mx else (K // a.group_size if a.group_size > 0 else 1)
+    if csm == 5:  # 128 x 128 weight blocks, (row, 128) activation blocks
+        kb, nb = (K + 127) // 128, (N + 127) // 128
+        if scales is not None:
+            check("scales", scales, need((kb, a.meta_stride_g), (nb, a.meta_stride_n)))
+        if scales_x is not None:
+            check("scales_x", scales_x, need((M, a.sx_stride_m), (kb, a.sx_stride_g)))
+        return
     if scales is not None:
         if mx or wgm >= 2:
             check("scales", scales, need((groups, a.meta_stride_g), (N, a.meta_stride_n)))
@@ -353,7 +365,7 @@ def matmul_workspace_need(args: MatmulArgs) -> int:
     return int(need)
 
 
-FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM"]
+FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM", "BLOCKQ_STREAM"]
 
 
 def matmul_family(args: MatmulArgs) -> str:
@@ -381,6 +393,19 @@ def scale_activations_per_token(x2d: torch.Tensor, y: torch.Tensor, scales: torc
             _stream_ptr(x2d.device),
         ),
         "gla_scale_activations_per_token",
+    )
+
+
+def scale_activations_per_block(x2d: torch.Tensor, y: torch.Tensor, scales: torch.Tensor):
+    _require_cuda(x2d, y, scales)
+    lib = load_library()
+    M, K = x2d.shape
+    _check(
+        lib.gla_scale_activations_per_block(
+            x2d.data_ptr(), _dt(x2d), x2d.stride(0), M, K, y.data_ptr(), _dt(y), scales.data_ptr(),
+            _stream_ptr(x2d.device),
+        ),
+        "gla_scale_activations_per_block",
     )
 
 

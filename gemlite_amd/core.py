@@ -24,7 +24,8 @@ from .dtypes import (
     TORCH_TO_DTYPE,
     is_mx_dtype,
 )
-from .quant_utils import scale_activations_mxfp4, scale_activations_mxfp8, scale_activations_per_token
+from .quant_utils import (scale_activations_mxfp4, scale_activations_mxfp8, scale_activations_per_block,
+                          scale_activations_per_token)
 
 logger = logging.getLogger(__name__)
 _FILE_LOCK = threading.Lock()
@@ -160,7 +161,9 @@ def forward_functional(
     kernel_input_dtype = input_dtype
     if scaled_activations:
         in_dt = DType(input_dtype)
-        if in_dt in FP8_INT8_DTYPES and channel_scale_mode != 5:
+        if in_dt in FP8_INT8_DTYPES and channel_scale_mode == 5:  # 128 x 128 block quantisation
+            x2d, scales_x = scale_activations_per_block(x2d, w_dtype=DTYPE_TO_TORCH[input_dtype])
+        elif in_dt in FP8_INT8_DTYPES:
             x2d, scales_x = scale_activations_per_token(x2d, w_dtype=DTYPE_TO_TORCH[input_dtype])
         elif in_dt == DType.MXFP4 and channel_scale_mode == 4:
             x2d, scales_x = scale_activations_mxfp4(x2d)

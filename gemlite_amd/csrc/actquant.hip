@@ -290,6 +290,87 @@ int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, 
     return check_hip(hipGetLastError(), "per-token activation quant launch");
 }
 
+// Per (row, 128-value block) dynamic quantisation to int8 / fp8-e4m3: s = max(amax / qmax, 1e-6),
+// y = clamp(x * (1 / s)); int8 rounds floor(y + 0.5) (reference: gemlite/quant_utils.py:2614-2676,
+// the kernel multiplies by the reciprocal of the scale).  Sixteen lanes share a block, eight
+// consecutive values each; a wave covers four consecutive blocks of a row-major [M, K/128] grid.
+template <int XDT, bool TO_INT8>
+__global__ __launch_bounds__(256) void per_block_kernel(const void* __restrict__ x, int64_t xsm, int M, int K,
+                                                        uint8_t* __restrict__ y, float* __restrict__ scales) {
+    const int lane = threadIdx.x & 63;
+    const int bpr = K / 128;
+    const int64_t blk = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 4 + (lane >> 4);
+    const bool live = blk < (int64_t)M * bpr;
+    const int row = live ? (int)(blk / bpr) : 0;
+    const int kb = live ? (int)(blk % bpr) : 0;
+    const int k = kb * 128 + (lane & 15) * 8;
+    const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+    float v[8];
+    decode_raw8<XDT>(load_raw8<XDT>(xrow, k), v);
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
+    const float qmax = TO_INT8 ? 127.0f : 448.0f;
+    const float qmin = TO_INT8 ? -128.0f : -448.0f;
+    const float s = fmaxf(amax / qmax, 1e-6f);
+    const float r = 1.0f / s;
+    if (!live) return;
+    if ((lane & 15) == 0) scales[(int64_t)row * bpr + kb] = s;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = fminf(fmaxf(v[j] * r, qmin), qmax);
+    uint32_t lo = 0, hi = 0;
+    if constexpr (TO_INT8) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            lo |= ((uint32_t)(int)floorf(v[j] + 0.5f) & 0xffu) << (8 * j);
+            hi |= ((uint32_t)(int)floorf(v[4 + j] + 0.5f) & 0xffu) << (8 * j);
+        }
+    } else {
+        lo = f32_to_fp8_pair(v[0], v[1]) | (f32_to_fp8_pair(v[2], v[3]) << 16);
+        hi = f32_to_fp8_pair(v[4], v[5]) | (f32_to_fp8_pair(v[6], v[7]) << 16);
+    }
+    *(uint2*)(y + (int64_t)row * K + k) = make_uint2(lo, hi);
+}
+
+int launch_act_per_block(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
+                         float* scales, hipStream_t stream) {
+    if (x == nullptr || y == nullptr || scales == nullptr || M < 0 || K <= 0) {
+        set_error("scale_activations_per_block: null pointer or bad size");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (y_dtype != GLA_DT_INT8 && y_dtype != GLA_DT_FP8) {
+        set_error("scale_activations_per_block: output type %d not supported (int8 or fp8-e4m3fn)", y_dtype);
+        return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (K % 128 != 0 || x_stride_m % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)y & 7)) {
+        set_error("scale_activations_per_block: K must be a multiple of 128, the row stride of 8, x 16-byte aligned");
+        return GLA_ERR_MISALIGNED_SHAPE;
+    }
+    if (M == 0) return GLA_OK;
+    const int64_t blocks = (int64_t)M * (K / 128);
+    dim3 grid((unsigned)((blocks + 15) / 16)), block(256);
+    const bool i8 = (y_dtype == GLA_DT_INT8);
+#define GLA_PB(XDT)                                                                                         \
+    do {                                                                                                    \
+        if (i8) hipLaunchKernelGGL((per_block_kernel<XDT, true>), grid, block, 0, stream, x, x_stride_m, M, K, \
+                                   (uint8_t*)y, scales);                                                    \
+        else hipLaunchKernelGGL((per_block_kernel<XDT, false>), grid, block, 0, stream, x, x_stride_m, M, K,  \
+                                (uint8_t*)y, scales);                                                       \
+    } while (0)
+    switch (x_dtype) {
+        case GLA_DT_FP16: GLA_PB(GLA_DT_FP16); break;
+        case GLA_DT_BF16: GLA_PB(GLA_DT_BF16); break;
+        case GLA_DT_FP32: GLA_PB(GLA_DT_FP32); break;
+        default:
+            set_error("scale_activations_per_block: input type %d not supported", x_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+#undef GLA_PB
+    return check_hip(hipGetLastError(), "per-block activation quant launch");
+}
+
 static int launch_act_mx(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
                          bool fp8, hipStream_t stream);
 

@@ -49,7 +49,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
     return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
 }
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM };
 
 int validate(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -129,6 +129,14 @@ int validate(const gla_matmul_args* p) {
         set_error("matmul: W_group_mode %d out of range", p->W_group_mode);
         return GLA_ERR_UNSUPPORTED_MODE;
     }
+    if (p->channel_scale_mode == GLA_CSM_BLOCK) {
+        if (!blockq_stream_eligible(*p)) {
+            set_error("matmul: channel_scale_mode 5 needs int8 or fp8 operands of one type, both K-contiguous with 16-byte "
+                      "aligned rows, K %% 128 == 0, W_group_mode 0 and fp32 block scales on both sides (K=%d)", p->K);
+            return GLA_ERR_UNSUPPORTED_MODE;
+        }
+        return GLA_OK;
+    }
     if (p->channel_scale_mode < GLA_CSM_NONE || p->channel_scale_mode > GLA_CSM_BOTH) {
         set_error("matmul: channel_scale_mode %d not supported for this input type", p->channel_scale_mode);
         return GLA_ERR_UNSUPPORTED_MODE;
@@ -154,6 +162,7 @@ Family choose(const gla_matmul_args& p, int type) {
     if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
     if (p.input_dtype == GLA_DT_MXFP8) return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;  // validated: one of the two
     if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16) return F_MX_STREAM;
+    if (p.channel_scale_mode == GLA_CSM_BLOCK) return F_BLOCKQ_STREAM;  // validated as eligible
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
     const bool small = type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16;
     if (small) {
@@ -231,6 +240,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_GEMM_KBYTES: return launch_gemm_kbytes(*args, s);
         case F_GEMM_MXFP8: return launch_gemm_mxfp8(*args, s);
         case F_MX_STREAM: return launch_mx_stream(*args, s);
+        case F_BLOCKQ_STREAM: return launch_blockq_stream(*args, s);
         default: return launch_generic(*args, s);
     }
 }
@@ -238,6 +248,11 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
 int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y,
                                     int y_dtype, float* scales, void* stream) {
     return launch_act_per_token(x, x_dtype, x_stride_m, M, K, y, y_dtype, scales, (hipStream_t)stream);
+}
+
+int gla_scale_activations_per_block(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y,
+                                    int y_dtype, float* scales, void* stream) {
+    return launch_act_per_block(x, x_dtype, x_stride_m, M, K, y, y_dtype, scales, (hipStream_t)stream);
 }
 
 int gla_scale_activations_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y,

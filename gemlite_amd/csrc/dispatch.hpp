@@ -43,8 +43,14 @@ int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p);
 bool mx_stream_eligible(const gla_matmul_args& p);
 int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream);
 
+// ---- streaming kernel for 128 x 128 block-quantised int8 / fp8 (blockq_stream.hip)
+bool blockq_stream_eligible(const gla_matmul_args& p);
+int launch_blockq_stream(const gla_matmul_args& p, hipStream_t stream);
+
 // ---- activation quantisation (actquant.hip) and bit packing (bitpack.hip) --
 int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
+                         float* scales, hipStream_t stream);
+int launch_act_per_block(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y, int y_dtype,
                          float* scales, hipStream_t stream);
 int launch_act_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, uint8_t* y, uint8_t* scales,
                      hipStream_t stream);

@@ -9,7 +9,7 @@ import torch
 
 from .core import GemLiteLinear
 from .dtypes import DType, TORCH_TO_DTYPE
-from .quant_utils import WeightQuantizerMXFP, quantize_weights_per_channel
+from .quant_utils import BLOCK_QUANT_SIZE, WeightQuantizerMXFP, quantize_weights_per_channel
 
 
 def cleanup_linear(linear_layer, del_orig=True):
@@ -296,13 +296,64 @@ class A8W8_dynamic:
     """Per-token dynamic activations x per-channel 8-bit weights, fp32 scales on both
     sides applied after the K sum (reference: gemlite/helper.py:509-691)."""
 
-    def __init__(self, device="cuda:0", dtype=None, fp8=False, fp32_scale=True):
+    def __init__(self, device="cuda:0", dtype=None, fp8=False, fp32_scale=True, block_quant=False):
         self.device = device
         self.dtype = dtype
         self.fp8 = fp8
         self.fp32_scale = fp32_scale
+        self.block_quant = block_quant
+
+    def _from_weights_block_quant(self, weight, bias=None, scales=None):
+        """128 x 128 block quantisation of the weights + one activation scale per (row, 128 values):
+        ``channel_scale_mode`` 5.  With ``scales`` ([ceil(N/128), ceil(K/128)] fp32) the weight is
+        taken as already quantised; otherwise it is quantised here per block
+        (reference: gemlite/helper.py:517-617)."""
+        B = BLOCK_QUANT_SIZE
+        w_dtype = self.fp8 if self.fp8 else torch.int8
+        input_dtype = TORCH_TO_DTYPE[w_dtype]
+        info = torch.finfo(w_dtype) if w_dtype.is_floating_point else torch.iinfo(w_dtype)
+        min_val, max_val = info.min, info.max
+        out_features, in_features = weight.shape
+        if scales is not None:
+            assert weight.dtype == w_dtype, f"Pre-quantized weight must be {w_dtype}, got {weight.dtype}"
+            want = ((out_features + B - 1) // B, (in_features + B - 1) // B)
+            assert tuple(scales.shape) == want, f"Pre-quantized scales must have shape {want}, got {tuple(scales.shape)}"
+            W_q = weight.contiguous().to(device=self.device)
+            scales = scales.to(device=self.device, dtype=torch.float32)
+            dtype = self.dtype if self.dtype is not None else torch.bfloat16
+        else:
+            dtype = weight.dtype if self.dtype is None else self.dtype
+            assert dtype in (torch.float16, torch.bfloat16, torch.float32), "Invalid weight dtype, should be floating point."
+            in_pad, out_pad = (in_features + B - 1) // B * B, (out_features + B - 1) // B * B
+            w = weight.to(dtype=torch.float32, device=self.device)
+            if in_pad != in_features or out_pad != out_features:
+                w = torch.nn.functional.pad(w, (0, in_pad - in_features, 0, out_pad - out_features))
+            w = w.view(out_pad // B, B, in_pad // B, B)
+            scales = (w.abs().amax(dim=(1, 3)) / max_val).clamp_(min=1e-6)
+            W_q = (w / scales[:, None, :, None]).clamp_(min=min_val, max=max_val)
+            W_q = W_q.to(w_dtype) if w_dtype.is_floating_point else W_q.round_().to(w_dtype)
+            W_q = W_q.view(out_pad, in_pad)[:out_features, :in_features].contiguous()
+        bias = bias.to(device=self.device, dtype=dtype) if bias is not None else None
+        layer = GemLiteLinear(
+            8, group_size=in_features, in_features=in_features, out_features=out_features,
+            input_dtype=input_dtype, output_dtype=TORCH_TO_DTYPE[dtype], acc_dtype=DType.FP32,
+            scaled_activations=True,
+        )
+        # pack() lays out the weights; the block scales replace its per-channel placeholder
+        layer.pack(W_q, torch.ones((out_features, 1), dtype=torch.float32, device=W_q.device), zeros=None, bias=bias)
+        layer._set_param("scales", scales.t().contiguous())   # [K/128, N/128]
+        layer.meta_dtype = DType.FP32
+        layer.W_group_mode, layer.channel_scale_mode = 0, 5
+        layer._set_param("metadata", torch.tensor(layer.get_meta_args(), device=W_q.device, dtype=torch.int32))
+        return layer
 
     def from_weights(self, weight, bias=None, scales=None):
+        if isinstance(weight, torch.nn.Parameter):
+            weight = weight.data
+        if isinstance(bias, torch.nn.Parameter):
+            bias = bias.data
+        if self.block_quant:
+            return self._from_weights_block_quant(weight, bias=bias, scales=scales)
         w_dtype = self.fp8 if self.fp8 else torch.int8
         input_dtype = TORCH_TO_DTYPE[w_dtype]
         out_features, in_features = weight.shape
@@ -329,13 +380,13 @@ class A8W8_dynamic:
 
 
 class A8W8_INT8_dynamic(A8W8_dynamic):
-    def __init__(self, device="cuda:0", dtype=None):
-        super().__init__(device=device, dtype=dtype, fp8=False)
+    def __init__(self, device="cuda:0", dtype=None, block_quant=False):
+        super().__init__(device=device, dtype=dtype, fp8=False, block_quant=block_quant)
 
 
 class A8W8_FP8_dynamic(A8W8_dynamic):
-    def __init__(self, device="cuda:0", dtype=None):
-        super().__init__(device=device, dtype=dtype, fp8=torch.float8_e4m3fn)
+    def __init__(self, device="cuda:0", dtype=None, fp8=torch.float8_e4m3fn, block_quant=False):
+        super().__init__(device=device, dtype=dtype, fp8=fp8, block_quant=block_quant)
 
 
 A8W8_int8_dynamic, A8W8_fp8_dynamic = A8W8_INT8_dynamic, A8W8_FP8_dynamic

@@ -46,6 +46,29 @@ def scale_activations_per_token(tensor: Tensor, w_dtype: torch.dtype, fp32_scale
     return y.view(x_shape), scales
 
 
+BLOCK_QUANT_SIZE = 128  # (reference: gemlite/triton_kernels/config.py:12)
+
+
+def scale_activations_per_block(tensor: Tensor, w_dtype: torch.dtype, block_size: int = BLOCK_QUANT_SIZE) -> Tuple[Tensor, Tensor]:
+    """Dynamic quantisation to int8 or fp8-e4m3fn with one fp32 scale per (row, ``block_size``
+    consecutive values).  Returns ``(y, scales)`` with ``y`` shaped like the input and ``scales``
+    ``[M, K / block_size]`` fp32 (reference: gemlite/quant_utils.py:2654-2676)."""
+    if w_dtype not in (torch.int8, torch.float8_e4m3fn):
+        raise NotImplementedError(f"per-block activation quantisation to {w_dtype} is not supported")
+    if block_size != BLOCK_QUANT_SIZE:
+        raise NotImplementedError(f"only blocks of {BLOCK_QUANT_SIZE} values are supported")
+    x_shape = tensor.shape
+    x2d = tensor.reshape(-1, x_shape[-1])
+    if x2d.stride(-1) != 1:
+        x2d = x2d.contiguous()
+    M, K = x2d.shape
+    assert K % block_size == 0, "K must be divisible by block_size for per-block activation quantization."
+    y = torch.empty((M, K), dtype=w_dtype, device=tensor.device)
+    scales = torch.empty((M, K // block_size), dtype=torch.float32, device=tensor.device)
+    _ext.scale_activations_per_block(x2d, y, scales)
+    return y.view(x_shape), scales
+
+
 def scale_activations_mxfp8(tensor: Tensor, w_dtype: torch.dtype = torch.float8_e4m3fn) -> Tuple[Tensor, Tensor]:
     """MXFP8 dynamic quantisation: ``([M, K] e4m3fn codes, [ceil32(M), K/32] uint8 e8m0)``
     (reference: gemlite/quant_utils.py:1025-1127)."""
@@ -84,7 +107,6 @@ def _not_built(name):
     return fn
 
 
-scale_activations_per_block = _not_built("scale_activations_per_block")
 scale_activations_nvfp4 = _not_built("scale_activations_nvfp4")
 
 

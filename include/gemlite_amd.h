@@ -73,6 +73,8 @@ extern "C" {
 #define GLA_CSM_ACTIVATION 2 /* out *= scales_x[m]                     */
 #define GLA_CSM_BOTH 3       /* out *= scales_x[m] * scales[n]         */
 #define GLA_CSM_MX 4         /* per-32 e8m0 micro-scales on both sides */
+#define GLA_CSM_BLOCK 5      /* fp32 scales per 128 x 128 weight block and per (row, 128) of x;
+                                scales: [K/128, ceil(N/128)], scales_x: [M, K/128] */
 
 /*
  * Arguments of one quantized matmul  out[M,N] = x[M,K] * dequant(w)[K,N].
@@ -158,6 +160,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_KBYTES 6  /* MFMA GEMM for 16-bit activations x unpacked 8-bit weight bytes */
 #define GLA_FAMILY_GEMM_MXFP8 7   /* MXFP8 weights x fp8 activations, MFMA GEMM */
 #define GLA_FAMILY_MX_STREAM 8    /* streaming kernel: weight-only MX layers, MXFP8 x MXFP4 */
+#define GLA_FAMILY_BLOCKQ_STREAM 9 /* streaming kernel: 128 x 128 block-quantised int8 / fp8 */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of
@@ -203,6 +206,14 @@ int gla_scale_activations_mxfp4(const void* x, int x_dtype, int64_t x_stride_m, 
  * are set to 127.  (reference: gemlite/quant_utils.py:1025-1127, exponent trick :697-705) */
 int gla_scale_activations_mxfp8(const void* x, int x_dtype, int64_t x_stride_m, int M, int K,
                                 uint8_t* y, uint8_t* scales, void* stream);
+
+/* Per-block dynamic activation quantisation for channel_scale_mode 5: one fp32
+ * scale max(amax / qmax, 1e-6) per (row, 128 consecutive k), y = clamp(x * (1 / scale))
+ * as int8 (rounded floor(v + 0.5)) or fp8-e4m3fn (nearest even).  y: [M, K] bytes
+ * contiguous; scales: [M, K/128] fp32 contiguous.  K must be a multiple of 128.
+ * (reference: gemlite/quant_utils.py:2614-2676) */
+int gla_scale_activations_per_block(const void* x, int x_dtype, int64_t x_stride_m, int M, int K,
+                                    void* y, int y_dtype, float* scales, void* stream);
 
 /* Pack rows x cols 8-bit codes into words of packing_bitwidth bits along the
  * column axis; out is [rows, cols/e] contiguous

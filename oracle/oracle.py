@@ -370,6 +370,58 @@ def matmul_mx_mixed(a, a_kind, a_scales, b_codes, b_kind, b_scales, scales_x=Non
     return out.astype(np.float32)
 
 
+def scale_activations_per_block(x, to_int8, block=128):
+    """One fp32 scale per (row, `block` values): s = max(amax / qmax, 1e-6); y = clamp(x * (1 / s));
+    int8: floor(y + 0.5) (the rounding the reference uses on AMD GPUs), fp8: e4m3fn cast
+    (reference: gemlite/quant_utils.py:2614-2676, :289-296).  Returns (codes [M, K], scales [M, K/block])."""
+    x = np.asarray(x, dtype=np.float32)
+    M, K = x.shape
+    qmax = np.float32(127.0 if to_int8 else 448.0)
+    qmin = np.float32(-128.0 if to_int8 else -448.0)
+    t = x.reshape(M, K // block, block)
+    s = np.maximum(np.abs(t).max(axis=2).astype(np.float32) / qmax, np.float32(1e-6)).astype(np.float32)
+    r = (np.float32(1.0) / s).astype(np.float32)
+    y = np.clip((t * r[:, :, None]).astype(np.float32), qmin, qmax)
+    if to_int8:
+        codes = np.floor(y + np.float32(0.5)).astype(np.int8)
+    else:
+        codes = e4m3fn_encode(y)
+    return codes.reshape(M, K), s
+
+
+def quantize_block_weights(W, to_int8, block=128):
+    """One fp32 scale per block x block tile of the [N, K] weight (edges padded with zeros):
+    s = max(amax / qmax, 1e-6); codes = clamp(W / s), int8 rounded half to even (torch.round), fp8
+    e4m3fn cast (reference: gemlite/helper.py:556-580).  Returns (codes [N, K], scales [ceil(N/b), ceil(K/b)])."""
+    W = np.asarray(W, dtype=np.float32)
+    N, K = W.shape
+    Np, Kp = -(-N // block) * block, -(-K // block) * block
+    Wp = np.zeros((Np, Kp), dtype=np.float32)
+    Wp[:N, :K] = W
+    t = Wp.reshape(Np // block, block, Kp // block, block)
+    qmax = np.float32(127.0 if to_int8 else 448.0)
+    qmin = np.float32(-128.0 if to_int8 else -448.0)
+    s = np.maximum(np.abs(t).max(axis=(1, 3)).astype(np.float32) / qmax, np.float32(1e-6)).astype(np.float32)
+    y = np.clip((t / s[:, None, :, None]).astype(np.float32), qmin, qmax)
+    if to_int8:
+        codes = np.rint(y).astype(np.int8)
+    else:
+        codes = e4m3fn_encode(y)
+    return codes.reshape(Np, Kp)[:N, :K].copy(), s
+
+
+def matmul_block_quant(a, scales_a, b, scales_b, block=128):
+    """out[m, n] = sum_kb (sum_{k in kb} a[m, k] b[n, k]) * scales_a[m, kb] * scales_b[n // block, kb]
+    with a, b the decoded code values (reference: gemlite/triton_kernels/gemm_kernels.py:441-450)."""
+    A = np.asarray(a, dtype=np.float64)
+    B = np.asarray(b, dtype=np.float64)
+    M, K = A.shape
+    N = B.shape[0]
+    sa = np.repeat(np.asarray(scales_a, dtype=np.float64), block, axis=1)[:, :K]
+    sb = np.repeat(np.repeat(np.asarray(scales_b, dtype=np.float64), block, axis=0)[:N], block, axis=1)[:, :K]
+    return ((A * sa) @ (B * sb).T).astype(np.float32)
+
+
 def quantize_per_channel(W, to_int8):
     """s = max(amax_row / qmax, 1e-6); W_q = clamp(W / s); int8 rounds half to even
     (torch.round_), fp8 casts (reference: gemlite/helper.py:635-657)."""

@@ -59,7 +59,15 @@ def oracle_forward(layer, x, matmul_x=None, scales_x=None):
     wgm, csm = layer.W_group_mode, layer.channel_scale_mode
     in_dt = layer.input_dtype
     xin = to_np(x).reshape(-1, x.shape[-1])
-    if in_dt in (DType.MXFP16, DType.MXBF16):   # weight-only MX: activations as they are, unit scales
+    if csm == 5:   # 128 x 128 block-quantised int8 / fp8
+        to_int8 = in_dt == DType.INT8
+        if matmul_x is None:
+            matmul_x, scales_x = orc.scale_activations_per_block(xin, to_int8)
+        Wb = layer.W_q.detach().cpu().t().contiguous()            # [N, K]
+        b = Wb.numpy() if to_int8 else orc.e4m3fn_decode(Wb.view(torch.uint8).numpy())
+        a = matmul_x if to_int8 else orc.e4m3fn_decode(matmul_x)
+        out = orc.matmul_block_quant(a, scales_x, b, to_np(layer.scales).T)
+    elif in_dt in (DType.MXFP16, DType.MXBF16):   # weight-only MX: activations as they are, unit scales
         sb = layer.scales.detach().cpu().contiguous().numpy()        # [N, K/32]
         if layer.elements_per_sample == 2:
             b, kind = orc.unpack_fp4_bytes(layer.W_q.detach().cpu().t().contiguous().numpy()), "e2m1"

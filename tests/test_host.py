@@ -461,3 +461,31 @@ def test_weight_only_and_mixed_mx_processors():
     lm = gemlite_amd.helper.A4W4_MXFP_dynamic(device="cpu", dtype=torch.bfloat16).from_weights(codes, scales=e8)
     assert _family(lm, 3, None, scales_x=torch.full((32, K2 // 32), 127, dtype=torch.uint8),
                    x=torch.zeros(3, K2 // 2, dtype=torch.uint8)) == "MX_STREAM"
+
+
+def test_block_quant_processor_packs_like_the_reference():
+    """A8W8 with block_quant=True: W_group_mode 0, channel_scale_mode 5, fp32 block scales stored
+    [K/128, N/128], accumulator type fp32, codes and scales equal to the oracle's per-block quantiser
+    (reference: gemlite/helper.py:517-617); pre-quantised weights are taken as they are."""
+    from oracle import oracle as orc
+    g = torch.Generator().manual_seed(9)
+    N, K = 200, 384
+    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    for proc, to_int8, wdt, in_dt in ((gemlite_amd.helper.A8W8_INT8_dynamic, True, torch.int8, DType.INT8),
+                                      (gemlite_amd.helper.A8W8_FP8_dynamic, False, torch.float8_e4m3fn, DType.FP8)):
+        l = proc(device="cpu", block_quant=True).from_weights(W)
+        assert (l.W_group_mode, l.channel_scale_mode) == (0, 5) and l.scaled_activations
+        assert l.input_dtype == in_dt and l.acc_dtype == DType.FP32 and l.meta_dtype == DType.FP32
+        assert l.W_q.shape == (K, N) and l.W_q.stride() == (1, K) and l.W_q.dtype == wdt
+        assert l.scales.shape == (3, 2) and l.scales.dtype == torch.float32 and l.scales.is_contiguous()
+        assert [int(v) for v in l.metadata.tolist()] == l.get_meta_args()
+        codes, s = orc.quantize_block_weights(W.float().numpy(), to_int8)
+        assert np.array_equal(l.scales.numpy(), s.T)
+        got = l.W_q.t().contiguous()
+        assert np.array_equal(got.numpy() if to_int8 else got.view(torch.uint8).numpy(), codes)
+        l2 = proc(device="cpu", dtype=torch.bfloat16, block_quant=True).from_weights(
+            l.W_q.t().contiguous(), scales=l.scales.t().contiguous())
+        assert torch.equal(l2.W_q.view(torch.uint8), l.W_q.view(torch.uint8)) and torch.equal(l2.scales, l.scales)
+        for M in (1, 7, 300):
+            xq = torch.zeros(M, K, dtype=wdt)
+            assert _family(l, M, None, scales_x=torch.ones(M, K // 128), x=xq) == "BLOCKQ_STREAM"

@@ -474,3 +474,60 @@ def test_matmul_mx_mixed_reduces_to_the_pinned_forms():
     up[:, 1] = 128
     blk = orc.e4m3fn_decode(a8[:, 32:64]).astype(np.float64) @ orc.e2m1_decode(b4[:, 32:64]).astype(np.float64).T
     assert np.array_equal(orc.matmul_mx_mixed(a8, "e4m3", None, b4, "e2m1", up), (base + blk).astype(np.float32))
+
+
+def test_block_quant_closed_forms():
+    """Per-block activation quantiser, 128 x 128 weight quantiser and the block-scaled matmul."""
+    rng = np.random.default_rng(21)
+    M, N, K = 5, 200, 384
+    x = rng.normal(size=(M, K)).astype(np.float32)
+    x[1, 128:256] = 0.0          # an all-zero block takes the floor scale
+    for to_int8, qmax in ((True, 127.0), (False, 448.0)):
+        codes, s = orc.scale_activations_per_block(x, to_int8)
+        assert codes.shape == (M, K) and s.shape == (M, 3) and s.dtype == np.float32
+        amax = np.abs(x.reshape(M, 3, 128)).max(axis=2)
+        assert np.array_equal(s, np.maximum(amax / np.float32(qmax), np.float32(1e-6)).astype(np.float32))
+        assert s[1, 1] == np.float32(1e-6)
+        vals = codes.astype(np.float32) if to_int8 else orc.e4m3fn_decode(codes)
+        back = vals.reshape(M, 3, 128) * s[:, :, None]
+        step = s[:, :, None] * (0.5 + 1e-3 if to_int8 else 1.0)  # int8: half a step; fp8: within 2^-4 relative
+        bound = step if to_int8 else np.maximum(np.abs(x.reshape(M, 3, 128)) * 2.0 ** -4, s[:, :, None] * 2.0 ** -9) * 1.01
+        assert np.all(np.abs(back - x.reshape(M, 3, 128)) <= bound)
+        # each block is the per-token quantiser applied to that block alone, up to x*(1/s) vs x/s
+        c_tok, s_tok = orc.scale_activations_per_token(x[:, :128], to_int8)
+        assert np.array_equal(s_tok[:, 0], s[:, 0])
+        assert np.mean(c_tok != codes[:, :128]) < 0.01
+    # the extreme value of a block maps to the end of the range
+    c8, s8 = orc.scale_activations_per_block(x, True)
+    i = np.abs(x[0, :128]).argmax()
+    assert abs(int(c8[0, i])) == 127
+    # weights: N = 200 is padded to 256; scales [2, 3]; per-block amax; a block of zeros -> 1e-6
+    W = (rng.normal(size=(N, K)) * 0.02).astype(np.float32)
+    W[:128, 256:] = 0.0
+    for to_int8, qmax in ((True, 127.0), (False, 448.0)):
+        codes, s = orc.quantize_block_weights(W, to_int8)
+        assert codes.shape == (N, K) and s.shape == (2, 3) and s[0, 2] == np.float32(1e-6)
+        assert np.isclose(s[1, 0], np.abs(W[128:, :128]).max() / qmax, rtol=1e-6)
+        vals = codes.astype(np.float32) if to_int8 else orc.e4m3fn_decode(codes)
+        deq = vals * np.repeat(np.repeat(s, 128, axis=0)[:N], 128, axis=1)
+        assert np.linalg.norm(deq - W) / np.linalg.norm(W) < (0.01 if to_int8 else 0.04)
+    # int8 rounds half to even on the weight side: 2.5 steps -> 2
+    Wt = np.zeros((128, 128), dtype=np.float32)
+    Wt[0, 0], Wt[0, 1], Wt[0, 2] = 127.0, 2.5, 3.5
+    ct, st = orc.quantize_block_weights(Wt, True)
+    assert st[0, 0] == 1.0 and list(ct[0, :3]) == [127, 2, 4]
+    # matmul: unit scales = plain integer matmul; doubling one activation block scale adds that block once more
+    a = rng.integers(-128, 128, size=(M, K)).astype(np.float32)
+    b = rng.integers(-128, 128, size=(N, K)).astype(np.float32)
+    ones_a, ones_b = np.ones((M, 3), np.float32), np.ones((2, 3), np.float32)
+    ref = a.astype(np.float64) @ b.astype(np.float64).T
+    assert np.array_equal(orc.matmul_block_quant(a, ones_a, b, ones_b), ref.astype(np.float32))
+    sa = ones_a.copy()
+    sa[:, 1] = 2.0
+    extra = a[:, 128:256].astype(np.float64) @ b[:, 128:256].astype(np.float64).T
+    assert np.array_equal(orc.matmul_block_quant(a, sa, b, ones_b), (ref + extra).astype(np.float32))
+    sb = ones_b.copy()
+    sb[1, :] = 0.5   # rows 128.. of the weight
+    want = ref.copy()
+    want[:, 128:] *= 0.5
+    assert np.array_equal(orc.matmul_block_quant(a, ones_a, b, sb), want.astype(np.float32))
