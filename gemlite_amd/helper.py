@@ -575,6 +575,57 @@ class A4W4_MXFP_dynamic:
         return self.from_weights(W_q.view(N, K), scales=scales.view(N, K // 32), bias=bias)
 
 
+class A16W158_INT:
+    """fp16/bf16 activations x ternary weights {-1, 0, 1} stored as 2-bit codes w + 1 with a scalar
+    zero point of 1 and one weight scale applied after the K sum (W_group_mode 1, channel_scale_mode 1)
+    (reference: gemlite/helper.py:1208-1262)."""
+
+    def __init__(self, device="cuda:0", dtype=None, fp32_scale=True):
+        self.device = device
+        self.dtype = dtype
+        self.fp32_scale = fp32_scale
+
+    def _layer(self, weight, weight_scale, bias, input_dtype, scaled_activations, csm):
+        if isinstance(weight, torch.nn.Parameter):
+            weight = weight.data
+        if isinstance(bias, torch.nn.Parameter):
+            bias = bias.data
+        dtype = weight.dtype if self.dtype is None else self.dtype
+        assert dtype in (torch.float16, torch.bfloat16, torch.float32), "Invalid weight.dtype, should be floating point."
+        weight = weight.to(dtype=dtype, device=self.device)
+        W_q = (weight + 1).to(torch.uint8)
+        out_features, in_features = W_q.shape
+        scale = float(weight_scale.item()) if isinstance(weight_scale, torch.Tensor) else float(weight_scale)
+        scales = torch.full((out_features, 1), scale, dtype=torch.float32 if self.fp32_scale else dtype, device=W_q.device)
+        bias = bias.to(device=self.device, dtype=dtype) if bias is not None else None
+        layer = GemLiteLinear(
+            2, group_size=in_features, in_features=in_features, out_features=out_features,
+            input_dtype=TORCH_TO_DTYPE[dtype] if input_dtype is None else input_dtype,
+            output_dtype=TORCH_TO_DTYPE[dtype], scaled_activations=scaled_activations,
+        )
+        layer.pack(W_q, scales=scales, zeros=1, bias=bias)
+        layer.W_group_mode, layer.channel_scale_mode = 1, csm
+        return layer
+
+    def from_weights(self, weight, weight_scale, bias=None):
+        return self._layer(weight, weight_scale, bias, None, False, 1)
+
+    def from_bitlinear(self, linear_layer, del_orig=True):
+        out_layer = self.from_weights(weight=linear_layer.weight, weight_scale=linear_layer.weight_scale,
+                                      bias=linear_layer.bias)
+        cleanup_linear(linear_layer, del_orig)
+        return out_layer
+
+
+class A8W158_INT_dynamic(A16W158_INT):
+    """int8 activations quantised per token x ternary weights, INT8 x INT8 -> INT32 accumulation, both
+    scales applied after the K sum (W_group_mode 1, channel_scale_mode 3)
+    (reference: gemlite/helper.py:1264-1321)."""
+
+    def from_weights(self, weight, weight_scale, bias=None):
+        return self._layer(weight, weight_scale, bias, DType.INT8, True, 3)
+
+
 default_batch_sizes = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096]
 
 

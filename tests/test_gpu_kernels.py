@@ -596,3 +596,31 @@ def test_a8w8_block_quantised(device, to_int8):
     assert np.allclose(layer.scales.cpu().numpy(), s.T, rtol=1e-6, atol=0)
     for M in (1, 2, 3, 8, 21):
         check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_ternary_weight_layers(device, dtype):
+    """A16W158_INT and A8W158_INT_dynamic: weights in {-1, 0, 1} as 2-bit codes with a scalar zero
+    point of 1 (reference: gemlite/helper.py:1208-1321).  The int8 x ternary sums are exact integers."""
+    N, K = 520, 2048
+    g = torch.Generator(device="cpu").manual_seed(3)
+    W = torch.randint(-1, 2, (N, K), generator=g).to(dtype)
+    layer = helper.A16W158_INT(device=device).from_weights(W, torch.tensor(0.037), bias=gen_x(1, N, dtype, seed=5).reshape(-1))
+    assert (layer.W_nbits, layer.W_group_mode, layer.channel_scale_mode) == (2, 1, 1)
+    for M in (1, 3, 16, 70):
+        check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
+    dyn = helper.A8W158_INT_dynamic(device=device).from_weights(W, torch.tensor(0.037))
+    assert (dyn.W_group_mode, dyn.channel_scale_mode, dyn.acc_dtype) == (1, 3, DType.INT32)
+    for M in (1, 9, 70):
+        x = gen_x(M, K, dtype, seed=M)
+        check_layer(dyn, x.to(device), dtype, types=["GEMM_SPLITK", "GEMM"])
+    # exact integer check of the accumulation: unit scales on both sides, int8-valued activations
+    unit = helper.A8W158_INT_dynamic(device=device).from_weights(W, torch.tensor(1.0))
+    unit.output_dtype = DType.FP32
+    xi = torch.randint(-127, 128, (5, K), generator=g).to(dtype)
+    xi[:, 0] = 127.0   # every row's amax is 127, so the activation scale is exactly 1
+    y = unit(xi.to(device))
+    torch.cuda.synchronize()
+    want = xi.double() @ W.double().T
+    assert np.array_equal(to_np(y).astype(np.float64), want.numpy())

@@ -489,3 +489,18 @@ def test_block_quant_processor_packs_like_the_reference():
         for M in (1, 7, 300):
             xq = torch.zeros(M, K, dtype=wdt)
             assert _family(l, M, None, scales_x=torch.ones(M, K // 128), x=xq) == "BLOCKQ_STREAM"
+
+
+def test_ternary_processors_pack_like_the_reference():
+    """(reference: gemlite/helper.py:1208-1321) 2-bit codes w + 1, scalar zero 1, fp32 channel scales."""
+    g = torch.Generator().manual_seed(0)
+    N, K = 256, 1024
+    W = torch.randint(-1, 2, (N, K), generator=g).to(torch.float16)
+    l = gemlite_amd.helper.A16W158_INT(device="cpu").from_weights(W, torch.tensor(0.037))
+    assert (l.W_nbits, l.group_size, l.W_group_mode, l.channel_scale_mode) == (2, K, 1, 1)
+    assert l.zeros.numel() == 1 and int(l.zeros) == 1 and l.scales.dtype == torch.float32 and not l.scaled_activations
+    assert torch.equal(gemlite_amd.unpack_over_cols(l.W_q.t().contiguous(), 2, K, torch.uint8), (W + 1).to(torch.uint8))
+    assert [_family(l, M, torch.float16) for M in (1, 16, 64)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN"]
+    d = gemlite_amd.helper.A8W158_INT_dynamic(device="cpu").from_weights(W, torch.tensor(0.037))
+    assert (d.W_group_mode, d.channel_scale_mode, d.input_dtype, d.acc_dtype) == (1, 3, DType.INT8, DType.INT32)
+    assert d.scaled_activations and d.output_dtype == DType.FP16
