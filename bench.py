@@ -237,6 +237,37 @@ def extra_points(lib, device):
     us = time_us(prepared(layer, xq1, sx1, y1), 50)
     out["gemv_a4w4_mxfp4_M1"] = {"N": N, "K": K, "us": round(us, 1),
                                  "GB/s": round((N * K // 2 + N * K // 32 + K // 2 + N * 2) / us / 1e3, 1)}
+    w_codes, w_scales = layer.W_q.data, layer.scales.data
+    del layer, x, xq, sx, y, xq1, sx1, y1
+
+    # Weight-only MXFP4 (bf16 activations as they are) on the same codes: the streaming MX kernel, M = 1, 2, 4
+    wo = helper.A16W4_MXFP(device=device, dtype=torch.bfloat16).from_packed_weights(
+        w_codes.t(), w_scales.view(torch.float8_e8m0fnu))
+    for M in (1, 2, 4):
+        xm = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+        ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+        us = time_us(prepared(wo, xm, None, ym), 50)
+        out[f"gemv_a16w4_mxfp_M{M}"] = {"N": N, "K": K, "us": round(us, 1),
+                                        "GB/s": round((N * K // 2 + N * K // 32 + M * K * 2 + M * N * 2) / us / 1e3, 1)}
+    out["gemv_a16w4_mxfp_M1"]["note"] = "134 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"
+    del wo, w_codes, w_scales, xm, ym
+
+    # 128 x 128 block-quantised fp8 (channel_scale_mode 5), N = K = 8192: per-block activation quantiser and the
+    # streaming kernel at M = 1
+    M, N, K = 4096, 8192, 8192
+    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
+    layer = helper.A8W8_FP8_dynamic(device=device, block_quant=True).from_weights(W)
+    del W
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    us = time_us(lambda: gemlite_amd.scale_activations_per_block(x, torch.float8_e4m3fn), 20)
+    out["actquant_per_block_fp8"] = {"M": M, "K": K, "us": round(us, 1),
+                                     "GB/s": round((M * K * 3 + M * K // 128 * 4) / us / 1e3, 1)}
+    xq1, sx1 = gemlite_amd.scale_activations_per_block(x[:1].contiguous(), torch.float8_e4m3fn)
+    y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
+    us = time_us(prepared(layer, xq1, sx1, y1), 50)
+    out["gemv_a8w8_fp8_block_quant_M1"] = {"N": N, "K": K, "us": round(us, 1),
+                                           "GB/s": round((N * K + N * K // 16384 * 4 + K + N * 2) / us / 1e3, 1),
+                                           "note": "64 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"}
     return out
 
 

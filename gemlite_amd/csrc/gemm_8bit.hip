@@ -40,9 +40,11 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4 };
+enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6 };
 // kMXFP8T: MXFP8 weights whose activations carry no block scales (their per-token scale is applied in the
 // epilogue), so no registers are spent on activation scale words and the 256-row tile fits
+// kBQF8 / kBQI8: fp8 / int8 with one fp32 scale per 128 x 128 weight block and per (activation row, 128 values):
+// the sum over two stages (128 values) goes to a second, fp32 accumulator scaled by both
 
 constexpr int kRowB8 = 64;  // bytes per LDS row = bytes of K per pipeline stage
 constexpr int kBN = 256;
@@ -87,7 +89,7 @@ __device__ __forceinline__ void wait_vmcnt8() {
 }
 
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
-constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 || mode == kMXFP8 || mode == kMXFP8T ? (bm + kBN) * 4 : 0); }
+constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 || mode == kMXFP8 || mode == kMXFP8T || mode == kBQF8 || mode == kBQI8 ? (bm + kBN) * 4 : 0); }
 
 // WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
 // (A 2-column variant with 4 waves of 128 x 128 and accumulators in AGPRs reads a third less from
@@ -103,9 +105,12 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr int TJ = WNC / 32;      // 32-column MFMA tiles per wave along N
     constexpr bool M8 = MODE == kMXFP8 || MODE == kMXFP8T;
     constexpr bool TOKEN = MODE == kMXFP8T;                 // no activation block scales
-    constexpr bool MX = MODE == kMXFP4 || M8;               // block scales ride along with every stage
-    // MXFP8: a 32-bit scale word of a row covers 128 values = two stages; MXFP4: one stage
-    constexpr int SSH = M8 ? 1 : 0;
+    constexpr bool BQ = MODE == kBQF8 || MODE == kBQI8;     // fp32 block scales, applied by the vector unit
+    constexpr bool F8 = MODE == kFP8 || MODE == kBQF8;      // plain fp8 operands, one 64-byte K-step per stage
+    constexpr bool I8 = MODE == kINT8 || MODE == kBQI8;
+    constexpr bool MX = MODE == kMXFP4 || M8 || BQ;         // block scales ride along with every stage
+    // MXFP8 and the fp32 block scales: a 32-bit scale word of a row covers 128 values = two stages; MXFP4: one stage
+    constexpr int SSH = (M8 || BQ) ? 1 : 0;
     constexpr int NW = kWavesM * WN;
     constexpr int RING = kRing8;
     constexpr int SLOT = slot_bytes8(MODE, BM);
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             } else {
                 int gn = n0 + (q - A_JOBS4) * 64 + lane;
                 if (gn > p.N - 1) gn = p.N - 1;
-                off4[i] = (unsigned)(gn * (int)p.msn);
+                off4[i] = (unsigned)((BQ ? gn / 128 : gn) * (int)p.msn);  // BQ: every column copies its block's word
             }
             // the LDS image keeps room for the activation scales of BM rows whether they are copied or not
             dst4[i] = S_OFF + (is_a4[i] ? q : q - A_JOBS4 + BM / 64) * 256;
@@ -207,8 +212,17 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     };
 
     // ---- accumulators
-    typedef typename std::conditional<MODE == kINT8, int16_t_v, float16_t>::type acc_t;
+    typedef typename std::conditional<I8, int16_t_v, float16_t>::type acc_t;
     acc_t acc[TI][TJ];
+    float16_t folded[BQ ? TI : 1][BQ ? TJ : 1];  // BQ: the scaled sum over the 128-blocks done so far
+    if constexpr (BQ) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) folded[i][j][e] = 0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -220,8 +234,8 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     const int sw = (r32 >> 2) & 3;  // chunk swizzle of this lane's rows (tile offsets are multiples of 32)
     // the two 16-byte chunks of a 64-byte row this lane feeds to the MFMAs of a stage:
     // fp8 (one K-step of 64 bytes): chunks 2kb, 2kb+1; int8 / fp4 (two K-steps of 32 bytes): chunks kb, 2+kb
-    const int c0 = ((MODE == kFP8 ? 2 * kb : kb) ^ sw) << 4;
-    const int c1 = ((MODE == kFP8 ? 2 * kb + 1 : 2 + kb) ^ sw) << 4;
+    const int c0 = ((F8 ? 2 * kb : kb) ^ sw) << 4;
+    const int c1 = ((F8 ? 2 * kb + 1 : 2 + kb) ^ sw) << 4;
     const int a_row0 = (wm * WM + r32) * kRowB8;
     const int b_row0 = B_OFF + (wn * WNC + r32) * kRowB8;
     const int sa_row0 = S_OFF + (wm * WM + r32) * 4;
@@ -253,7 +267,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             // MXFP4: half-wave kb multiplies blocks kb and 2 + kb of the stage: shift them into bytes 0 and 2.
             // MXFP8: it multiplies with the scale of block kb of the stage, byte 2 par + kb of the word.
             const int q = r - 2 * (TI + TJ) + (TOKEN ? TI : 0);   // TOKEN: weight scale words only
-            const int sh = M8 ? 8 * (2 * par + kb) : 8 * kb;
+            const int sh = BQ ? 0 : (M8 ? 8 * (2 * par + kb) : 8 * kb);  // BQ: the word is the fp32 scale
             if (q < TI) {
                 if constexpr (!TOKEN) fsa[B][q] = *(const unsigned*)(base + sa_row0 + q * 128) >> sh;
             } else {
@@ -281,12 +295,12 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         for (int r = 0; r < NRD; ++r) load_one(slot, buf_tag, r, par);
     };
     // MFMA q of a stage's NM.  fp8: one K-step of 64 bytes per tile pair; int8 / fp4: two K-steps of 32
-    constexpr int NM = TI * TJ * (MODE == kFP8 || M8 ? 1 : 2);
+    constexpr int NM = TI * TJ * (F8 || M8 ? 1 : 2);
     auto multiply_one = [&](int limit, auto buf_tag, auto scale_tag, int q) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;    // fragment buffer
         constexpr int SB = decltype(scale_tag)::value; // scale buffer (MXFP4)
         const int s2 = q / (TI * TJ), i = (q % (TI * TJ)) / TJ, j = q % TJ;
-        if constexpr (MODE == kFP8) {
+        if constexpr (F8) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
         } else if constexpr (TOKEN) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0,
@@ -299,11 +313,11 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         } else {
             // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
             // must not live across control flow)
-            const bool valid = MODE != kINT8 || s2 * 32 < limit;
+            const bool valid = !I8 || s2 * 32 < limit;
             u32x4 af = fa[B][i].c[s2];
             if (!valid) af = u32x4{0, 0, 0, 0};
             const u32x4 bf = fb[B][j].c[s2];
-            if constexpr (MODE == kINT8) {
+            if constexpr (I8) {
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w},
                                                                   int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w}, acc[i][j], 0, 0, 0);
             } else {
@@ -348,6 +362,20 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         load_frags(0, tag0{}, k_first & 1);
     }
 
+    // BQ: tile t = i * TJ + j has summed a whole 128-block (an even and an odd stage; splits start on even
+    // stages, so the odd ones are those multiplied from register buffer 1, whose scale words are the block's):
+    // add it, scaled, to the fp32 result and start the next block from zero
+    auto fold_one = [&](int t) __attribute__((always_inline)) {
+        if constexpr (BQ) {
+            const int i = t / TJ, j = t % TJ;
+            const float sc = __builtin_bit_cast(float, fsa[1][i]) * __builtin_bit_cast(float, fsb[1][j]);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                folded[i][j][e] = __builtin_fmaf((float)acc[i][j][e], sc, folded[i][j][e]);
+                acc[i][j][e] = 0;
+            }
+        }
+    };
     int slot = 0;  // ring slot of the stage being multiplied
     auto step = [&](int k, auto buf_tag) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
@@ -376,8 +404,13 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                 for (int c = q * LPS / NM; c < (q + 1) * LPS / NM; ++c) issue_one(k + RING, slot, c);
 #pragma unroll
                 for (int r = q * NRD / RS; r < (q + 1) * NRD / RS && r < NRD; ++r) load_one(next, other{}, r, (k_first + k + 1) & 1);
+                // a finished tile is folded one slice after its last MFMA, in the shadow of the next one
+                if constexpr (BQ && B == 1) {
+                    if (q > NM - TI * TJ) fold_one(q - (NM - TI * TJ) - 1);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (BQ && B == 1) fold_one(TI * TJ - 1);
         } else {
             const int refill = slot == 0 ? RING - 1 : slot - 1;
             constexpr int H = NM / 2, HS = H / 2, R1 = TI + TJ, R2 = 2 * (TI + TJ);
@@ -409,7 +442,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // 4g .. 4g+3, the four adjacent output columns 8g + 4kb .. + 3, which leave in one store.
     const int n_wave = n0 + wn * WNC + 4 * kb;
     if (p.S > 1) {  // partial tile, raw 32-bit accumulators; the reduction kernel finishes
-        typedef typename std::conditional<MODE == kINT8, int32_t, float>::type raw_t;
+        typedef typename std::conditional<MODE == kINT8, int32_t, float>::type raw_t;  // BQ: the scaled fp32 sums
         typedef raw_t raw4_t __attribute__((ext_vector_type(4)));
         raw_t* part = (raw_t*)p.partials + (size_t)blockIdx.y * p.M * p.N;
         const bool wide = (p.N & 3) == 0;
@@ -423,19 +456,29 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                 for (int g = 0; g < 4; ++g) {
                     const int n = n_wave + j * 32 + 8 * g;
                     raw_t* dst = part + (size_t)m * p.N + n;
+                    raw_t v[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        if constexpr (BQ) v[t] = folded[i][j][4 * g + t];
+                        else v[t] = acc[i][j][4 * g + t];
+                    }
                     if (wide && n + 3 < p.N) {
-                        *(raw4_t*)dst = raw4_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                        *(raw4_t*)dst = raw4_t{v[0], v[1], v[2], v[3]};
                     } else {
 #pragma unroll
                         for (int t = 0; t < 4; ++t)
-                            if (n + t < p.N) dst[t] = acc[i][j][4 * g + t];
+                            if (n + t < p.N) dst[t] = v[t];
                     }
                 }
         }
         return;
     }
     const bool col_scale = !MX && (p.csm & 1);
-    const bool row_scale = MODE != kMXFP4 && (p.csm & 2);
+    const bool row_scale = MODE != kMXFP4 && !BQ && (p.csm & 2);
+    auto value = [&](int i, int j, int e) __attribute__((always_inline)) -> float {
+        if constexpr (BQ) return folded[i][j][e];
+        else return (float)acc[i][j][e];
+    };
     float sb[TJ][16];
 #pragma unroll
     for (int j = 0; j < TJ; ++j)
@@ -467,7 +510,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                         } else {
                             float v[4];
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) v[t] = (float)acc[i][j][4 * g + t] * (sa * sb[j][4 * g + t]);
+                            for (int t = 0; t < 4; ++t) v[t] = value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]);
                             if constexpr (DT == GLA_DT_FP32) {
                                 *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
                             } else {
@@ -487,7 +530,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                         for (int t = 0; t < 4; ++t) {
                             if (n + t >= p.N) continue;
                             if constexpr (DT == GLA_DT_INT32) ((int32_t*)p.out)[o + t] = (int32_t)acc[i][j][4 * g + t];
-                            else store_typed<DT>(p.out, o + t, (float)acc[i][j][4 * g + t] * (sa * sb[j][4 * g + t]));
+                            else store_typed<DT>(p.out, o + t, value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]));
                         }
                     }
                 }
@@ -537,7 +580,7 @@ int launch_bm(const Gemm8Args& a, hipStream_t stream) {
     if (rc == GLA_OK && a.S > 1) {
         const int64_t items = (int64_t)a.M * a.N;
         Gemm8Args f = a;
-        if (MODE == kMXFP4) f.csm = 0;  // block scales were applied inside the MFMAs
+        if (MODE == kMXFP4 || MODE == kBQF8 || MODE == kBQI8) f.csm = 0;  // block scales were applied in the main kernel
         hipLaunchKernelGGL((splitk_finish8_kernel<MODE == kINT8>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
                            stream, f);
         rc = check_hip(hipGetLastError(), "gemm_8bit split-K reduction launch");
@@ -658,10 +701,61 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     return launch_mode<kFP8>(a, g.bm, stream);
 }
 
+static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+// ---- 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5) above 16 rows ----------------
+// (reference: gemlite/triton_kernels/gemm_kernels.py:396-400, :441-450.)  Tiles of 64 or 128 rows: the
+// second accumulator leaves no registers for the 256-row tile.  K splits hold whole 128-blocks (an even
+// number of stages) and their partials are the scaled fp32 sums, which the reduction kernel only adds.
+static Plan8 plan_blockq(const gla_matmul_args& p) {
+    const int cfg = p.tile_config > 0 ? p.tile_config : 0;
+    int bm = cfg % 1000;
+    if (bm != 64 && bm != 128) bm = p.M > 64 ? 128 : 64;
+    Plan8 g = plan8(p.M, p.N, p.K, (cfg / 1000) * 1000 + bm);
+    if (g.S > 1 && (g.sps & 1)) {
+        g.sps += 1;
+        g.S = ceil_div(ceil_div(p.K, kRowB8), g.sps);
+    }
+    return g;
+}
+
+bool gemm_blockq_eligible(const gla_matmul_args& p) {
+    if (!blockq_stream_eligible(p) || p.M <= 16 || p.out_stride_n != 1) return false;
+    if (p.meta_stride_n < 0 || p.meta_stride_g < 0 || p.sx_stride_m < 0 || p.sx_stride_g < 0) return false;
+    if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
+    if ((int64_t)p.M * p.sx_stride_m * 4 >= (1ll << 31) || (int64_t)(p.N / 128 + 1) * p.meta_stride_n * 4 >= (1ll << 31)) return false;
+    return true;
+}
+
+int64_t gemm_blockq_workspace_bytes(const gla_matmul_args& p) {
+    const Plan8 g = plan_blockq(p);
+    return g.S > 1 ? kWsReserved8 + align256((int64_t)g.S * p.M * p.N * 4) : 0;
+}
+
+int launch_gemm_blockq(const gla_matmul_args& p, hipStream_t stream) {
+    if (!gemm_blockq_eligible(p)) {
+        set_error("gemm_blockq: operands not eligible (see blockq_stream; more than 16 rows, unit output column stride)");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    Gemm8Args a;
+    a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.out = p.out;
+    a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
+    // block scales travel with the stages like micro-scales: byte strides per row / per 128-block of K
+    a.scales = p.scales; a.msn = p.meta_stride_n * 4; a.sw_stage = p.meta_stride_g * 4;
+    a.ascales = p.scales_x; a.asxm = p.sx_stride_m * 4; a.sx_stage = p.sx_stride_g * 4;
+    a.scales_x = nullptr; a.sxm = 0; a.csm = 0;  // nothing left for the epilogue
+    a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
+    const Plan8 g = plan_blockq(p);
+    const int rc = attach_plan(p, g, a);
+    if (rc != GLA_OK) return rc;
+    if (p.input_dtype == GLA_DT_INT8)
+        return g.bm == 128 ? launch_bm<kBQI8, 128, 4>(a, stream) : launch_bm<kBQI8, 64, 4>(a, stream);
+    return g.bm == 128 ? launch_bm<kBQF8, 128, 4>(a, stream) : launch_bm<kBQF8, 64, 4>(a, stream);
+}
+
 // MXFP4 scales regrouped by stage pay off once the GEMM itself takes much longer than regrouping
 // the weight scales (a pass over N x K/32 bytes): from the 128-row tile on.
 static bool mx_scales_staged(const gla_matmul_args& p, const Plan8& g) { return g.bm >= 128; }
-static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
 int64_t gemm_8bit_workspace_bytes(const gla_matmul_args& p) {
     const bool mx = p.input_dtype == GLA_DT_MXFP4;

@@ -594,8 +594,26 @@ def test_a8w8_block_quantised(device, to_int8):
     # the one-time weight quantiser is torch code: its fp32 division on the GPU may differ from the CPU's in the
     # last place (the CPU test compares it exactly); the matmul is checked against the layer's own tensors
     assert np.allclose(layer.scales.cpu().numpy(), s.T, rtol=1e-6, atol=0)
-    for M in (1, 2, 3, 8, 21):
+    for M in (1, 2, 3, 8, 16, 21, 64, 100, 130, 300):   # streaming kernel up to 16 rows, MFMA GEMM above
         check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("to_int8", [True, False])
+@pytest.mark.parametrize("K", [2176, 4096])
+def test_a8w8_block_quantised_split_k(device, to_int8, K):
+    """Few output tiles and a long K: the MFMA kernel splits K on whole 128-blocks (K = 2176 is 17
+    blocks, split 9 + 8); block scales that differ a lot from block to block make a misplaced scale visible."""
+    N = 520
+    W = gen_x(N, K, torch.bfloat16, seed=73, std=0.02)
+    W[:, 128:256] *= 16.0
+    W[:, K - 128:] *= 0.125
+    proc = helper.A8W8_INT8_dynamic if to_int8 else helper.A8W8_FP8_dynamic
+    layer = proc(device=device, block_quant=True).from_weights(W)
+    for M in (24, 70, 200):
+        x = gen_x(M, K, torch.bfloat16, seed=M)
+        x[:, 256:384] *= 8.0
+        check_layer(layer, x.to(device), torch.bfloat16, types=["GEMM"])
 
 
 @pytest.mark.gpu
