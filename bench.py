@@ -252,22 +252,27 @@ def extra_points(lib, device):
     out["gemv_a16w4_mxfp_M1"]["note"] = "134 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"
     del wo, w_codes, w_scales, xm, ym
 
-    # 128 x 128 block-quantised fp8 (channel_scale_mode 5), N = K = 8192: per-block activation quantiser and the
-    # streaming kernel at M = 1
+    # 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5), N = K = 8192: per-block activation quantiser,
+    # the MFMA GEMM at M = 4096 and the streaming kernel at M = 1
     M, N, K = 4096, 8192, 8192
     W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
-    layer = helper.A8W8_FP8_dynamic(device=device, block_quant=True).from_weights(W)
-    del W
     x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
-    us = time_us(lambda: gemlite_amd.scale_activations_per_block(x, torch.float8_e4m3fn), 20)
-    out["actquant_per_block_fp8"] = {"M": M, "K": K, "us": round(us, 1),
-                                     "GB/s": round((M * K * 3 + M * K // 128 * 4) / us / 1e3, 1)}
-    xq1, sx1 = gemlite_amd.scale_activations_per_block(x[:1].contiguous(), torch.float8_e4m3fn)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
     y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
-    us = time_us(prepared(layer, xq1, sx1, y1), 50)
-    out["gemv_a8w8_fp8_block_quant_M1"] = {"N": N, "K": K, "us": round(us, 1),
-                                           "GB/s": round((N * K + N * K // 16384 * 4 + K + N * 2) / us / 1e3, 1),
-                                           "note": "64 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"}
+    for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
+        layer = proc(device=device, block_quant=True).from_weights(W)
+        xq, sx = gemlite_amd.scale_activations_per_block(x, wdt)
+        us = time_us(prepared(layer, xq, sx, y), 30)
+        point(f"gemm_a8w8_{name}_block_quant", M, N, K, us, 5000.0, name)
+        us = time_us(lambda: gemlite_amd.scale_activations_per_block(x, wdt), 20)
+        out[f"actquant_per_block_{name}"] = {"M": M, "K": K, "us": round(us, 1),
+                                            "GB/s": round((M * K * 3 + M * K // 128 * 4) / us / 1e3, 1)}
+        xq1, sx1 = gemlite_amd.scale_activations_per_block(x[:1].contiguous(), wdt)
+        us = time_us(prepared(layer, xq1, sx1, y1), 50)
+        out[f"gemv_a8w8_{name}_block_quant_M1"] = {
+            "N": N, "K": K, "us": round(us, 1), "GB/s": round((N * K + N * K // 16384 * 4 + K + N * 2) / us / 1e3, 1),
+            "note": "64 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"}
+        del layer, xq, sx, xq1, sx1
     return out
 
 

@@ -43,7 +43,7 @@ int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p);
 bool mx_stream_eligible(const gla_matmul_args& p);
 int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream);
 
-// ---- 128 x 128 block-quantised int8 / fp8 above 16 rows: MFMA GEMM (gemm_8bit.hip)
+// ---- 128 x 128 block-quantised int8 / fp8 above 4 rows: MFMA GEMM (gemm_8bit.hip)
 bool gemm_blockq_eligible(const gla_matmul_args& p);
 int launch_gemm_blockq(const gla_matmul_args& p, hipStream_t stream);
 int64_t gemm_blockq_workspace_bytes(const gla_matmul_args& p);

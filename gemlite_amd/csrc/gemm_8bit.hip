@@ -300,8 +300,16 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         constexpr int B = decltype(buf_tag)::value;    // fragment buffer
         constexpr int SB = decltype(scale_tag)::value; // scale buffer (MXFP4)
         const int s2 = q / (TI * TJ), i = (q % (TI * TJ)) / TJ, j = q % TJ;
+        // BQ: the first MFMA of a 128-block (even stage = register buffer 0, first K-step) starts from zero
+        // instead of the accumulator, which spares the vector unit clearing it after every fold
+        constexpr bool FRESH_STAGE = BQ && B == 0;
         if constexpr (F8) {
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0, 127, 0, 127);
+            acc_t cin = acc[i][j];
+            if constexpr (FRESH_STAGE) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) cin[e] = 0;
+            }
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, cin, 0, 0, 0, 127, 0, 127);
         } else if constexpr (TOKEN) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0,
                                                                         (int)fsb[SB][j], 0, 127);
@@ -318,8 +326,13 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
             if (!valid) af = u32x4{0, 0, 0, 0};
             const u32x4 bf = fb[B][j].c[s2];
             if constexpr (I8) {
+                acc_t cin = acc[i][j];
+                if (FRESH_STAGE && s2 == 0) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) cin[e] = 0;
+                }
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w},
-                                                                  int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w}, acc[i][j], 0, 0, 0);
+                                                                  int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w}, cin, 0, 0, 0);
             } else {
                 // fp4 operands occupy the first four of the eight operand registers; the rest is not read
                 const int4_t a4 = int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w};
@@ -364,16 +377,13 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
 
     // BQ: tile t = i * TJ + j has summed a whole 128-block (an even and an odd stage; splits start on even
     // stages, so the odd ones are those multiplied from register buffer 1, whose scale words are the block's):
-    // add it, scaled, to the fp32 result and start the next block from zero
+    // add it, scaled, to the fp32 result (the next block's first MFMA starts from zero)
     auto fold_one = [&](int t) __attribute__((always_inline)) {
         if constexpr (BQ) {
             const int i = t / TJ, j = t % TJ;
             const float sc = __builtin_bit_cast(float, fsa[1][i]) * __builtin_bit_cast(float, fsb[1][j]);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                folded[i][j][e] = __builtin_fmaf((float)acc[i][j][e], sc, folded[i][j][e]);
-                acc[i][j][e] = 0;
-            }
+            for (int e = 0; e < 16; ++e) folded[i][j][e] = __builtin_fmaf((float)acc[i][j][e], sc, folded[i][j][e]);
         }
     };
     int slot = 0;  // ring slot of the stage being multiplied
@@ -703,7 +713,7 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
 
 static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
-// ---- 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5) above 16 rows ----------------
+// ---- 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5) above 4 rows ----------------
 // (reference: gemlite/triton_kernels/gemm_kernels.py:396-400, :441-450.)  Tiles of 64 or 128 rows: the
 // second accumulator leaves no registers for the 256-row tile.  K splits hold whole 128-blocks (an even
 // number of stages) and their partials are the scaled fp32 sums, which the reduction kernel only adds.
@@ -720,7 +730,7 @@ static Plan8 plan_blockq(const gla_matmul_args& p) {
 }
 
 bool gemm_blockq_eligible(const gla_matmul_args& p) {
-    if (!blockq_stream_eligible(p) || p.M <= 16 || p.out_stride_n != 1) return false;
+    if (!blockq_stream_eligible(p) || p.M <= 4 || p.out_stride_n != 1) return false;
     if (p.meta_stride_n < 0 || p.meta_stride_g < 0 || p.sx_stride_m < 0 || p.sx_stride_g < 0) return false;
     if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
     if ((int64_t)p.M * p.sx_stride_m * 4 >= (1ll << 31) || (int64_t)(p.N / 128 + 1) * p.meta_stride_n * 4 >= (1ll << 31)) return false;
@@ -734,7 +744,7 @@ int64_t gemm_blockq_workspace_bytes(const gla_matmul_args& p) {
 
 int launch_gemm_blockq(const gla_matmul_args& p, hipStream_t stream) {
     if (!gemm_blockq_eligible(p)) {
-        set_error("gemm_blockq: operands not eligible (see blockq_stream; more than 16 rows, unit output column stride)");
+        set_error("gemm_blockq: operands not eligible (see blockq_stream; more than 4 rows, unit output column stride)");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     Gemm8Args a;

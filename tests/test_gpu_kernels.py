@@ -594,7 +594,7 @@ def test_a8w8_block_quantised(device, to_int8):
     # the one-time weight quantiser is torch code: its fp32 division on the GPU may differ from the CPU's in the
     # last place (the CPU test compares it exactly); the matmul is checked against the layer's own tensors
     assert np.allclose(layer.scales.cpu().numpy(), s.T, rtol=1e-6, atol=0)
-    for M in (1, 2, 3, 8, 16, 21, 64, 100, 130, 300):   # streaming kernel up to 16 rows, MFMA GEMM above
+    for M in (1, 2, 3, 4, 5, 8, 16, 21, 64, 100, 130, 300):   # streaming kernel up to 4 rows, MFMA GEMM above
         check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
 
 
