@@ -22,7 +22,8 @@ from .core import (
     get_type_id,
 )
 from .dtypes import DTYPE_TO_TORCH, DType, is_mx_dtype
-from .quant_utils import scale_activations_mxfp4, scale_activations_per_token
+from .quant_utils import (scale_activations_mxfp4, scale_activations_mxfp8, scale_activations_per_block,
+                          scale_activations_per_token)
 
 
 def candidate_configs(family: str, M: int, K: int) -> List[int]:
@@ -41,6 +42,10 @@ def candidate_configs(family: str, M: int, K: int) -> List[int]:
         bms = [64] if M <= 64 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 1024)]
+    if family == "GEMM_BLOCKQ":      # the second accumulator rules out the 256-row tile
+        bms = [64] if M <= 64 else [64, 128]
+        splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
+        return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 1024)]
     return [-1]
 
 
@@ -52,6 +57,12 @@ def _prepare_inputs(layer: GemLiteLinear, M: int, device):
         x = torch.randn((M, layer.in_features), generator=g).to(torch.bfloat16).to(device)
         if in_dt == DType.MXFP4:
             return scale_activations_mxfp4(x)
+        if in_dt == DType.MXFP8:
+            if layer.channel_scale_mode == 4:
+                return scale_activations_mxfp8(x)
+            return scale_activations_per_token(x, w_dtype=torch.float8_e4m3fn)
+        if layer.channel_scale_mode == 5:
+            return scale_activations_per_block(x, w_dtype=DTYPE_TO_TORCH[in_dt.value])
         return scale_activations_per_token(x, w_dtype=DTYPE_TO_TORCH[in_dt.value])
     if layer.compute_dtype == torch.int8:
         return torch.randint(-128, 128, (M, layer.in_features), generator=g, dtype=torch.int32).to(torch.int8).to(device), None

@@ -107,3 +107,44 @@ def test_a16w4_prefill_4096_cubed(device):
     want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], 128)
     err = rel_frob(y[:, cols], want)
     assert err <= FROB_TOL and err <= TIGHT_FP16, err
+
+
+@pytest.mark.parametrize("to_int8", [True, False])
+def test_a8w8_block_quantised_4096x8192x8192(device, to_int8):
+    """128 x 128 block-quantised int8 / fp8 at M = 4096, N = K = 8192 (the matrix-core kernel, 128-row tiles):
+    activation codes and scales bit for bit on a row sample; sampled output columns from exact sums per block."""
+    M, N, K = 4096, 8192, 8192
+    W = gen_x(N, K, torch.bfloat16, seed=21, std=0.02)
+    codes, sw = orc.quantize_block_weights(to_np(W), to_int8)          # [N, K], [N/128, K/128]
+    wdt = torch.int8 if to_int8 else torch.float8_e4m3fn
+    wq = torch.from_numpy(codes) if to_int8 else torch.from_numpy(codes).view(torch.float8_e4m3fn)
+    proc = (helper.A8W8_INT8_dynamic if to_int8 else helper.A8W8_FP8_dynamic)(device=device, dtype=torch.bfloat16, block_quant=True)
+    layer = proc.from_weights(wq, scales=torch.from_numpy(sw))
+    x = gen_x(M, K, torch.bfloat16, seed=22)
+    y = to_np(layer(x.to(device)))
+    xq, sx = gemlite_amd.scale_activations_per_block(x.to(device), wdt)
+    rows = np.arange(0, M, 61)
+    want_q, want_s = orc.scale_activations_per_block(to_np(x)[rows], to_int8)
+    got_q = xq.cpu().numpy()[rows] if to_int8 else xq.view(torch.uint8).cpu().numpy()[rows]
+    assert np.array_equal(got_q, want_q) and np.array_equal(sx.cpu().numpy()[rows], want_s)
+    cols = sample_cols(N, seed=23)
+    a = xq.cpu().numpy() if to_int8 else orc.e4m3fn_decode(xq.view(torch.uint8).cpu().numpy())
+    b = codes[cols] if to_int8 else orc.e4m3fn_decode(codes[cols])
+    sa = np.repeat(sx.cpu().numpy().astype(np.float64), 128, axis=1)
+    sb = np.repeat(sw[cols // 128].astype(np.float64), 128, axis=1)
+    want = (a.astype(np.float64) * sa) @ (b.astype(np.float64) * sb).T
+    assert rel_frob(y[:, cols], want.astype(np.float32)) <= TIGHT_BF16
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_a16w4_mxfp_weight_only_16384_square(device, M):
+    """bf16 activations x MXFP4 weights, N = K = 16384 (the streaming MX kernel)."""
+    N = K = 16384
+    W = gen_x(N, K, torch.bfloat16, seed=9, std=0.02)
+    codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+    layer = helper.A16W4_MXFP(device=device, dtype=torch.bfloat16).from_weights(torch.from_numpy(codes), torch.from_numpy(e8))
+    x = gen_x(M, K, torch.bfloat16, seed=M)
+    y = to_np(layer(x.to(device)))
+    cols = sample_cols(N, seed=M)
+    want = orc.matmul_mx_mixed(to_np(x), "float", None, codes[cols], "e2m1", e8[cols])
+    assert rel_frob(y[:, cols], want) <= TIGHT_BF16
