@@ -49,7 +49,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
     return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
 }
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX };
 
 int validate(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -161,7 +161,8 @@ int validate(const gla_matmul_args* p) {
 Family choose(const gla_matmul_args& p, int type) {
     if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
     if (p.input_dtype == GLA_DT_MXFP8) return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;  // validated: one of the two
-    if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16) return F_MX_STREAM;
+    if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)  // validated as eligible for the streaming kernel
+        return gemm_kbytes_mx_eligible(p) ? F_GEMM_KBYTES_MX : F_MX_STREAM;
     if (p.channel_scale_mode == GLA_CSM_BLOCK)  // validated as eligible for the streaming kernel at least
         return gemm_blockq_eligible(p) ? F_GEMM_BLOCKQ : F_BLOCKQ_STREAM;
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
@@ -224,6 +225,7 @@ int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
         case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(*args);
         case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(*args);
         case F_GEMM_BLOCKQ: return gemm_blockq_workspace_bytes(*args);
+        case F_GEMM_KBYTES_MX: return gemm_kbytes_mx_workspace_bytes(*args);
         default: return 0;
     }
 }
@@ -244,6 +246,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_MX_STREAM: return launch_mx_stream(*args, s);
         case F_BLOCKQ_STREAM: return launch_blockq_stream(*args, s);
         case F_GEMM_BLOCKQ: return launch_gemm_blockq(*args, s);
+        case F_GEMM_KBYTES_MX: return launch_gemm_kbytes_mx(*args, s);
         default: return launch_generic(*args, s);
     }
 }

@@ -46,6 +46,10 @@ constexpr int kRowBb = 64;   // LDS row of the weight tile: 64 bytes
 constexpr int kBNb = 256;
 constexpr int kWavesNb = 4;
 constexpr int64_t kWsReservedB = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
+// Weight kinds beyond the element-type ids: micro-scaled weights of weight-only MX layers, fp8-e4m3 bytes or
+// e2m1 nibble pairs with one e8m0 scale per 32 values along K.  The block scale is applied by the
+// conversion instruction (v_cvt_scalef32_pk_*), so the 16-bit operand is the dequantised weight.
+constexpr int kWMX8 = 100, kWMX4 = 101;
 
 struct GemmKbArgs {
     const uint16_t* x;
@@ -61,6 +65,8 @@ struct GemmKbArgs {
     int tiles_m, tiles_n;
     int S, sps;
     float* partials;
+    const uint8_t* bscales;  // micro-scaled weights: e8m0 block scales [N, K/32], K contiguous
+    int64_t bsn;             // ... bytes from one row's scales to the next
 };
 
 __device__ __forceinline__ void tile_coords_kb(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -118,6 +124,39 @@ __device__ __forceinline__ u32x4b bytes_to_operand(uint32_t d0, uint32_t d1) {
     return o;
 }
 
+// micro-scaled weights: 8 codes (two dwords of fp8, one of fp4) times the block scale 2^(e - 127), whose e8m0
+// byte sits in the exponent field of `scale` (which is all the conversion instruction reads of it)
+template <int WDT, bool BF16>
+__device__ __forceinline__ u32x4b mx_to_operand(uint32_t d0, uint32_t d1, float scale) {
+    u32x4b o;
+    if constexpr (WDT == kWMX8) {
+        if constexpr (BF16) {
+            o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d0, scale, false));
+            o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d0, scale, true));
+            o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d1, scale, false));
+            o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d1, scale, true));
+        } else {
+            o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, scale, false));
+            o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d0, scale, true));
+            o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, scale, false));
+            o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(d1, scale, true));
+        }
+    } else {
+        if constexpr (BF16) {
+            o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d0, scale, 0));
+            o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d0, scale, 1));
+            o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d0, scale, 2));
+            o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d0, scale, 3));
+        } else {
+            o[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, scale, 0));
+            o[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, scale, 1));
+            o[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, scale, 2));
+            o[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(d0, scale, 3));
+        }
+    }
+    return o;
+}
+
 template <bool BF16>
 __device__ __forceinline__ float16_t mfma32b(const u32x4b& a, const u32x4b& b, float16_t c) {
     if constexpr (BF16)
@@ -127,9 +166,14 @@ __device__ __forceinline__ float16_t mfma32b(const u32x4b& a, const u32x4b& b, f
 }
 
 constexpr int ring_slots_kb(int bm) { return bm >= 256 ? 3 : 4; }
-constexpr int slot_bytes_kb(int bm) { return bm * kRowAb + kBNb * kRowBb; }
+// weight bytes per row and stage: 64 codes are 64 bytes, or 32 for nibble pairs; micro-scaled weights add one
+// 32-bit word of block scales per row (it covers 128 values, two stages)
+constexpr int row_bytes_kb(int wdt) { return wdt == kWMX4 ? 32 : kRowBb; }
+constexpr int slot_bytes_kb(int bm, int wdt = 0) {
+    return bm * kRowAb + kBNb * row_bytes_kb(wdt) + (wdt == kWMX8 || wdt == kWMX4 ? kBNb * 4 : 0);
+}
 
-// WDT: GLA_DT_INT8, GLA_DT_UINT8 or GLA_DT_FP8; TI = 32-row MFMA tiles per wave (1, 2 or 4)
+// WDT: GLA_DT_INT8, GLA_DT_UINT8, GLA_DT_FP8, kWMX8 or kWMX4; TI = 32-row MFMA tiles per wave (1, 2 or 4)
 template <int WDT, bool BF16, int WAVES_M, int TI>
 __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kbytes_kernel(GemmKbArgs p) {
     constexpr int TJ = 2;
@@ -137,11 +181,17 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
     constexpr int BM = WAVES_M * WM;
     constexpr int NW = WAVES_M * kWavesNb;
     constexpr int RING = ring_slots_kb(BM);
-    constexpr int SLOT = slot_bytes_kb(BM);
+    constexpr bool MXW = WDT == kWMX8 || WDT == kWMX4;
+    constexpr bool FP4 = WDT == kWMX4;
+    constexpr int ROWB = row_bytes_kb(WDT);
+    constexpr int SLOT = slot_bytes_kb(BM, WDT);
     constexpr int B_OFF = BM * kRowAb;
+    constexpr int S_OFF = B_OFF + kBNb * ROWB;  // micro-scaled weights: one scale word per weight row
     constexpr int A_JOBS = BM / 8;            // 16-byte copy instructions for the A tile (8 rows x 128 bytes each)
-    constexpr int JOBS16 = A_JOBS + kBNb / 16;  // ... and the weight tile (16 rows x 64 bytes each)
-    constexpr int LPS = (JOBS16 + NW - 1) / NW; // copy instructions per wave per stage
+    constexpr int JOBS16 = A_JOBS + (FP4 ? kBNb / 32 : kBNb / 16);  // ... and the weight tile (16 rows x 64 bytes, or 32 rows x 32 bytes, each)
+    constexpr int J16 = (JOBS16 + NW - 1) / NW;
+    constexpr int J4 = MXW ? (kBNb / 64 + NW - 1) / NW : 0;  // 4-byte copies of scale words, 64 rows each
+    constexpr int LPS = J16 + J4;             // copy instructions per wave per stage
     static_assert(RING * LPS < 64, "outstanding copies must fit the vmcnt counter");
 
     extern __shared__ __align__(16) unsigned char smem[];
@@ -157,11 +207,11 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
     // activation tile, lane (row l/8, position l%8) fetches the chunk that belongs at that position of
     // the swizzled row; otherwise rows 16(q - A_JOBS).. of the weight tile, lane (row l/4, position l%4).
     // A source address is a wave-uniform base that advances per stage plus a 32-bit lane offset.
-    unsigned off16[LPS];
-    int dst16[LPS];
-    bool is_a16[LPS];
+    unsigned off16[J16];
+    int dst16[J16];
+    bool is_a16[J16];
 #pragma unroll
-    for (int i = 0; i < LPS; ++i) {
+    for (int i = 0; i < J16; ++i) {
         int q = wave + NW * i;
         if (q > JOBS16 - 1) q = JOBS16 - 1;  // surplus jobs repeat the last one: same data, same place
         is_a16[i] = q < A_JOBS;
@@ -172,6 +222,13 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
             if (gm > p.M - 1) gm = p.M - 1;
             off16[i] = (unsigned)(gm * (int)p.xsm + chunk * 8) * 2u;
             dst16[i] = q * 8 * kRowAb;
+        } else if constexpr (FP4) {
+            // 32 rows of two 16-byte chunks: lane (chunk l/32, row l%32), so that the job's LDS image is
+            // [chunk][row] and the 32 lanes of a half-wave later read 32 consecutive 16-byte slots
+            int gn = n0 + (q - A_JOBS) * 32 + (lane & 31);
+            if (gn > p.N - 1) gn = p.N - 1;
+            off16[i] = (unsigned)(gn * (int)p.wsn + (lane >> 5) * 16);
+            dst16[i] = B_OFF + (q - A_JOBS) * 1024;
         } else {
             const int row = (q - A_JOBS) * 16 + (lane >> 2);
             const int chunk = (lane & 3) ^ ((row >> 2) & 3);
@@ -179,6 +236,20 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
             if (gn > p.N - 1) gn = p.N - 1;
             off16[i] = (unsigned)(gn * (int)p.wsn + chunk * 16);
             dst16[i] = B_OFF + (q - A_JOBS) * 16 * kRowBb;
+        }
+    }
+    // micro-scaled weights: job q copies the scale word (4 blocks of 32 values = two stages) of 64 weight rows
+    unsigned off4[MXW ? J4 : 1];
+    int dst4[MXW ? J4 : 1];
+    if constexpr (MXW) {
+#pragma unroll
+        for (int i = 0; i < J4; ++i) {
+            int q = wave + NW * i;
+            if (q > kBNb / 64 - 1) q = kBNb / 64 - 1;
+            int gn = n0 + q * 64 + lane;
+            if (gn > p.N - 1) gn = p.N - 1;
+            off4[i] = (unsigned)(gn * (int)p.bsn);
+            dst4[i] = S_OFF + q * 256;
         }
     }
     const int total_steps = p.K / kBKb;
@@ -192,12 +263,19 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
         ++ik;
         unsigned char* base = smem + slot * SLOT;
         const unsigned char* xk = (const unsigned char*)p.x + (int64_t)kk * (kBKb * 2);
-        const unsigned char* wk = p.w + (int64_t)kk * kBKb;
+        const unsigned char* wk = p.w + (int64_t)kk * ROWB;
 #pragma unroll
-        for (int i = 0; i < LPS; ++i) {
+        for (int i = 0; i < J16; ++i) {
             const unsigned char* src = (is_a16[i] ? xk : wk) + off16[i];
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(base + dst16[i]), 16, 0, 0);
+        }
+        if constexpr (MXW) {
+            const unsigned char* sk = p.bscales + (int64_t)(kk >> 1) * 4;
+#pragma unroll
+            for (int i = 0; i < J4; ++i)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
+                                                 (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
         }
     };
 
@@ -211,7 +289,10 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
 
     const int swa = (r32 >> 1) & 7, swb = (r32 >> 2) & 3;  // chunk swizzles of this lane's rows (tile offsets are multiples of 32)
     const int a_row0 = (wm * WM + r32) * kRowAb;
-    const int b_row0 = B_OFF + (wn * 32 * TJ + r32) * kRowBb + 8 * kb;
+    const int b_row0 = FP4 ? B_OFF + wn * TJ * 1024 + r32 * 16 + 4 * kb   // [job = 32 rows][chunk][row] image
+                           : B_OFF + (wn * 32 * TJ + r32) * kRowBb + 8 * kb;
+    const int s_row0 = S_OFF + (wn * 32 * TJ + r32) * 4;
+    uint32_t sword[MXW ? TJ : 1];  // scale words of the stage whose K-steps are being converted
 
     struct Raw {
         u32x4b a[TI];   // activation chunk of the lane's row in each row tile
@@ -224,13 +305,34 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
 #pragma unroll
         for (int i = 0; i < TI; ++i) r.a[i] = *(const u32x4b*)(base + a_row0 + i * 32 * kRowAb + (((2 * s + kb) ^ swa) << 4));
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) r.w[j] = *(const u32x2b*)(base + b_row0 + j * 32 * kRowBb + ((s ^ swb) << 4));
+        for (int j = 0; j < TJ; ++j) {
+            if constexpr (FP4) {  // K-step s: bytes 8 s .. 8 s + 7 of the row = chunk s / 2, half s % 2; 4 of them per lane
+                r.w[j].x = *(const uint32_t*)(base + b_row0 + j * 1024 + (s >> 1) * 512 + (s & 1) * 8);
+                r.w[j].y = 0;
+            } else {
+                r.w[j] = *(const u32x2b*)(base + b_row0 + j * 32 * kRowBb + ((s ^ swb) << 4));
+            }
+        }
+        if constexpr (MXW) {
+            if (s == 0) {
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) sword[j] = *(const uint32_t*)(base + s_row0 + j * 128);
+            }
+        }
     };
-    auto unpack = [&](const Raw& r, Ops& o) __attribute__((always_inline)) {
+    // (s, par: the K-step just read and the parity of its stage, which pick the block's byte of the scale word)
+    auto unpack = [&](const Raw& r, Ops& o, int s, int par) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < TI; ++i) o.af[i] = r.a[i];
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) o.bq[j] = bytes_to_operand<WDT, BF16>(r.w[j].x, r.w[j].y);
+        for (int j = 0; j < TJ; ++j) {
+            if constexpr (MXW) {
+                const uint32_t e = (sword[j] >> (8 * (2 * par + (s >> 1)))) & 0xffu;
+                o.bq[j] = mx_to_operand<WDT, BF16>(r.w[j].x, r.w[j].y, __builtin_bit_cast(float, e << 23));
+            } else {
+                o.bq[j] = bytes_to_operand<WDT, BF16>(r.w[j].x, r.w[j].y);
+            }
+        }
     };
 
     // ---- pipeline (see the header): RING stages in flight, bare barriers, explicit waits
@@ -243,7 +345,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     read_raw(smem, 0, raw);
-    unpack(raw, ops[0]);
+    unpack(raw, ops[0], 0, k_first & 1);
 
     constexpr int NMF = TI * TJ;
     constexpr int NVA = 16 * TJ;  // VALU instructions of a conversion, roughly
@@ -253,6 +355,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
         const unsigned char* base = smem + slot * SLOT;
         const int next = slot == RING - 1 ? 0 : slot + 1;
         const unsigned char* nbase = smem + next * SLOT;
+        const int par = (k_first + k) & 1;
         auto kstep = [&](auto s_tag) __attribute__((always_inline)) {
             constexpr int s = decltype(s_tag)::value;
             if constexpr (s == 3) {
@@ -271,7 +374,7 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
             for (int j = 0; j < TJ; ++j)
 #pragma unroll
                 for (int i = 0; i < TI; ++i) acc[i][j] = mfma32b<BF16>(ops[s & 1].bq[j], ops[s & 1].af[i], acc[i][j]);
-            unpack(raw, ops[(s + 1) & 1]);
+            unpack(raw, ops[(s + 1) & 1], s == 3 ? 0 : s + 1, s == 3 ? par ^ 1 : par);
             __builtin_amdgcn_sched_group_barrier(0x100, TI + TJ, 0);  // the LDS reads first
 #pragma unroll
             for (int q = 0; q < NMF; ++q) {
@@ -387,7 +490,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kb_kernel(GemmKbArgs p) {
 template <int WDT, bool BF16, int WAVES_M, int TI>
 int launch_kb(const GemmKbArgs& a, hipStream_t stream) {
     constexpr int BM = WAVES_M * 32 * TI;
-    const size_t smem = (size_t)ring_slots_kb(BM) * slot_bytes_kb(BM);
+    const size_t smem = (size_t)ring_slots_kb(BM) * slot_bytes_kb(BM, WDT);
     static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
     auto kern = gemm_kbytes_kernel<WDT, BF16, WAVES_M, TI>;
     if (once.first()) {
@@ -469,6 +572,62 @@ int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p) {
     return g.S > 1 ? kWsReservedB + (int64_t)g.S * p.M * p.N * 4 : 0;
 }
 
+// ---- weight-only MX layers above a few rows: fp16 / bf16 activations x MXFP8 / MXFP4 weights ------------
+// (reference: gemlite/triton_kernels/gemm_kernels.py:509-737 with 16-bit activations and unit activation
+// scales, gemlite/helper.py:199-237.)  The conversion instruction applies the block scale, so the operand is
+// the dequantised weight in the activations' type: exact in bf16; in fp16 as far as code x 2^(e-127) is a
+// finite normal fp16 number, which weights of trained layers are.
+bool gemm_kbytes_mx_eligible(const gla_matmul_args& p) {
+    if (!(p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)) return false;
+    if (p.M <= 4 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_NONE || p.scales == nullptr) return false;
+    const bool fp4 = p.elements_per_sample == 2 && p.W_nbits == 4;
+    const bool fp8 = p.elements_per_sample == 1 && p.W_nbits == 8 && p.w_dtype == GLA_DT_FP8;
+    if (!fp4 && !fp8) return false;
+    switch (p.output_dtype) {
+        case GLA_DT_FP32: case GLA_DT_FP16: case GLA_DT_BF16: case GLA_DT_MXFP16: case GLA_DT_MXBF16: break;
+        default: return false;
+    }
+    if (p.w_stride_k != 1 || p.x_stride_k != 1 || p.out_stride_n != 1 || p.meta_stride_g != 1) return false;
+    if (p.K % 128 != 0 || p.w_stride_n % 16 != 0 || p.x_stride_m % 8 != 0 || p.meta_stride_n % 4 != 0) return false;
+    if (((uintptr_t)p.w & 15) || ((uintptr_t)p.x & 15) || ((uintptr_t)p.scales & 3)) return false;
+    if ((int64_t)p.M * p.x_stride_m >= (1ll << 30) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
+    if ((int64_t)p.N * p.meta_stride_n >= (1ll << 31)) return false;
+    return true;
+}
+
+int64_t gemm_kbytes_mx_workspace_bytes(const gla_matmul_args& p) { return gemm_kbytes_workspace_bytes(p); }
+
+int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream) {
+    if (!gemm_kbytes_mx_eligible(p)) {
+        set_error("gemm_kbytes_mx: operands not eligible (K-contiguous MXFP8 / MXFP4 weights, K %% 128 == 0, more than 4 rows)");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    GemmKbArgs a;
+    a.x = (const uint16_t*)p.x; a.w = (const uint8_t*)p.w; a.scales = nullptr; a.scales_x = nullptr; a.out = p.out;
+    a.M = p.M; a.N = p.N; a.K = p.K;
+    a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = 0; a.sxm = 0;
+    a.col_scale = 0; a.row_scale = 0;
+    a.bscales = (const uint8_t*)p.scales; a.bsn = p.meta_stride_n;
+    a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
+    a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
+    const KbPlan g = kb_plan(p);
+    a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps;
+    a.partials = nullptr;
+    if (g.S > 1) {
+        const int64_t need = gemm_kbytes_workspace_bytes(p);
+        if (p.workspace == nullptr || (int64_t)p.workspace_bytes < need) {
+            set_error("gemm_kbytes_mx: workspace of %lld bytes required, %llu given", (long long)need,
+                      (unsigned long long)p.workspace_bytes);
+            return GLA_ERR_WORKSPACE_TOO_SMALL;
+        }
+        a.partials = (float*)((char*)p.workspace + kWsReservedB);
+    }
+    const bool bf16 = p.input_dtype == GLA_DT_MXBF16;
+    if (p.elements_per_sample == 2)
+        return bf16 ? launch_kb_m<kWMX4, true>(a, g.bm, stream) : launch_kb_m<kWMX4, false>(a, g.bm, stream);
+    return bf16 ? launch_kb_m<kWMX8, true>(a, g.bm, stream) : launch_kb_m<kWMX8, false>(a, g.bm, stream);
+}
+
 int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream) {
     GemmKbArgs a;
     a.x = (const uint16_t*)p.x; a.w = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
@@ -477,6 +636,7 @@ int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream) {
     a.col_scale = (p.W_group_mode == GLA_WGM_SCALE ? 1 : 0) + ((p.channel_scale_mode & 1) ? 1 : 0);
     a.row_scale = (p.channel_scale_mode & 2) ? 1 : 0;
     a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
+    a.bscales = nullptr; a.bsn = 0;
     const KbPlan g = kb_plan(p);
     a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps;
     a.partials = nullptr;

@@ -525,7 +525,8 @@ def test_weight_only_mxfp_layers(device, dtype, W_nbits):
     layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
     want = orc.quantize_mxfp8_weights(to_np(W.to(dtype))) if W_nbits == 8 else orc.quantize_mxfp4_weights(to_np(W.to(dtype)))
     assert np.array_equal(layer.scales.cpu().numpy(), want[1])
-    for M in (1, 2, 3, 7, 33):
+    # streaming kernel up to 4 rows; above, the matrix-core kernel (64-, 128- and 256-row tiles, split K)
+    for M in (1, 2, 3, 4, 5, 7, 33, 70, 130, 300):
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=["GEMV", "GEMM_SPLITK", "GEMM"])
     # a one-hot activation row picks out one dequantised weight column exactly
     x = torch.zeros(1, K, dtype=dtype)
@@ -535,6 +536,27 @@ def test_weight_only_mxfp_layers(device, dtype, W_nbits):
     torch.cuda.synchronize()
     y_ref = oracle_forward(layer, x)
     assert np.array_equal(to_np(y), round_like(y_ref, dtype))
+    # ... and through the matrix-core kernel: row r of a batch of 40 is one-hot at a position of its own
+    x = torch.zeros(40, K, dtype=dtype)
+    for r in range(40):
+        x[r, (97 * r + 5) % K] = 1.0
+    y = layer(x.to(device))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(y), round_like(oracle_forward(layer, x), dtype))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("W_nbits", [8, 4])
+def test_weight_only_mxfp_layers_k_not_a_multiple_of_128(device, dtype, W_nbits):
+    """K = 1056 (33 blocks): every batch size stays on the streaming kernel."""
+    N, K = 264, 1056
+    lin = torch.nn.Linear(K, N, bias=False, dtype=dtype)
+    lin.weight.data = gen_x(N, K, torch.bfloat16, seed=53, std=0.03).to(dtype)
+    cls = helper.A16W8_MXFP if W_nbits == 8 else helper.A16W4_MXFP
+    layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
+    for M in (1, 6, 9, 40):
+        check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=["GEMM_SPLITK", "GEMM"])
 
 
 @pytest.mark.gpu
