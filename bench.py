@@ -250,6 +250,11 @@ def extra_points(lib, device):
         out[f"gemv_a16w4_mxfp_M{M}"] = {"N": N, "K": K, "us": round(us, 1),
                                         "GB/s": round((N * K // 2 + N * K // 32 + M * K * 2 + M * N * 2) / us / 1e3, 1)}
     out["gemv_a16w4_mxfp_M1"]["note"] = "134 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"
+    # ... and at M = 4096 on the matrix cores (weights converted to bf16 fragments in registers)
+    xm = torch.randn((4096, K), generator=g).to(torch.bfloat16).to(device)
+    ym = torch.empty((4096, N), dtype=torch.bfloat16, device=device)
+    us = time_us(prepared(wo, xm, None, ym), 20)
+    point("gemm_a16w4_mxfp_bf16", 4096, N, K, us, 2500.0, "bf16")
     del wo, w_codes, w_scales, xm, ym
 
     # 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5), N = K = 8192: per-block activation quantiser,

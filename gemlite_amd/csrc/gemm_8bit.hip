@@ -2,7 +2,11 @@
 //   fp8-e4m3 x fp8-e4m3 -> fp32      (v_mfma_f32_32x32x64_f8f6f4, unit block scales)
 //   int8 x int8 -> int32             (v_mfma_i32_32x32x32_i8, exact)
 //   MXFP4 x MXFP4 -> fp32            (v_mfma_scale_f32_32x32x64_f8f6f4 with one e8m0 scale per
-//                                     32 K-values on either operand)
+//                                     32 K-values on either operand; MXFP8 likewise)
+//   fp8 / int8 with fp32 scales per 128 x 128 weight block and per (activation row, 128 values):
+//                                     the sum over each 128 values of K is folded, scaled, into a
+//                                     second fp32 accumulator (channel_scale_mode 5,
+//                                     reference: gemlite/triton_kernels/gemm_kernels.py:441-450)
 // and a per-row / per-column scale epilogue.  The prefill path of dynamically quantised A8W8
 // and A4W4 layers.
 //

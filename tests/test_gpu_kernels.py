@@ -525,7 +525,7 @@ def test_weight_only_mxfp_layers(device, dtype, W_nbits):
     layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
     want = orc.quantize_mxfp8_weights(to_np(W.to(dtype))) if W_nbits == 8 else orc.quantize_mxfp4_weights(to_np(W.to(dtype)))
     assert np.array_equal(layer.scales.cpu().numpy(), want[1])
-    # streaming kernel up to 4 rows; above, the matrix-core kernel (64-, 128- and 256-row tiles, split K)
+    # streaming kernel up to 2 rows; above, the matrix-core kernel (64-, 128- and 256-row tiles, split K)
     for M in (1, 2, 3, 4, 5, 7, 33, 70, 130, 300):
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=["GEMV", "GEMM_SPLITK", "GEMM"])
     # a one-hot activation row picks out one dequantised weight column exactly

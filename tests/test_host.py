@@ -412,7 +412,7 @@ def test_weight_only_and_mixed_mx_processors():
     """A16W8_MXFP / A16W4_MXFP keep fp16 / bf16 activations (input and output type MXFP16 / MXBF16,
     W_group_mode 2, channel_scale_mode 0; reference: gemlite/helper.py:199-237, 384-420);
     A8W4_MXFP_dynamic is MXFP8 activations x MXFP4 weights (reference: gemlite/helper.py:950-1040).
-    They run the streaming MX kernel; weight-only layers take the matrix cores above 4 rows."""
+    They run the streaming MX kernel; weight-only layers take the matrix cores above 2 rows."""
     g = torch.Generator().manual_seed(5)
     N, K = 64, 256
     W = (torch.randn((N, K), generator=g) * 0.03).to(torch.bfloat16)
@@ -429,8 +429,8 @@ def test_weight_only_and_mixed_mx_processors():
             assert l.scales.shape == (N, K // 32) and l.scales.dtype == torch.uint8 and l.scales.stride() == (K // 32, 1)
             assert l.bias.dtype == dtype
             assert gemlite_amd.DTYPE_TO_TORCH[l.get_meta_args()[6]] == dtype
-            # streaming kernel up to 4 rows, matrix cores above (K = 256 is a multiple of 128)
-            for M, fam in ((1, "MX_STREAM"), (4, "MX_STREAM"), (5, "GEMM_KBYTES_MX"), (100, "GEMM_KBYTES_MX")):
+            # streaming kernel up to 2 rows, matrix cores above (K = 256 is a multiple of 128)
+            for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (3, "GEMM_KBYTES_MX"), (100, "GEMM_KBYTES_MX")):
                 m = l.get_meta_args()
                 x = torch.zeros(M, K, dtype=dtype)
                 out = torch.zeros(M, N, dtype=dtype)
