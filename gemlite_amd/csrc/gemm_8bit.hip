@@ -44,9 +44,11 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6 };
+enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6, kMX84 = 7, kMX84T = 8 };
 // kMXFP8T: MXFP8 weights whose activations carry no block scales (their per-token scale is applied in the
 // epilogue), so no registers are spent on activation scale words and the 256-row tile fits
+// kMX84 / kMX84T: fp8 activations (with MXFP8 micro-scales / per token) x MXFP4 weights: the mixed form of the
+// scaled MFMA; a stage's weight tile has rows of 32 bytes (64 e2m1 values)
 // kBQF8 / kBQI8: fp8 / int8 with one fp32 scale per 128 x 128 weight block and per (activation row, 128 values):
 // the sum over two stages (128 values) goes to a second, fp32 accumulator scaled by both
 
@@ -93,7 +95,10 @@ __device__ __forceinline__ void wait_vmcnt8() {
 }
 
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
-constexpr int slot_bytes8(int mode, int bm) { return (bm + kBN) * kRowB8 + (mode == kMXFP4 || mode == kMXFP8 || mode == kMXFP8T || mode == kBQF8 || mode == kBQI8 ? (bm + kBN) * 4 : 0); }
+constexpr int slot_bytes8(int mode, int bm) {
+    const bool w4 = mode == kMX84 || mode == kMX84T;
+    return bm * kRowB8 + kBN * (w4 ? 32 : kRowB8) + (mode == kFP8 || mode == kINT8 ? 0 : (bm + kBN) * 4);
+}
 
 // WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
 // (A 2-column variant with 4 waves of 128 x 128 and accumulators in AGPRs reads a third less from
@@ -107,8 +112,9 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr int TI = WM / 32;       // 32-row MFMA tiles per wave along M
     constexpr int WNC = kBN / WN;     // wave tile columns
     constexpr int TJ = WNC / 32;      // 32-column MFMA tiles per wave along N
-    constexpr bool M8 = MODE == kMXFP8 || MODE == kMXFP8T;
-    constexpr bool TOKEN = MODE == kMXFP8T;                 // no activation block scales
+    constexpr bool W4 = MODE == kMX84 || MODE == kMX84T;    // MXFP4 weights under fp8 activations
+    constexpr bool M8 = MODE == kMXFP8 || MODE == kMXFP8T || W4;
+    constexpr bool TOKEN = MODE == kMXFP8T || MODE == kMX84T;  // no activation block scales
     constexpr bool BQ = MODE == kBQF8 || MODE == kBQI8;     // fp32 block scales, applied by the vector unit
     constexpr bool F8 = MODE == kFP8 || MODE == kBQF8;      // plain fp8 operands, one 64-byte K-step per stage
     constexpr bool I8 = MODE == kINT8 || MODE == kBQI8;
@@ -118,9 +124,10 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr int NW = kWavesM * WN;
     constexpr int RING = kRing8;
     constexpr int SLOT = slot_bytes8(MODE, BM);
-    constexpr int B_OFF = BM * kRowB8, S_OFF = (BM + kBN) * kRowB8;
+    constexpr int ROWW = W4 ? 32 : kRowB8;    // bytes of a weight row per stage
+    constexpr int B_OFF = BM * kRowB8, S_OFF = BM * kRowB8 + kBN * ROWW;
     constexpr int A_JOBS = BM / 16;           // 16-byte copy instructions for the A tile (16 rows each)
-    constexpr int JOBS16 = A_JOBS + kBN / 16; // ... and the B tile
+    constexpr int JOBS16 = A_JOBS + (W4 ? kBN / 32 : kBN / 16); // ... and the B tile (W4: 32 rows of two chunks each)
     constexpr int J16 = (JOBS16 + NW - 1) / NW;
     constexpr int A_JOBS4 = TOKEN ? 0 : BM / 64;
     constexpr int JOBS4 = A_JOBS4 + kBN / 64; // micro-scaled: 4-byte copies of block scales, 64 rows each
@@ -152,7 +159,15 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         is_a16[i] = q < A_JOBS;
         const int row = (is_a16[i] ? q : q - A_JOBS) * 16 + (lane >> 2);
         chunk16[i] = ((lane & 3) ^ ((row >> 2) & 3)) * 16;
-        if (is_a16[i]) {
+        if (W4 && !is_a16[i]) {
+            // 32 weight rows of two 16-byte chunks: lane (chunk l/32, row l%32); the job's LDS image is
+            // [chunk][row], so a half-wave later reads 32 consecutive 16-byte slots
+            int gn = n0 + (q - A_JOBS) * 32 + (lane & 31);
+            if (gn > p.N - 1) gn = p.N - 1;
+            chunk16[i] = (lane >> 5) * 16;
+            off16[i] = (unsigned)(gn * (int)p.ldb);
+            dst16[i] = B_OFF + (q - A_JOBS) * 1024;
+        } else if (is_a16[i]) {
             int gm = m0 + row;
             if (gm > p.M - 1) gm = p.M - 1;
             off16[i] = (unsigned)(gm * (int)p.lda);
@@ -200,7 +215,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         unsigned char* base = smem + slot * SLOT;
         if (c < J16) {
             const int limit = p.Kb - kk * kRowB8;
-            const uint8_t* src = (is_a16[c] ? p.a : p.b) + kk * kRowB8 + (off16[c] + (unsigned)(chunk16[c] < limit ? chunk16[c] : 0));
+            const uint8_t* src = (is_a16[c] ? p.a : p.b) + kk * (is_a16[c] ? kRowB8 : ROWW) + (off16[c] + (unsigned)(chunk16[c] < limit ? chunk16[c] : 0));
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(base + dst16[c]), 16, 0, 0);
         } else if constexpr (MX) {
@@ -241,7 +256,8 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     const int c0 = ((F8 ? 2 * kb : kb) ^ sw) << 4;
     const int c1 = ((F8 ? 2 * kb + 1 : 2 + kb) ^ sw) << 4;
     const int a_row0 = (wm * WM + r32) * kRowB8;
-    const int b_row0 = B_OFF + (wn * WNC + r32) * kRowB8;
+    // W4: [32-row job][chunk][row] image, the half-wave's chunk kb is K-block kb of the stage
+    const int b_row0 = W4 ? B_OFF + (wn * TJ) * 1024 + kb * 512 + r32 * 16 : B_OFF + (wn * WNC + r32) * kRowB8;
     const int sa_row0 = S_OFF + (wm * WM + r32) * 4;
     const int sb_row0 = S_OFF + (BM + wn * WNC + r32) * 4;
 
@@ -263,7 +279,11 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         constexpr int B = decltype(buf_tag)::value;
         const unsigned char* base = smem + slot * SLOT;
         if (r < 2 * TJ) {
-            fb[B][r / 2].c[r % 2] = *(const u32x4*)(base + b_row0 + (r / 2) * 32 * kRowB8 + (r % 2 ? c1 : c0));
+            if constexpr (W4) {
+                if (r % 2 == 0) fb[B][r / 2].c[0] = *(const u32x4*)(base + b_row0 + (r / 2) * 1024);
+            } else {
+                fb[B][r / 2].c[r % 2] = *(const u32x4*)(base + b_row0 + (r / 2) * 32 * kRowB8 + (r % 2 ? c1 : c0));
+            }
         } else if (r < 2 * (TI + TJ)) {
             const int q = r - 2 * TJ;
             fa[B][q / 2].c[q % 2] = *(const u32x4*)(base + a_row0 + (q / 2) * 32 * kRowB8 + (q % 2 ? c1 : c0));
@@ -314,6 +334,16 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                 for (int e = 0; e < 16; ++e) cin[e] = 0;
             }
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, cin, 0, 0, 0, 127, 0, 127);
+        } else if constexpr (W4) {
+            // mixed formats: e2m1 weights (the first four operand registers, K-block kb in half-wave kb) x e4m3
+            // activations (chunk pair (kb, 2 + kb) as for MXFP8); each half-wave's scale byte is that of block kb
+            const int4_t b4 = int4_t{(int)fb[B][j].c[0].x, (int)fb[B][j].c[0].y, (int)fb[B][j].c[0].z, (int)fb[B][j].c[0].w};
+            const int8_t_v b8 = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
+            if constexpr (TOKEN)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, fa[B][i].v8, acc[i][j], 4, 0, 0, (int)fsb[SB][j], 0, 127);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, fa[B][i].v8, acc[i][j], 4, 0, 0, (int)fsb[SB][j], 0,
+                                                                            (int)fsa[SB][i]);
         } else if constexpr (TOKEN) {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[B][j].v8, fa[B][i].v8, acc[i][j], 0, 0, 0,
                                                                         (int)fsb[SB][j], 0, 127);
@@ -833,7 +863,9 @@ int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
 bool gemm_mxfp8_eligible(const gla_matmul_args& p) {
     if (p.input_dtype != GLA_DT_MXFP8) return false;
     if (!(p.channel_scale_mode == GLA_CSM_MX || p.channel_scale_mode == GLA_CSM_ACTIVATION)) return false;
-    if (p.W_nbits != 8 || p.elements_per_sample != 1 || p.group_size != 32 || p.w_dtype != GLA_DT_FP8) return false;
+    const bool w8 = p.W_nbits == 8 && p.elements_per_sample == 1 && p.w_dtype == GLA_DT_FP8;
+    const bool w4 = p.W_nbits == 4 && p.elements_per_sample == 2;  // MXFP4 weights: the mixed fp8 x fp4 MFMA
+    if (!(w8 || w4) || p.group_size != 32) return false;
     if (p.scales == nullptr || p.scales_x == nullptr) return false;
     if (p.w_stride_k != 1 || p.x_stride_k != 1 || p.out_stride_n != 1) return false;
     if (p.meta_stride_g != 1 || p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3)) return false;
@@ -897,6 +929,7 @@ int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
         if (act_blocks) { a.ascales = sx; a.asxm = 4; a.sx_stage = (int64_t)p.M * 4; }
         else { a.ascales = sw; }
     }
+    if (p.elements_per_sample == 2) return act_blocks ? launch_mode<kMX84>(a, g.bm, stream) : launch_mode<kMX84T>(a, g.bm, stream);
     return act_blocks ? launch_mode<kMXFP8>(a, g.bm, stream) : launch_mode<kMXFP8T>(a, g.bm, stream);
 }
 

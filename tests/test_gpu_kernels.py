@@ -561,17 +561,24 @@ def test_weight_only_mxfp_layers_k_not_a_multiple_of_128(device, dtype, W_nbits)
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("post_scale", [True, False])
-def test_a8w4_mxfp8_activations_mxfp4_weights(device, post_scale):
+@pytest.mark.parametrize("K", [1056, 1024, 2432])
+def test_a8w4_mxfp8_activations_mxfp4_weights(device, post_scale, K):
     """MXFP8 activations (per token, or with micro-scales) x MXFP4 weights
-    (reference processor A8W4_MXFP_dynamic, gemlite/helper.py:950-1040)."""
-    N, K = 520, 1056   # 33 blocks: not a multiple of the 128 the matrix-core kernels want
+    (reference processor A8W4_MXFP_dynamic, gemlite/helper.py:950-1040).  K = 1056 is 33 blocks, not a
+    multiple of the 128 the matrix-core kernel wants, and streams; the others run the mixed fp8 x fp4 MFMA
+    (K = 2432 is 19 words of scales: an odd number of stage pairs)."""
+    N = 520
     W = gen_x(N, K, torch.bfloat16, seed=61, std=0.03)
+    W[:, 32:64] *= 8.0     # block scales that differ from block to block
+    W[:, 96:128] *= 0.125
     codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
     layer = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=post_scale).from_weights(
         torch.from_numpy(codes), scales=torch.from_numpy(e8))
     assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 2 if post_scale else 4)
-    for M in (1, 5, 33, 70):
-        check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
+    for M in (1, 5, 33, 70, 130, 300):
+        x = gen_x(M, K, torch.bfloat16, seed=M)
+        x[:, 64:96] *= 16.0
+        check_layer(layer, x.to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
 
 
 @pytest.mark.gpu
