@@ -255,7 +255,13 @@ def extra_points(lib, device):
     ym = torch.empty((4096, N), dtype=torch.bfloat16, device=device)
     us = time_us(prepared(wo, xm, None, ym), 20)
     point("gemm_a16w4_mxfp_bf16", 4096, N, K, us, 2500.0, "bf16")
-    del wo, w_codes, w_scales, xm, ym
+    # ... and under fp8 activations quantised per token (A8W4_MXFP_dynamic): the mixed fp8 x fp4 scaled MFMA
+    a84 = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_packed_weights(
+        w_codes.t(), scales=w_scales.view(torch.float8_e8m0fnu))
+    xq, sx = gemlite_amd.scale_activations_per_token(xm, torch.float8_e4m3fn)
+    us = time_us(prepared(a84, xq, sx, ym), 20)
+    point("gemm_a8w4_mxfp", 4096, N, K, us, 5000.0, "fp8")
+    del wo, a84, xq, sx, w_codes, w_scales, xm, ym
 
     # 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5), N = K = 8192: per-block activation quantiser,
     # the MFMA GEMM at M = 4096 and the streaming kernel at M = 1

@@ -20,11 +20,11 @@
 // dot instruction; the block's partial sum is then scaled once by the product of its two block
 // scales, as the scaled matrix instruction does.  A shuffle tree sums the lanes.
 //
-// The combinations that have a matrix-core kernel do not come here (MXFP4 x MXFP4, fp8 x MXFP8, and
-// weight-only MX layers from 3 rows up when K is a multiple of 128); this kernel is the decode path
-// of the weight-only MX layers and the path at any batch size for MXFP8 activations x MXFP4 weights
-// and for a K that the matrix-core kernels do not take (not tuned above a few rows: every group of
-// eight activation rows streams the weights again).
+// The combinations that have a matrix-core kernel do not come here (MXFP4 x MXFP4, fp8 x MXFP8, and,
+// from 3 rows up when K is a multiple of 128, weight-only MX layers and fp8 x MXFP4); this kernel is
+// the decode path of the weight-only MX layers and of MXFP8 activations x MXFP4 weights, and the
+// path at any batch size for a K that the matrix-core kernels do not take (not tuned above a few
+// rows: every group of eight activation rows streams the weights again).
 #include "common.hpp"
 #include "dispatch.hpp"
 

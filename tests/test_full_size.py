@@ -148,3 +148,24 @@ def test_a16w4_mxfp_weight_only_16384_square(device, M):
     cols = sample_cols(N, seed=M)
     want = orc.matmul_mx_mixed(to_np(x), "float", None, codes[cols], "e2m1", e8[cols])
     assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+
+
+@pytest.mark.parametrize("post_scale,M", [(True, 1), (True, 1024), (False, 32), (False, 1024)])
+def test_a8w4_mxfp_16384_square(device, post_scale, M):
+    """MXFP8 activations (per token / micro-scaled) x MXFP4 weights, N = K = 16384: streaming kernel at M = 1,
+    the mixed fp8 x fp4 MFMA above."""
+    N = K = 16384
+    W = gen_x(N, K, torch.bfloat16, seed=9, std=0.02)
+    codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+    layer = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=post_scale).from_weights(
+        torch.from_numpy(codes), scales=torch.from_numpy(e8))
+    x = gen_x(M, K, torch.bfloat16, seed=M)
+    y = to_np(layer(x.to(device)))
+    cols = sample_cols(N, seed=M)
+    if post_scale:
+        aq, sx = orc.scale_activations_per_token(to_np(x), False)
+        want = orc.matmul_mx_mixed(aq, "e4m3", None, codes[cols], "e2m1", e8[cols], scales_x=sx)
+    else:
+        aq, sa = orc.scale_activations_mxfp8(to_np(x))
+        want = orc.matmul_mx_mixed(aq, "e4m3", sa[:M], codes[cols], "e2m1", e8[cols])
+    assert rel_frob(y[:, cols], want) <= TIGHT_BF16

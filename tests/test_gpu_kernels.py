@@ -575,7 +575,7 @@ def test_a8w4_mxfp8_activations_mxfp4_weights(device, post_scale, K):
     layer = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=post_scale).from_weights(
         torch.from_numpy(codes), scales=torch.from_numpy(e8))
     assert (layer.W_group_mode, layer.channel_scale_mode) == (0, 2 if post_scale else 4)
-    for M in (1, 5, 33, 70, 130, 300):
+    for M in (1, 2, 3, 5, 33, 70, 130, 300):
         x = gen_x(M, K, torch.bfloat16, seed=M)
         x[:, 64:96] *= 16.0
         check_layer(layer, x.to(device), torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])

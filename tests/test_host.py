@@ -451,10 +451,11 @@ def test_weight_only_and_mixed_mx_processors():
             lin, del_orig=False)
         assert l.input_dtype == DType.MXFP8 and l.scaled_activations and (l.W_nbits, l.elements_per_sample) == (4, 2)
         assert (l.W_group_mode, l.channel_scale_mode) == (0, csm)
-        for M in (1, 64):   # K = 256 is a multiple of 128: the mixed fp8 x fp4 matrix-core kernel
+        # streaming up to 2 rows; above (K = 256 is a multiple of 128) the mixed fp8 x fp4 matrix-core kernel
+        for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (3, "GEMM_MXFP8"), (64, "GEMM_MXFP8")):
             xq = torch.zeros(M, K, dtype=torch.float8_e4m3fn)
             sx = torch.ones(M, 1) if post_scale else torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
-            assert _family(l, M, None, scales_x=sx, x=xq) == "GEMM_MXFP8"
+            assert _family(l, M, None, scales_x=sx, x=xq) == fam
     # MXFP4 x MXFP4 whose K is a multiple of 32 but not of 128 streams too (the matrix-core kernel wants 128)
     K2 = 96
     codes = torch.randint(0, 16, (N, K2), generator=g).to(torch.uint8)
