@@ -26,6 +26,14 @@ def _layers(device):
     lin.weight.data = W
     yield "MXFP4", helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device)), \
         torch.bfloat16, (40,)
+    lin = torch.nn.Linear(2048, 1032, bias=True, dtype=torch.bfloat16)
+    lin.weight.data = W
+    yield "A16W4_MXFP", helper.A16W4_MXFP(device=device, dtype=torch.bfloat16).from_linear(lin.to(device), del_orig=False), \
+        torch.bfloat16, (1, 6)         # streaming kernel; split-K matrix-core kernel with its finishing kernel
+    yield "A8W4_MXFP", helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=False).from_linear(
+        lin.to(device), del_orig=False), torch.bfloat16, (2, 150)   # MXFP8 quantiser + streaming / mixed MFMA with staged scales
+    yield "A8W8 block-quantised", helper.A8W8_FP8_dynamic(device=device, block_quant=True).from_weights(W.to(device)), \
+        torch.bfloat16, (3, 40)        # per-block quantiser + streaming / split-K MFMA with the second accumulator
 
 
 def test_forward_replays_from_a_graph(device):

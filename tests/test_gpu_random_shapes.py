@@ -90,3 +90,39 @@ def test_mx_random_shapes(device, seed):
     layer = proc.from_linear(lin.to(device))
     for M in row_counts(rng, 2, 3):
         check(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, f"MX{'FP4' if fp4 else 'FP8'} {dtype} M={M} N={N} K={K}")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_weight_only_mx_and_mixed_random_shapes(device, seed):
+    """Weight-only MX layers (fp16 / bf16 x MXFP8 / MXFP4) and MXFP8 activations x MXFP4 weights: K a multiple of
+    32 (streaming kernel at every batch size) or of 128 (matrix cores from 3 rows up)."""
+    rng = np.random.default_rng(5000 + seed)
+    dtype = [torch.bfloat16, torch.float16][seed % 2]
+    kind = seed % 4   # 0: A16W4_MXFP, 1: A16W8_MXFP, 2: A8W4 per token, 3: A8W4 micro-scaled activations
+    K = (128 if seed < 6 else 32) * int(rng.integers(1, 33))
+    N = 8 * int(rng.integers(4, 200))
+    lin = torch.nn.Linear(K, N, bias=bool(seed % 3 == 0), dtype=dtype)
+    lin.weight.data = gen_x(N, K, dtype, seed=seed, std=0.02)
+    if kind == 0:
+        proc = helper.A16W4_MXFP(device=device, dtype=dtype)
+    elif kind == 1:
+        proc = helper.A16W8_MXFP(device=device, dtype=dtype)
+    else:
+        proc = helper.A8W4_MXFP_dynamic(device=device, dtype=dtype, post_scale=(kind == 2))
+    layer = proc.from_linear(lin.to(device))
+    for M in row_counts(rng, 3, 3):
+        check(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, f"MX kind {kind} {dtype} M={M} N={N} K={K}")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_block_quantised_random_shapes(device, seed):
+    rng = np.random.default_rng(6000 + seed)
+    to_int8 = bool(seed % 2)
+    dtype = [torch.bfloat16, torch.float16][(seed // 2) % 2]
+    K = 128 * int(rng.integers(1, 40))
+    N = 8 * int(rng.integers(4, 300))
+    W = gen_x(N, K, dtype, seed=seed, std=0.02)
+    proc = (helper.A8W8_INT8_dynamic if to_int8 else helper.A8W8_FP8_dynamic)(device=device, block_quant=True)
+    layer = proc.from_weights(W)
+    for M in row_counts(rng, 3, 3):
+        check(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, f"block-quant {'int8' if to_int8 else 'fp8'} {dtype} M={M} N={N} K={K}")
