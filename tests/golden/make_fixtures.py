@@ -96,7 +96,36 @@ def main():
     y = orc.matmul_mx(orc.unpack_fp4_bytes(a_packed), a_scales[:5], codes, e8)
     np.savez_compressed(os.path.join(HERE, "mxfp4.npz"), W=W, w_codes=codes, w_scales=e8, x=xa,
                         x_packed=a_packed, x_scales=a_scales, y=y)
+    mx_and_block_quant()
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
+
+
+def mx_and_block_quant():
+    """Weight-only MX layers, MXFP8 activations x MXFP4 weights, MXFP8 quantisers, and 128 x 128 block
+    quantisation (own generator, so that the files above do not depend on this section)."""
+    rng = np.random.default_rng(20240608)
+    N, K, M = 40, 256, 6
+    W = orc.round_to_bf16(rng.normal(0, 0.02, size=(N, K)).astype(np.float32))
+    W[:, 32:64] *= 8.0
+    x = orc.round_to_bf16(rng.normal(0, 1, size=(M, K)).astype(np.float32))
+    c4, e4 = orc.quantize_mxfp4_weights(W)
+    c8, e8 = orc.quantize_mxfp8_weights(W)
+    xq8, xs8 = orc.scale_activations_mxfp8(x)
+    xqt, xst = orc.scale_activations_per_token(x, False)
+    out = dict(W=W, x=x, w4_codes=c4, w4_scales=e4, w8_codes=c8, w8_scales=e8,
+               x_mxfp8_codes=xq8, x_mxfp8_scales=xs8, x_token_codes=xqt, x_token_scales=xst,
+               y_a16w4=orc.matmul_mx_mixed(x, "float", None, c4, "e2m1", e4),
+               y_a16w8=orc.matmul_mx_mixed(x, "float", None, c8, "e4m3", e8),
+               y_a8w4_token=orc.matmul_mx_mixed(xqt, "e4m3", None, c4, "e2m1", e4, scales_x=xst),
+               y_a8w4_mx=orc.matmul_mx_mixed(xq8, "e4m3", xs8[:M], c4, "e2m1", e4))
+    for name, to_int8 in (("int8", True), ("fp8", False)):
+        wq, ws = orc.quantize_block_weights(W, to_int8)
+        aq, asx = orc.scale_activations_per_block(x, to_int8)
+        a = aq if to_int8 else orc.e4m3fn_decode(aq)
+        b = wq if to_int8 else orc.e4m3fn_decode(wq)
+        out.update({f"bq_{name}_w_codes": wq, f"bq_{name}_w_scales": ws, f"bq_{name}_x_codes": aq,
+                    f"bq_{name}_x_scales": asx, f"bq_{name}_y": orc.matmul_block_quant(a, asx, b, ws)})
+    np.savez_compressed(os.path.join(HERE, "mx_blockq.npz"), **out)
 
 
 if __name__ == "__main__":

@@ -164,3 +164,67 @@ def test_hip_int8_and_mxfp4_products_match_golden(device):
         torch.from_numpy(m["w_codes"]).to(device), scales=torch.from_numpy(m["w_scales"]).to(device))
     y = layer(torch.from_numpy(m["x"]).to(torch.bfloat16).to(device))
     assert rel_frob(y.float().cpu().numpy(), m["y"]) <= 6e-3
+
+
+def test_oracle_reproduces_mx_and_block_quant():
+    z = load("mx_blockq.npz")
+    W, x = z["W"], z["x"]
+    M = x.shape[0]
+    c4, e4 = orc.quantize_mxfp4_weights(W)
+    c8, e8 = orc.quantize_mxfp8_weights(W)
+    assert np.array_equal(c4, z["w4_codes"]) and np.array_equal(e4, z["w4_scales"])
+    assert np.array_equal(c8, z["w8_codes"]) and np.array_equal(e8, z["w8_scales"])
+    xq8, xs8 = orc.scale_activations_mxfp8(x)
+    assert np.array_equal(xq8, z["x_mxfp8_codes"]) and np.array_equal(xs8, z["x_mxfp8_scales"])
+    assert np.array_equal(orc.matmul_mx_mixed(x, "float", None, c4, "e2m1", e4), z["y_a16w4"])
+    assert np.array_equal(orc.matmul_mx_mixed(x, "float", None, c8, "e4m3", e8), z["y_a16w8"])
+    assert np.array_equal(orc.matmul_mx_mixed(z["x_token_codes"], "e4m3", None, c4, "e2m1", e4, scales_x=z["x_token_scales"]),
+                          z["y_a8w4_token"])
+    assert np.array_equal(orc.matmul_mx_mixed(xq8, "e4m3", xs8[:M], c4, "e2m1", e4), z["y_a8w4_mx"])
+    # whatever produced the numbers: each result is the float matmul up to the formats' quantisation error,
+    # and the dequantised weights are within half a code step of the originals
+    ref = x.astype(np.float64) @ W.astype(np.float64).T
+    for key, tol in (("y_a16w4", 0.2), ("y_a16w8", 0.05), ("y_a8w4_token", 0.2), ("y_a8w4_mx", 0.2)):
+        assert rel_frob(z[key], ref) < tol, key
+    deq8 = orc.e4m3fn_decode(z["w8_codes"]) * np.repeat(orc.e8m0_decode(z["w8_scales"]), 32, axis=1)
+    assert np.all(np.abs(deq8 - W) <= np.abs(W) * 2.0 ** -4 + 1e-9)
+    for name, to_int8, tol in (("int8", True, 0.02), ("fp8", False, 0.06)):
+        wq, ws = orc.quantize_block_weights(W, to_int8)
+        aq, asx = orc.scale_activations_per_block(x, to_int8)
+        assert np.array_equal(wq, z[f"bq_{name}_w_codes"]) and np.array_equal(ws, z[f"bq_{name}_w_scales"])
+        assert np.array_equal(aq, z[f"bq_{name}_x_codes"]) and np.array_equal(asx, z[f"bq_{name}_x_scales"])
+        assert ws.shape == (1, 2) and asx.shape == (M, 2)
+        assert rel_frob(z[f"bq_{name}_y"], ref) < tol, name
+
+
+@pytest.mark.gpu
+def test_hip_mx_and_block_quant_match_golden(device):
+    import gemlite_amd
+    from gemlite_amd import helper
+    z = load("mx_blockq.npz")
+    x = torch.from_numpy(z["x"]).to(torch.bfloat16).to(device)
+    M = x.shape[0]
+    # quantisers: bit for bit
+    q, s = gemlite_amd.scale_activations_mxfp8(x)
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy(), z["x_mxfp8_codes"]) and np.array_equal(s.cpu().numpy(), z["x_mxfp8_scales"])
+    for name, dt in (("int8", torch.int8), ("fp8", torch.float8_e4m3fn)):
+        q, s = gemlite_amd.scale_activations_per_block(x, dt)
+        got = q.cpu().numpy() if dt == torch.int8 else q.view(torch.uint8).cpu().numpy()
+        assert np.array_equal(got, z[f"bq_{name}_x_codes"]) and np.array_equal(s.cpu().numpy(), z[f"bq_{name}_x_scales"])
+    w4, e4 = torch.from_numpy(z["w4_codes"]), torch.from_numpy(z["w4_scales"])
+    w8 = torch.from_numpy(z["w8_codes"]).view(torch.float8_e4m3fn)
+    cases = [
+        ("y_a16w4", helper.A16W4_MXFP(device=device, dtype=torch.bfloat16).from_weights(w4, e4)),
+        ("y_a16w8", helper.A16W8_MXFP(device=device, dtype=torch.bfloat16).from_weights(w8, torch.from_numpy(z["w8_scales"]))),
+        ("y_a8w4_token", helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_weights(w4, scales=e4)),
+        ("y_a8w4_mx", helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16, post_scale=False).from_weights(w4, scales=e4)),
+        ("bq_int8_y", helper.A8W8_INT8_dynamic(device=device, dtype=torch.bfloat16, block_quant=True).from_weights(
+            torch.from_numpy(z["bq_int8_w_codes"]), scales=torch.from_numpy(z["bq_int8_w_scales"]))),
+        ("bq_fp8_y", helper.A8W8_FP8_dynamic(device=device, dtype=torch.bfloat16, block_quant=True).from_weights(
+            torch.from_numpy(z["bq_fp8_w_codes"]).view(torch.float8_e4m3fn), scales=torch.from_numpy(z["bq_fp8_w_scales"]))),
+    ]
+    for key, layer in cases:
+        for rows in (M, 2):   # 6 rows: matrix-core kernels; 2 rows: the streaming kernels
+            y = layer(x[:rows])
+            torch.cuda.synchronize()
+            assert rel_frob(y.float().cpu().numpy(), z[key][:rows]) <= 6e-3, (key, rows)
