@@ -34,11 +34,11 @@ def candidate_configs(family: str, M: int, K: int) -> List[int]:
         bms = [32, 64] if M <= 32 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 512)]
-    if family == "GEMM_KBYTES":      # BM + 1000 * K splits
+    if family in ("GEMM_KBYTES", "GEMM_KBYTES_MX"):      # BM + 1000 * K splits
         bms = [64] if M <= 64 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 512)]
-    if family in ("GEMM_8BIT", "GEMM_MXFP4"):
+    if family in ("GEMM_8BIT", "GEMM_MXFP4", "GEMM_MXFP8"):
         bms = [64] if M <= 64 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 1024)]
