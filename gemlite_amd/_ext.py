@@ -74,6 +74,9 @@ class MatmulArgs(ctypes.Structure):
         ("zero_is_scalar", ctypes.c_int32),
         ("sx_dtype", ctypes.c_int32),
         ("tile_config", ctypes.c_int32),
+        ("bias", ctypes.c_void_p),
+        ("bias_dtype", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -227,7 +230,7 @@ def _dt(t: Optional[torch.Tensor], default: int = 0) -> int:
 def build_matmul_args(
     x, W_q, scales, zeros, scales_x, out, *,
     W_nbits, group_size, unpack_mask, elements_per_sample, input_dtype, output_dtype, acc_dtype, meta_dtype,
-    channel_scale_mode, W_group_mode, data_contiguous, matmul_type=MATMUL_AUTO, tile_config=-1,
+    channel_scale_mode, W_group_mode, data_contiguous, matmul_type=MATMUL_AUTO, tile_config=-1, bias=None,
 ) -> MatmulArgs:
     """Fill a ``gla_matmul_args`` from tensors and the reference's meta ints."""
     a = MatmulArgs()
@@ -278,6 +281,14 @@ def build_matmul_args(
     a.zero_is_scalar = int(has_zeros and zeros.numel() == 1)
     a.sx_dtype = _dt(scales_x, DType.FP32.value)
     a.tile_config = int(tile_config)
+    if bias is not None:
+        if bias.numel() < N or bias.stride(-1) != 1:
+            raise ValueError(f"bias: need {N} contiguous elements, got shape {tuple(bias.shape)} strides {bias.stride()}")
+        a.bias = bias.data_ptr()
+        a.bias_dtype = _dt(bias)
+    else:
+        a.bias = None
+        a.bias_dtype = 0
     _check_operand_bounds(a, x, W_q, scales if has_scales else None, zeros if has_zeros else None, scales_x, out, mx)
     return a
 

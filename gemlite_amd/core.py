@@ -194,14 +194,18 @@ def forward_functional(
     else:
         matmul_type_str = get_matmul_type(M, W_nbits, mx)
 
-    out = GEMLITE_TRITON_MAPPING[matmul_type_str].forward(
+    # the library adds a floating-point bias itself (in the GEMV epilogue, or with one small launch after
+    # the other kernels); anything else is added here like the reference does (gemlite/core.py:271-272)
+    fused_bias = bias is not None and bias.dtype in _BIAS_DTYPES and DTYPE_TO_TORCH[output_dtype] in _BIAS_DTYPES \
+        and bias.dim() == 1 and bias.is_contiguous() and bias.device == x2d.device
+    out = _KERNEL_FORWARD[matmul_type_str](
         x2d, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
         kernel_input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
-        data_contiguous, get_type_id(input_dtype, W_nbits),
+        data_contiguous, get_type_id(input_dtype, W_nbits), bias=bias if fused_bias else None,
     )
 
     out = out.view(out_shape)
-    if bias is not None:
+    if bias is not None and not fused_bias:
         out += bias
     return out
 
@@ -227,7 +231,7 @@ def _kernel_forward(matmul_type_str):
 
     def forward(x, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
                 input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
-                data_contiguous, type_id, meta_scale=0.0):
+                data_contiguous, type_id, meta_scale=0.0, bias=None):
         M, K, N = x.shape[0], W_q.shape[0] * elements_per_sample, W_q.shape[1]
         out = torch.empty((M, N), dtype=DTYPE_TO_TORCH[int(output_dtype)], device=x.device)
         if M == 0:
@@ -240,7 +244,7 @@ def _kernel_forward(matmul_type_str):
         key = (id(W_q), W_q.shape, W_q.stride(), _thread_id(), matmul_type_id, x.shape, x.stride(), x.dtype, sx_key,
                x.device.index, W_nbits, group_size,
                unpack_mask, elements_per_sample, input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode,
-               W_group_mode, data_contiguous, tile)
+               W_group_mode, data_contiguous, tile, None if bias is None else (bias.data_ptr(), bias.dtype))
         hit = _PREPARED.get(key)
         if hit is not None:
             args, need, w_ptr, s_ptr, z_ptr = hit
@@ -255,7 +259,7 @@ def _kernel_forward(matmul_type_str):
             elements_per_sample=elements_per_sample, input_dtype=input_dtype, output_dtype=output_dtype,
             acc_dtype=acc_dtype, meta_dtype=meta_dtype, channel_scale_mode=channel_scale_mode,
             W_group_mode=W_group_mode, data_contiguous=data_contiguous,
-            matmul_type=matmul_type_id, tile_config=tile,
+            matmul_type=matmul_type_id, tile_config=tile, bias=bias,
         )
         need = _ext.matmul_workspace_need(args)
         _ext.matmul_prepared(args, need, args.x, args.out, args.scales_x, x.device)
@@ -267,11 +271,25 @@ def _kernel_forward(matmul_type_str):
     return forward
 
 
+_BIAS_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
+_KERNEL_FORWARD = {}  # matmul type -> forward with the extra `bias` argument (what forward_functional calls)
+
+
 def _kernel_class(matmul_type_str):
+    inner = _KERNEL_FORWARD[matmul_type_str] = _kernel_forward(matmul_type_str)
+
+    def forward(x, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
+                input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
+                data_contiguous, type_id, meta_scale=0.0):
+        # the reference's argument list, which has no bias
+        return inner(x, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
+                     input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
+                     data_contiguous, type_id, meta_scale)
+
     return type(matmul_type_str.lower(), (), {
         "kernel": ["gla_matmul"],
         "matmul_type": matmul_type_str,
-        "forward": staticmethod(_kernel_forward(matmul_type_str)),
+        "forward": staticmethod(forward),
         "__doc__": f"Kernel plug-in for matmul type {matmul_type_str}: forward(x, W_q, scales, zeros, scales_x, "
                    "W_nbits, ..., type_id) -> Tensor[M, N], backed by the C ABI.",
     })

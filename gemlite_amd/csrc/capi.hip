@@ -69,6 +69,15 @@ int validate(const gla_matmul_args* p) {
         set_error("matmul: x, w and out must not be NULL");
         return GLA_ERR_INVALID_ARGUMENT;
     }
+    if (p->bias != nullptr) {
+        const int odt = p->output_dtype;
+        const bool float_out = odt == GLA_DT_FP32 || odt == GLA_DT_FP16 || odt == GLA_DT_BF16 || odt == GLA_DT_MXFP16 || odt == GLA_DT_MXBF16;
+        const bool float_bias = p->bias_dtype == GLA_DT_FP32 || p->bias_dtype == GLA_DT_FP16 || p->bias_dtype == GLA_DT_BF16;
+        if (!float_out || !float_bias) {
+            set_error("matmul: a bias needs a floating-point output (type %d) and an fp16, bf16 or fp32 bias (type %d)", odt, p->bias_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+        }
+    }
     if (p->matmul_type < GLA_MATMUL_AUTO || p->matmul_type > GLA_MATMUL_GEMM) {
         set_error("matmul: matmul_type %d out of range", p->matmul_type);
         return GLA_ERR_UNSUPPORTED_MODE;
@@ -239,20 +248,24 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
     if (rc != GLA_OK) return rc;
     if (args->M == 0) return GLA_OK;
     hipStream_t s = (hipStream_t)stream;
-    switch (choose(*args, resolve_type(*args))) {
-        case F_GEMV_PACKED: return launch_gemv_packed(*args, s);
-        case F_GEMV_KMAJOR: return launch_gemv_kmajor(*args, s);
-        case F_GEMM_WN: return launch_gemm_wn(*args, s);
-        case F_GEMM_8BIT: return launch_gemm_8bit(*args, s);
-        case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
-        case F_GEMM_KBYTES: return launch_gemm_kbytes(*args, s);
-        case F_GEMM_MXFP8: return launch_gemm_mxfp8(*args, s);
-        case F_MX_STREAM: return launch_mx_stream(*args, s);
-        case F_BLOCKQ_STREAM: return launch_blockq_stream(*args, s);
-        case F_GEMM_BLOCKQ: return launch_gemm_blockq(*args, s);
-        case F_GEMM_KBYTES_MX: return launch_gemm_kbytes_mx(*args, s);
-        default: return launch_generic(*args, s);
+    const Family f = choose(*args, resolve_type(*args));
+    int rc2;
+    switch (f) {
+        case F_GEMV_PACKED: return launch_gemv_packed(*args, s);  // adds the bias in its epilogue
+        case F_GEMV_KMAJOR: rc2 = launch_gemv_kmajor(*args, s); break;
+        case F_GEMM_WN: rc2 = launch_gemm_wn(*args, s); break;
+        case F_GEMM_8BIT: rc2 = launch_gemm_8bit(*args, s); break;
+        case F_GEMM_MXFP4: rc2 = launch_gemm_mxfp4(*args, s); break;
+        case F_GEMM_KBYTES: rc2 = launch_gemm_kbytes(*args, s); break;
+        case F_GEMM_MXFP8: rc2 = launch_gemm_mxfp8(*args, s); break;
+        case F_MX_STREAM: rc2 = launch_mx_stream(*args, s); break;
+        case F_BLOCKQ_STREAM: rc2 = launch_blockq_stream(*args, s); break;
+        case F_GEMM_BLOCKQ: rc2 = launch_gemm_blockq(*args, s); break;
+        case F_GEMM_KBYTES_MX: rc2 = launch_gemm_kbytes_mx(*args, s); break;
+        default: rc2 = launch_generic(*args, s); break;
     }
+    if (rc2 == GLA_OK && args->bias != nullptr) rc2 = launch_bias_add(*args, s);
+    return rc2;
 }
 
 int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y,

@@ -120,6 +120,13 @@ __device__ __forceinline__ void store_from_float(void* p, int dt, int64_t idx, f
     }
 }
 
+// `v` as the output type `dt` holds it (fp16 / bf16 rounding; fp32 as it is).
+__device__ __forceinline__ float round_to_dtype(int dt, float v) {
+    if (dt == GLA_DT_FP16) return half_bits_to_float(float_to_half_bits(v));
+    if (dt == GLA_DT_BF16) return bf16_bits_to_float(float_to_bf16_bits(v));
+    return v;
+}
+
 // Store with the element type fixed at compile time (DT is a GLA_DT_* id).
 template <int DT>
 __device__ __forceinline__ void store_typed(void* p, int64_t idx, float v) {

@@ -7,6 +7,8 @@ namespace gla {
 
 // ---- layout-agnostic path (generic.hip) -----------------------------------
 int launch_generic(const gla_matmul_args& p, hipStream_t stream);
+// out += bias on the finished output, for the families that do not add the bias in their epilogue
+int launch_bias_add(const gla_matmul_args& p, hipStream_t stream);
 
 // ---- streaming GEMV on 32-bit packed words, N fastest (gemv_packed.hip) ----
 // tile_config (when >= 1000) = waves per workgroup * 1000 + load batches per wave.

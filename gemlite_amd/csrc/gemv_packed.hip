@@ -69,6 +69,8 @@ struct GemvArgs {
     int fl_log2;  // log2(FL)
     int wgm, csm, meta_dt, z_dt, z_scalar, out_dt, sx_dt;
     int64_t wsk, xsm, osm, msg, sxm;
+    const void* bias;  // [N] or NULL: added to the result rounded to the output type
+    int bias_dt;
 };
 
 template <bool BF16>
@@ -159,6 +161,8 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
     constexpr int NT = (RT + kWaves - 1) / kWaves;  // output rows per thread
     const int n_out = n0 + lane;
     const bool col_ok = n_out < a.N;
+    // loaded before the reduction, so that its latency is not the kernel's tail
+    const float bias = (a.bias != nullptr && col_ok) ? load_as_float(a.bias, a.bias_dt, n_out) : 0.0f;
     float total[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -233,6 +237,7 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
             v *= load_as_float(a.scales_x, a.sx_dt, (int64_t)(m0 + m) * a.sxm) *
                  load_as_float(a.scales, a.meta_dt, n_out);
         }
+        if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + bias;  // `out += bias` on the rounded output
         store_from_float(a.out, a.out_dt, (int64_t)(m0 + m) * a.osm + n_out, v);
     }
     GLA_STAMP(5);
@@ -939,6 +944,7 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
 #endif
     a.w = (const uint32_t*)p.w; a.x = p.x; a.scales = p.scales; a.zeros = p.zeros; a.scales_x = p.scales_x;
     a.out = p.out; a.partials = nullptr; a.counters = nullptr;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     if (g.S > 1) {
         const int64_t need = gemv_packed_workspace_bytes(p);
         if (p.workspace == nullptr || (int64_t)p.workspace_bytes < need) {

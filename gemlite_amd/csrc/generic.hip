@@ -176,7 +176,26 @@ __global__ __launch_bounds__(64) void generic_mxfp4_kernel(GenericArgs a) {
     }
 }
 
+// out[m, n] = cast(out[m, n] + bias[n]): the reference's `out += bias` on the finished output
+// (reference: gemlite/core.py:271-272), for the kernel families that do not add the bias themselves.
+__global__ __launch_bounds__(256) void bias_add_kernel(void* out, const void* bias, int M, int N, int64_t osm, int64_t osn,
+                                                       int out_dt, int bias_dt) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)M * N) return;
+    const int m = (int)(idx / N), n = (int)(idx % N);
+    const int64_t o = (int64_t)m * osm + (int64_t)n * osn;
+    store_from_float(out, out_dt, o, load_as_float(out, out_dt, o) + load_as_float(bias, bias_dt, n));
+}
+
 }  // namespace
+
+int launch_bias_add(const gla_matmul_args& p, hipStream_t stream) {
+    const int out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
+    const int64_t items = (int64_t)p.M * p.N;
+    hipLaunchKernelGGL(bias_add_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, p.out, p.bias, p.M, p.N,
+                       p.out_stride_m, p.out_stride_n, out_dt, p.bias_dtype);
+    return check_hip(hipGetLastError(), "bias add launch");
+}
 
 int launch_generic(const gla_matmul_args& p, hipStream_t stream) {
     GenericArgs a;

@@ -130,6 +130,14 @@ typedef struct gla_matmul_args {
     int32_t zero_is_scalar; /* zeros holds a single element */
     int32_t sx_dtype;       /* element type of scales_x (FP32 or UINT8/E8M0) */
     int32_t tile_config;    /* -1 = library heuristic, else an id from gla_select_config */
+
+    /* Optional bias [N] (fp16, bf16 or fp32), or NULL: out = cast(cast(acc ...) + bias[n]), i.e. added to the
+     * result already rounded to the output type, as the reference's `out += bias` does
+     * (reference: gemlite/core.py:271-272).  Float output types only.  The streaming GEMV on packed codes
+     * adds it in its epilogue; the other kernel families are followed by one small launch on the same stream. */
+    const void* bias;
+    int32_t bias_dtype;
+    int32_t reserved0;
 } gla_matmul_args;
 
 /* Library identification.  No reference counterpart. */

@@ -671,3 +671,44 @@ def test_ternary_weight_layers(device, dtype):
     torch.cuda.synchronize()
     want = xi.double() @ W.double().T
     assert np.array_equal(to_np(y).astype(np.float64), want.numpy())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_bias_is_added_to_the_rounded_output_like_the_reference(device, dtype):
+    """`out += bias` on the output already rounded to its type (reference: gemlite/core.py:271-272): a layer with
+    a bias must equal the same layer without one plus the bias, bit for bit, whether the kernel adds it in its
+    epilogue (packed-code GEMV, up to 16 rows) or the library adds it with a launch of its own."""
+    N, K = 1032, 2048
+    bias = gen_x(1, N, dtype, seed=77).reshape(-1).to(device)
+    W_q, s, z = gen_int_case(N, K, 4, 128, dtype, seed=5)
+    in_dt = DType.FP16 if dtype == torch.float16 else DType.BF16
+    W = gen_x(N, K, torch.bfloat16, seed=6, std=0.02)
+    lin = torch.nn.Linear(K, N, bias=False, dtype=dtype)
+    lin.weight.data = W.to(dtype)
+
+    def pair(make):
+        a, b = make(), make()
+        b.bias = torch.nn.Parameter(bias.clone(), requires_grad=False)
+        return a, b
+
+    cases = {
+        "A16W4": pair(lambda: GemLiteLinear(4, 128, K, N, in_dt, in_dt).pack(W_q.to(device), s.to(device), z.to(device))),
+        "A8W8 fp8": pair(lambda: helper.A8W8_FP8_dynamic(device=device).from_weights(W.to(dtype))),
+        "A16W4_MXFP": pair(lambda: helper.A16W4_MXFP(device=device, dtype=dtype).from_linear(lin.to(device), del_orig=False)),
+        "block-quantised": pair(lambda: helper.A8W8_FP8_dynamic(device=device, block_quant=True).from_weights(W.to(dtype))),
+    }
+    for name, (plain, biased) in cases.items():
+        for M in (1, 2, 5, 16, 70):
+            x = gen_x(M, K, dtype, seed=M).to(device)
+            want = plain(x) + bias
+            got = biased(x)
+            torch.cuda.synchronize()
+            assert got.dtype == want.dtype and torch.equal(got, want), (name, M)
+    # a bias the library does not take (fp32 bias on an fp16 output is fine; an integer output is not) still works
+    y32 = cases["A16W4"][1]
+    y32.bias = torch.nn.Parameter(bias.float(), requires_grad=False)
+    x = gen_x(3, K, dtype, seed=3).to(device)
+    got = y32(x)
+    torch.cuda.synchronize()
+    assert torch.equal(got, (cases["A16W4"][0](x).float() + bias.float()).to(dtype))
