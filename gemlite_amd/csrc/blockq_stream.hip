@@ -32,6 +32,8 @@ struct BqArgs {
     int M, N, pieces;  // pieces = K / 16
     int64_t xsm, wsn, osm, osn, msg, msn, sxm, sxg;
     int out_dt;
+    const void* bias;  // [N] or NULL: added to the result rounded to the output type
+    int bias_dt;
 };
 
 typedef uint32_t u32x4q __attribute__((ext_vector_type(4)));
@@ -110,8 +112,10 @@ __global__ __launch_bounds__(256) void blockq_stream_kernel(BqArgs a) {
             float v = acc[r][c];
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) v += wave_xor(v, off);
-            if (lane == 0 && m < a.M && n0 + c < a.N)
+            if (lane == 0 && m < a.M && n0 + c < a.N) {
+                if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + load_as_float(a.bias, a.bias_dt, n0 + c);
                 store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)(n0 + c) * a.osn, v);
+            }
         }
     }
 }
@@ -154,6 +158,7 @@ int launch_blockq_stream(const gla_matmul_args& p, hipStream_t stream) {
     a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.osn = p.out_stride_n;
     a.msg = p.meta_stride_g; a.msn = p.meta_stride_n; a.sxm = p.sx_stride_m; a.sxg = p.sx_stride_g;
     a.out_dt = p.output_dtype;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     const int rm = p.M >= 5 ? 8 : (p.M >= 3 ? 4 : p.M);
     dim3 grid(ceil_div(p.N, 4 * kColsQ), ceil_div(p.M, rm));
     if (p.input_dtype == GLA_DT_FP8) launch_rows_q<true>(a, rm, grid, stream);

@@ -252,14 +252,14 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
     int rc2;
     switch (f) {
         case F_GEMV_PACKED: return launch_gemv_packed(*args, s);  // adds the bias in its epilogue
-        case F_GEMV_KMAJOR: rc2 = launch_gemv_kmajor(*args, s); break;
+        case F_GEMV_KMAJOR: return launch_gemv_kmajor(*args, s);  // adds the bias in its epilogue
         case F_GEMM_WN: rc2 = launch_gemm_wn(*args, s); break;
         case F_GEMM_8BIT: rc2 = launch_gemm_8bit(*args, s); break;
         case F_GEMM_MXFP4: rc2 = launch_gemm_mxfp4(*args, s); break;
         case F_GEMM_KBYTES: rc2 = launch_gemm_kbytes(*args, s); break;
         case F_GEMM_MXFP8: rc2 = launch_gemm_mxfp8(*args, s); break;
-        case F_MX_STREAM: rc2 = launch_mx_stream(*args, s); break;
-        case F_BLOCKQ_STREAM: rc2 = launch_blockq_stream(*args, s); break;
+        case F_MX_STREAM: return launch_mx_stream(*args, s);  // adds the bias in its epilogue
+        case F_BLOCKQ_STREAM: return launch_blockq_stream(*args, s);  // adds the bias in its epilogue
         case F_GEMM_BLOCKQ: rc2 = launch_gemm_blockq(*args, s); break;
         case F_GEMM_KBYTES_MX: rc2 = launch_gemm_kbytes_mx(*args, s); break;
         default: rc2 = launch_generic(*args, s); break;

@@ -45,7 +45,15 @@ struct GemvKArgs {
     int M, N, K;
     int64_t xsm, wsn, osm, msn, sxm;
     int wgm, csm, meta_dt, z_dt, z_scalar, out_dt, sx_dt;
+    const void* bias;  // [N] or NULL: added to the result rounded to the output type
+    int bias_dt;
 };
+
+// store v, or with a bias round(v) + bias[n]: the reference's `out += bias` on the rounded output
+__device__ __forceinline__ void store_result(const GemvKArgs& a, int m, int n, float v) {
+    if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + load_as_float(a.bias, a.bias_dt, n);
+    store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + n, v);
+}
 
 // 16 codes (one 128-bit load) -> 16 floats.  Signed bytes come out biased by +128.
 template <int WDT>
@@ -170,7 +178,7 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     float post = 1.0f;
     if (a.csm & 1) post *= load_as_float(a.scales, a.meta_dt, (int64_t)n * a.msn);
     if (a.csm & 2) post *= load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
-    store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + n, v * post);
+    store_result(a, m, n, v * post);
 }
 
 // ---- 3..16 rows: the same streaming on the matrix cores.  A workgroup of 16 waves owns 16 weight
@@ -317,7 +325,7 @@ __global__ __launch_bounds__(kWavesKM * 64) void gemv_kmajor_mfma_kernel(GemvKAr
             }
             float post = sxm;
             if (a.csm & 1) post *= load_as_float(a.scales, a.meta_dt, (int64_t)n * a.msn);
-            store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + n, v * post);
+            store_result(a, m, n, v * post);
         }
     }
 }
@@ -372,6 +380,7 @@ int launch_gemv_kmajor(const gla_matmul_args& p, hipStream_t stream) {
     a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = p.meta_stride_n; a.sxm = p.sx_stride_m;
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.z_scalar = p.zero_is_scalar; a.out_dt = p.output_dtype; a.sx_dt = p.sx_dtype;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     const bool bf16 = p.input_dtype == GLA_DT_BF16;
     switch (p.w_dtype) {
         case GLA_DT_INT8: return bf16 ? launch_k<GLA_DT_INT8, true>(a, stream) : launch_k<GLA_DT_INT8, false>(a, stream);

@@ -44,6 +44,8 @@ struct MxArgs {
     int M, N, KB;  // KB = K / 32
     int64_t xsm_bytes, wsn_bytes, osm, osn, msg, msn, sxm, sxg;
     int csm, out_dt;
+    const void* bias;  // [N] or NULL: added to the result rounded to the output type
+    int bias_dt;
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -188,8 +190,11 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
             float v = acc[r][c];
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) v += wave_xor(v, off);
-            if (lane == 0 && m < a.M && n0 + c < a.N)
-                store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)(n0 + c) * a.osn, v * rs);
+            if (lane == 0 && m < a.M && n0 + c < a.N) {
+                v *= rs;
+                if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + load_as_float(a.bias, a.bias_dt, n0 + c);
+                store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)(n0 + c) * a.osn, v);
+            }
         }
     }
 }
@@ -259,6 +264,7 @@ int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream) {
     a.osm = p.out_stride_m; a.osn = p.out_stride_n;
     a.msg = p.meta_stride_g; a.msn = p.meta_stride_n; a.sxm = p.sx_stride_m; a.sxg = p.sx_stride_g;
     a.csm = p.channel_scale_mode;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
     const int rm = p.M >= 5 ? 8 : (p.M >= 3 ? 4 : p.M);
     const int bk = p.elements_per_sample == 2 ? B_FP4 : B_FP8;

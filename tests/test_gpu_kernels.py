@@ -697,6 +697,9 @@ def test_bias_is_added_to_the_rounded_output_like_the_reference(device, dtype):
         "A8W8 fp8": pair(lambda: helper.A8W8_FP8_dynamic(device=device).from_weights(W.to(dtype))),
         "A16W4_MXFP": pair(lambda: helper.A16W4_MXFP(device=device, dtype=dtype).from_linear(lin.to(device), del_orig=False)),
         "block-quantised": pair(lambda: helper.A8W8_FP8_dynamic(device=device, block_quant=True).from_weights(W.to(dtype))),
+        "A16W8 bytes": pair(lambda: helper.A16W8_INT8(device=device, dtype=dtype).from_weights(
+            *gemlite_amd.quantize_weights_per_channel(W.to(dtype), torch.int8)[:1],
+            scales=gemlite_amd.quantize_weights_per_channel(W.to(dtype), torch.int8)[1])),
     }
     for name, (plain, biased) in cases.items():
         for M in (1, 2, 5, 16, 70):
