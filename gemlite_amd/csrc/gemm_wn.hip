@@ -64,6 +64,8 @@ struct GemmWnArgs {
     int S;    // K splits (gridDim.y)
     int sps;  // pipeline stages per split
     float* partials;  // [S][M][N] when S > 1
+    const void* bias;  // [N] or NULL: added to the result rounded to the output type
+    int bias_dt;
 };
 
 __device__ __forceinline__ void tile_coords_wn(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -556,6 +558,9 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
             float sb[RUN];
 #pragma unroll
             for (int c = 0; c < RUN; ++c) sb[c] = ((p.csm & 1) && col + c < p.N) ? load_as_float(p.scales, p.meta_dt, col + c) : 1.0f;
+            float bv[RUN];
+#pragma unroll
+            for (int c = 0; c < RUN; ++c) bv[c] = (p.bias != nullptr && col + c < p.N) ? load_as_float(p.bias, p.bias_dt, col + c) : 0.0f;
 #pragma unroll
             for (int i = 0; i < TI; ++i) {
                 const int m = m0 + wm * WM + i * 32 + r32;
@@ -563,6 +568,10 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
                 float v[RUN];
 #pragma unroll
                 for (int c = 0; c < RUN; ++c) v[c] = acc[i][c % TJ][4 * g + c / TJ] * (sa[i] * sb[c]);
+                if (p.bias != nullptr) {  // `out += bias` on the rounded output
+#pragma unroll
+                    for (int c = 0; c < RUN; ++c) v[c] = round_to_dtype(DT, v[c]) + bv[c];
+                }
                 const int64_t o = (int64_t)m * p.osm + col;
                 constexpr int PER = 16 / ES;  // elements per 16-byte store
 #pragma unroll
@@ -609,7 +618,9 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmWnArgs p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const float sb = (p.csm & 1) ? load_as_float(p.scales, p.meta_dt, n + j) : 1.0f;
-        store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n + j, v[j] * (sa * sb));
+        float r = v[j] * (sa * sb);
+        if (p.bias != nullptr) r = round_to_dtype(p.out_dt, r) + load_as_float(p.bias, p.bias_dt, n + j);
+        store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n + j, r);
     }
 }
 
@@ -732,6 +743,7 @@ int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream) {
     a.xsm = p.x_stride_m; a.wsk = p.w_stride_k; a.osm = p.out_stride_m; a.msg = p.meta_stride_g; a.sxm = p.sx_stride_m;
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.z_scalar = p.zero_is_scalar; a.out_dt = p.output_dtype; a.sx_dt = p.sx_dtype;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     const WnPlan g = wn_plan(p);
     a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps;
     a.partials = nullptr;
