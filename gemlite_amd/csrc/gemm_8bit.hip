@@ -72,8 +72,6 @@ struct Gemm8Args {
     int S;     // K splits (gridDim.y)
     int sps;   // pipeline stages per split
     void* partials;  // [S][M][N] 32-bit accumulators when S > 1
-    const void* bias;  // [N] or NULL: added to the result rounded to the output type
-    int bias_dt;
 };
 
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -557,10 +555,6 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                             float v[4];
 #pragma unroll
                             for (int t = 0; t < 4; ++t) v[t] = value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]);
-                            if (p.bias != nullptr) {  // `out += bias` on the rounded output
-#pragma unroll
-                                for (int t = 0; t < 4; ++t) v[t] = round_to_dtype(DT, v[t]) + load_as_float(p.bias, p.bias_dt, n + t);
-                            }
                             if constexpr (DT == GLA_DT_FP32) {
                                 *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
                             } else {
@@ -580,11 +574,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                         for (int t = 0; t < 4; ++t) {
                             if (n + t >= p.N) continue;
                             if constexpr (DT == GLA_DT_INT32) ((int32_t*)p.out)[o + t] = (int32_t)acc[i][j][4 * g + t];
-                            else {
-                                float r = value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]);
-                                if (p.bias != nullptr) r = round_to_dtype(DT, r) + load_as_float(p.bias, p.bias_dt, n + t);
-                                store_typed<DT>(p.out, o + t, r);
-                            }
+                            else store_typed<DT>(p.out, o + t, value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]));
                         }
                     }
                 }
@@ -611,17 +601,11 @@ __global__ __launch_bounds__(256) void splitk_finish8_kernel(Gemm8Args p) {
         int32_t v = 0;
         for (int s = 0; s < p.S; ++s) v += ((const int32_t*)p.partials)[s * slab + idx];
         if (p.out_dt == GLA_DT_INT32) ((int32_t*)p.out)[o] = v;
-        else {
-            float r = (float)v * scale;
-            if (p.bias != nullptr) r = round_to_dtype(p.out_dt, r) + load_as_float(p.bias, p.bias_dt, n);
-            store_from_float(p.out, p.out_dt, o, r);
-        }
+        else store_from_float(p.out, p.out_dt, o, (float)v * scale);
     } else {
         float v = 0.0f;
         for (int s = 0; s < p.S; ++s) v += ((const float*)p.partials)[s * slab + idx];
-        float r = v * scale;
-        if (p.bias != nullptr) r = round_to_dtype(p.out_dt, r) + load_as_float(p.bias, p.bias_dt, n);
-        store_from_float(p.out, p.out_dt, o, r);
+        store_from_float(p.out, p.out_dt, o, v * scale);
     }
 }
 
@@ -750,7 +734,6 @@ bool gemm_8bit_eligible(const gla_matmul_args& p) {
 
 int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     Gemm8Args a;
-    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
@@ -799,7 +782,6 @@ int launch_gemm_blockq(const gla_matmul_args& p, hipStream_t stream) {
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     Gemm8Args a;
-    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     // block scales travel with the stages like micro-scales: byte strides per row / per 128-block of K
@@ -850,7 +832,6 @@ bool gemm_mxfp4_eligible(const gla_matmul_args& p) {
 
 int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
     Gemm8Args a;
-    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K / 2; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.csm = 0; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
@@ -921,7 +902,6 @@ int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p) {
 
 int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
     Gemm8Args a;
-    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     const bool act_blocks = p.channel_scale_mode == GLA_CSM_MX;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;

@@ -70,8 +70,6 @@ struct GemmKbArgs {
     float* partials;
     const uint8_t* bscales;  // micro-scaled weights: e8m0 block scales [N, K/32], K contiguous
     int64_t bsn;             // ... bytes from one row's scales to the next
-    const void* bias;        // [N] or NULL: added to the result rounded to the output type
-    int bias_dt;
 };
 
 __device__ __forceinline__ void tile_coords_kb(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -453,11 +451,6 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
                     float v[4];
 #pragma unroll
                     for (int t = 0; t < 4; ++t) v[t] = acc[i][j][4 * g + t] * (sa * sb[j][4 * g + t]);
-                    if (p.bias != nullptr) {  // `out += bias` on the rounded output
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            if (n + t < p.N) v[t] = round_to_dtype(DT, v[t]) + load_as_float(p.bias, p.bias_dt, n + t);
-                    }
                     if (wide && n + 3 < p.N) {
                         if constexpr (DT == GLA_DT_FP32) {
                             *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
@@ -494,9 +487,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kb_kernel(GemmKbArgs p) {
         const float s = load_as_float(p.scales, p.meta_dt, (int64_t)n * p.msn);
         sc *= p.col_scale == 2 ? s * s : s;
     }
-    float r = v * sc;
-    if (p.bias != nullptr) r = round_to_dtype(p.out_dt, r) + load_as_float(p.bias, p.bias_dt, n);
-    store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n, r);
+    store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n, v * sc);
 }
 
 template <int WDT, bool BF16, int WAVES_M, int TI>
@@ -620,7 +611,6 @@ int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream) {
     a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = 0; a.sxm = 0;
     a.col_scale = 0; a.row_scale = 0;
     a.bscales = (const uint8_t*)p.scales; a.bsn = p.meta_stride_n;
-    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
     const KbPlan g = kb_plan(p);
@@ -650,7 +640,6 @@ int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream) {
     a.row_scale = (p.channel_scale_mode & 2) ? 1 : 0;
     a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
     a.bscales = nullptr; a.bsn = 0;
-    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     const KbPlan g = kb_plan(p);
     a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps;
     a.partials = nullptr;

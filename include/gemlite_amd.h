@@ -133,9 +133,9 @@ typedef struct gla_matmul_args {
 
     /* Optional bias [N] (fp16, bf16 or fp32), or NULL: out = cast(cast(acc ...) + bias[n]), i.e. added to the
      * result already rounded to the output type, as the reference's `out += bias` does
-     * (reference: gemlite/core.py:271-272).  Float output types only.  The tuned kernel families
-     * add it in their epilogue (or split-K finishing kernel); the layout-agnostic kernel is followed by one
-     * small launch on the same stream. */
+     * (reference: gemlite/core.py:271-272).  Float output types only.  The streaming (decode) kernels
+     * and the packed-code GEMM add it in their epilogue; the other kernels are followed by one small launch
+     * on the same stream. */
     const void* bias;
     int32_t bias_dtype;
     int32_t reserved0;
