@@ -191,34 +191,55 @@ def get_closest_m(M: int) -> int:
 
 
 # ---------------------------------------------------------------------------
-# workspace: one zero-initialised scratch tensor per device, grown on demand
+# workspace: one zero-initialised scratch tensor per (device, stream), grown on demand
 # ---------------------------------------------------------------------------
 _workspaces = {}
 _retired_workspaces = []  # outgrown buffers stay allocated: a captured HIP graph may still point at them
+_workspace_lock = threading.Lock()
 
 
-def get_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+def _workspace_key(device: torch.device, stream: int):
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return (device.type, index, int(stream))
+
+
+def get_workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> torch.Tensor:
     """Scratch memory for split-K partials, ticket counters and regrouped block scales.
+
+    Keyed by the device and the raw handle of the stream the launch goes to (the current stream when
+    ``stream`` is None): kernels on one stream run in order and may share scratch, kernels on
+    different streams may overlap and must not, so each stream that launches a matmul needing
+    scratch gets a buffer of its own.  A graph captured on a stream keeps pointing at that stream's
+    buffer, whichever stream replays it.
 
     Growing replaces the buffer (at least doubling, so the outgrown ones add up to less than the
     live one) and never frees the old one.  Growing while the stream is being captured into a graph
     is refused: the fill that zeroes the new buffer would become a node of the graph.  Run the
-    layer once before capturing it.
+    layer once on that stream before capturing it.
     """
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    if stream is None:
+        stream = _stream_ptr(device)
+    key = _workspace_key(device, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError(
-                f"gemlite_amd: the workspace has to grow to {int(nbytes)} bytes while a graph is being captured; "
-                "run the layer once at this shape before capturing"
-            )
-        size = max(int(nbytes), 8 << 20, 0 if ws is None else 2 * ws.numel())
-        if ws is not None:
-            _retired_workspaces.append(ws)
-        ws = torch.zeros(size, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+        with _workspace_lock:
+            ws = _workspaces.get(key)
+            if ws is None or ws.numel() < nbytes:
+                if torch.cuda.is_current_stream_capturing():
+                    raise RuntimeError(
+                        f"gemlite_amd: the workspace of this stream has to grow to {int(nbytes)} bytes while a graph "
+                        "is being captured; run the layer once at this shape on the capture stream before capturing"
+                    )
+                size = max(int(nbytes), 8 << 20, 0 if ws is None else 2 * ws.numel())
+                if ws is not None:
+                    _retired_workspaces.append(ws)
+                ws = _new_workspace(size, device)
+                _workspaces[key] = ws
     return ws
+
+
+def _new_workspace(size: int, device: torch.device) -> torch.Tensor:
+    return torch.zeros(size, dtype=torch.uint8, device=device)
 
 
 def _dt(t: Optional[torch.Tensor], default: int = 0) -> int:
@@ -345,11 +366,12 @@ def matmul(args: MatmulArgs, device: torch.device):
     need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))
     if need < 0:
         _check(int(need), "gla_matmul_workspace_bytes")
+    stream = _stream_ptr(device)
     if need > 0:
-        ws = get_workspace(device, need)
+        ws = get_workspace(device, need, stream)
         args.workspace = ws.data_ptr()
         args.workspace_bytes = ws.numel()
-    _check(lib.gla_matmul(ctypes.byref(args), _stream_ptr(device)), "gla_matmul")
+    _check(lib.gla_matmul(ctypes.byref(args), stream), "gla_matmul")
 
 
 def matmul_prepared(args: MatmulArgs, need: int, x_ptr: int, out_ptr: int, sx_ptr, device: torch.device):
@@ -360,11 +382,12 @@ def matmul_prepared(args: MatmulArgs, need: int, x_ptr: int, out_ptr: int, sx_pt
     args.x = x_ptr
     args.out = out_ptr
     args.scales_x = sx_ptr
+    stream = _stream_ptr(device)
     if need > 0:
-        ws = get_workspace(device, need)
+        ws = get_workspace(device, need, stream)
         args.workspace = ws.data_ptr()
         args.workspace_bytes = ws.numel()
-    status = load_library().gla_matmul(ctypes.byref(args), _stream_ptr(device))
+    status = load_library().gla_matmul(ctypes.byref(args), stream)
     if status != GLA_OK:
         _check(status, "gla_matmul")
 

@@ -299,8 +299,10 @@ GEMLITE_TRITON_MAPPING = {name: _kernel_class(name) for name in GEMLITE_MATMUL_T
 
 
 # The same function as a torch custom op with a fake (meta) implementation, so that graphs traced
-# by torch.compile can hold it as one opaque node (reference: gemlite/core.py:193-200, :276-285).
-# The module's forward calls the plain function: eager decode steps do not pay the op dispatch.
+# by torch.compile hold it as one opaque node instead of tracing into ctypes
+# (reference: gemlite/core.py:193-200, :276-285).  The module's forward goes through the op while
+# a graph is being traced and calls the plain function otherwise: eager decode steps do not pay the
+# op dispatch (~10 us per call against a ~7 us kernel).
 def _make_custom_op():
     try:
         @torch.library.custom_op("gemlite::forward_functional", mutates_args=())
@@ -310,15 +312,25 @@ def _make_custom_op():
 
         @forward_functional_op.register_fake
         def _(x, bias, tensor_args, meta_args, matmul_type=-1):
+            # the dtype forward_functional really returns (the reference's fake says x.dtype, which
+            # is the same thing for every processor it ships: output type = activation type)
             out_features = tensor_args[0].shape[1]
             return torch.empty(x.shape[:-1] + (out_features,), device=x.device, dtype=DTYPE_TO_TORCH[int(meta_args[6])])
 
         return forward_functional_op
-    except Exception:  # the name is taken (the reference package is loaded in this process) or torch is too old
+    except Exception as exc:  # the name is taken (the reference package is loaded in this process) or torch is too old
+        logger.warning("gemlite_amd: torch custom op gemlite::forward_functional was not registered (%s); "
+                       "torch.compile will trace into the plain Python forward", exc)
         return None
 
 
 forward_functional_op = _make_custom_op()
+
+
+def _dispatch_forward(x, bias, tensor_args, meta_args, matmul_type=-1):
+    if forward_functional_op is not None and torch.compiler.is_compiling():
+        return forward_functional_op(x, bias, tensor_args, meta_args, matmul_type)
+    return forward_functional(x, bias, tensor_args, meta_args, matmul_type)
 
 
 # ---------------------------------------------------------------------------
@@ -568,13 +580,13 @@ class GemLiteLinear(torch.nn.Module):
     # --------------------------------------------------------------- forward
     def forward_manual(self, x: Tensor, matmul_type: str = "GEMM") -> Tensor:
         """(reference: gemlite/core.py:820-827)"""
-        return forward_functional(
+        return _dispatch_forward(
             x, self.bias, self.get_tensor_args(), self.get_meta_args(), GEMLITE_MATMUL_TYPES_MAPPING[matmul_type]
         )
 
     def forward_auto_no_warmup(self, x: Tensor) -> Tensor:
         """(reference: gemlite/core.py:830-836)"""
-        return forward_functional(x, self.bias, self.get_tensor_args(), self.get_meta_args())
+        return _dispatch_forward(x, self.bias, self.get_tensor_args(), self.get_meta_args())
 
     # ------------------------------------------------------------ state dict
     def _save_to_state_dict(self, destination, prefix, keep_vars):
@@ -584,6 +596,14 @@ class GemLiteLinear(torch.nn.Module):
         if isinstance(w, Tensor) and w.numel() > 0 and self.elements_per_sample is not None:
             self._set_param("metadata", torch.tensor(self.get_meta_args(), device=w.device, dtype=torch.int32))
         super()._save_to_state_dict(destination, prefix, keep_vars)
+        # Micro-scaled layers keep their e8m0 scales [N, K/32] row-major in memory (K-contiguous, what the
+        # MFMA kernels read).  The reference holds the same shape as the transposed view of a
+        # [K/32, N] buffer (gemlite/core.py:752) and torch.save keeps strides, so the checkpoint
+        # gets that stride order; loading accepts either (_apply_state_dict).
+        sc = destination.get(prefix + "scales")
+        if (isinstance(sc, Tensor) and sc.dim() == 2 and sc.numel() > 0 and self.elements_per_sample is not None
+                and is_mx_dtype(self.input_dtype) and sc.stride(-1) == 1 and sc.shape[0] > 1):
+            destination[prefix + "scales"] = sc.detach().t().contiguous().t()
 
     def _apply_state_dict(self, sd):
         """Populate the module from short-keyed checkpoint tensors

@@ -86,6 +86,15 @@ int validate(const gla_matmul_args* p) {
         set_error("matmul: K=%d not divisible by elements_per_sample=%d", p->K, p->elements_per_sample);
         return GLA_ERR_MISALIGNED_SHAPE;
     }
+    if (is_mx(p->input_dtype)) {  // every micro-scaled kernel stores fp32, fp16 or bf16
+        int odt = p->output_dtype;
+        if (odt == GLA_DT_MXFP16) odt = GLA_DT_FP16;  // the reference's weight-only MX processors say it this way
+        if (odt == GLA_DT_MXBF16) odt = GLA_DT_BF16;
+        if (odt != GLA_DT_FP32 && odt != GLA_DT_FP16 && odt != GLA_DT_BF16) {
+            set_error("matmul: micro-scaled inputs need an fp32, fp16 or bf16 output (type %d)", p->output_dtype);
+            return GLA_ERR_UNSUPPORTED_DTYPE;
+        }
+    }
     if (p->input_dtype == GLA_DT_MXFP4) {
         if (p->K % 32 != 0) {
             set_error("matmul: MXFP4 needs K %% 32 == 0 (K=%d)", p->K);

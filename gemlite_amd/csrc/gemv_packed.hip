@@ -33,19 +33,7 @@ constexpr int kTileN = 64;  // output columns per workgroup
 constexpr int kBatch = 8;   // 128-bit loads in flight per lane
 constexpr int64_t kCounterBytes = 256 * 1024;  // fixed ticket-counter region at the start of the workspace
 
-#ifndef GLA_EXP
-#define GLA_EXP 0  // lab-only experiment switches; 0 in every product build
-#endif
-#ifdef GLA_TRACE
-#define GLA_STAMP(i) do { if (threadIdx.x == 0) a.trace[((size_t)blockIdx.x) * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define GLA_STAMP(i) do { } while (0)
-#endif
-
 struct GemvArgs {
-#ifdef GLA_TRACE
-    long long* trace;
-#endif
     const uint32_t* w;
     const void* x;
     const void* scales;
@@ -146,7 +134,6 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int cg = lane & 15, kb = lane >> 4;
-    GLA_STAMP(2);
     // ---- reduce the waves: lane (cg, kb) holds rows 4*kb + i of columns 4*cg + j
     if (RT == 16 || kb == 0) {
 #pragma unroll
@@ -174,8 +161,6 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
         }
         total[t] = v;
     }
-
-    GLA_STAMP(3);
     if (a.S > 1) {
         // publish this slab's partial, then take a ticket; the last slab to arrive sums all
 #pragma unroll
@@ -194,7 +179,6 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
             ticket = __hip_atomic_fetch_add(a.counters + blockIdx.y * a.tiles + tile, 1u, __ATOMIC_RELAXED,
                                             __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        GLA_STAMP(4);
         if (ticket != (unsigned)(a.S - 1)) return;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -240,7 +224,6 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
         if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + bias;  // `out += bias` on the rounded output
         store_from_float(a.out, a.out_dt, (int64_t)(m0 + m) * a.osm + n_out, v);
     }
-    GLA_STAMP(5);
 }
 
 // BITS: code width.  BF16: activation type.  RT: rows of x per pass (1, 2, 4 or 16).
@@ -260,8 +243,6 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
     float2* mt = (float2*)(xs + (size_t)SRW * RT * T);  // [GW][64] (s, zz)
     float* red = (float*)(mt + (size_t)a.GW * kTileN);  // [kWaves][RT][64]
     __shared__ unsigned ticket;
-
-    GLA_STAMP(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int cg = lane & 15, kb = lane >> 4;
@@ -404,7 +385,6 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
         }
     }
     __syncthreads();
-    GLA_STAMP(1);
 
     // ---- main loop
     float acc[4][RI];
@@ -507,8 +487,6 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     float2* mtw = (float2*)smem + (size_t)(threadIdx.x >> 6) * nfb * kTileN;  // [nfb][64], this wave's
     float* red = (float*)((float2*)smem + (size_t)kWaves * nfb * kTileN);     // [kWaves][RT][64]
     __shared__ unsigned ticket;
-
-    GLA_STAMP(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int cg = lane & 15, kb = lane >> 4;
@@ -547,7 +525,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     };
 
     auto issue = [&](int ib, Batch& b) {
-        if (fast_meta && !(GLA_EXP & 4)) {
+        if (fast_meta) {
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
                 const int item = lane + 64 * p;
@@ -722,13 +700,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
             process(ib, cur);
         }
     }
-    GLA_STAMP(1);
     wg_finish<RT, kWaves, RI>(a, acc, red, ticket, tile, split, m0, n0);
 }
-
-#ifdef GLA_TRACE
-long long* g_trace = nullptr;
-#endif
 
 int row_tile(int M) { return M >= 3 ? 16 : (M == 2 ? 2 : 1); }
 
@@ -939,9 +912,6 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
         return GLA_ERR_MISALIGNED_SHAPE;
     }
     GemvArgs a;
-#ifdef GLA_TRACE
-    a.trace = g_trace;
-#endif
     a.w = (const uint32_t*)p.w; a.x = p.x; a.scales = p.scales; a.zeros = p.zeros; a.scales_x = p.scales_x;
     a.out = p.out; a.partials = nullptr; a.counters = nullptr;
     a.bias = p.bias; a.bias_dt = p.bias_dtype;

@@ -25,6 +25,30 @@ def rel_frob(y, y_ref):
     return float(np.linalg.norm(y - y_ref) / (denom if denom > 0 else 1.0))
 
 
+# Elementwise bound next to the global norm: |y - y_ref| <= atol_rms * rms(y_ref) + rtol * |y_ref|.
+# A correct kernel's error is output rounding (half an ulp: 2^-9 bf16, 2^-12 fp16, relative to the
+# element) plus fp32 accumulation noise and, where weights are dequantised to 16 bits before the MFMA,
+# their rounding (a few 1e-4 of the rms in fp16, 2e-3 in bf16).  A wrong tail column, row tile or MFMA
+# tile is off by about the rms itself and fails this whatever its share of the whole norm.
+ELEMENTWISE = {"bf16": (2.5e-2, 2.0 ** -7), "fp16": (5e-3, 2.0 ** -10), "fp32": (1e-3, 1e-4)}
+
+
+def elementwise_excess(y, y_ref, kind):
+    """Largest |y - y_ref| / (atol_rms * rms + rtol * |y_ref|); <= 1 passes."""
+    atol_rms, rtol = ELEMENTWISE[kind]
+    y = np.asarray(y, dtype=np.float64)
+    y_ref = np.asarray(y_ref, dtype=np.float64)
+    if y_ref.size == 0:
+        return 0.0
+    rms = float(np.sqrt(np.mean(y_ref * y_ref)))
+    bound = atol_rms * (rms if rms > 0 else 1.0) + rtol * np.abs(y_ref)
+    return float(np.max(np.abs(y - y_ref) / bound))
+
+
+def kind_of(dtype):
+    return {torch.bfloat16: "bf16", torch.float16: "fp16", torch.float32: "fp32"}[dtype]
+
+
 def gen_int_case(N, K, W_nbits, group_size, dtype, seed=0, scale_std=0.02, channelwise=False):
     """Seeded weights in the distributions of the benchmark configs: codes uniform over the
     bit range, scales |N(0, std)|, zeros uniform over the middle of the range."""

@@ -8,7 +8,7 @@ import torch
 import gemlite_amd
 from gemlite_amd import DType, GemLiteLinear, helper
 from oracle import oracle as orc
-from parity import FROB_TOL, gen_int_case, gen_x, rel_frob, to_np
+from parity import FROB_TOL, elementwise_excess, gen_int_case, gen_x, rel_frob, to_np
 
 pytestmark = pytest.mark.gpu
 TIGHT_BF16, TIGHT_FP16 = 6e-3, 1.5e-3
@@ -35,6 +35,7 @@ def test_a16wn_bf16_16384_square(device, nbits, gs, M):
     want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], gs)
     err = rel_frob(y[:, cols], want)
     assert err <= FROB_TOL and err <= TIGHT_BF16, err
+    assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0
 
 
 @pytest.mark.parametrize("fp8", [False, True])
@@ -62,9 +63,32 @@ def test_a8w8_dynamic_4096x8192x8192(device, fp8):
     acc = a.astype(np.float64) @ b.astype(np.float64).T
     want = acc * sx.cpu().numpy().astype(np.float64) * to_np(sw).astype(np.float64).reshape(-1)[cols][None, :]
     assert rel_frob(y[:, cols], want.astype(np.float32)) <= TIGHT_BF16
+    assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0
 
 
-@pytest.mark.parametrize("M", [1, 32, 1024])
+def test_int8_x_int8_int32_exact_4096x8192x8192(device):
+    """INT8 x INT8 -> INT32 at M = 4096, N = K = 8192 with the accumulators as the output: sampled
+    columns, all rows, bit for bit against exact sums (|sum| <= 8192 * 2^14 < 2^53, so float64 BLAS is
+    exact) (reference epilogue: gemlite/triton_kernels/gemm_kernels.py:479-488 with channel_scale_mode 0)."""
+    M, N, K = 4096, 8192, 8192
+    g = torch.Generator().manual_seed(41)
+    W = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    x = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    layer = GemLiteLinear(8, None, K, N, DType.INT8, DType.INT32).pack(W.to(device), None, None)
+    assert layer.acc_dtype == DType.INT32 and layer.W_group_mode == 0 and layer.channel_scale_mode == 0
+    y = layer(x.to(device))
+    assert y.dtype == torch.int32 and y.shape == (M, N)
+    y = y.cpu().numpy()
+    cols = sample_cols(N, count=96, seed=42)
+    want = (x.numpy().astype(np.float64) @ W.numpy()[cols].astype(np.float64).T).astype(np.int64)
+    assert np.array_equal(y[:, cols].astype(np.int64), want)
+    # every tile of the output is touched by a cheap invariant too: the row sums over all columns
+    # equal x @ (sum of weight rows), exactly
+    wsum = W.numpy().astype(np.float64).sum(axis=0)
+    assert np.array_equal(y.astype(np.int64).sum(axis=1), (x.numpy().astype(np.float64) @ wsum).astype(np.int64))
+
+
+@pytest.mark.parametrize("M", [1, 32, 1024, 8192])
 def test_a4w4_mxfp4_16384_square(device, M):
     N = K = 16384
     W = gen_x(N, K, torch.bfloat16, seed=9, std=0.02)
@@ -73,10 +97,16 @@ def test_a4w4_mxfp4_16384_square(device, M):
         torch.from_numpy(codes), scales=torch.from_numpy(e8))
     x = gen_x(M, K, torch.bfloat16, seed=M)
     y = to_np(layer(x.to(device)))
-    a_packed, sa = orc.scale_activations_mxfp4(to_np(x))
+    # the activation quantiser works row by row, so at the largest batch the oracle follows a sample of
+    # rows: the first and last 256-row tiles whole, every 13th row between
+    rows = np.arange(M) if M <= 1024 else np.unique(np.concatenate([np.arange(256), np.arange(256, M - 256, 13),
+                                                                     np.arange(M - 256, M)]))
+    a_packed, sa = orc.scale_activations_mxfp4(to_np(x)[rows])
     cols = sample_cols(N, seed=M)
-    want = orc.matmul_mx(orc.unpack_fp4_bytes(a_packed), sa[:M], codes[cols], e8[cols])
-    assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+    want = orc.matmul_mx(orc.unpack_fp4_bytes(a_packed), sa[:len(rows)], codes[cols], e8[cols])
+    got = y[rows][:, cols]
+    assert rel_frob(got, want) <= TIGHT_BF16
+    assert elementwise_excess(got, want, "bf16") <= 1.0
 
 
 @pytest.mark.parametrize("M", [1, 1024])
@@ -92,6 +122,7 @@ def test_a8w8_mxfp8_8192_square(device, M):
     cols = sample_cols(N, seed=M)
     want = orc.matmul_mxfp8_weights(orc.e4m3fn_decode(aq), sx, codes[cols], e8[cols])
     assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+    assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0
 
 
 def test_a16w4_prefill_4096_cubed(device):
@@ -107,6 +138,7 @@ def test_a16w4_prefill_4096_cubed(device):
     want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], 128)
     err = rel_frob(y[:, cols], want)
     assert err <= FROB_TOL and err <= TIGHT_FP16, err
+    assert elementwise_excess(y[:, cols], want, "fp16") <= 1.0
 
 
 @pytest.mark.parametrize("to_int8", [True, False])
@@ -134,6 +166,7 @@ def test_a8w8_block_quantised_4096x8192x8192(device, to_int8):
     sb = np.repeat(sw[cols // 128].astype(np.float64), 128, axis=1)
     want = (a.astype(np.float64) * sa) @ (b.astype(np.float64) * sb).T
     assert rel_frob(y[:, cols], want.astype(np.float32)) <= TIGHT_BF16
+    assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0
 
 
 @pytest.mark.parametrize("M", [1, 4, 16])
@@ -148,6 +181,7 @@ def test_a16w4_mxfp_weight_only_16384_square(device, M):
     cols = sample_cols(N, seed=M)
     want = orc.matmul_mx_mixed(to_np(x), "float", None, codes[cols], "e2m1", e8[cols])
     assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+    assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0
 
 
 @pytest.mark.parametrize("post_scale,M", [(True, 1), (True, 1024), (False, 32), (False, 1024)])
@@ -169,3 +203,4 @@ def test_a8w4_mxfp_16384_square(device, post_scale, M):
         aq, sa = orc.scale_activations_mxfp8(to_np(x))
         want = orc.matmul_mx_mixed(aq, "e4m3", sa[:M], codes[cols], "e2m1", e8[cols])
     assert rel_frob(y[:, cols], want) <= TIGHT_BF16
+    assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0

@@ -10,7 +10,8 @@ import gemlite_amd
 from gemlite_amd import DType, GemLiteLinear, helper
 from gemlite_amd.bitpack import pack_weights_over_cols_hip, unpack_over_cols_hip
 from oracle import oracle as orc
-from parity import FROB_TOL, gen_int_case, gen_x, oracle_forward, rel_frob, round_like, to_np
+from parity import (FROB_TOL, elementwise_excess, gen_int_case, gen_x, kind_of, oracle_forward, rel_frob, round_like,
+                    to_np)
 
 pytestmark = pytest.mark.gpu
 
@@ -34,12 +35,15 @@ def check_layer(layer, x, tol_dtype, types=ALL_TYPES, exact=False):
             err = rel_frob(y_np, y_ref)
             assert err <= FROB_TOL, (mt, err)
             assert err <= TIGHT[tol_dtype], (mt, err)
+            ex = elementwise_excess(y_np, y_ref, kind_of(y.dtype))
+            assert ex <= 1.0, (mt, "elementwise", ex)
     y_auto = layer(x)
     torch.cuda.synchronize()
     if exact:
         assert np.array_equal(to_np(y_auto).reshape(y_ref.shape), y_ref)
     else:
         assert rel_frob(to_np(y_auto).reshape(y_ref.shape), y_ref) <= TIGHT[tol_dtype]
+        assert elementwise_excess(to_np(y_auto).reshape(y_ref.shape), y_ref, kind_of(y_auto.dtype)) <= 1.0
 
 
 # ------------------------------------------------------------------ bit packing

@@ -506,3 +506,92 @@ def test_ternary_processors_pack_like_the_reference():
     d = gemlite_amd.helper.A8W158_INT_dynamic(device="cpu").from_weights(W, torch.tensor(0.037))
     assert (d.W_group_mode, d.channel_scale_mode, d.input_dtype, d.acc_dtype) == (1, 3, DType.INT8, DType.INT32)
     assert d.scaled_activations and d.output_dtype == DType.FP16
+
+
+# ------------------------------------------------------------------ workspace keyed by (device, stream)
+def test_workspace_is_per_stream(monkeypatch):
+    """Two streams never share scratch; one stream keeps its buffer across calls, grows by replacement and
+    never frees the outgrown one (a captured graph may still point at it)."""
+    monkeypatch.setattr(_ext, "_new_workspace", lambda size, device: torch.zeros(size, dtype=torch.uint8))
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
+    monkeypatch.setattr(_ext, "_workspaces", {})
+    monkeypatch.setattr(_ext, "_retired_workspaces", [])
+    dev = torch.device("cuda", 0)
+    a = _ext.get_workspace(dev, 1024, stream=0x1000)
+    b = _ext.get_workspace(dev, 1024, stream=0x2000)
+    assert a.data_ptr() != b.data_ptr()
+    assert _ext.get_workspace(dev, 4096, stream=0x1000) is a          # within the 8 MiB floor: same buffer
+    big = _ext.get_workspace(dev, 20 << 20, stream=0x1000)
+    assert big is not a and big.numel() >= 20 << 20 and a in _ext._retired_workspaces
+    assert _ext.get_workspace(dev, 1024, stream=0x2000) is b
+    assert _ext.get_workspace(torch.device("cuda", 1), 1024, stream=0x1000) is not big
+    # growing under capture is refused
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    with pytest.raises(RuntimeError, match="captured"):
+        _ext.get_workspace(dev, 1024, stream=0x3000)
+    assert _ext.get_workspace(dev, 1024, stream=0x2000) is b           # an existing buffer is still served
+
+
+# ------------------------------------------------------------------ torch custom op
+def test_custom_op_fake_shape_and_dtype():
+    """The registered op's fake implementation (what torch.compile sees) returns [..., N] in the layer's
+    output type, on the input's device, without touching any kernel."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from gemlite_amd import core
+
+    assert core.forward_functional_op is not None
+    meta = [0, 4, 128, 15, 8, DType.BF16.value, DType.BF16.value, DType.FP32.value, DType.BF16.value, 0, 4, 1]
+    with FakeTensorMode():
+        x = torch.empty((3, 5, 256), dtype=torch.bfloat16)
+        W_q = torch.empty((32, 96), dtype=torch.int32)
+        s = torch.empty((2, 96), dtype=torch.bfloat16)
+        out = core.forward_functional_op(x, None, [W_q, s, s, torch.empty((), dtype=torch.float32)], meta, -1)
+        assert tuple(out.shape) == (3, 5, 96) and out.dtype == torch.bfloat16 and out.device == x.device
+        meta[6] = DType.FP32.value
+        out = torch.ops.gemlite.forward_functional(x, None, [W_q, s, s, torch.empty((), dtype=torch.float32)], meta, 4)
+        assert out.dtype == torch.float32
+    # eager calls take the plain function; the op is only used while a graph is being traced
+    assert not torch.compiler.is_compiling()
+
+
+# ------------------------------------------------------------------ patch_model
+class _CountingProcessor:
+    def __init__(self):
+        self.seen = []
+
+    def from_linear(self, layer):
+        self.seen.append(layer.name)
+        return torch.nn.Identity()
+
+
+def test_patch_model_replaces_linears_and_skips_named_modules():
+    from gemlite_amd import helper
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = torch.nn.Linear(32, 32)
+            self.norm = torch.nn.LayerNorm(32)
+            self.mlp = torch.nn.Sequential(torch.nn.Linear(32, 64), torch.nn.ReLU(), torch.nn.Linear(64, 32))
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Block(), Block()])
+            self.lm_head = torch.nn.Linear(32, 100)
+            self.visual = torch.nn.Sequential(torch.nn.Linear(32, 32))
+
+    proc = _CountingProcessor()
+    model = helper.patch_model(Model(), device="cpu", processor=proc)
+    assert sorted(proc.seen) == sorted(
+        [f"layers.{i}.{n}" for i in (0, 1) for n in ("q_proj", "mlp.0", "mlp.2")])
+    assert isinstance(model.layers[0].q_proj, torch.nn.Identity) and isinstance(model.layers[1].mlp[2], torch.nn.Identity)
+    assert isinstance(model.lm_head, torch.nn.Linear) and isinstance(model.visual[0], torch.nn.Linear)
+    assert isinstance(model.layers[0].norm, torch.nn.LayerNorm)
+
+    class HqqOnly:
+        def from_hqqlinear(self, layer):
+            return layer
+
+    with pytest.raises(ImportError):
+        helper.patch_model(Model(), device="cpu", processor=HqqOnly())

@@ -330,6 +330,44 @@ def test_quantize_per_channel():
     assert np.array_equal(tq8.view(torch.uint8).numpy(), q8) and np.array_equal(ts8.numpy(), s8)
 
 
+def test_weight_quantizer_ties_by_hand():
+    """Known answers written out by hand, independent of any quantiser code.
+
+    MXFP4 weights (reference: gemlite/quant_utils.py:80-88): `searchsorted` without `right=True`
+    returns the first threshold >= |v|, so a value exactly on a threshold takes the LOWER e2m1
+    value.  A block whose amax is 6 has scale 2^0, so the values below are their own quotients.
+    Negative values that round to zero lose their sign (index of the first match of -0.0 == 0.0).
+    INT8 per channel (reference: gemlite/helper.py:651-657): `round_()` is round-half-to-even;
+    a row whose amax is 127 has scale 1."""
+    block = np.zeros(32, dtype=np.float32)
+    vals = [6.0, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.25, -0.75, -1.25, -1.75, -2.5, -3.5, -5.0, -6.0,
+            0.26, 0.76, 2.51, 5.01, -0.0, 0.0]
+    want = [7, 0, 1, 2, 3, 4, 5, 6, 0, 9, 10, 11, 12, 13, 14, 15,
+            1, 2, 5, 7, 0, 0]
+    block[:len(vals)] = vals
+    for scale_exp in (0, -7, 5):   # the same quotients under other block scales (powers of two: exact)
+        codes, e = orc.quantize_mxfp4_weights((block * np.float32(2.0 ** scale_exp)).reshape(1, 32))
+        assert e.tolist() == [[127 + scale_exp]]
+        assert codes[0, :len(vals)].tolist() == want, scale_exp
+        assert not np.any(codes[0, len(vals):])
+
+    row = np.zeros(16, dtype=np.float32)
+    v8 = [127.0, 0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, -3.5, 2.49, 2.51, -126.5, 126.5]
+    w8 = [127, 0, 2, 2, 4, 0, -2, -2, -4, 2, 3, -126, 126]
+    row[:len(v8)] = v8
+    q, s = orc.quantize_per_channel(row.reshape(1, 16), True)
+    assert s.tolist() == [[1.0]] and q[0, :len(v8)].tolist() == w8
+    # the same row scaled by a power of two: same codes, scaled scale
+    q, s = orc.quantize_per_channel((row * np.float32(0.125)).reshape(1, 16), True)
+    assert s.tolist() == [[0.125]] and q[0, :len(v8)].tolist() == w8
+    # fp8: amax 448 -> scale 1; 17, 19 lie halfway between e4m3 neighbours (16, 18, 20) -> nearest even mantissa
+    row8 = np.zeros(16, dtype=np.float32)
+    row8[:5] = [448.0, 17.0, 19.0, -17.0, 1.0]
+    q8, s8 = orc.quantize_per_channel(row8.reshape(1, 16), False)
+    assert s8.tolist() == [[1.0]]
+    assert orc.e4m3fn_decode(q8)[0, :5].tolist() == [448.0, 16.0, 20.0, -16.0, 1.0]
+
+
 # ------------------------------------------------------------------ host logic
 def test_matmul_type_table():
     # the decision table in the reference's source, including every batch size of the benchmark configs
