@@ -93,6 +93,7 @@ SYMBOLS = {
     "gla_matmul_family": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
     "gla_probe_mfma": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                       ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]),
+    "gla_probe_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "gla_matmul_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),
     "gla_scale_activations_per_token": (
@@ -196,6 +197,7 @@ def get_closest_m(M: int) -> int:
 _workspaces = {}
 _retired_workspaces = []  # outgrown buffers stay allocated: a captured HIP graph may still point at them
 _workspace_lock = threading.Lock()
+_last_eager_key = {}  # (thread, device index) -> key of the stream that thread last launched on outside a capture
 
 
 def _workspace_key(device: torch.device, stream: int):
@@ -209,32 +211,45 @@ def get_workspace(device: torch.device, nbytes: int, stream: Optional[int] = Non
     Keyed by the device and the raw handle of the stream the launch goes to (the current stream when
     ``stream`` is None): kernels on one stream run in order and may share scratch, kernels on
     different streams may overlap and must not, so each stream that launches a matmul needing
-    scratch gets a buffer of its own.  A graph captured on a stream keeps pointing at that stream's
-    buffer, whichever stream replays it.
+    scratch gets a buffer of its own.
+
+    While a graph is being captured nothing can be allocated or zero-filled (the fill would become a
+    node of the graph).  A capture stream that has no buffer of its own (torch.cuda.graph captures
+    on an internal stream) therefore takes the buffer of the stream this thread last launched on
+    outside a capture - the stream the layer was warmed up on, and normally the one that replays the
+    graph, so the two stay ordered.  A graph replayed on another stream while that stream is busy
+    with matmuls would race with them; capture on an explicit, warmed-up stream in that case.  If no
+    buffer is large enough the capture is refused: run the layer once at this shape first.
 
     Growing replaces the buffer (at least doubling, so the outgrown ones add up to less than the
-    live one) and never frees the old one.  Growing while the stream is being captured into a graph
-    is refused: the fill that zeroes the new buffer would become a node of the graph.  Run the
-    layer once on that stream before capturing it.
+    live one) and never frees the old one: a captured graph may still point at it.
     """
     if stream is None:
         stream = _stream_ptr(device)
     key = _workspace_key(device, stream)
+    capturing = torch.cuda.is_current_stream_capturing()
+    owner = (threading.get_ident(), key[1])
+    if not capturing:
+        _last_eager_key[owner] = key
     ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        with _workspace_lock:
-            ws = _workspaces.get(key)
-            if ws is None or ws.numel() < nbytes:
-                if torch.cuda.is_current_stream_capturing():
-                    raise RuntimeError(
-                        f"gemlite_amd: the workspace of this stream has to grow to {int(nbytes)} bytes while a graph "
-                        "is being captured; run the layer once at this shape on the capture stream before capturing"
-                    )
-                size = max(int(nbytes), 8 << 20, 0 if ws is None else 2 * ws.numel())
-                if ws is not None:
-                    _retired_workspaces.append(ws)
-                ws = _new_workspace(size, device)
-                _workspaces[key] = ws
+    if ws is not None and ws.numel() >= nbytes:
+        return ws
+    if capturing:
+        fallback = _workspaces.get(_last_eager_key.get(owner))
+        if fallback is not None and fallback.numel() >= nbytes:
+            return fallback
+        raise RuntimeError(
+            f"gemlite_amd: a workspace of {int(nbytes)} bytes is needed while a graph is being captured and none "
+            "that large exists yet; run the layer once at this shape before capturing"
+        )
+    with _workspace_lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            size = max(int(nbytes), 8 << 20, 0 if ws is None else 2 * ws.numel())
+            if ws is not None:
+                _retired_workspaces.append(ws)
+            ws = _new_workspace(size, device)
+            _workspaces[key] = ws
     return ws
 
 

@@ -230,6 +230,10 @@ int gla_probe_mfma(int dtype, int random_operands, int iters, void* sink, double
     return gla::launch_probe_mfma(dtype, random_operands, iters, sink, flops, (hipStream_t)stream);
 }
 
+int gla_probe_read(const void* buf, int64_t bytes, void* sink, void* stream) {
+    return gla::launch_probe_read(buf, bytes, sink, (hipStream_t)stream);
+}
+
 int gla_matmul_family(const gla_matmul_args* args) {
     const int rc = validate(args);
     if (rc != GLA_OK) return rc;

@@ -152,6 +152,28 @@ __device__ __forceinline__ T wave_xor(T v, int mask) {
 
 static inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
+// Workspace layout shared by every family.  The first kWsPrivateBytes belong to the streaming GEMV
+// kernels alone: kWsCounterBytes of ticket counters, then their tagged partial slots.  Nothing else
+// ever writes there, so "all counters zero, all slots invalid" holds between launches (the buffer
+// starts zero-filled and the last-arriving workgroup of a column tile clears what it consumed).
+// Every other use of the workspace (split-K partials of the GEMMs, regrouped block scales, GEMV
+// partials too large for the slot region) starts at kWsPrivateBytes.
+constexpr int64_t kWsCounterBytes = 256 * 1024;
+constexpr int64_t kWsPrivateBytes = 4 << 20;
+
+// 128-bit load that is not kept in the caches on its way in (weights are read once per launch;
+// measured on MI355X: 5-9 % more streaming bandwidth than a plain load).
+__device__ __forceinline__ uint4 load_streaming_u4(const void* p) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const u4 v = __builtin_nontemporal_load((const u4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 load_streaming_u2(const void* p) {
+    typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+    const u2 v = __builtin_nontemporal_load((const u2*)p);
+    return make_uint2(v.x, v.y);
+}
+
 // ---------------------------------------------------------------------------
 // kernel-family launchers (host); each returns a GLA_* status
 // ---------------------------------------------------------------------------

@@ -80,5 +80,7 @@ int64_t gemm_kbytes_mx_workspace_bytes(const gla_matmul_args& p);
 
 // ---- diagnostic: sustained matrix rate (probe.hip) ---------------------------
 int launch_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, hipStream_t stream);
+// ---- diagnostic: streaming-read ceiling (probe.hip) --------------------------
+int launch_probe_read(const void* buf, int64_t bytes, void* sink, hipStream_t stream);
 
 }  // namespace gla

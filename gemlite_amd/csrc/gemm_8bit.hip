@@ -673,7 +673,7 @@ __global__ __launch_bounds__(256) void mx_scales_by_stage_kernel(const uint8_t* 
     }
 }
 
-constexpr int64_t kWsReserved8 = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
+constexpr int64_t kWsReserved8 = kWsPrivateBytes;  // the start of the workspace belongs to the GEMV family (common.hpp)
 
 Plan8 plan8(int M, int N, int Kb, int tile_config) {
     Plan8 g;

@@ -48,7 +48,7 @@ constexpr int kRowAb = 128;  // LDS row of the activation tile: 64 fp16/bf16 val
 constexpr int kRowBb = 64;   // LDS row of the weight tile: 64 bytes
 constexpr int kBNb = 256;
 constexpr int kWavesNb = 4;
-constexpr int64_t kWsReservedB = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
+constexpr int64_t kWsReservedB = kWsPrivateBytes;  // the start of the workspace belongs to the GEMV family (common.hpp)
 // Weight kinds beyond the element-type ids: micro-scaled weights of weight-only MX layers, fp8-e4m3 bytes or
 // e2m1 nibble pairs with one e8m0 scale per 32 values along K.  The block scale is applied by the
 // conversion instruction (v_cvt_scalef32_pk_*), so the 16-bit operand is the dequantised weight.

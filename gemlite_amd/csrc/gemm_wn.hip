@@ -47,7 +47,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kBKw = 64;    // K per pipeline stage
 constexpr int kRowW = 128;  // LDS row: 64 fp16/bf16 values
 constexpr int kBNw = 256;   // workgroup tile columns: 256 / (32 TJ) wave columns of TJ 32-column MFMA tiles
-constexpr int64_t kWsReserved = 256 * 1024;  // start of the workspace: ticket counters of the GEMV family
+constexpr int64_t kWsReserved = kWsPrivateBytes;  // the start of the workspace belongs to the GEMV family (common.hpp)
 
 struct GemmWnArgs {
     const uint16_t* x;

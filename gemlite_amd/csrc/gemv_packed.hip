@@ -21,7 +21,12 @@
 //    five dequant modes are a choice of (s, zz), staged per slab in LDS.
 //  * The K reduction is deterministic: k-blocks inside the MFMA, waves through LDS, slabs by
 //    fp32 partials in a workspace that the last-arriving workgroup of a column tile sums in
-//    slab order (no float atomics).
+//    slab order (no float atomics).  A partial travels as a 64-bit slot (value, tag) written with
+//    one atomic store, so a reader sees either the whole slot or none of it: a workgroup publishes
+//    its slots, takes a ticket and reads the other slabs' slots in the same breath, and the one
+//    whose ticket says "last" already holds every partial that had landed (it polls the few that
+//    had not).  One memory round trip ends the kernel instead of three (store-and-wait, ticket,
+//    load), which at decode sizes is a quarter of the kernel.
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -31,7 +36,14 @@ namespace {
 
 constexpr int kTileN = 64;  // output columns per workgroup
 constexpr int kBatch = 8;   // 128-bit loads in flight per lane
-constexpr int64_t kCounterBytes = 256 * 1024;  // fixed ticket-counter region at the start of the workspace
+constexpr int64_t kCounterBytes = kWsCounterBytes;  // ticket-counter region at the start of the workspace
+constexpr int kCounterStride = 32;  // words between the counters of two column tiles: a 128-byte line each.  The atomic
+                                    // unit takes the adds to one line one after the other; with the counters of 32 tiles in
+                                    // one line, the 256 tickets of a launch queued up there for ~2 us
+constexpr int64_t kSlotBytes = kWsPrivateBytes - kWsCounterBytes;  // tagged partial slots, private to this family
+constexpr uint32_t kSlotValid = 0x7fc5a11du;  // tag of a published slot; a consumed slot is all zeros
+constexpr int kSpinLimit = 1 << 22;           // polls of a slot whose store is in flight (it has been issued)
+constexpr int kSpec = 8;                      // slots read ahead of the ticket
 
 struct GemvArgs {
     const uint32_t* w;
@@ -40,7 +52,8 @@ struct GemvArgs {
     const void* zeros;
     const void* scales_x;
     void* out;
-    float* partials;
+    float* partials;             // [S][Mp][N] fp32 (plain protocol: problems whose slots do not fit the private region)
+    unsigned long long* slots;   // [S][Mp][N] (value, tag) (tagged protocol), or NULL
     unsigned* counters;
     int M, N, K;
     int R;      // word rows = K / E
@@ -128,9 +141,11 @@ __device__ __forceinline__ uint32_t pick(const uint4& v, int j) {
 // Shared end of both kernels: sum the waves of the workgroup through LDS, combine the K slabs
 // (last-arriving workgroup of a column tile sums the partials in slab order), apply the channel
 // scales and store.  Lane (cg, kb) holds rows 4*kb + i of columns 4*cg + j in acc[j][i].
+// kWaves = 0: the number of waves is blockDim.x / 64 (any count from 4 to 16; RT <= 4 only).
 template <int RT, int kWaves, int RI>
 __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI], float* red, unsigned& ticket,
                                           int tile, int split, int m0, int n0) {
+    const int waves = kWaves ? kWaves : (int)(blockDim.x >> 6);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int cg = lane & 15, kb = lane >> 4;
@@ -145,7 +160,8 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
     }
     __syncthreads();
 
-    constexpr int NT = (RT + kWaves - 1) / kWaves;  // output rows per thread
+    // output rows per thread; a run-time wave count is at least 4 (row tiles up to 4) or 8 (the 16-row tile)
+    constexpr int NT = kWaves ? (RT + kWaves - 1) / kWaves : (RT <= 4 ? 1 : 2);
     const int n_out = n0 + lane;
     const bool col_ok = n_out < a.N;
     // loaded before the reduction, so that its latency is not the kernel's tail
@@ -153,19 +169,96 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
     float total[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int m = wv + t * kWaves;
+        const int m = wv + t * waves;
         float v = 0.0f;
         if (m < RT) {
-#pragma unroll
-            for (int w2 = 0; w2 < kWaves; ++w2) v += red[((size_t)w2 * RT + m) * kTileN + lane];
+            for (int w2 = 0; w2 < waves; ++w2) v += red[((size_t)w2 * RT + m) * kTileN + lane];
         }
         total[t] = v;
     }
-    if (a.S > 1) {
-        // publish this slab's partial, then take a ticket; the last slab to arrive sums all
+
+    if (a.S > 1 && a.slots != nullptr) {
+        // ---- tagged protocol.  Publish (value, tag) slots, then ticket and read-ahead together.
+        const size_t stride = (size_t)a.Mp * a.N;
+        unsigned long long* mine[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const int m = wv + t * kWaves;
+            const int m = wv + t * waves;
+            mine[t] = a.slots + (size_t)(m0 + (m < RT ? m : 0)) * a.N + (col_ok ? n_out : 0);
+            if (m < RT && col_ok)
+                __hip_atomic_store(mine[t] + (size_t)split * stride,
+                                   ((unsigned long long)kSlotValid << 32) | __builtin_bit_cast(uint32_t, total[t]),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();  // every wave of this workgroup has issued its slot stores
+        // The ticket is issued here and awaited below, after the read-ahead loads have been issued
+        // too: written as __hip_atomic_fetch_add the compiler waits for the returned value on the
+        // spot (it funnels the one-lane add through a wave-wide reduction), which would put the
+        // ticket's round trip in front of the loads' instead of beside it.  Same instruction and
+        // cache policy as the compiler emits for an agent-scope relaxed fetch-add.
+        unsigned tk = 0;
+        if (tid == 0) {
+            unsigned* cnt = a.counters + (size_t)(blockIdx.y * a.tiles + tile) * kCounterStride;
+            const unsigned one = 1u;
+            asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(tk) : "v"(cnt), "v"(one) : "memory");
+        }
+        // Read ahead the first kSpec slabs' slots while the ticket is on its way (one output row per
+        // thread only: more rows would cost more registers than the round trip is worth).
+        unsigned long long ahead[kSpec];
+        if constexpr (NT == 1) {
+            const bool live = (wv < RT) && col_ok;
+#pragma unroll
+            for (int u = 0; u < kSpec; ++u) {
+                ahead[u] = 0ull;
+                if (live && u < a.S && u != split)
+                    ahead[u] = __hip_atomic_load(mine[0] + (size_t)u * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(tk) : : "memory");  // ticket and read-ahead have returned
+        if (tid == 0) ticket = tk;
+        __syncthreads();
+        if (ticket != (unsigned)(a.S - 1)) return;
+        // ---- last arriver: every other slab's stores were issued before its ticket, so a slot that is
+        // not valid yet is in flight and a bounded poll gets it.  Sum in slab order.
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int m = wv + t * waves;
+            if (!(m < RT && col_ok)) continue;
+            float v = 0.0f;
+            for (int sl = 0; sl < a.S; ++sl) {
+                if (sl == split) {
+                    v += total[t];
+                    continue;
+                }
+                unsigned long long q = 0ull;
+                if constexpr (NT == 1) {
+                    if (sl < kSpec) {
+#pragma unroll
+                        for (int u = 0; u < kSpec; ++u)
+                            if (u == sl) q = ahead[u];
+                    }
+                }
+                unsigned long long* src = mine[t] + (size_t)sl * stride;
+                for (int tries = 0; (uint32_t)(q >> 32) != kSlotValid && tries < kSpinLimit; ++tries)
+                    q = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // a slot that never turned valid cannot happen with a healthy memory system; make it loud
+                v += (uint32_t)(q >> 32) == kSlotValid ? __builtin_bit_cast(float, (uint32_t)q)
+                                                       : __builtin_bit_cast(float, 0x7fc00000u);
+            }
+            total[t] = v;
+            // leave the slots invalid and the counter at zero for the next launch
+            for (int sl = 0; sl < a.S; ++sl)
+                __hip_atomic_store(mine[t] + (size_t)sl * stride, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (tid == 0)
+            __hip_atomic_store(a.counters + (size_t)(blockIdx.y * a.tiles + tile) * kCounterStride, 0u, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    } else if (a.S > 1) {
+        // ---- plain protocol (partials too large for the slot region): publish this slab's partial, wait
+        // for it to land, then take a ticket; the last slab to arrive sums all
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int m = wv + t * waves;
             if (m < RT && col_ok)
                 __hip_atomic_store(a.partials + ((size_t)split * a.Mp + (m0 + m)) * a.N + n_out, total[t],
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -176,41 +269,41 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0)
-            ticket = __hip_atomic_fetch_add(a.counters + blockIdx.y * a.tiles + tile, 1u, __ATOMIC_RELAXED,
+            ticket = __hip_atomic_fetch_add(a.counters + (size_t)(blockIdx.y * a.tiles + tile) * kCounterStride, 1u, __ATOMIC_RELAXED,
                                             __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (ticket != (unsigned)(a.S - 1)) return;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const int m = wv + t * kWaves;
+            const int m = wv + t * waves;
             float v = 0.0f;
             if (m < RT && col_ok) {
                 const float* p = a.partials + (size_t)(m0 + m) * a.N + n_out;
                 const size_t stride = (size_t)a.Mp * a.N;
-                int s = 0;
-                for (; s + 8 <= a.S; s += 8) {  // loads of a batch are independent; the sum keeps slab order
+                int sl = 0;
+                for (; sl + 8 <= a.S; sl += 8) {  // loads of a batch are independent; the sum keeps slab order
                     float q[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u)
-                        q[u] = __hip_atomic_load(p + (size_t)(s + u) * stride, __ATOMIC_RELAXED,
+                        q[u] = __hip_atomic_load(p + (size_t)(sl + u) * stride, __ATOMIC_RELAXED,
                                                  __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                     for (int u = 0; u < 8; ++u) v += q[u];
                 }
-                for (; s < a.S; ++s)
-                    v += __hip_atomic_load(p + (size_t)s * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (; sl < a.S; ++sl)
+                    v += __hip_atomic_load(p + (size_t)sl * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             total[t] = v;
         }
         if (tid == 0)
-            __hip_atomic_store(a.counters + blockIdx.y * a.tiles + tile, 0u, __ATOMIC_RELAXED,
+            __hip_atomic_store(a.counters + (size_t)(blockIdx.y * a.tiles + tile) * kCounterStride, 0u, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue: channel scales, cast, store
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int m = wv + t * kWaves;
+        const int m = wv + t * waves;
         if (m >= RT || !col_ok || (m0 + m) >= a.M) continue;
         float v = total[t];
         if (a.csm == GLA_CSM_WEIGHT) {
@@ -296,7 +389,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
     for (int u = 0; u < kBatch; ++u) {
         int row = r0 + (lsr0 + 4 * (u / LW)) * LW + (u % LW);
         if (row > a.R - 1) row = a.R - 1;  // activation rows there are staged as zeros
-        buf[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
+        buf[u] = load_streaming_u4(wbase + (int64_t)row * a.wsk);
     }
     // keep every load above in flight before anything below consumes one of them
     __builtin_amdgcn_sched_barrier(0);
@@ -412,7 +505,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
             for (int u = 0; u < kBatch; ++u) {
                 int row = r0 + (lsr0 + 4 * (ib + IPB + u / LW)) * LW + (u % LW);
                 if (row > a.R - 1) row = a.R - 1;
-                buf[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
+                buf[u] = load_streaming_u4(wbase + (int64_t)row * a.wsk);
             }
         }
 #pragma unroll
@@ -468,8 +561,10 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
 // table), so waves run independently until the final reduction and compute overlaps the stream.
 // LOOP = false: exactly one batch of kBatch loads per lane (everything in flight at once).
 // ---------------------------------------------------------------------------------------------
+// kWaves = 0: the wave count is blockDim.x / 64, any number from 4 to 16 (row tiles up to 4), so that
+// the K slabs of a column tile can be cut equal: 56 wave-batches are 4 slabs of 14 waves, not 16/16/16/8.
 template <int BITS, bool BF16, int RT, int kWaves, bool LOOP>
-__global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
+__global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kernel(GemvArgs a) {
     using SH = Shape<BITS>;
     constexpr int E = SH::E, LW = SH::LW, T = SH::T;  // T MFMA K-steps per super row (2 for 2-bit codes)
     static_assert(BITS == 2 || BITS == 4 || BITS == 8, "direct variant: 2-, 4- and 8-bit codes");
@@ -484,8 +579,9 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
 
     extern __shared__ __align__(16) unsigned char smem[];
     const int nfb = a.nfb;                                        // flush blocks per batch
+    const int waves = kWaves ? kWaves : (int)(blockDim.x >> 6);
     float2* mtw = (float2*)smem + (size_t)(threadIdx.x >> 6) * nfb * kTileN;  // [nfb][64], this wave's
-    float* red = (float*)((float2*)smem + (size_t)kWaves * nfb * kTileN);     // [kWaves][RT][64]
+    float* red = (float*)((float2*)smem + (size_t)waves * nfb * kTileN);      // [waves][RT][64]
     __shared__ unsigned ticket;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
@@ -495,8 +591,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
     const int m0 = blockIdx.y * RT;
     const int n0 = tile * kTileN;
     const int r0 = split * a.RW;
-    const int SRWW = a.RW / LW / kWaves;  // super rows per wave
-    const int nit = SRWW / 4;             // wave iterations
+    const int SRWW = a.RW / LW / waves;  // super rows per wave
+    const int nit = SRWW / 4;            // wave iterations
     const int lsr0 = wv * SRWW + kb;
     const int g0w = (r0 + wv * SRWW * LW) / a.gr;  // first group this wave touches
 
@@ -535,8 +631,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
                 int n = n0 + (item & 15) * 4;
                 if (n > a.N - 4) n = a.N - 4;
                 if (p == 0 || nfb > 4) {
-                    b.sr[p] = *(const uint2*)((const uint16_t*)a.scales + (int64_t)g * a.msg + n);
-                    b.zr[p] = *(const uint2*)((const uint16_t*)a.zeros + (int64_t)g * a.msg + n);
+                    b.sr[p] = load_streaming_u2((const uint16_t*)a.scales + (int64_t)g * a.msg + n);
+                    b.zr[p] = load_streaming_u2((const uint16_t*)a.zeros + (int64_t)g * a.msg + n);
                 }
             }
         }
@@ -553,7 +649,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_direct_kernel(GemvArgs a) {
         for (int u = 0; u < kBatch; ++u) {
             int row = r0 + (lsr0 + 4 * (ib + u / LW)) * LW + (u % LW);
             if (row > a.R - 1) row = a.R - 1;
-            b.wr[u] = *(const uint4*)(wbase + (int64_t)row * a.wsk);
+            b.wr[u] = load_streaming_u4(wbase + (int64_t)row * a.wsk);
         }
     };
 
@@ -746,18 +842,27 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     if (p.tile_config >= 1000) {
         waves = p.tile_config / 1000;
         nb = p.tile_config % 1000;
-        if (!(waves == 4 || waves == 8 || waves == 16) || waves > max_waves || nb < 1) return false;
+        const bool any_count = can_direct && nb == 1 && waves >= (g.RT <= 4 ? 4 : 8) && waves <= 16;
+        if (!(waves == 4 || waves == 8 || waves == 16 || any_count) || waves > max_waves || nb < 1) return false;
     } else {
         // Slabs along K: enough workgroups to cover the CUs, and few enough wave-batches per
         // workgroup that every load of the kernel is in flight at once (one batch per wave).
-        int s_min = ceil_div(128, g.tiles * g.mchunks);
-        if (s_min < 1) s_min = 1;
+        // A chip's worth of workgroups (256 CUs) unless the column tiles alone nearly give that: with
+        // 200+ tiles a second slab buys little bandwidth and costs the combining round trip.
+        const int cols = g.tiles * g.mchunks;
+        int s_min = cols >= 192 ? 1 : ceil_div(g.RT <= 4 ? 256 : 128, cols);  // the 16-row tile: half as many, larger workgroups
         int want_s = ceil_div(units, max_waves);
         if (want_s < s_min) want_s = s_min;
         if (want_s > units) want_s = units;
         int per_wg = ceil_div(units, want_s);  // wave-batches per workgroup
-        waves = per_wg <= 4 ? 4 : (per_wg <= 8 && max_waves >= 8 ? 8 : max_waves);
-        nb = ceil_div(per_wg, waves);
+        if (can_direct && per_wg <= max_waves && (g.RT <= 4 || per_wg > 8)) {
+            // one batch per wave and exactly as many waves as batches: equal slabs
+            waves = per_wg < 4 ? 4 : per_wg;
+            nb = 1;
+        } else {
+            waves = per_wg <= 4 ? 4 : (per_wg <= 8 && max_waves >= 8 ? 8 : max_waves);
+            nb = ceil_div(per_wg, waves);
+        }
     }
     g.direct = can_direct;
     if (g.direct && nb > 1 && waves != 4) {  // the looping direct variant runs 4 waves
@@ -786,7 +891,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
         if (nb > 1) {
             --nb;
         } else if (waves > 4) {
-            waves /= 2;
+            waves = waves > 8 ? 8 : 4;
         } else {
             return false;
         }
@@ -796,7 +901,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     const bool split8 = p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16;
     if (split8 && !g.direct) return false;
     // a ragged last slab is fine in either variant: rows past K multiply zeroed activations
-    if (g.S > 1 && (int64_t)g.tiles * g.mchunks * 4 > kCounterBytes) return false;
+    if (g.S > 1 && (int64_t)g.tiles * g.mchunks * kCounterStride * 4 > kCounterBytes) return false;
     return true;
 }
 
@@ -817,8 +922,17 @@ void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
             } else if (g.waves == 8)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 8, false>), grid, dim3(512), g.smem, stream, a);
-            else
+            else if (g.waves == 4)
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, false>), grid, dim3(256), g.smem, stream, a);
+            else {
+                if constexpr (RT == 16) {  // a cross-wave buffer of up to 60 KiB
+                    static DeviceOnce once;
+                    if (once.first())
+                        (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 0, false>,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
+                }
+                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 0, false>), grid, dim3(g.waves * 64), g.smem, stream, a);
+            }
             return;
         }
     }
@@ -898,11 +1012,16 @@ int gemv_packed_default_config(const gla_matmul_args& p) {
     return g.waves * 1000 + g.nb;
 }
 
+// Tagged slots when they fit the region no other kernel writes; else fp32 partials behind it.
+static bool slots_fit(const Geometry& g, const gla_matmul_args& p) {
+    return (int64_t)g.S * g.Mp * p.N * 8 <= kSlotBytes;
+}
+
 int64_t gemv_packed_workspace_bytes(const gla_matmul_args& p) {
     Geometry g;
     if (!geometry(p, g)) return 0;
     if (g.S <= 1) return 0;
-    return kCounterBytes + (int64_t)g.S * g.Mp * p.N * 4;
+    return slots_fit(g, p) ? kWsPrivateBytes : kWsPrivateBytes + (int64_t)g.S * g.Mp * p.N * 4;
 }
 
 int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
@@ -913,7 +1032,7 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
     }
     GemvArgs a;
     a.w = (const uint32_t*)p.w; a.x = p.x; a.scales = p.scales; a.zeros = p.zeros; a.scales_x = p.scales_x;
-    a.out = p.out; a.partials = nullptr; a.counters = nullptr;
+    a.out = p.out; a.partials = nullptr; a.slots = nullptr; a.counters = nullptr;
     a.bias = p.bias; a.bias_dt = p.bias_dtype;
     if (g.S > 1) {
         const int64_t need = gemv_packed_workspace_bytes(p);
@@ -923,7 +1042,8 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
             return GLA_ERR_WORKSPACE_TOO_SMALL;
         }
         a.counters = (unsigned*)p.workspace;
-        a.partials = (float*)((char*)p.workspace + kCounterBytes);
+        if (slots_fit(g, p)) a.slots = (unsigned long long*)((char*)p.workspace + kCounterBytes);
+        else a.partials = (float*)((char*)p.workspace + kWsPrivateBytes);
     }
     a.M = p.M; a.N = p.N; a.K = p.K; a.R = g.R; a.RW = g.RW; a.S = g.S; a.tiles = g.tiles; a.Mp = g.Mp;
     a.gr = g.gr; a.G = g.G; a.GW = g.GW; a.FL = g.FL; a.waves = g.waves; a.nfb = g.nfb;

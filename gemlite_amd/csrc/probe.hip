@@ -1,8 +1,15 @@
-// Diagnostic: the matrix rate the device sustains.  A register-only loop of independent MFMAs on
+// Diagnostics, no counterpart in the reference.
+//
+// (1) The matrix rate the device sustains.  A register-only loop of independent MFMAs on
 // every SIMD, no memory traffic.  With zero operands this reaches the datasheet rate; with random
 // operand bits the same loop runs into the board's power limit and the clock drops, which is the
 // ceiling any GEMM on real data sees.  Timed by the caller (events around the launch).
-// No counterpart in the reference.
+//
+// (2) The rate at which a kernel can read a buffer once: every workgroup streams one contiguous
+// chunk with 128-bit non-temporal loads, eight in flight per lane, and folds what it read into a
+// value it never stores.  Launched over rotated buffers by the caller, it is the ceiling a
+// weight-streaming kernel of that footprint can reach on the box at hand (launch ramp and tail
+// included).
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -60,7 +67,40 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, int random_o
     if (s == 123.456f) sink[0] = s;  // keeps the loop alive; never true for these operands in practice
 }
 
+// chunked read: workgroup b owns 16-byte pieces [b * per, (b + 1) * per)
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ p, size_t n16, float* sink) {
+    constexpr int U = 8;
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t lo = per * blockIdx.x;
+    size_t hi = lo + per;
+    if (hi > n16) hi = n16;
+    unsigned acc = 0;
+    for (size_t i = lo + threadIdx.x; i < hi; i += (size_t)256 * U) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            size_t j = i + (size_t)u * 256;
+            if (j >= hi) j = hi - 1;
+            v[u] = load_streaming_u4(p + j);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (acc == 0x12345678u) sink[0] = 1.0f;  // keeps the loads alive; the buffers the callers use never fold to this
+}
+
 }  // namespace
+
+int launch_probe_read(const void* buf, int64_t bytes, void* sink, hipStream_t stream) {
+    if (buf == nullptr || sink == nullptr || bytes < 16 || (bytes & 15) || ((uintptr_t)buf & 15)) {
+        set_error("gla_probe_read: a 16-byte aligned device buffer of a multiple of 16 bytes and a 4-byte sink are required");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    // four workgroups of four waves per CU; twice that once every workgroup still streams 128 KiB or more
+    const int grid = bytes >= ((int64_t)256 << 20) ? 2048 : 1024;
+    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, (const uint4*)buf, (size_t)(bytes / 16), (float*)sink);
+    return check_hip(hipGetLastError(), "gla_probe_read launch");
+}
 
 int launch_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, hipStream_t stream) {
     if (iters < 1 || sink == nullptr) {

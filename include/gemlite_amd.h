@@ -184,6 +184,14 @@ int gla_matmul_family(const gla_matmul_args* args);
  * at most sustain.  sink: 4 bytes of device memory (never written in practice). */
 int gla_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, void* stream);
 
+/* Diagnostic, no counterpart in the reference: one kernel that reads `bytes` bytes of `buf` once
+ * (contiguous chunk per workgroup, 128-bit non-temporal loads, eight in flight per lane) and stores
+ * nothing.  Timed by the caller over rotated buffers, it gives the rate at which a kernel can
+ * stream a footprint of that size on the device at hand, launch ramp and tail included: the
+ * ceiling of the weight-streaming kernels.  buf: 16-byte aligned device memory, bytes a multiple
+ * of 16; sink: 4 bytes of device memory (never written in practice). */
+int gla_probe_read(const void* buf, int64_t bytes, void* sink, void* stream);
+
 /* Scratch bytes gla_matmul needs for these arguments (0 if none).  The scratch
  * must be zero-filled once when it is allocated; the library leaves it zeroed
  * where it needs zeros.  (Plays the role of the reference's pre-zeroed output

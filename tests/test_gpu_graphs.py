@@ -70,3 +70,27 @@ def test_workspace_growth_is_refused_during_capture_and_keeps_old_buffers(device
     grown = _ext.get_workspace(device, bigger)
     assert grown.numel() >= 2 * ws.numel() and grown.data_ptr() != ws.data_ptr()
     assert any(r.data_ptr() == ws.data_ptr() for r in _ext._retired_workspaces)
+
+
+def test_two_streams_use_separate_scratch(device):
+    """Split-K launches (fp32 partials + ticket counters in the workspace) issued from two streams at the same
+    time: each stream has a workspace of its own, so every result equals the single-stream one bit for bit."""
+    W_q, s, z = gen_int_case(1024, 8192, 4, 128, torch.float16, seed=5)
+    layer_a = GemLiteLinear(4, 128, 8192, 1024, DType.FP16, DType.FP16).pack(W_q.to(device), s.to(device), z.to(device))
+    W_q, s, z = gen_int_case(2048, 4096, 4, 128, torch.float16, seed=6)
+    layer_b = GemLiteLinear(4, 128, 4096, 2048, DType.FP16, DType.FP16).pack(W_q.to(device), s.to(device), z.to(device))
+    xa, xb = gen_x(1, 8192, torch.float16, seed=7).to(device), gen_x(3, 4096, torch.float16, seed=8).to(device)
+    want_a, want_b = layer_a(xa).clone(), layer_b(xb).clone()
+    torch.cuda.synchronize()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a, outs_b = [], []
+    for _ in range(200):
+        with torch.cuda.stream(sa):
+            outs_a.append(layer_a(xa))
+        with torch.cuda.stream(sb):
+            outs_b.append(layer_b(xb))
+    torch.cuda.synchronize()
+    key_a = _ext._workspace_key(device, sa.cuda_stream)
+    key_b = _ext._workspace_key(device, sb.cuda_stream)
+    assert _ext._workspaces[key_a].data_ptr() != _ext._workspaces[key_b].data_ptr()
+    assert all(torch.equal(o, want_a) for o in outs_a) and all(torch.equal(o, want_b) for o in outs_b)

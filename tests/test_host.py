@@ -516,6 +516,7 @@ def test_workspace_is_per_stream(monkeypatch):
     monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
     monkeypatch.setattr(_ext, "_workspaces", {})
     monkeypatch.setattr(_ext, "_retired_workspaces", [])
+    monkeypatch.setattr(_ext, "_last_eager_key", {})
     dev = torch.device("cuda", 0)
     a = _ext.get_workspace(dev, 1024, stream=0x1000)
     b = _ext.get_workspace(dev, 1024, stream=0x2000)
@@ -525,11 +526,14 @@ def test_workspace_is_per_stream(monkeypatch):
     assert big is not a and big.numel() >= 20 << 20 and a in _ext._retired_workspaces
     assert _ext.get_workspace(dev, 1024, stream=0x2000) is b
     assert _ext.get_workspace(torch.device("cuda", 1), 1024, stream=0x1000) is not big
-    # growing under capture is refused
+    # under capture nothing is allocated: a stream with a buffer keeps it, a stream without one takes the
+    # buffer of the stream this thread last launched on eagerly, and a request no buffer can serve is refused
     monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    assert _ext.get_workspace(dev, 1024, stream=0x1000) is big
+    assert _ext.get_workspace(dev, 1024, stream=0x3000) is b           # last eager launch went to stream 0x2000
     with pytest.raises(RuntimeError, match="captured"):
-        _ext.get_workspace(dev, 1024, stream=0x3000)
-    assert _ext.get_workspace(dev, 1024, stream=0x2000) is b           # an existing buffer is still served
+        _ext.get_workspace(dev, 9 << 20, stream=0x3000)                # b holds 8 MiB
+    assert 0x3000 not in [k[2] for k in _ext._workspaces]
 
 
 # ------------------------------------------------------------------ torch custom op
