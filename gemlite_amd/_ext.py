@@ -96,6 +96,8 @@ SYMBOLS = {
     "gla_probe_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "gla_matmul_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),
+    "gla_matmul_static": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),
+    "gla_static_scratch_bytes": (ctypes.c_int64, []),
     "gla_scale_activations_per_token": (
         ctypes.c_int,
         [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,

@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -282,6 +284,91 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
     }
     if (rc2 == GLA_OK && args->bias != nullptr) rc2 = launch_bias_add(*args, s);
     return rc2;
+}
+
+// ---- gla_matmul without a caller's workspace --------------------------------------------------
+// The scratch that gla_matmul takes as `workspace` (split-K partials, ticket counters, regrouped
+// block scales) lives here in a device array that the code object brings along: nothing is
+// allocated, at set-up or per call.  Each GPU has its own copy at its own address; the array's
+// name is only a host-side handle for hipGetSymbolAddress, and everything below uses the address
+// that call returned for the current device.
+}  // extern "C"
+
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[GLA_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+constexpr size_t kCounterRegionBytes = (size_t)kWsPrivateBytes;  // ticket counters and partial slots of the streaming kernels: must start at zero
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+__global__ void clear_words_kernel(uint32_t* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// Address of this device's copy of `scratch`; the first call on a device looks it up and clears the
+// counter region with a kernel on `stream` (a fill kernel, not a memset: the call may be recorded
+// into a graph).  Every later kernel that takes tickets leaves its counters at zero again.
+int static_scratch(hipStream_t stream, void** out) {
+    int dev = 0;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc != GLA_OK) return rc;
+    if (dev < 0 || dev >= kMaxDevices) {
+        set_error("gla_matmul_static: device index %d is outside the %d devices this entry point keeps scratch for", dev,
+                  kMaxDevices);
+        return GLA_ERR_NO_DEVICE;
+    }
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        static std::mutex mu;
+        std::lock_guard<std::mutex> lock(mu);
+        ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+        if (ptr == nullptr) {
+            rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+            if (rc != GLA_OK) return rc;
+            if (ptr == nullptr) {
+                set_error("gla_matmul_static: the device array has no address on device %d", dev);
+                return GLA_ERR_LAUNCH_FAILED;
+            }
+            const size_t words = kCounterRegionBytes / 4;
+            hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream,
+                               (uint32_t*)ptr, words);
+            rc = check_hip(hipGetLastError(), "gla_matmul_static: clearing the ticket counters");
+            if (rc != GLA_OK) return rc;
+            g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+        }
+    }
+    *out = ptr;
+    return GLA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t gla_static_scratch_bytes(void) { return (int64_t)GLA_STATIC_SCRATCH_BYTES; }
+
+int gla_matmul_static(const gla_matmul_args* args, void* stream) {
+    const int64_t need = gla_matmul_workspace_bytes(args);
+    if (need < 0) return (int)need;
+    if (need > (int64_t)GLA_STATIC_SCRATCH_BYTES) {
+        set_error("gla_matmul_static: this problem (M=%d N=%d K=%d) needs %lld bytes of scratch; the built-in array holds "
+                  "%lld. Use gla_matmul with a workspace of that size", args->M, args->N, args->K, (long long)need,
+                  (long long)GLA_STATIC_SCRATCH_BYTES);
+        return GLA_ERR_WORKSPACE_TOO_SMALL;
+    }
+    gla_matmul_args a = *args;
+    a.workspace = nullptr;
+    a.workspace_bytes = 0;
+    if (need > 0) {
+        void* ptr = nullptr;
+        const int rc = static_scratch((hipStream_t)stream, &ptr);
+        if (rc != GLA_OK) return rc;
+        a.workspace = ptr;
+        a.workspace_bytes = (uint64_t)GLA_STATIC_SCRATCH_BYTES;
+    }
+    return gla_matmul(&a, stream);
 }
 
 int gla_scale_activations_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, int K, void* y,

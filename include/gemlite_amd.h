@@ -201,6 +201,21 @@ int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args);
 /* Launch one quantized matmul (reference: the five launchers listed above). */
 int gla_matmul(const gla_matmul_args* args, void* stream);
 
+/* gla_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, same kernels and bit-identical results, except that `workspace` / `workspace_bytes` of
+ * the struct are ignored: the scratch is a device array of GLA_STATIC_SCRATCH_BYTES bytes that the
+ * library's code object carries (each GPU the library runs on holds its own copy until the process
+ * ends).  The call allocates and frees nothing.  A problem whose gla_matmul_workspace_bytes()
+ * exceeds GLA_STATIC_SCRATCH_BYTES is refused with GLA_ERR_WORKSPACE_TOO_SMALL.  The first call on
+ * a device that needs scratch looks the array's address up and clears its ticket counters with a
+ * small kernel on `stream`.  All calls on one GPU share the array: calls that may overlap in time
+ * on one GPU (two streams, two graphs replayed concurrently) race and must use gla_matmul with
+ * workspaces of their own. */
+#define GLA_STATIC_SCRATCH_BYTES (72u << 20)
+int64_t gla_static_scratch_bytes(void);
+int gla_matmul_static(const gla_matmul_args* args, void* stream);
+
 /* Per-token dynamic activation quantisation to fp8-e4m3fn or int8:
  *   s[m] = max(amax(|x[m,:]|) / qmax, 1e-6);  y = clamp(x / s, qmin, qmax);
  *   int8 rounds with floor(y + 0.5).

@@ -536,6 +536,27 @@ def test_workspace_is_per_stream(monkeypatch):
     assert 0x3000 not in [k[2] for k in _ext._workspaces]
 
 
+def test_static_scratch_entry_point_refuses_oversize_without_a_gpu():
+    lib = _ext.load_library()
+    assert lib.gla_static_scratch_bytes() == 72 << 20
+    a = _ext.MatmulArgs()
+    a.struct_size = ctypes.sizeof(a)
+    a.matmul_type = 3
+    a.M, a.N, a.K = 512, 16384, 16384
+    for f in ("x", "w", "scales", "zeros", "out"):
+        setattr(a, f, 1 << 20)  # never dereferenced: the size check comes first
+    a.x_stride_m, a.x_stride_k, a.w_stride_k, a.w_stride_n = 16384, 1, 16384, 1
+    a.out_stride_m, a.out_stride_n, a.meta_stride_g, a.meta_stride_n = 16384, 1, 16384, 1
+    a.W_nbits, a.group_size, a.unpack_mask, a.elements_per_sample = 2, 64, 3, 16
+    a.input_dtype = a.output_dtype = a.meta_dtype = a.zeros_dtype = DType.BF16.value
+    a.acc_dtype, a.channel_scale_mode, a.W_group_mode, a.data_contiguous = DType.FP32.value, 0, 4, 1
+    a.w_dtype, a.tile_config = DType.INT32.value, 4256
+    need = lib.gla_matmul_workspace_bytes(ctypes.byref(a))
+    assert need > 72 << 20
+    assert lib.gla_matmul_static(ctypes.byref(a), None) == -5
+    assert b"gla_matmul_static" in lib.gla_last_error() and str(need).encode() in lib.gla_last_error()
+
+
 # ------------------------------------------------------------------ torch custom op
 def test_custom_op_fake_shape_and_dtype():
     """The registered op's fake implementation (what torch.compile sees) returns [..., N] in the layer's
