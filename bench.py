@@ -8,6 +8,13 @@ A16W4 (HQQ asymmetric, group 128, 32-bit packing, fp16), launched through the C 
 cache level holds the weights between steps.  The metric is algorithmic bytes per step (every
 operand read once, the output written once) divided by the time per step.
 
+`extra` carries the other points of the benchmark table, each measured in the same run: the
+4096^2 decode GEMV, the 16384^2 8-bit channel-wise and 2-bit group-64 layers at M = 1/16/64/512,
+fp8 / int8 / MXFP4 GEMMs, MXFP4 at M = 1/32/1024/8192, the activation quantisers, and the rate at
+which a plain read kernel streams the same footprints on this box.  Every bandwidth-bound point
+rotates over distinct copies of its operands that add up to more than 512 MB, twice the 256 MB
+Infinity Cache, and is timed as a HIP-graph replay with one launch per copy.
+
 Prints ONE JSON line (see the `out` dict at the end).
 """
 import argparse
@@ -26,14 +33,15 @@ import gemlite_amd  # noqa: E402
 from gemlite_amd import DType, GemLiteLinear, _ext  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+ROTATE_BYTES = 600e6   # distinct operand bytes a bandwidth-bound point cycles through (> 2 x 256 MB)
 
 SHAPES = [(14336, 4096), (4096, 14336)]  # (N, K): up / down projection
 GROUP = 128
 
 
-def algorithmic_bytes(N, K, M=1, nbits=4, gs=GROUP):
-    """W_q + scales + zeros + x + out, each touched once (fp16 metadata and activations)."""
-    return N * K * nbits // 8 + 2 * (N * K // gs) * 2 + M * K * 2 + M * N * 2
+def algorithmic_bytes(N, K, M=1, nbits=4, gs=GROUP, elt=2):
+    """W_q + scales + zeros + x + out, each touched once (16-bit metadata and activations)."""
+    return N * K * nbits // 8 + 2 * (N * K // gs) * elt + M * K * elt + M * N * elt
 
 
 def make_layer(N, K, seed, device):
@@ -55,23 +63,28 @@ def clone_layer(layer):
 class Launch:
     """A prepared `gla_matmul` call: argument struct built once, launched on the current stream."""
 
-    def __init__(self, lib, layer, x, out, device):
+    def __init__(self, lib, layer, x, out, device, scales_x=None):
         m = layer.get_meta_args()
         self.lib = lib
+        in_dt = m[5]
+        if scales_x is None and not gemlite_amd.dtypes.is_mx_dtype(in_dt):
+            in_dt = gemlite_amd.TORCH_TO_DTYPE[x.dtype].value  # the kernels read x as the type it has
+        elif scales_x is None:  # weight-only MX layer
+            in_dt = DType.MXFP16.value if x.dtype == torch.float16 else DType.MXBF16.value
         self.args = _ext.build_matmul_args(
-            x, layer.W_q, layer.scales, layer.zeros, None, out,
-            W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5],
+            x, layer.W_q, layer.scales, layer.zeros, scales_x, out,
+            W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=in_dt,
             output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
-            data_contiguous=m[11],  # matmul type left to the dispatcher (RevSplit-K up to 4 rows, Split-K GEMM above)
+            data_contiguous=m[11],  # matmul type left to the dispatcher
         )
         need = lib.gla_matmul_workspace_bytes(ctypes.byref(self.args))
         if need < 0:
             raise RuntimeError(lib.gla_last_error().decode())
         if need > 0:
-            ws = _ext.get_workspace(device, need)
-            self.args.workspace = ws.data_ptr()
+            ws = _ext.get_workspace(device, need, stream=0)   # one buffer for everything this script launches:
+            self.args.workspace = ws.data_ptr()               # all of it runs in order on one stream
             self.args.workspace_bytes = ws.numel()
-        self.keep = (layer, x, out)
+        self.keep = (layer, x, out, scales_x)
 
     def __call__(self):
         rc = self.lib.gla_matmul(ctypes.byref(self.args), torch.cuda.current_stream().cuda_stream)
@@ -79,48 +92,96 @@ class Launch:
             raise RuntimeError(self.lib.gla_last_error().decode())
 
 
-def time_us(fn, reps, warm=25):
-    """Average microseconds per call of `fn` on the current stream (events on that stream)."""
-    for _ in range(warm):
-        fn()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / reps
+class Timer:
+    """Event timing on the stream the work is launched on (a side stream, also used for capture)."""
+
+    def __init__(self):
+        self.side = torch.cuda.Stream()
+
+    def graph_us(self, fns, reps):
+        """Average microseconds per call: one graph holding every callable of `fns` once, replayed `reps` times."""
+        with torch.cuda.stream(self.side):
+            for f in fns[:2]:
+                f()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=self.side):
+                for f in fns:
+                    f()
+            gr.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(self.side)
+            for _ in range(reps):
+                gr.replay()
+            e1.record(self.side)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * len(fns))
+
+    def eager_us(self, fn, reps, warm=3):
+        with torch.cuda.stream(self.side):
+            for _ in range(warm):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(self.side)
+            for _ in range(reps):
+                fn()
+            e1.record(self.side)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
 
 
-def extra_points(lib, device):
-    """The other points of the benchmark table, measured briefly (synthetic data, same C ABI):
-    GEMM TFLOP/s at M=4096 for each operand format, activation quantisers, the 4096^2 decode GEMV."""
+def copies_for(nbytes):
+    return max(2, int(ROTATE_BYTES // nbytes) + 1)
+
+
+def bw_point(us, nbytes, **more):
+    gbs = nbytes / us / 1e3
+    return {"us": round(us, 2), "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "bytes": int(nbytes), **more}
+
+
+def extra_points(lib, device, T, quick):
+    """The other points of the benchmark table (synthetic data, same C ABI)."""
     from gemlite_amd import helper
     out = {}
     g = torch.Generator(device="cpu").manual_seed(7)
+    stream = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
 
-    def prepared(layer, x, scales_x, y):
-        m = layer.get_meta_args()
-        args = _ext.build_matmul_args(
-            x, layer.W_q, layer.scales, layer.zeros, scales_x, y,
-            W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5],
-            output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
-            data_contiguous=m[11])
-        need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))
-        if need > 0:
-            ws = _ext.get_workspace(device, need)
-            args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+    # ---- what a plain read kernel streams on this box (launch ramp and tail included), rotated buffers
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+    ceil = {}
+    for label, nbytes in (("9MB", 8929280), ("31MB", 31232000), ("268MB", 268435456)):
+        n = copies_for(nbytes)
+        bufs = [torch.full((nbytes // 4,), 0x01010101, dtype=torch.int32, device=device) for _ in range(n)]
 
-        def run():
-            if lib.gla_matmul(ctypes.byref(args), torch.cuda.current_stream().cuda_stream) != 0:
-                raise RuntimeError(lib.gla_last_error().decode())
-        return run
+        def reader(b):
+            def run():
+                if lib.gla_probe_read(b.data_ptr(), b.numel() * 4, sink.data_ptr(), stream()) != 0:
+                    raise RuntimeError(lib.gla_last_error().decode())
+            return run
+        us = T.graph_us([reader(b) for b in bufs], 4 if nbytes > 1e8 else 10)
+        ceil[label] = bw_point(us, nbytes, copies=n)
+        del bufs
+    out["read_ceiling"] = {"kernel": "gla_probe_read (contiguous chunks, 128-bit non-temporal loads, nothing stored)", **ceil}
+    torch.cuda.empty_cache()
+
+    # ---- C1: A16W4 gs128 fp16, K = N = 4096, M = 1 (and the same layer at M = 4096 below)
+    N = K = 4096
+    base, _ = make_layer(N, K, seed=11, device=device)
+    nbytes = algorithmic_bytes(N, K)
+    layers = [base] + [clone_layer(base) for _ in range(copies_for(nbytes) - 1)]
+    x1 = torch.randn((1, K), generator=g).to(torch.float16).to(device)
+    y1 = torch.empty((1, N), dtype=torch.float16, device=device)
+    us = T.graph_us([Launch(lib, l, x1, y1, device) for l in layers], 10)
+    out["gemv_a16w4_gs128_4096sq_M1"] = bw_point(
+        us, nbytes, copies=len(layers), frac_of_read_ceiling=round(nbytes / us / 1e3 / ceil["9MB"]["GB/s"], 4))
+    del layers
 
     # Sustained matrix rate of this board: a register-only MFMA loop (no memory traffic) with zero and
     # with random operand bits.  With random bits the power limit lowers the clock; that rate, not the
     # datasheet one, is what a GEMM on real data can at most reach here.
-    sink = torch.zeros(1, dtype=torch.float32, device=device)
     probe = {}
     for name, dt in (("fp16", 1), ("bf16", 2), ("fp8", 3), ("int8", 4), ("mxfp4", 17)):
         rates = {}
@@ -128,15 +189,14 @@ def extra_points(lib, device):
             flops = ctypes.c_double(0.0)
 
             def run():
-                if lib.gla_probe_mfma(dt, rnd, 60000, sink.data_ptr(), ctypes.byref(flops),
-                                      torch.cuda.current_stream().cuda_stream) != 0:
+                if lib.gla_probe_mfma(dt, rnd, 60000, sink.data_ptr(), ctypes.byref(flops), stream()) != 0:
                     raise RuntimeError(lib.gla_last_error().decode())
-            us = time_us(run, 3, warm=1)
+            us = T.eager_us(run, 3, warm=1)
             rates[label + "_TFLOP/s"] = round(flops.value / us / 1e6, 1)
         probe[name] = rates
     out["mfma_probe"] = probe
 
-    def point(name, M, N, K, us, peak_tf, kind, us_zero=None):
+    def gemm_point(name, M, N, K, us, peak_tf, kind, us_zero=None, us_e2e=None):
         tf = 2.0 * M * N * K / us / 1e6
         sustained = probe[kind]["random_operands_TFLOP/s"]
         out[name] = {"M": M, "N": N, "K": K, "us": round(us, 1), "TFLOP/s": round(tf, 1),
@@ -147,153 +207,178 @@ def extra_points(lib, device):
             # switching power, so the clock stays up; the gap to `us` is the board's power limit
             out[name]["us_zero_operands"] = round(us_zero, 1)
             out[name]["frac_of_peak_zero_operands"] = round(2.0 * M * N * K / us_zero / 1e6 / peak_tf, 4)
+        if us_e2e is not None:
+            out[name]["us_with_activation_quantiser"] = round(us_e2e, 1)
 
     def zeroed(run, *tensors):
         """Time `run` again with the given operand tensors zero-filled (they are scratch copies)."""
         for t in tensors:
             t.view(torch.uint8).zero_()
-        return time_us(run, 30)
+        return T.eager_us(run, 20)
 
     # A16W4 gs128 fp16, M = 4096 (fused-dequant MFMA GEMM)
-    M, N, K = 4096, 4096, 4096
-    layer, _ = make_layer(N, K, seed=11, device=device)
+    M = 4096
     x = torch.randn((M, K), generator=g).to(torch.float16).to(device)
     y = torch.empty((M, N), dtype=torch.float16, device=device)
-    run = prepared(layer, x, None, y)
-    us = time_us(run, 50)
-    point("gemm_a16w4_gs128_fp16", M, N, K, us, 2500.0, "fp16", zeroed(run, x, layer.W_q.data))
-    del layer, x, y
+    run = Launch(lib, base, x, y, device)
+    us = T.eager_us(run, 40)
+    gemm_point("gemm_a16w4_gs128_fp16", M, N, K, us, 2500.0, "fp16", zeroed(run, x, base.W_q.data))
+    del base, x, y, run
 
-    # A8W8 fp8 / int8 dynamic, M = 4096, N = K = 8192: activation quantiser + GEMM
+    # ---- C3: bf16 activations, K = N = 16384: 8-bit channel-wise and 2-bit group-64 weights, M = 1 / 16 / 64 / 512
+    N = K = 16384
+    for tag, nbits, gs in (("a16w8_channelwise", 8, K), ("a16w2_gs64", 2, 64)):
+        W_q = torch.randint(0, 2 ** nbits, (N, K), dtype=torch.uint8, device=device)
+        groups = N * K // gs
+        sc = (torch.randn((groups, 1), device=device) * 0.01).abs().clamp_(min=1e-4).to(torch.bfloat16)
+        zr = (torch.rand((groups, 1), device=device) * (2 ** nbits) / 4 + (2 ** nbits) * 3 / 8).to(torch.bfloat16)
+        layer = helper.A16Wn(device=device, post_scale=True).from_weights(W_q, sc, zr, nbits, gs)
+        del W_q
+        wbytes = N * K * nbits // 8 + 2 * groups * 2   # codes + scales + zeros
+        layers = [layer] + [clone_layer(layer) for _ in range(copies_for(wbytes) - 1)]
+        for M in (1, 16, 64, 512):
+            if quick and M in (16, 64):
+                continue
+            xm = torch.randn((M, K), device=device).to(torch.bfloat16)
+            ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+            us = T.graph_us([Launch(lib, l, xm, ym, device) for l in layers], 4)
+            nbytes = wbytes + M * K * 2 + M * N * 2
+            if M <= 16:
+                out[f"gemv_{tag}_16384sq_M{M}"] = bw_point(us, nbytes, copies=len(layers))
+            else:
+                gemm_point(f"gemm_{tag}_16384sq_M{M}", M, N, K, us, 2500.0, "bf16")
+                out[f"gemm_{tag}_16384sq_M{M}"].update({"GB/s": round(nbytes / us / 1e3, 1),
+                                                        "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del layers, layer
+        torch.cuda.empty_cache()
+
+    # ---- C4: A8W8 fp8 / int8 dynamic, M = 4096, N = K = 8192: activation quantiser + GEMM
     M, N, K = 4096, 8192, 8192
     W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
-    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    xs = [torch.randn((M, K), device=device).to(torch.bfloat16) for _ in range(copies_for(M * K * 3))]
+    x = xs[0]
     y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
     for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
         layer = proc(device=device).from_weights(W)
         xq, sx = gemlite_amd.scale_activations_per_token(x, wdt)
-        run = prepared(layer, xq, sx, y)
-        us = time_us(run, 50)
-        point(f"gemm_a8w8_{name}", M, N, K, us, 5000.0, name, zeroed(run, xq, layer.W_q.data))
-        us = time_us(lambda: gemlite_amd.scale_activations_per_token(x, wdt), 20)
-        out[f"actquant_per_token_{name}"] = {"M": M, "K": K, "us": round(us, 1),
-                                            "GB/s": round((M * K * 3 + M * 4) / us / 1e3, 1)}
-        del layer, xq, sx
-    del W, x, y
-
-    # A8W8 MXFP8 weights, fp8 activations quantised per token (the reference processor's default), M = 4096, N = K = 8192
-    M, N, K = 4096, 8192, 8192
+        run = Launch(lib, layer, xq, y, device, scales_x=sx)
+        us = T.eager_us(run, 40)
+        us_e2e = T.eager_us(lambda: layer(x), 20)
+        gemm_point(f"gemm_a8w8_{name}", M, N, K, us, 5000.0, name, zeroed(run, xq, layer.W_q.data), us_e2e)
+        # the quantiser alone, reading a different activation matrix every launch
+        xq_o, sx_o = torch.empty_like(xq), torch.empty_like(sx)
+        fns = [(lambda xi=xi: _ext.scale_activations_per_token(xi, xq_o, sx_o)) for xi in xs]
+        us = T.graph_us(fns, 6)
+        out[f"actquant_per_token_{name}"] = bw_point(us, M * K * 3 + M * 4, M=M, K=K, copies=len(xs))
+        del layer, xq, sx, run
+    # MXFP8 weights, fp8 activations quantised per token (the reference processor's default)
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
-    lin.weight.data = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
-    layer = helper.A8W8_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
-    del lin
-    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    lin.weight.data = W
+    layer = helper.A8W8_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device), del_orig=False)
     xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn)
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    run = prepared(layer, xq, sx, y)
-    us = time_us(run, 50)
-    point("gemm_a8w8_mxfp8", M, N, K, us, 5000.0, "fp8", zeroed(run, xq, layer.W_q.data))
-    del layer, x, xq, sx, y
+    run = Launch(lib, layer, xq, y, device, scales_x=sx)
+    us = T.eager_us(run, 40)
+    gemm_point("gemm_a8w8_mxfp8", M, N, K, us, 5000.0, "fp8", zeroed(run, xq, layer.W_q.data))
+    del layer, lin, xq, sx, run
+    # 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5)
+    if not quick:
+        for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
+            layer = proc(device=device, block_quant=True).from_weights(W)
+            xq, sx = gemlite_amd.scale_activations_per_block(x, wdt)
+            us = T.eager_us(Launch(lib, layer, xq, y, device, scales_x=sx), 30)
+            gemm_point(f"gemm_a8w8_{name}_block_quant", M, N, K, us, 5000.0, name)
+            xq_o, sx_o = torch.empty_like(xq), torch.empty_like(sx)
+            us = T.graph_us([(lambda xi=xi: _ext.scale_activations_per_block(xi, xq_o, sx_o)) for xi in xs], 6)
+            out[f"actquant_per_block_{name}"] = bw_point(us, M * K * 3 + M * K // 128 * 4, M=M, K=K, copies=len(xs))
+            del layer, xq, sx
+        # A16W8 weight-only int8 bytes (unpacked), bf16: M = 4096 (MFMA GEMM) and M = 1 (streaming, rotated)
+        layer = helper.A16W8_INT8(device=device, post_scale=True).from_weights(W)
+        us = T.eager_us(Launch(lib, layer, x, y, device), 20)
+        gemm_point("gemm_a16w8_int8_bytes_bf16", M, N, K, us, 2500.0, "bf16")
+        wbytes = N * K + N * 4
+        layers = [layer] + [clone_layer(layer) for _ in range(copies_for(wbytes) - 1)]
+        x1 = x[:1].contiguous()
+        y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
+        us = T.graph_us([Launch(lib, l, x1, y1, device) for l in layers], 6)
+        out["gemv_a16w8_int8_bytes_M1"] = bw_point(us, wbytes + K * 2 + N * 2, N=N, K=K, copies=len(layers))
+        del layers, layer
+    del W, xs, x, y
+    torch.cuda.empty_cache()
 
-    # A16W8 weight-only int8 bytes (unpacked), bf16, N = K = 8192: M = 4096 (MFMA GEMM) and M = 1 (streaming)
-    M, N, K = 4096, 8192, 8192
-    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
-    layer = helper.A16W8_INT8(device=device, post_scale=True).from_weights(W)
-    del W
-    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    run = prepared(layer, x, None, y)
-    us = time_us(run, 30)
-    point("gemm_a16w8_int8_bytes_bf16", M, N, K, us, 2500.0, "bf16")
-    x1 = x[:1].contiguous()
-    y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
-    us = time_us(prepared(layer, x1, None, y1), 50)
-    out["gemv_a16w8_int8_bytes_M1"] = {"N": N, "K": K, "us": round(us, 1), "GB/s": round((N * K + N * 4 + K * 2 + N * 2) / us / 1e3, 1),
-                                       "note": "64 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"}
-    del layer, x, y, x1, y1
-
-    # A4W4 MXFP4 dynamic, M = 4096, N = K = 16384
-    M, N, K = 4096, 16384, 16384
+    # ---- C5: MXFP4 x MXFP4, K = N = 16384, M = 1 / 32 / 1024 / 4096 / 8192
+    N = K = 16384
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
     lin.weight.data = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
     layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
     del lin
-    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
-    xq, sx = gemlite_amd.scale_activations_mxfp4(x)
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    run = prepared(layer, xq, sx, y)
-    us = time_us(run, 30)
-    w_saved = layer.W_q.data.clone()
-    point("gemm_a4w4_mxfp4", M, N, K, us, 10100.0, "mxfp4", zeroed(run, xq, layer.W_q.data))
-    layer.W_q.data.copy_(w_saved)
-    del w_saved
-    us = time_us(lambda: gemlite_amd.scale_activations_mxfp4(x), 20)
-    out["actquant_mxfp4"] = {"M": M, "K": K, "us": round(us, 1),
-                             "GB/s": round((M * K * 2 + M * K // 2 + M * K // 32) / us / 1e3, 1)}
-    # the same layer at M = 1: weight-streaming, HBM-bound
-    x1 = torch.randn((1, K), generator=g).to(torch.bfloat16).to(device)
-    xq1, sx1 = gemlite_amd.scale_activations_mxfp4(x1)
-    y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
-    us = time_us(prepared(layer, xq1, sx1, y1), 50)
-    out["gemv_a4w4_mxfp4_M1"] = {"N": N, "K": K, "us": round(us, 1),
-                                 "GB/s": round((N * K // 2 + N * K // 32 + K // 2 + N * 2) / us / 1e3, 1)}
-    w_codes, w_scales = layer.W_q.data, layer.scales.data
-    del layer, x, xq, sx, y, xq1, sx1, y1
-
-    # Weight-only MXFP4 (bf16 activations as they are) on the same codes: the streaming MX kernel, M = 1, 2, 4
-    wo = helper.A16W4_MXFP(device=device, dtype=torch.bfloat16).from_packed_weights(
-        w_codes.t(), w_scales.view(torch.float8_e8m0fnu))
-    for M in (1, 2, 4):
-        xm = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+    wbytes = N * K // 2 + N * K // 32
+    layers = [layer] + [clone_layer(layer) for _ in range(copies_for(wbytes) - 1)]
+    for M in (1, 32):
+        xm = torch.randn((M, K), device=device).to(torch.bfloat16)
+        xq, sx = gemlite_amd.scale_activations_mxfp4(xm)
         ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-        us = time_us(prepared(wo, xm, None, ym), 50)
-        out[f"gemv_a16w4_mxfp_M{M}"] = {"N": N, "K": K, "us": round(us, 1),
-                                        "GB/s": round((N * K // 2 + N * K // 32 + M * K * 2 + M * N * 2) / us / 1e3, 1)}
-    out["gemv_a16w4_mxfp_M1"]["note"] = "134 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"
-    # ... and at M = 4096 on the matrix cores (weights converted to bf16 fragments in registers)
-    xm = torch.randn((4096, K), generator=g).to(torch.bfloat16).to(device)
-    ym = torch.empty((4096, N), dtype=torch.bfloat16, device=device)
-    us = time_us(prepared(wo, xm, None, ym), 20)
-    point("gemm_a16w4_mxfp_bf16", 4096, N, K, us, 2500.0, "bf16")
-    # ... and under fp8 activations quantised per token (A8W4_MXFP_dynamic): the mixed fp8 x fp4 scaled MFMA
-    a84 = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_packed_weights(
-        w_codes.t(), scales=w_scales.view(torch.float8_e8m0fnu))
-    xq, sx = gemlite_amd.scale_activations_per_token(xm, torch.float8_e4m3fn)
-    us = time_us(prepared(a84, xq, sx, ym), 20)
-    point("gemm_a8w4_mxfp", 4096, N, K, us, 5000.0, "fp8")
-    del wo, a84, xq, sx, w_codes, w_scales, xm, ym
+        us = T.graph_us([Launch(lib, l, xq, ym, device, scales_x=sx) for l in layers], 6)
+        out[f"gemv_a4w4_mxfp4_16384sq_M{M}"] = bw_point(us, wbytes + M * K // 2 + M * K // 32 + M * N * 2, copies=len(layers))
+    w_saved = layer.W_q.data.clone()
+    for M in (1024, 4096, 8192):
+        if quick and M == 1024:
+            continue
+        xm = torch.randn((M, K), device=device).to(torch.bfloat16)
+        xq, sx = gemlite_amd.scale_activations_mxfp4(xm)
+        ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+        run = Launch(lib, layer, xq, ym, device, scales_x=sx)
+        us = T.eager_us(run, 12)
+        us_e2e = T.eager_us(lambda: layer(xm), 8)
+        us_zero = None
+        if M == 4096:
+            us_zero = zeroed(run, xq, layer.W_q.data)
+            layer.W_q.data.copy_(w_saved)
+        gemm_point(f"gemm_a4w4_mxfp4_M{M}" if M != 4096 else "gemm_a4w4_mxfp4", M, N, K, us, 10100.0, "mxfp4", us_zero, us_e2e)
+        if M == 4096:
+            xs = [xm] + [torch.randn((M, K), device=device).to(torch.bfloat16) for _ in range(copies_for(M * K * 2.5) - 1)]
+            xq_o, sx_o = torch.empty_like(xq), torch.empty_like(sx)
+            us = T.graph_us([(lambda xi=xi: _ext.scale_activations_mxfp4(xi, xq_o, sx_o)) for xi in xs], 4)
+            out["actquant_mxfp4"] = bw_point(us, M * K * 2 + M * K // 2 + M * K // 32, M=M, K=K, copies=len(xs))
+            del xs
+        del xm, xq, sx, ym, run
+    del w_saved
+    w_codes, w_scales = layer.W_q.data, layer.scales.data
+    del layers
 
-    # 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5), N = K = 8192: per-block activation quantiser,
-    # the MFMA GEMM at M = 4096 and the streaming kernel at M = 1
-    M, N, K = 4096, 8192, 8192
-    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
-    x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-    y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
-    for name, proc, wdt in (("fp8", helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), ("int8", helper.A8W8_INT8_dynamic, torch.int8)):
-        layer = proc(device=device, block_quant=True).from_weights(W)
-        xq, sx = gemlite_amd.scale_activations_per_block(x, wdt)
-        us = time_us(prepared(layer, xq, sx, y), 30)
-        point(f"gemm_a8w8_{name}_block_quant", M, N, K, us, 5000.0, name)
-        us = time_us(lambda: gemlite_amd.scale_activations_per_block(x, wdt), 20)
-        out[f"actquant_per_block_{name}"] = {"M": M, "K": K, "us": round(us, 1),
-                                            "GB/s": round((M * K * 3 + M * K // 128 * 4) / us / 1e3, 1)}
-        xq1, sx1 = gemlite_amd.scale_activations_per_block(x[:1].contiguous(), wdt)
-        us = time_us(prepared(layer, xq1, sx1, y1), 50)
-        out[f"gemv_a8w8_{name}_block_quant_M1"] = {
-            "N": N, "K": K, "us": round(us, 1), "GB/s": round((N * K + N * K // 16384 * 4 + K + N * 2) / us / 1e3, 1),
-            "note": "64 MB of weights, same buffer every call: served partly by the 256 MB Infinity Cache"}
-        del layer, xq, sx, xq1, sx1
+    if not quick:
+        # Weight-only MXFP4 (bf16 activations as they are) on the same codes, rotated: M = 1, 2, 4, 8
+        wo = helper.A16W4_MXFP(device=device, dtype=torch.bfloat16).from_packed_weights(
+            w_codes.t(), w_scales.view(torch.float8_e8m0fnu))
+        wos = [wo] + [clone_layer(wo) for _ in range(copies_for(wbytes) - 1)]
+        for M in (1, 2, 4, 8):
+            xm = torch.randn((M, K), device=device).to(torch.bfloat16)
+            ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
+            us = T.graph_us([Launch(lib, l, xm, ym, device) for l in wos], 4)
+            out[f"gemv_a16w4_mxfp_M{M}"] = bw_point(us, wbytes + M * K * 2 + M * N * 2, copies=len(wos))
+        del wos
+        # ... at M = 4096 on the matrix cores (weights converted to bf16 fragments in registers)
+        xm = torch.randn((4096, K), device=device).to(torch.bfloat16)
+        ym = torch.empty((4096, N), dtype=torch.bfloat16, device=device)
+        us = T.eager_us(Launch(lib, wo, xm, ym, device), 10)
+        gemm_point("gemm_a16w4_mxfp_bf16", 4096, N, K, us, 2500.0, "bf16")
+        # ... and under fp8 activations quantised per token (A8W4_MXFP_dynamic): the mixed fp8 x fp4 scaled MFMA
+        a84 = helper.A8W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_packed_weights(
+            w_codes.t(), scales=w_scales.view(torch.float8_e8m0fnu))
+        xq, sx = gemlite_amd.scale_activations_per_token(xm, torch.float8_e4m3fn)
+        us = T.eager_us(Launch(lib, a84, xq, ym, device, scales_x=sx), 10)
+        gemm_point("gemm_a8w4_mxfp", 4096, N, K, us, 5000.0, "fp8")
     return out
 
 
 def cpu_baseline(host_tensors, x_host, y_gpu, threads):
-    """The reference's CPU path (HQQ dequantize + fp32 matmul) as restated in oracle/oracle_c.c,
-    timed on this box's host cores on whole steps of the same workload; also the parity check."""
+    """The reference's CPU path (HQQ dequantize + fp32 matmul) on this box's host cores, on whole steps of the
+    same workload: the C restatement (oracle/oracle_c.c, OpenMP), which also gives the parity check, and
+    the same two operations written with torch (`W = (W_q - z) * s`; `x @ W.T`), as a user of the reference
+    without a GPU would run them."""
     import numpy as np
 
     lib = ctypes.CDLL(os.path.join(ROOT, "oracle", "liboracle_c.so"))
-    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
     i64 = ctypes.c_int64
     arrs = []
     for (W_q, scales, zeros) in host_tensors:
@@ -311,18 +396,34 @@ def cpu_baseline(host_tensors, x_host, y_gpu, threads):
             v = np.ascontiguousarray(y.astype(np.float16).astype(np.float32))  # fp16 hand-over like the GPU chain
         return v
 
+    def timed(fn, budget_s, max_reps):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > budget_s or reps >= max_reps:
+                return dt / reps, reps
+
     x32 = np.ascontiguousarray(x_host.float().numpy())
-    y_ref = step(x32)  # warm-up + reference output
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        step(x32)
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt > 10.0 or reps >= 20:
-            break
-    sec = dt / reps
+    y_ref = step(x32)
+    sec, reps = timed(lambda: step(x32), 10.0, 20)
     err = float(np.linalg.norm(y_gpu.astype(np.float64) - y_ref) / np.linalg.norm(y_ref))
-    return sec, reps, err
+
+    torch.set_num_threads(threads)
+    tl = [(W_q.view(W_q.shape[0], -1, GROUP), s.float().view(W_q.shape[0], -1, 1), z.float().view(W_q.shape[0], -1, 1))
+          for (W_q, s, z) in host_tensors]
+
+    def torch_step():
+        v = x_host.float()
+        for (q, s, z) in tl:
+            W = ((q.float() - z) * s).view(q.shape[0], -1)
+            v = (v @ W.t()).to(torch.float16).float()
+        return v
+
+    sec_torch, reps_torch = timed(torch_step, 10.0, 20)
+    return sec, reps, err, sec_torch, reps_torch
 
 
 def main():
@@ -333,6 +434,7 @@ def main():
     ap.add_argument("--rotate-gb", type=float, default=3.0, help="total bytes of distinct weight copies")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary benchmark points")
+    ap.add_argument("--quick-extra", action="store_true", help="a subset of the secondary points")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 256 MiB device copy (a kernel of known traffic, to scale profiler byte counters)")
     a = ap.parse_args()
@@ -343,6 +445,7 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     lib = _ext.load_library()
+    T = Timer()
 
     step_bytes = sum(algorithmic_bytes(N, K) for N, K in SHAPES)
     copies = max(2, int(a.rotate_gb * 1e9 // step_bytes) + 1)
@@ -369,95 +472,51 @@ def main():
             down()
 
     # ---- warm-up (eager), then graphs of the timed steps
-    run_steps(0, a.warmup)
-    torch.cuda.synchronize()
-
-    chunk = min(a.steps, 256)
-    full, rem = divmod(a.steps, chunk)
-    side = torch.cuda.Stream()
-    graphs = []
+    side = T.side
     with torch.cuda.stream(side):
-        run_steps(0, 2)
+        run_steps(0, a.warmup)
         torch.cuda.synchronize()
+        chunk = min(a.steps, 256)
+        full, rem = divmod(a.steps, chunk)
+        graphs = []
         for n_steps in ([chunk] if full else []) + ([rem] if rem else []):
             gr = torch.cuda.CUDAGraph()
             with torch.cuda.graph(gr, stream=side):
                 run_steps(0, n_steps)
             graphs.append(gr)
-    torch.cuda.synchronize()
-    for gr in graphs:  # one untimed replay each
-        gr.replay()
-    torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        for gr in graphs:  # one untimed replay each
+            gr.replay()
+        torch.cuda.synchronize()
 
-    # ---- timed region: exactly a.steps steps
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    if full:
-        for _ in range(full):
-            graphs[0].replay()
-    if rem:
-        graphs[-1].replay()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+        # ---- timed region: exactly a.steps steps
+        t0 = time.perf_counter()
+        if full:
+            for _ in range(full):
+                graphs[0].replay()
+        if rem:
+            graphs[-1].replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / a.steps
     value = step_bytes / (elapsed / a.steps) / 1e9
+    y_gpu = y.float().cpu().numpy()
 
-    # ---- launch duration of the dominant kernel (the 4096 -> 14336 GEMV): HIP events on the
-    # launch stream around a timed region that holds only that kernel, one launch per weight copy
-    def kernel_avg_us(which, reps=8):
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(gr, stream=side):
-                for i in range(copies):
-                    launches[i][which]()
-            gr.replay()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(side)
-            for _ in range(reps):
-                gr.replay()
-            e1.record(side)
-            torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / (reps * copies)
-
-    up_avg = kernel_avg_us(0)
-    down_avg = kernel_avg_us(1)
+    # ---- launch duration of each of the two kernels of a step: HIP events on the launch stream around a
+    # graph that holds only that kernel, one launch per weight copy
+    up_avg = T.graph_us([l[0] for l in launches], 8)
+    down_avg = T.graph_us([l[1] for l in launches], 8)
 
     # the other batch sizes of the decode configuration (same weights, same rotation, graph replay)
-    def batch_avg_us(M, which, reps=4):
-        N, K = SHAPES[which]
-        xm = torch.randn((M, K), generator=g).to(torch.float16).to(device)
-        om = torch.empty((M, N), dtype=torch.float16, device=device)
-        ls = [Launch(lib, s[which], xm, om, device) for s in sets]
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            for l in ls[:2]:
-                l()
-            torch.cuda.synchronize()
-            with torch.cuda.graph(gr, stream=side):
-                for l in ls:
-                    l()
-            gr.replay()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(side)
-            for _ in range(reps):
-                gr.replay()
-            e1.record(side)
-            torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / (reps * copies)
-
     batch_points = {}
     if not a.no_extra:
         for M in (2, 4, 8, 16):
             for which, name in ((0, "up"), (1, "down")):
-                us = batch_avg_us(M, which)
-                batch_points[f"gemv_mlp_{name}_M{M}"] = {
-                    "us": round(us, 2), "GB/s": round(algorithmic_bytes(*SHAPES[which], M=M) / us / 1e3, 1)}
-    kbytes = algorithmic_bytes(*SHAPES[0])
-    achieved = kbytes / (up_avg * 1e-6) / 1e9
-
-    y_gpu = y.float().cpu().numpy()
+                N, K = SHAPES[which]
+                xm = torch.randn((M, K), generator=g).to(torch.float16).to(device)
+                om = torch.empty((M, N), dtype=torch.float16, device=device)
+                us = T.graph_us([Launch(lib, s[which], xm, om, device) for s in sets], 4)
+                batch_points[f"gemv_mlp_{name}_M{M}"] = bw_point(us, algorithmic_bytes(N, K, M=M))
 
     if a.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device)
@@ -467,6 +526,13 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # the roofline object describes the heavier of the two launches of a step (same bytes, more time)
+    kbytes = [algorithmic_bytes(*s) for s in SHAPES]
+    heavy = 1 if down_avg >= up_avg else 0
+    heavy_us = max(up_avg, down_avg)
+    achieved = kbytes[heavy] / (heavy_us * 1e-6) / 1e9
+    names = ["4096->14336 (up projection, 224 workgroups, K in one slab)",
+             "14336->4096 (down projection, 64 column tiles x 4 K slabs)"]
     out = {
         "metric": "A16W4 gs128 GEMV GB/s (%HBM peak) @M=1",
         "value": round(value, 1),
@@ -489,43 +555,52 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_direct_kernel<4-bit, fp16, M=1> on 4096->14336",
+            "kernel": "gemv_direct_kernel<4-bit, fp16, M=1> on " + names[heavy],
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "bytes_per_launch": kbytes,
-            "avg_launch_us": round(up_avg, 3),
+            "bytes_per_launch": kbytes[heavy],
+            "avg_launch_us": round(heavy_us, 3),
             "traffic": None,
         },
         "extra": {
+            "up_proj_avg_launch_us": round(up_avg, 3),
+            "up_proj_GBps": round(kbytes[0] / (up_avg * 1e-6) / 1e9, 1),
             "down_proj_avg_launch_us": round(down_avg, 3),
-            "down_proj_GBps": round(algorithmic_bytes(*SHAPES[1]) / (down_avg * 1e-6) / 1e9, 1),
+            "down_proj_GBps": round(kbytes[1] / (down_avg * 1e-6) / 1e9, 1),
             **batch_points,
         },
     }
 
-    # traffic per launch of the dominant kernel as read from the HBM byte counters, when a profile holds it
+    # traffic per launch of that kernel as read from the HBM byte counters, when a profile holds it
     traffic_file = os.path.join(ROOT, "profiles", "gemv_direct_a16w4_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file) as f:
-            out["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+            out["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch_down" if heavy else "hbm_bytes_per_launch")
 
     if not a.no_extra:
         del launches, sets, base
         torch.cuda.empty_cache()
-        out["extra"].update(extra_points(lib, device))
+        out["extra"].update(extra_points(lib, device, T, a.quick_extra))
+        rc = out["extra"]["read_ceiling"]["31MB"]["GB/s"]
+        out["roofline"]["frac_of_read_ceiling_on_this_box"] = round(achieved / rc, 4)
 
     if not a.no_cpu:
-        threads = min(os.cpu_count() or 1, 16)
-        sec, reps, err = cpu_baseline(host, x_host, y_gpu, threads)
+        cores = os.cpu_count() or 1
+        threads = min(cores, 16)   # the box's CPU share for one GPU
+        sec, reps, err, sec_torch, reps_torch = cpu_baseline(host, x_host, y_gpu, threads)
         out["cpu_baseline"] = {
             "value": round(step_bytes / sec / 1e9, 3),
             "unit": "GB/s",
-            "cores": threads,
+            "cores": cores,
+            "threads": threads,
             "kind": "port",
-            "sample": f"{reps} whole steps (HQQ dequantize of both weight matrices + fp32 matmul), "
+            "sample": f"{reps} whole steps (HQQ dequantize of both weight matrices + fp32 matmul, C/OpenMP restatement), "
                       f"{sec * 1e3:.1f} ms per step",
+            "torch_fp32_dequant_matmul": {
+                "value": round(step_bytes / sec_torch / 1e9, 3), "unit": "GB/s", "threads": threads,
+                "sample": f"{reps_torch} whole steps of ((W_q - z) * s) then x @ W.T in torch fp32, {sec_torch * 1e3:.1f} ms per step"},
         }
         out["extra"]["gpu_vs_cpu_rel_frobenius_err"] = round(err, 6)
     print(json.dumps(out))

@@ -51,6 +51,8 @@ int matmul_type_for(int M, int W_nbits, int mx) {
     return W_nbits < 8 ? GLA_MATMUL_GEMV_REVSPLITK : GLA_MATMUL_GEMV_SPLITK;
 }
 
+constexpr int kMxStreamRows = 2;  // MXFP4 x MXFP4: rows up to which the streaming kernel is chosen
+
 enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX };
 
 int validate(const gla_matmul_args* p) {
@@ -179,10 +181,15 @@ int validate(const gla_matmul_args* p) {
 }
 
 Family choose(const gla_matmul_args& p, int type) {
-    if (p.input_dtype == GLA_DT_MXFP4) return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
+    if (p.input_dtype == GLA_DT_MXFP4) {
+        // decode sizes: the streaming kernel (weights read once, straight into registers) beats the split-K matrix-core
+        // path, whose tiles are at least 64 rows tall
+        if (p.M <= kMxStreamRows && p.tile_config < 1000 && mx_stream_eligible(p)) return F_MX_STREAM;
+        return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
+    }
     if (p.input_dtype == GLA_DT_MXFP8) {  // validated: eligible for one of the two at least
-        // MXFP4 weights under fp8 activations: up to 2 rows the streaming kernel is the faster one (16384^2: 44 against 61 us)
-        if (p.elements_per_sample == 2 && p.M <= 2 && mx_stream_eligible(p)) return F_MX_STREAM;
+        // MXFP4 weights under fp8 activations: up to 4 rows the streaming kernel is the faster one (16384^2, M=4: 54 against 66 us)
+        if (p.elements_per_sample == 2 && p.M <= 4 && mx_stream_eligible(p)) return F_MX_STREAM;
         return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;
     }
     if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)  // validated as eligible for the streaming kernel

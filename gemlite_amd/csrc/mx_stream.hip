@@ -20,11 +20,11 @@
 // dot instruction; the block's partial sum is then scaled once by the product of its two block
 // scales, as the scaled matrix instruction does.  A shuffle tree sums the lanes.
 //
-// The combinations that have a matrix-core kernel do not come here (MXFP4 x MXFP4, fp8 x MXFP8, and,
-// from 3 rows up when K is a multiple of 128, weight-only MX layers and fp8 x MXFP4); this kernel is
-// the decode path of the weight-only MX layers and of MXFP8 activations x MXFP4 weights, and the
-// path at any batch size for a K that the matrix-core kernels do not take (not tuned above a few
-// rows: every group of eight activation rows streams the weights again).
+// This is the decode path of every micro-scaled layer: MXFP4 x MXFP4 up to 2 rows, weight-only MX
+// layers up to 3, fp8 activations x MXFP4 weights up to 4 (above that the matrix-core kernels are
+// faster: the conversions and dot products here cost vector-unit time per row), fp8 x MXFP8 never;
+// and the path at any batch size for a K that the matrix-core kernels do not take (not tuned above
+// a few rows: every group of eight activation rows streams the weights again).
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -67,8 +67,7 @@ __device__ __forceinline__ float dot2(typename Pair<BF>::type a, typename Pair<B
 
 // The 32 values of one block as 16 pairs (k, k+1), from e2m1 nibbles (16 bytes) ...
 template <bool BF>
-__device__ __forceinline__ void block_from_fp4(const uint8_t* p, typename Pair<BF>::type (&v)[16]) {
-    const u32x4 q = *(const u32x4*)p;
+__device__ __forceinline__ void block_from_fp4(const u32x4 q, typename Pair<BF>::type (&v)[16]) {
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
         if constexpr (BF) {
@@ -87,8 +86,7 @@ __device__ __forceinline__ void block_from_fp4(const uint8_t* p, typename Pair<B
 
 // ... from e4m3 bytes (32 bytes) ...
 template <bool BF>
-__device__ __forceinline__ void block_from_fp8(const uint8_t* p, typename Pair<BF>::type (&v)[16]) {
-    const u32x4 q0 = *(const u32x4*)p, q1 = *(const u32x4*)(p + 16);
+__device__ __forceinline__ void block_from_fp8(const u32x4 q0, const u32x4 q1, typename Pair<BF>::type (&v)[16]) {
 #pragma unroll
     for (int d = 0; d < 8; ++d) {
         const uint32_t w = d < 4 ? q0[d & 3] : q1[d & 3];
@@ -104,10 +102,10 @@ __device__ __forceinline__ void block_from_fp8(const uint8_t* p, typename Pair<B
 
 // ... or taken as they lie (64 bytes of fp16 / bf16).
 template <bool BF>
-__device__ __forceinline__ void block_from_16bit(const uint8_t* p, typename Pair<BF>::type (&v)[16]) {
+__device__ __forceinline__ void block_from_16bit(const u32x4 (&raw)[4], typename Pair<BF>::type (&v)[16]) {
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-        const u32x4 q = *(const u32x4*)(p + 16 * d);
+        const u32x4 q = raw[d];
         // element copies first: a bit cast applied to `q[j]` directly took element 0 for every j
         const uint32_t q0 = q.x, q1 = q.y, q2 = q.z, q3 = q.w;
         v[4 * d + 0] = __builtin_bit_cast(typename Pair<BF>::type, q0);
@@ -145,27 +143,74 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) acc[r][c] = 0.0f;
 
-    for (int blk = lane; blk < a.KB; blk += 64) {
+    // One step = the wave's 64 blocks at blk, blk + 64, ...; the weight bytes and scale bytes of step
+    // i + 1 (and the activation blocks too while they fit eight 16-byte registers) are requested before step i is
+    // multiplied, so that a wave always has two steps' loads in flight.  Weights are read once per
+    // launch: streaming (non-temporal) loads.
+    constexpr int WQ = kBBytes / 16;  // 16-byte pieces of a weight block
+    constexpr int AQ = kABytes / 16;
+    constexpr bool XPRE = RM * AQ <= 8;  // activation blocks ride along with the prefetch (up to 8 registers quads)
+    struct Step {
+        u32x4 w[NC][WQ];
+        uint8_t s[NC];
+        u32x4 x[XPRE ? RM : 1][AQ];
+        uint8_t sa[XPRE ? RM : 1];
+    };
+    auto fetch = [&](int blk, Step& st) __attribute__((always_inline)) {
+        const int b = blk < a.KB ? blk : a.KB - 1;  // lanes past the end re-read the last block and drop it
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+#pragma unroll
+            for (int q = 0; q < WQ; ++q) {
+                const uint4 t = load_streaming_u4(wrow[c] + (int64_t)b * kBBytes + 16 * q);
+                st.w[c][q] = u32x4{t.x, t.y, t.z, t.w};
+            }
+            st.s[c] = srow[c][(int64_t)b * a.msg];
+        }
+        if constexpr (XPRE) {
+#pragma unroll
+            for (int r = 0; r < RM; ++r) {
+                const int m = m0 + r < a.M ? m0 + r : a.M - 1;
+                const uint8_t* xp = a.x + (int64_t)m * a.xsm_bytes + (int64_t)b * kABytes;
+#pragma unroll
+                for (int q = 0; q < AQ; ++q) st.x[r][q] = *(const u32x4*)(xp + 16 * q);
+                st.sa[r] = a.csm == GLA_CSM_MX ? ((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)b * a.sxg] : (uint8_t)127;
+            }
+        }
+    };
+    auto to_pairs_a = [&](const u32x4 (&raw)[AQ], pair_t (&xv)[16]) __attribute__((always_inline)) {
+        if constexpr (AK == A_FP4) block_from_fp4<BF>(raw[0], xv);
+        else if constexpr (AK == A_FP8) block_from_fp8<BF>(raw[0], raw[1], xv);
+        else block_from_16bit<BF>(raw, xv);
+    };
+    auto multiply = [&](int blk, const Step& st) __attribute__((always_inline)) {
+        if (blk >= a.KB) return;
         pair_t wv[NC][16];
         float sw[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            if constexpr (BK == B_FP4) block_from_fp4<BF>(wrow[c] + (int64_t)blk * kBBytes, wv[c]);
-            else block_from_fp8<BF>(wrow[c] + (int64_t)blk * kBBytes, wv[c]);
-            sw[c] = e8m0_to_float(srow[c][(int64_t)blk * a.msg]);
+            if constexpr (BK == B_FP4) block_from_fp4<BF>(st.w[c][0], wv[c]);
+            else block_from_fp8<BF>(st.w[c][0], st.w[c][WQ - 1], wv[c]);
+            sw[c] = e8m0_to_float(st.s[c]);
         }
 #pragma unroll
         for (int r = 0; r < RM; ++r) {
             const int m = m0 + r;
             if (m < a.M) {
-                const uint8_t* xp = a.x + (int64_t)m * a.xsm_bytes + (int64_t)blk * kABytes;
                 pair_t xv[16];
-                if constexpr (AK == A_FP4) block_from_fp4<BF>(xp, xv);
-                else if constexpr (AK == A_FP8) block_from_fp8<BF>(xp, xv);
-                else block_from_16bit<BF>(xp, xv);
                 float sa = 1.0f;
-                if (a.csm == GLA_CSM_MX)
-                    sa = e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)blk * a.sxg]);
+                if constexpr (XPRE) {
+                    to_pairs_a(st.x[r], xv);
+                    if (a.csm == GLA_CSM_MX) sa = e8m0_to_float(st.sa[r]);
+                } else {
+                    const uint8_t* xp = a.x + (int64_t)m * a.xsm_bytes + (int64_t)blk * kABytes;
+                    u32x4 raw[AQ];
+#pragma unroll
+                    for (int q = 0; q < AQ; ++q) raw[q] = *(const u32x4*)(xp + 16 * q);
+                    to_pairs_a(raw, xv);
+                    if (a.csm == GLA_CSM_MX)
+                        sa = e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)blk * a.sxg]);
+                }
 #pragma unroll
                 for (int c = 0; c < NC; ++c) {
                     float p0 = 0.0f, p1 = 0.0f;
@@ -177,6 +222,16 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
                     acc[r][c] = __builtin_fmaf(p0 + p1, sw[c] * sa, acc[r][c]);
                 }
             }
+        }
+    };
+    {
+        Step cur, nxt;
+        fetch(lane, cur);
+        for (int blk = lane; blk < a.KB + lane; blk += 128) {  // two steps per trip: the buffers alternate
+            fetch(blk + 64, nxt);
+            multiply(blk, cur);
+            fetch(blk + 128, cur);
+            multiply(blk + 64, nxt);
         }
     }
 
