@@ -370,6 +370,40 @@ def extra_points(lib, device, T, quick):
     return out
 
 
+def run_point(name, lib, device, T):
+    """One GEMM point alone, a few launches: the workload of the per-kernel counter profiles under profiles/."""
+    from gemlite_amd import helper
+    g = torch.Generator(device="cpu").manual_seed(7)
+    if name in ("gemm_a8w8_fp8", "gemm_a8w8_int8"):
+        M, N, K = 4096, 8192, 8192
+        W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
+        x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+        fp8 = name.endswith("fp8")
+        layer = (helper.A8W8_FP8_dynamic if fp8 else helper.A8W8_INT8_dynamic)(device=device).from_weights(W)
+        xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn if fp8 else torch.int8)
+        peak = 5000.0
+    elif name in ("gemm_a4w4_mxfp4", "gemm_a4w4_mxfp4_M8192"):
+        M, N, K = (8192 if name.endswith("8192") else 4096), 16384, 16384
+        lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+        lin.weight.data = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+        layer = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
+        x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
+        xq, sx = gemlite_amd.scale_activations_mxfp4(x)
+        peak = 10100.0
+    elif name == "gemm_a16w4_gs128_fp16":
+        M = N = K = 4096
+        layer, _ = make_layer(N, K, seed=11, device=device)
+        xq, sx = torch.randn((M, K), generator=g).to(torch.float16).to(device), None
+        peak = 2500.0
+    else:
+        sys.exit(f"bench.py: unknown --point {name}")
+    y = torch.empty((M, N), dtype=torch.float16 if name == "gemm_a16w4_gs128_fp16" else torch.bfloat16, device=device)
+    us = T.eager_us(Launch(lib, layer, xq, y, device, scales_x=sx), 10)
+    tf = 2.0 * M * N * K / us / 1e6
+    print(json.dumps({"point": name, "M": M, "N": N, "K": K, "us": round(us, 1), "TFLOP/s": round(tf, 1),
+                      "frac_of_peak": round(tf / peak, 4)}))
+
+
 def cpu_baseline(host_tensors, x_host, y_gpu, threads):
     """The reference's CPU path (HQQ dequantize + fp32 matmul) on this box's host cores, on whole steps of the
     same workload: the C restatement (oracle/oracle_c.c, OpenMP), which also gives the parity check, and
@@ -435,6 +469,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary benchmark points")
     ap.add_argument("--quick-extra", action="store_true", help="a subset of the secondary points")
+    ap.add_argument("--point", default=None,
+                    help="run one GEMM point alone (gemm_a8w8_fp8, gemm_a8w8_int8, gemm_a4w4_mxfp4, gemm_a4w4_mxfp4_M8192, "
+                         "gemm_a16w4_gs128_fp16) for a profiler, print its line and exit")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 256 MiB device copy (a kernel of known traffic, to scale profiler byte counters)")
     a = ap.parse_args()
@@ -446,6 +483,9 @@ def main():
     torch.cuda.set_device(device)
     lib = _ext.load_library()
     T = Timer()
+    if a.point:
+        run_point(a.point, lib, device, T)
+        return
 
     step_bytes = sum(algorithmic_bytes(N, K) for N, K in SHAPES)
     copies = max(2, int(a.rotate_gb * 1e9 // step_bytes) + 1)

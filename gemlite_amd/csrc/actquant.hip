@@ -64,14 +64,28 @@ struct Raw8<GLA_DT_FP32> {
     uint4 a, b;
 };
 
+// (plain loads: the part of a long row that a wave reads twice should stay in the L2 between the passes)
 template <int XDT>
-__device__ __forceinline__ Raw8<XDT> load_raw8(const void* row, int k) {
+__device__ __forceinline__ Raw8<XDT> load_raw8_cached(const void* row, int k) {
     Raw8<XDT> r;
     if constexpr (XDT == GLA_DT_FP32) {
         r.a = ((const uint4*)((const float*)row + k))[0];
         r.b = ((const uint4*)((const float*)row + k))[1];
     } else {
         r.a = *(const uint4*)((const uint16_t*)row + k);
+    }
+    return r;
+}
+
+// (streaming loads: read once)
+template <int XDT>
+__device__ __forceinline__ Raw8<XDT> load_raw8(const void* row, int k) {
+    Raw8<XDT> r;
+    if constexpr (XDT == GLA_DT_FP32) {
+        r.a = load_streaming_u4((const float*)row + k);
+        r.b = load_streaming_u4((const float*)row + k + 4);
+    } else {
+        r.a = load_streaming_u4((const uint16_t*)row + k);
     }
     return r;
 }
@@ -153,7 +167,7 @@ __global__ __launch_bounds__(256) void per_token_kernel(const void* __restrict__
     }
     for (int c = lane + RC * kWave; c < chunks; c += kWave) {
         float v[8];
-        decode_raw8<XDT>(load_raw8<XDT>(xrow, c * 8), v);
+        decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
 #pragma unroll
         for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
     }
@@ -174,7 +188,7 @@ __global__ __launch_bounds__(256) void per_token_kernel(const void* __restrict__
     }
     for (int c = lane + RC * kWave; c < chunks; c += kWave) {
         float v[8];
-        decode_raw8<XDT>(load_raw8<XDT>(xrow, c * 8), v);
+        decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
         *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
     }
 }
@@ -187,69 +201,109 @@ __device__ __forceinline__ uint32_t e2m1_code(float v) {
     return (v >= 0.0f) ? idx : (idx + 8u);
 }
 
-// Four lanes share one 32-value group (8 values each): a wave covers 16 groups = 512 values.
+// Four lanes share one 32-value group (8 values each): a wave step covers 16 groups = 512 values, and a
+// wave takes kMxSteps consecutive steps of the row-major [M_pad, steps per row] grid, all of whose loads
+// it issues before it converts anything (one step per wave left a CU with too few bytes in flight).
 // FP8OUT: MXFP8 (codes are e4m3fn bytes, y is [M, K]; the largest magnitude is 448) instead of MXFP4
 // (e2m1 nibbles, y is [M, K/2]; 6).
+constexpr int kMxSteps = 8;
+
 template <int XDT, bool FP8OUT>
 __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, int64_t xsm, int M, int M_pad, int K,
                                                     uint8_t* __restrict__ y, uint8_t* __restrict__ scales) {
     const int groups = K / 32;
-    const int gpr = (groups + 15) / 16;  // wave-chunks per row
-    const int64_t wave_id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int gpr = (groups + 15) / 16;  // wave steps per row
+    const int64_t total = (int64_t)M_pad * gpr;
+    const int64_t first = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * kMxSteps;
     const int lane = threadIdx.x & 63;
-    const int row = (int)(wave_id / gpr);
-    const int g = (int)(wave_id % gpr) * 16 + (lane >> 2);
-    if (row >= M_pad) return;
-    if (row >= M) {  // padding rows carry the identity scale and no codes
-        if ((lane & 3) == 0 && g < groups) scales[(int64_t)row * groups + g] = 127;
-        return;
-    }
-    const bool active = g < groups;
-    const int k = g * 32 + (lane & 3) * 8;
-    float v[8];
-    if (active) {
-        const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
-        load8<XDT>(xrow, k, v);
-    } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = 0.0f;
-    }
-    float amax = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
+    if (first >= total) return;
 
-    const uint32_t bits = __builtin_bit_cast(uint32_t, amax / (FP8OUT ? 448.0f : 6.0f));
-    uint32_t e = (bits >> 23) & 0xffu;
-    e += (bits & 0x7fffffu) ? 1u : 0u;
-    e = e > 254u ? 254u : e;
-    e = e < 97u ? 97u : e;
-    const float s = __builtin_bit_cast(float, e << 23);
-
-    if (!active) return;
-    uint32_t packed = 0;
-    // s is a power of two, so v / s is an exact exponent shift: ldexp gives the same value (signed zeros
-    // and denormal results included) in one instruction instead of a division sequence
-    const int down = 127 - (int)e;
-    (void)s;
-    if constexpr (FP8OUT) {
-        uint32_t w[2];
+    Raw8<XDT> raw[kMxSteps];
+    int rows[kMxSteps], gs[kMxSteps];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            float q[4];
+    for (int u = 0; u < kMxSteps; ++u) {
+        const int64_t id = first + u < total ? first + u : total - 1;  // surplus steps repeat the last one (same values, same place)
+        rows[u] = (int)(id / gpr);
+        gs[u] = (int)(id % gpr) * 16 + (lane >> 2);
+        // loads stay in bounds: padding rows and groups past the row read the first chunk of row 0 and drop it
+        const bool live = rows[u] < M && gs[u] < groups;
+        const char* xrow = (const char*)x + (int64_t)(live ? rows[u] : 0) * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+        raw[u] = load_raw8<XDT>(xrow, live ? gs[u] * 32 + (lane & 3) * 8 : 0);
+    }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) q[j] = fminf(fmaxf(__builtin_ldexpf(v[4 * h + j], down), -448.0f), 448.0f);
-            w[h] = f32_to_fp8_pair(q[0], q[1]) | (f32_to_fp8_pair(q[2], q[3]) << 16);
+    for (int u = 0; u < kMxSteps; ++u) {
+        const int row = rows[u], g = gs[u];
+        if (row >= M) {  // padding rows carry the identity scale and no codes
+            if ((lane & 3) == 0 && g < groups) scales[(int64_t)row * groups + g] = 127;
+            continue;
         }
-        *(uint2*)(y + (int64_t)row * K + k) = make_uint2(w[0], w[1]);
-        if ((lane & 3) == 0) scales[(int64_t)row * groups + g] = (uint8_t)e;
-        return;
-    }
+        const bool active = g < groups;
+        const int k = g * 32 + (lane & 3) * 8;
+        float v[8];
+        decode_raw8<XDT>(raw[u], v);
+        if (!active) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) packed |= e2m1_code(__builtin_ldexpf(v[j], down)) << (4 * j);
-    *(uint32_t*)(y + (int64_t)row * (K / 2) + k / 2) = packed;
-    if ((lane & 3) == 0) scales[(int64_t)row * groups + g] = (uint8_t)e;
+            for (int j = 0; j < 8; ++j) v[j] = 0.0f;
+        }
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
+
+        const uint32_t bits = __builtin_bit_cast(uint32_t, amax / (FP8OUT ? 448.0f : 6.0f));
+        uint32_t e = (bits >> 23) & 0xffu;
+        e += (bits & 0x7fffffu) ? 1u : 0u;
+        e = e > 254u ? 254u : e;
+        e = e < 97u ? 97u : e;
+
+        if (!active) continue;
+        // the scale is a power of two, so v / s is an exact exponent shift: ldexp gives the same value (signed
+        // zeros and denormal results included) in one instruction instead of a division sequence
+        const int down = 127 - (int)e;
+        if constexpr (FP8OUT) {
+            uint32_t w[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float q[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) q[j] = fminf(fmaxf(__builtin_ldexpf(v[4 * h + j], down), -448.0f), 448.0f);
+                w[h] = f32_to_fp8_pair(q[0], q[1]) | (f32_to_fp8_pair(q[2], q[3]) << 16);
+            }
+            *(uint2*)(y + (int64_t)row * K + k) = make_uint2(w[0], w[1]);
+        } else {
+            // The hardware conversion divides by the block scale and rounds to nearest even; the reference
+            // counts the thresholds strictly below |x / s|, i.e. rounds ties toward zero, and gives -0.0 the
+            // code 0.  The two differ at exact ties whose upper neighbour is the even one (0.75, 1.75 and
+            // 3.5 times the scale: those go one ulp toward zero first) and at -0.0 (x + 0.0 is +0.0 for both
+            // zeros and x otherwise).  An input that is not a number takes the reference's route.
+            const float sc = __builtin_bit_cast(float, e << 23);
+            const uint32_t shift = (e - 127u) << 23;
+            const uint32_t t1 = 0x3f400000u + shift, t2 = 0x3fe00000u + shift, t3 = 0x40600000u + shift;
+            bool odd = false;
+            float w[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float z = v[j] + 0.0f;
+                const uint32_t zb = __builtin_bit_cast(uint32_t, z), mag = zb & 0x7fffffffu;
+                const bool tie = mag == t1 || mag == t2 || mag == t3;
+                w[j] = __builtin_bit_cast(float, zb - (tie ? 1u : 0u));
+                odd |= mag > 0x7f800000u;
+            }
+            uint32_t packed = 0;
+            if (__builtin_expect(!odd, 1)) {
+                packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, w[0], w[1], sc, 0);
+                packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, w[2], w[3], sc, 1);
+                packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, w[4], w[5], sc, 2);
+                packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, w[6], w[7], sc, 3);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) packed |= e2m1_code(__builtin_ldexpf(v[j], down)) << (4 * j);
+            }
+            *(uint32_t*)(y + (int64_t)row * (K / 2) + k / 2) = packed;
+        }
+        if ((lane & 3) == 0) scales[(int64_t)row * groups + g] = (uint8_t)e;
+    }
 }
 
 }  // namespace
@@ -398,7 +452,7 @@ static int launch_act_mx(const void* x, int x_dtype, int64_t x_stride_m, int M, 
     const int M_pad = (M + 31) / 32 * 32;
     const int groups = K / 32;
     const int gpr = (groups + 15) / 16;
-    const int64_t waves = (int64_t)M_pad * gpr;
+    const int64_t waves = ((int64_t)M_pad * gpr + kMxSteps - 1) / kMxSteps;
     dim3 grid((unsigned)((waves + 3) / 4)), block(256);
     switch (x_dtype) {
         case GLA_DT_FP16:

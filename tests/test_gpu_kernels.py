@@ -107,6 +107,27 @@ def test_mxfp4_quant_bit_exact(device, dtype, shape):
     assert np.array_equal(y.cpu().numpy(), y_ref)
 
 
+@pytest.mark.parametrize("amax_exp", [-9, -3, 0, 4, 12])
+def test_mxfp4_quant_every_fp16_value(device, amax_exp):
+    """Every finite fp16 value (both zeros, subnormals, every exact tie) up to the block maximum, under a block
+    scale pinned by one element 6 * 2^amax_exp per group of 32: codes and scales equal the oracle's bit for bit."""
+    top = 6.0 * 2.0 ** amax_exp
+    allv = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    allv = allv[torch.isfinite(allv) & (allv.float().abs() <= top)]
+    pad = (-allv.numel()) % 31
+    allv = torch.cat([allv, torch.zeros(pad, dtype=torch.float16)])
+    groups = allv.view(-1, 31)
+    x = torch.cat([torch.full((groups.shape[0], 1), top, dtype=torch.float16), groups], dim=1).reshape(1, -1)
+    # rows of 128 groups, so that several rows and wave steps are exercised
+    cols = 32 * 128
+    x = torch.cat([x, torch.zeros((1, (-x.shape[1]) % cols), dtype=torch.float16)], dim=1).view(-1, cols)
+    for dtype in (torch.float16, torch.float32):
+        y, s = gemlite_amd.scale_activations_mxfp4(x.to(dtype).to(device))
+        y_ref, s_ref = orc.scale_activations_mxfp4(to_np(x))
+        assert np.array_equal(s.cpu().numpy(), s_ref)
+        assert np.array_equal(y.cpu().numpy(), y_ref)
+
+
 def test_mxfp4_quant_zero_and_tiny_groups(device):
     x = torch.zeros((2, 64), dtype=torch.bfloat16)
     x[1, 32:] = 1e-30
