@@ -273,19 +273,18 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
     const Family f = choose(*args, resolve_type(*args));
     int rc2;
     switch (f) {
-        // The streaming kernels and the packed-code GEMM add the bias in their epilogue (the `return`s); the 8-bit and
-        // byte-weight MFMA GEMMs do not: a bias branch in their epilogues made the compiler spill accumulators
-        // (576 bytes of scratch per lane, 25-35 % more time), so they are followed by the elementwise launch below.
+        // Every family adds the bias in its epilogue or split-K finishing kernel (the `return`s) except the byte-weight
+        // MFMA GEMM and the generic kernel, which are followed by the elementwise launch below.
         case F_GEMV_PACKED: return launch_gemv_packed(*args, s);
         case F_GEMV_KMAJOR: return launch_gemv_kmajor(*args, s);
         case F_GEMM_WN: return launch_gemm_wn(*args, s);
-        case F_GEMM_8BIT: rc2 = launch_gemm_8bit(*args, s); break;
-        case F_GEMM_MXFP4: rc2 = launch_gemm_mxfp4(*args, s); break;
+        case F_GEMM_8BIT: return launch_gemm_8bit(*args, s);
+        case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
         case F_GEMM_KBYTES: rc2 = launch_gemm_kbytes(*args, s); break;
-        case F_GEMM_MXFP8: rc2 = launch_gemm_mxfp8(*args, s); break;
+        case F_GEMM_MXFP8: return launch_gemm_mxfp8(*args, s);
         case F_MX_STREAM: return launch_mx_stream(*args, s);
         case F_BLOCKQ_STREAM: return launch_blockq_stream(*args, s);
-        case F_GEMM_BLOCKQ: rc2 = launch_gemm_blockq(*args, s); break;
+        case F_GEMM_BLOCKQ: return launch_gemm_blockq(*args, s);
         case F_GEMM_KBYTES_MX: rc2 = launch_gemm_kbytes_mx(*args, s); break;
         default: rc2 = launch_generic(*args, s); break;
     }

@@ -48,12 +48,20 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
     return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
 
-// round-to-nearest-even float -> bf16 bits (NaN kept quiet)
-__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+// Two floats -> two bf16 in one register (lo in bits 15:0), round to nearest even: one v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// round-to-nearest-even float -> bf16 bits
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) { return (uint16_t)pack_bf16x2(f, 0.0f); }
+
+// Two floats -> two fp16 in one register (lo in bits 15:0), round to nearest even.
+__device__ __forceinline__ uint32_t pack_half2(float lo, float hi) {
+    const half2_t v = {(half_t)lo, (half_t)hi};
+    return __builtin_bit_cast(uint32_t, v);
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint16_t b) {

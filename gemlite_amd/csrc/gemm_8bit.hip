@@ -72,6 +72,8 @@ struct Gemm8Args {
     int S;     // K splits (gridDim.y)
     int sps;   // pipeline stages per split
     void* partials;  // [S][M][N] 32-bit accumulators when S > 1
+    const void* bias;  // [N] or NULL: added to the result rounded to the output type (float outputs)
+    int bias_dt;
 };
 
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -106,7 +108,9 @@ constexpr int slot_bytes8(int mode, int bm) {
 // measured slower.  LDS bandwidth is not what limits these loops: 128-bit reads sustain well over
 // 200 bytes per clock and CU, the loop needs about 35.  With random operands the board's power
 // limit is: the clock falls to about 1.55 GHz under these kernels.)
-template <int MODE, int BM, int WN>
+// BIAS: the epilogue adds p.bias.  A separate instantiation: the extra rounding and the bias loads cost the
+// 256-row tile 10-35 % when they are compiled into the one kernel and merely switched off at run time.
+template <int MODE, int BM, int WN, bool BIAS = false>
 __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args p) {
     constexpr int WM = BM / kWavesM;  // wave tile rows
     constexpr int TI = WM / 32;       // 32-row MFMA tiles per wave along M
@@ -523,14 +527,40 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         if constexpr (BQ) return folded[i][j][e];
         else return (float)acc[i][j][e];
     };
+    // The element type is tested once per vector, outside the loops, so that a lane's 16 * TJ loads
+    // are issued back to back and waited for together.
+    auto load_cols = [&](float (&dst)[TJ][16], const void* base, int dt, float fill) __attribute__((always_inline)) {
+        auto each = [&](auto get) __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int n = n_wave + j * 32 + 8 * (e / 4) + (e % 4);
+                    dst[j][e] = n < p.N ? get(n) : fill;
+                }
+        };
+        if (dt == GLA_DT_FP32) each([&](int n) { return ((const float*)base)[n]; });
+        else if (dt == GLA_DT_BF16) each([&](int n) { return bf16_bits_to_float(((const uint16_t*)base)[n]); });
+        else if (dt == GLA_DT_FP16) each([&](int n) { return (float)((const half_t*)base)[n]; });
+        else each([&](int n) { return load_as_float(base, dt, n); });
+    };
     float sb[TJ][16];
+    if (col_scale) {
+        load_cols(sb, p.scales, p.meta_dt, 1.0f);
+    } else {
 #pragma unroll
-    for (int j = 0; j < TJ; ++j)
+        for (int j = 0; j < TJ; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int n = n_wave + j * 32 + 8 * (e / 4) + (e % 4);
-            sb[j][e] = (col_scale && n < p.N) ? load_as_float(p.scales, p.meta_dt, n) : 1.0f;
-        }
+            for (int e = 0; e < 16; ++e) sb[j][e] = 1.0f;
+    }
+    // Bias: out = cast(cast(v) + bias[n]) like the reference's `out += bias` on the rounded output
+    // (reference: gemlite/core.py:271-272).
+    float bb[BIAS ? TJ : 1][16];
+    if constexpr (BIAS) load_cols(bb, p.bias, p.bias_dt, 0.0f);
+    auto biased = [&](auto dt_tag, float v, int j, int e) __attribute__((always_inline)) -> float {
+        if constexpr (BIAS) return round_to_dtype(decltype(dt_tag)::value, v) + bb[j][e];
+        else return v;
+    };
     auto emit = [&](auto dt_tag) {
         constexpr int DT = decltype(dt_tag)::value;
         constexpr int ES = (DT == GLA_DT_FP16 || DT == GLA_DT_BF16) ? 2 : 4;
@@ -554,17 +584,17 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                         } else {
                             float v[4];
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) v[t] = value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]);
+                            for (int t = 0; t < 4; ++t) v[t] = biased(dt_tag, value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]), j, 4 * g + t);
                             if constexpr (DT == GLA_DT_FP32) {
                                 *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
                             } else {
                                 uint32_t lo, hi;
                                 if constexpr (DT == GLA_DT_FP16) {
-                                    lo = float_to_half_bits(v[0]) | ((uint32_t)float_to_half_bits(v[1]) << 16);
-                                    hi = float_to_half_bits(v[2]) | ((uint32_t)float_to_half_bits(v[3]) << 16);
+                                    lo = pack_half2(v[0], v[1]);
+                                    hi = pack_half2(v[2], v[3]);
                                 } else {
-                                    lo = float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-                                    hi = float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+                                    lo = pack_bf16x2(v[0], v[1]);
+                                    hi = pack_bf16x2(v[2], v[3]);
                                 }
                                 *(u32x2*)((uint16_t*)p.out + o) = u32x2{lo, hi};
                             }
@@ -574,7 +604,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                         for (int t = 0; t < 4; ++t) {
                             if (n + t >= p.N) continue;
                             if constexpr (DT == GLA_DT_INT32) ((int32_t*)p.out)[o + t] = (int32_t)acc[i][j][4 * g + t];
-                            else store_typed<DT>(p.out, o + t, value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]));
+                            else store_typed<DT>(p.out, o + t, biased(dt_tag, value(i, j, 4 * g + t) * (sa * sb[j][4 * g + t]), j, 4 * g + t));
                         }
                     }
                 }
@@ -584,6 +614,11 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     else if (p.out_dt == GLA_DT_BF16) emit(std::integral_constant<int, GLA_DT_BF16>{});
     else if (p.out_dt == GLA_DT_INT32) emit(std::integral_constant<int, GLA_DT_INT32>{});
     else emit(std::integral_constant<int, GLA_DT_FP32>{});
+}
+
+__device__ __forceinline__ float with_bias(const Gemm8Args& p, int n, float v) {
+    if (p.bias == nullptr) return v;
+    return round_to_dtype(p.out_dt, v) + load_as_float(p.bias, p.bias_dt, n);
 }
 
 // Sum the K splits in order (exactly, for integer accumulators), apply the channel scales and store.
@@ -601,19 +636,23 @@ __global__ __launch_bounds__(256) void splitk_finish8_kernel(Gemm8Args p) {
         int32_t v = 0;
         for (int s = 0; s < p.S; ++s) v += ((const int32_t*)p.partials)[s * slab + idx];
         if (p.out_dt == GLA_DT_INT32) ((int32_t*)p.out)[o] = v;
-        else store_from_float(p.out, p.out_dt, o, (float)v * scale);
+        else store_from_float(p.out, p.out_dt, o, with_bias(p, n, (float)v * scale));
     } else {
         float v = 0.0f;
         for (int s = 0; s < p.S; ++s) v += ((const float*)p.partials)[s * slab + idx];
-        store_from_float(p.out, p.out_dt, o, v * scale);
+        store_from_float(p.out, p.out_dt, o, with_bias(p, n, v * scale));
     }
 }
 
-template <int MODE, int BM, int WN>
+template <int MODE, int BM, int WN, bool BIAS = false>
 int launch_bm(const Gemm8Args& a, hipStream_t stream) {
+    if constexpr (!BIAS) {
+        // with a bias and an unsplit K the epilogue adds it (a split K leaves it to the finishing kernel)
+        if (a.bias != nullptr && a.S == 1 && a.out_dt != GLA_DT_INT32) return launch_bm<MODE, BM, WN, true>(a, stream);
+    }
     const size_t smem = (size_t)kRing8 * slot_bytes8(MODE, BM);
     static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
-    auto kern = gemm_8bit_kernel<MODE, BM, WN>;
+    auto kern = gemm_8bit_kernel<MODE, BM, WN, BIAS>;
     if (once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "gemm_8bit: raising the dynamic LDS limit");
@@ -734,6 +773,7 @@ bool gemm_8bit_eligible(const gla_matmul_args& p) {
 
 int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     Gemm8Args a;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
@@ -782,6 +822,7 @@ int launch_gemm_blockq(const gla_matmul_args& p, hipStream_t stream) {
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     Gemm8Args a;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     // block scales travel with the stages like micro-scales: byte strides per row / per 128-block of K
@@ -832,6 +873,7 @@ bool gemm_mxfp4_eligible(const gla_matmul_args& p) {
 
 int launch_gemm_mxfp4(const gla_matmul_args& p, hipStream_t stream) {
     Gemm8Args a;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K / 2; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;
     a.sxm = p.sx_stride_m; a.msn = p.meta_stride_n; a.csm = 0; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
@@ -902,6 +944,7 @@ int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p) {
 
 int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
     Gemm8Args a;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
     const bool act_blocks = p.channel_scale_mode == GLA_CSM_MX;
     a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.Kb = p.K; a.lda = p.x_stride_m; a.ldb = p.w_stride_n; a.osm = p.out_stride_m;

@@ -455,11 +455,11 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
                         if constexpr (DT == GLA_DT_FP32) {
                             *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
                         } else if constexpr (DT == GLA_DT_FP16) {
-                            *(u32x2b*)((uint16_t*)p.out + o) = u32x2b{float_to_half_bits(v[0]) | ((uint32_t)float_to_half_bits(v[1]) << 16),
-                                                                       float_to_half_bits(v[2]) | ((uint32_t)float_to_half_bits(v[3]) << 16)};
+                            *(u32x2b*)((uint16_t*)p.out + o) = u32x2b{pack_half2(v[0], v[1]),
+                                                                       pack_half2(v[2], v[3])};
                         } else {
-                            *(u32x2b*)((uint16_t*)p.out + o) = u32x2b{float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16),
-                                                                       float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16)};
+                            *(u32x2b*)((uint16_t*)p.out + o) = u32x2b{pack_bf16x2(v[0], v[1]),
+                                                                       pack_bf16x2(v[2], v[3])};
                         }
                     } else {
 #pragma unroll

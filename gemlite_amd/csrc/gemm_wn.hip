@@ -584,9 +584,9 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
 #pragma unroll
                             for (int q = 0; q < 4; ++q) {
                                 if constexpr (DT == GLA_DT_FP16)
-                                    w[q] = float_to_half_bits(v[c + 2 * q]) | ((uint32_t)float_to_half_bits(v[c + 2 * q + 1]) << 16);
+                                    w[q] = pack_half2(v[c + 2 * q], v[c + 2 * q + 1]);
                                 else
-                                    w[q] = float_to_bf16_bits(v[c + 2 * q]) | ((uint32_t)float_to_bf16_bits(v[c + 2 * q + 1]) << 16);
+                                    w[q] = pack_bf16x2(v[c + 2 * q], v[c + 2 * q + 1]);
                             }
                             *(u32x4*)((uint16_t*)p.out + o + c) = w;
                         }

@@ -703,7 +703,8 @@ def test_ternary_weight_layers(device, dtype):
 def test_bias_is_added_to_the_rounded_output_like_the_reference(device, dtype):
     """`out += bias` on the output already rounded to its type (reference: gemlite/core.py:271-272): a layer with
     a bias must equal the same layer without one plus the bias, bit for bit, whether the kernel adds it in its
-    epilogue (packed-code GEMV, up to 16 rows) or the library adds it with a launch of its own."""
+    epilogue or split-K finishing kernel (every family but the byte-weight MFMA GEMM) or the library adds it with a
+    launch of its own."""
     N, K = 1032, 2048
     bias = gen_x(1, N, dtype, seed=77).reshape(-1).to(device)
     W_q, s, z = gen_int_case(N, K, 4, 128, dtype, seed=5)
@@ -722,12 +723,16 @@ def test_bias_is_added_to_the_rounded_output_like_the_reference(device, dtype):
         "A8W8 fp8": pair(lambda: helper.A8W8_FP8_dynamic(device=device).from_weights(W.to(dtype))),
         "A16W4_MXFP": pair(lambda: helper.A16W4_MXFP(device=device, dtype=dtype).from_linear(lin.to(device), del_orig=False)),
         "block-quantised": pair(lambda: helper.A8W8_FP8_dynamic(device=device, block_quant=True).from_weights(W.to(dtype))),
+        "A8W8 int8": pair(lambda: helper.A8W8_INT8_dynamic(device=device).from_weights(W.to(dtype))),
+        "A4W4 MXFP4": pair(lambda: helper.A4W4_MXFP_dynamic(device=device, dtype=dtype).from_linear(lin.to(device), del_orig=False)),
+        "A8W8 MXFP8": pair(lambda: helper.A8W8_MXFP_dynamic(device=device, dtype=dtype).from_linear(lin.to(device), del_orig=False)),
+        "A8W4 MXFP": pair(lambda: helper.A8W4_MXFP_dynamic(device=device, dtype=dtype).from_linear(lin.to(device), del_orig=False)),
         "A16W8 bytes": pair(lambda: helper.A16W8_INT8(device=device, dtype=dtype).from_weights(
             *gemlite_amd.quantize_weights_per_channel(W.to(dtype), torch.int8)[:1],
             scales=gemlite_amd.quantize_weights_per_channel(W.to(dtype), torch.int8)[1])),
     }
     for name, (plain, biased) in cases.items():
-        for M in (1, 2, 5, 16, 70):
+        for M in (1, 2, 5, 16, 70, 300):   # streaming kernels, split-K with a finishing kernel, 64- / 128- / 256-row tiles
             x = gen_x(M, K, dtype, seed=M).to(device)
             want = plain(x) + bias
             got = biased(x)
