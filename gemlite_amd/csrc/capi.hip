@@ -188,8 +188,9 @@ Family choose(const gla_matmul_args& p, int type) {
         return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
     }
     if (p.input_dtype == GLA_DT_MXFP8) {  // validated: eligible for one of the two at least
-        // MXFP4 weights under fp8 activations: up to 4 rows the streaming kernel is the faster one (16384^2, M=4: 54 against 66 us)
-        if (p.elements_per_sample == 2 && p.M <= 4 && mx_stream_eligible(p)) return F_MX_STREAM;
+        // MXFP4 weights under fp8 activations: up to 2 rows the streaming kernel is the faster one (16384^2, M=2: 33
+        // against 42 us; M=3: 47 against 42 us)
+        if (p.elements_per_sample == 2 && p.M <= 2 && mx_stream_eligible(p)) return F_MX_STREAM;
         return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;
     }
     if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)  // validated as eligible for the streaming kernel

@@ -141,7 +141,12 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
 
     extern __shared__ __align__(16) unsigned char smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // The wave index as a scalar: what depends on it alone (which operand a copy job serves, and with it
+    // the choice between two kernel arguments) is then decided by scalar selects.  Left in a vector
+    // register, such a choice becomes a load of the chosen argument inside the K loop, and the wait for
+    // it drains every copy in flight.
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     int tm, tn;
     tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
@@ -214,17 +219,37 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // stage (always inside the row) and are never multiplied.  Stages past the end of K copy the
     // last one again so that every step issues the same number of copies.
     // copy c (0 <= c < LPS) of stage k into ring slot `slot`
+    // The operand a job copies from, chosen once, here, between two argument values held in scalar
+    // registers.  (Written as a choice between p.a and p.b at the point of use, the compiler selects
+    // between the arguments' addresses and loads the chosen one inside the K loop.)
+    const uint8_t *arg_a = p.a, *arg_b = p.b;
+    asm volatile("" : "+s"(arg_a), "+s"(arg_b));
+    const uint8_t* src16[J16];
+#pragma unroll
+    for (int i = 0; i < J16; ++i) src16[i] = is_a16[i] ? arg_a : arg_b;
+    const uint8_t* src4[MX ? J4 : 1];
+    int64_t stage4[MX ? J4 : 1];
+    if constexpr (MX) {
+        const uint8_t *arg_sx = (const uint8_t*)p.ascales, *arg_sw = (const uint8_t*)p.scales;
+        int64_t arg_xs = p.sx_stage, arg_ws = p.sw_stage;
+        asm volatile("" : "+s"(arg_sx), "+s"(arg_sw), "+s"(arg_xs), "+s"(arg_ws));
+#pragma unroll
+        for (int i = 0; i < J4; ++i) {
+            src4[i] = is_a4[i] ? arg_sx : arg_sw;
+            stage4[i] = is_a4[i] ? arg_xs : arg_ws;
+        }
+    }
     auto issue_one = [&](int k, int slot, int c) __attribute__((always_inline)) {
         const int kk = k_first + (k > steps - 1 ? steps - 1 : k);  // absolute stage
         unsigned char* base = smem + slot * SLOT;
         if (c < J16) {
             const int limit = p.Kb - kk * kRowB8;
-            const uint8_t* src = (is_a16[c] ? p.a : p.b) + kk * (is_a16[c] ? kRowB8 : ROWW) + (off16[c] + (unsigned)(chunk16[c] < limit ? chunk16[c] : 0));
+            const uint8_t* src = src16[c] + kk * (is_a16[c] ? kRowB8 : ROWW) + (off16[c] + (unsigned)(chunk16[c] < limit ? chunk16[c] : 0));
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                              (__attribute__((address_space(3))) void*)(base + dst16[c]), 16, 0, 0);
         } else if constexpr (MX) {
             const int i = c - J16;
-            const uint8_t* sk = is_a4[i] ? (const uint8_t*)p.ascales + (kk >> SSH) * p.sx_stage : (const uint8_t*)p.scales + (kk >> SSH) * p.sw_stage;
+            const uint8_t* sk = src4[i] + (kk >> SSH) * stage4[i];
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sk + off4[i]),
                                              (__attribute__((address_space(3))) void*)(base + dst4[i]), 4, 0, 0);
         }
@@ -787,7 +812,7 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
 
 static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
-// ---- 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5) above 4 rows ----------------
+// ---- 128 x 128 block-quantised fp8 / int8 (channel_scale_mode 5) from 2 rows up ----------------
 // (reference: gemlite/triton_kernels/gemm_kernels.py:396-400, :441-450.)  Tiles of 64 or 128 rows: the
 // second accumulator leaves no registers for the 256-row tile.  K splits hold whole 128-blocks (an even
 // number of stages) and their partials are the scaled fp32 sums, which the reduction kernel only adds.
@@ -804,7 +829,7 @@ static Plan8 plan_blockq(const gla_matmul_args& p) {
 }
 
 bool gemm_blockq_eligible(const gla_matmul_args& p) {
-    if (!blockq_stream_eligible(p) || p.M <= 4 || p.out_stride_n != 1) return false;
+    if (!blockq_stream_eligible(p) || p.M <= 1 || p.out_stride_n != 1) return false;
     if (p.meta_stride_n < 0 || p.meta_stride_g < 0 || p.sx_stride_m < 0 || p.sx_stride_g < 0) return false;
     if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
     if ((int64_t)p.M * p.sx_stride_m * 4 >= (1ll << 31) || (int64_t)(p.N / 128 + 1) * p.meta_stride_n * 4 >= (1ll << 31)) return false;
@@ -818,7 +843,7 @@ int64_t gemm_blockq_workspace_bytes(const gla_matmul_args& p) {
 
 int launch_gemm_blockq(const gla_matmul_args& p, hipStream_t stream) {
     if (!gemm_blockq_eligible(p)) {
-        set_error("gemm_blockq: operands not eligible (see blockq_stream; more than 4 rows, unit output column stride)");
+        set_error("gemm_blockq: operands not eligible (see blockq_stream; more than 1 row, unit output column stride)");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     Gemm8Args a;
@@ -923,9 +948,14 @@ bool gemm_mxfp8_eligible(const gla_matmul_args& p) {
 
 // with block scales on both sides the 256-row tile has no registers for the scale words next to two
 // fragment buffers of 8-register operands
+// Left to choose, 64 rows or fewer take the 128-row tile too: it reads the scales regrouped by stage, the
+// 64-row tile reads them where the caller keeps them (16384^2, M=8: MXFP4 weights 42 against 54 us, MXFP8
+// weights 59 against 66 us).
 static Plan8 plan_mxfp8(const gla_matmul_args& p) {
     Plan8 g = plan8(p.M, p.N, p.K, p.tile_config);
-    if (g.bm == 256 && p.channel_scale_mode == GLA_CSM_MX) {
+    const int asked = p.tile_config > 0 ? p.tile_config % 1000 : 0;
+    const bool chosen_here = !(asked == 64 || asked == 128 || asked == 256);
+    if ((g.bm == 256 && p.channel_scale_mode == GLA_CSM_MX) || (g.bm == 64 && chosen_here)) {
         const int cfg = (p.tile_config > 0 ? p.tile_config / 1000 : 0) * 1000 + 128;
         g = plan8(p.M, p.N, p.K, cfg);
     }

@@ -575,14 +575,14 @@ int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p) {
     return g.S > 1 ? kWsReservedB + (int64_t)g.S * p.M * p.N * 4 : 0;
 }
 
-// ---- weight-only MX layers above 3 rows: fp16 / bf16 activations x MXFP8 / MXFP4 weights ------------
+// ---- weight-only MX layers above 2 rows: fp16 / bf16 activations x MXFP8 / MXFP4 weights ------------
 // (reference: gemlite/triton_kernels/gemm_kernels.py:509-737 with 16-bit activations and unit activation
 // scales, gemlite/helper.py:199-237.)  The conversion instruction applies the block scale, so the operand is
 // the dequantised weight in the activations' type: exact in bf16; in fp16 as far as code x 2^(e-127) is a
 // finite normal fp16 number, which weights of trained layers are.
 bool gemm_kbytes_mx_eligible(const gla_matmul_args& p) {
     if (!(p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)) return false;
-    if (p.M <= 3 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_NONE || p.scales == nullptr) return false;
+    if (p.M <= 2 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_NONE || p.scales == nullptr) return false;
     const bool fp4 = p.elements_per_sample == 2 && p.W_nbits == 4;
     const bool fp8 = p.elements_per_sample == 1 && p.W_nbits == 8 && p.w_dtype == GLA_DT_FP8;
     if (!fp4 && !fp8) return false;
@@ -602,7 +602,7 @@ int64_t gemm_kbytes_mx_workspace_bytes(const gla_matmul_args& p) { return gemm_k
 
 int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream) {
     if (!gemm_kbytes_mx_eligible(p)) {
-        set_error("gemm_kbytes_mx: operands not eligible (K-contiguous MXFP8 / MXFP4 weights, K %% 128 == 0, more than 3 rows)");
+        set_error("gemm_kbytes_mx: operands not eligible (K-contiguous MXFP8 / MXFP4 weights, K %% 128 == 0, more than 2 rows)");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     GemmKbArgs a;

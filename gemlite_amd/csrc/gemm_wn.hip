@@ -676,9 +676,9 @@ WnPlan wn_plan(const gla_matmul_args& p) {
         // enough workgroups for 256 CUs, but no split shorter than 8 stages (512 K-values) and at
         // most 32 splits
         const int tiles = g.tiles_m * g.tiles_n;
-        // 2-bit codes on short tiles are bound by unpacking on one wave per SIMD: two workgroups per CU
-        // (16384^2, M=64: 72 against 90 us)
-        const int target = (p.W_nbits == 2 && g.bm <= 64) ? 512 : 256;
+        // short tiles (4 waves) are bound by unpacking on one wave per SIMD: two workgroups per CU
+        // (16384^2, 2-bit, M=64: 72 against 90 us; 4-bit, M=32: 47 against 56 us)
+        const int target = g.bm <= 64 ? 512 : 256;
         want = tiles * 2 > target ? 1 : ceil_div(target, tiles);
         const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
         if (want > max_s) want = max_s;

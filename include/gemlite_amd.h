@@ -170,8 +170,8 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_MXFP8 7   /* MXFP8 weights x fp8 activations, MFMA GEMM */
 #define GLA_FAMILY_MX_STREAM 8    /* streaming kernel: weight-only MX layers, MXFP8 x MXFP4 */
 #define GLA_FAMILY_BLOCKQ_STREAM 9 /* streaming kernel: 128 x 128 block-quantised int8 / fp8 */
-#define GLA_FAMILY_GEMM_BLOCKQ 10  /* the same above 4 rows: MFMA GEMM with a second, scaled accumulator */
-#define GLA_FAMILY_GEMM_KBYTES_MX 11 /* weight-only MX layers above 3 rows: MFMA GEMM, block scale applied on conversion */
+#define GLA_FAMILY_GEMM_BLOCKQ 10  /* the same from 2 rows up: MFMA GEMM with a second, scaled accumulator */
+#define GLA_FAMILY_GEMM_KBYTES_MX 11 /* weight-only MX layers above 2 rows: MFMA GEMM, block scale applied on conversion */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of

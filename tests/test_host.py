@@ -430,7 +430,7 @@ def test_weight_only_and_mixed_mx_processors():
             assert l.bias.dtype == dtype
             assert gemlite_amd.DTYPE_TO_TORCH[l.get_meta_args()[6]] == dtype
             # streaming kernel up to 2 rows, matrix cores above (K = 256 is a multiple of 128)
-            for M, fam in ((1, "MX_STREAM"), (3, "MX_STREAM"), (4, "GEMM_KBYTES_MX"), (100, "GEMM_KBYTES_MX")):
+            for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (3, "GEMM_KBYTES_MX"), (100, "GEMM_KBYTES_MX")):
                 m = l.get_meta_args()
                 x = torch.zeros(M, K, dtype=dtype)
                 out = torch.zeros(M, N, dtype=dtype)
@@ -452,7 +452,7 @@ def test_weight_only_and_mixed_mx_processors():
         assert l.input_dtype == DType.MXFP8 and l.scaled_activations and (l.W_nbits, l.elements_per_sample) == (4, 2)
         assert (l.W_group_mode, l.channel_scale_mode) == (0, csm)
         # streaming up to 2 rows; above (K = 256 is a multiple of 128) the mixed fp8 x fp4 matrix-core kernel
-        for M, fam in ((1, "MX_STREAM"), (4, "MX_STREAM"), (5, "GEMM_MXFP8"), (64, "GEMM_MXFP8")):
+        for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (3, "GEMM_MXFP8"), (64, "GEMM_MXFP8")):
             xq = torch.zeros(M, K, dtype=torch.float8_e4m3fn)
             sx = torch.ones(M, 1) if post_scale else torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
             assert _family(l, M, None, scales_x=sx, x=xq) == fam
@@ -488,7 +488,7 @@ def test_block_quant_processor_packs_like_the_reference():
         l2 = proc(device="cpu", dtype=torch.bfloat16, block_quant=True).from_weights(
             l.W_q.t().contiguous(), scales=l.scales.t().contiguous())
         assert torch.equal(l2.W_q.view(torch.uint8), l.W_q.view(torch.uint8)) and torch.equal(l2.scales, l.scales)
-        for M, fam in ((1, "BLOCKQ_STREAM"), (4, "BLOCKQ_STREAM"), (5, "GEMM_BLOCKQ"), (300, "GEMM_BLOCKQ")):
+        for M, fam in ((1, "BLOCKQ_STREAM"), (2, "GEMM_BLOCKQ"), (5, "GEMM_BLOCKQ"), (300, "GEMM_BLOCKQ")):
             xq = torch.zeros(M, K, dtype=wdt)
             assert _family(l, M, None, scales_x=torch.ones(M, K // 128), x=xq) == fam
 
