@@ -442,7 +442,7 @@ def cpu_baseline(host_tensors, x_host, y_gpu, threads):
 
     x32 = np.ascontiguousarray(x_host.float().numpy())
     y_ref = step(x32)
-    sec, reps = timed(lambda: step(x32), 10.0, 20)
+    sec, reps = timed(lambda: step(x32), 10.0, 2000)  # about 10 s of CPU work
     err = float(np.linalg.norm(y_gpu.astype(np.float64) - y_ref) / np.linalg.norm(y_ref))
 
     torch.set_num_threads(threads)
@@ -456,7 +456,7 @@ def cpu_baseline(host_tensors, x_host, y_gpu, threads):
             v = (v @ W.t()).to(torch.float16).float()
         return v
 
-    sec_torch, reps_torch = timed(torch_step, 10.0, 20)
+    sec_torch, reps_torch = timed(torch_step, 6.0, 200)
     return sec, reps, err, sec_torch, reps_torch
 
 

@@ -416,7 +416,7 @@ def matmul_workspace_need(args: MatmulArgs) -> int:
     return int(need)
 
 
-FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM", "BLOCKQ_STREAM", "GEMM_BLOCKQ", "GEMM_KBYTES_MX"]
+FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM", "BLOCKQ_STREAM", "GEMM_BLOCKQ", "GEMM_KBYTES_MX", "MX_SKINNY"]
 
 
 def matmul_family(args: MatmulArgs) -> str:

@@ -74,6 +74,9 @@ int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream);
 int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p);
 
 // ---- weight-only MX layers above 2 rows: the same MFMA GEMM with micro-scaled weights (gemm_kbytes.hip)
+// ---- weight-only MX layers at 3..16 rows: weights straight into registers, matrix cores (mx_skinny.hip)
+bool mx_skinny_eligible(const gla_matmul_args& p);
+int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream);
 bool gemm_kbytes_mx_eligible(const gla_matmul_args& p);
 int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream);
 int64_t gemm_kbytes_mx_workspace_bytes(const gla_matmul_args& p);

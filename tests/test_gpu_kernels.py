@@ -550,8 +550,9 @@ def test_weight_only_mxfp_layers(device, dtype, W_nbits):
     layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
     want = orc.quantize_mxfp8_weights(to_np(W.to(dtype))) if W_nbits == 8 else orc.quantize_mxfp4_weights(to_np(W.to(dtype)))
     assert np.array_equal(layer.scales.cpu().numpy(), want[1])
-    # streaming kernel up to 2 rows; above, the matrix-core kernel (64-, 128- and 256-row tiles, split K)
-    for M in (1, 2, 3, 4, 5, 7, 33, 70, 130, 300):
+    # streaming kernel up to 2 rows; 3..16 rows: weights straight into registers and to the matrix cores;
+    # above, the tiled matrix-core kernel (64-, 128- and 256-row tiles, split K)
+    for M in (1, 2, 3, 4, 5, 7, 11, 16, 17, 33, 70, 130, 300):
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=["GEMV", "GEMM_SPLITK", "GEMM"])
     # a one-hot activation row picks out one dequantised weight column exactly
     x = torch.zeros(1, K, dtype=dtype)
@@ -561,10 +562,36 @@ def test_weight_only_mxfp_layers(device, dtype, W_nbits):
     torch.cuda.synchronize()
     y_ref = oracle_forward(layer, x)
     assert np.array_equal(to_np(y), round_like(y_ref, dtype))
-    # ... and through the matrix-core kernel: row r of a batch of 40 is one-hot at a position of its own
-    x = torch.zeros(40, K, dtype=dtype)
-    for r in range(40):
-        x[r, (97 * r + 5) % K] = 1.0
+    # ... and through the matrix-core kernels (13 rows: the skinny one, 40: the tiled one): row r of the batch is
+    # one-hot at a position of its own
+    for rows in (13, 40):
+        x = torch.zeros(rows, K, dtype=dtype)
+        for r in range(rows):
+            x[r, (97 * r + 5) % K] = 1.0
+        y = layer(x.to(device))
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(y), round_like(oracle_forward(layer, x), dtype))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("W_nbits", [8, 4])
+def test_weight_only_mxfp_skinny_kernel_on_wide_layers(device, W_nbits):
+    """3..16 rows on layers wide enough for two and four 16-row tiles per wave (N = 16400 leaves the last
+    workgroup a ragged tile; K = 2432 = 19 steps of 128 ends inside the second chunk of activations)."""
+    N, K = 16400, 2432
+    dtype = torch.bfloat16
+    lin = torch.nn.Linear(K, N, bias=True, dtype=dtype)
+    lin.weight.data = gen_x(N, K, torch.bfloat16, seed=57, std=0.03)
+    lin.weight.data[:, 64:96] *= 16.0   # block scales that differ along K
+    lin.bias.data = gen_x(1, N, dtype, seed=58).reshape(-1)
+    cls = helper.A16W8_MXFP if W_nbits == 8 else helper.A16W4_MXFP
+    layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
+    for M in (3, 9, 16):
+        check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=["GEMM"])
+    x = torch.zeros(11, K, dtype=dtype)
+    for r in range(11):
+        x[r, (211 * r + 7) % K] = 1.0
+    layer.bias = None
     y = layer(x.to(device))
     torch.cuda.synchronize()
     assert np.array_equal(to_np(y), round_like(oracle_forward(layer, x), dtype))

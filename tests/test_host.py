@@ -429,8 +429,8 @@ def test_weight_only_and_mixed_mx_processors():
             assert l.scales.shape == (N, K // 32) and l.scales.dtype == torch.uint8 and l.scales.stride() == (K // 32, 1)
             assert l.bias.dtype == dtype
             assert gemlite_amd.DTYPE_TO_TORCH[l.get_meta_args()[6]] == dtype
-            # streaming kernel up to 2 rows, matrix cores above (K = 256 is a multiple of 128)
-            for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (3, "GEMM_KBYTES_MX"), (100, "GEMM_KBYTES_MX")):
+            # streaming kernel up to 2 rows, weights straight to the matrix cores up to 16, the tiled GEMM above (K = 256 is a multiple of 128)
+            for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (3, "MX_SKINNY"), (16, "MX_SKINNY"), (17, "GEMM_KBYTES_MX"), (100, "GEMM_KBYTES_MX")):
                 m = l.get_meta_args()
                 x = torch.zeros(M, K, dtype=dtype)
                 out = torch.zeros(M, N, dtype=dtype)
