@@ -26,7 +26,8 @@
 //    its slots, takes a ticket and reads the other slabs' slots in the same breath, and the one
 //    whose ticket says "last" already holds every partial that had landed (it polls the few that
 //    had not).  One memory round trip ends the kernel instead of three (store-and-wait, ticket,
-//    load), which at decode sizes is a quarter of the kernel.
+//    load); measured on the 4096^2 launch the tail after the last weight load is then about 1.6 us
+//    (ticket 0.25, one re-poll 0.6, LDS reduction and store 0.75) of 6 us.
 #include "common.hpp"
 #include "dispatch.hpp"
 
