@@ -136,60 +136,74 @@ __device__ __forceinline__ uint2 quantise8(float (&v)[8], float s) {
 template <int XDT>
 constexpr int row_cache() { return XDT == GLA_DT_FP32 ? 8 : 16; }
 
-// One wave per row.  The amax pass keeps the raw row in registers; the part of a
-// longer row that does not fit is read again (from L2) in the quantise pass.
+// One wave per row.  The amax pass keeps the raw row in registers; the part of a longer row that does not
+// fit is read again (from L2) in the quantise pass.  (kRowsPerWave = 2, the loads of a wave's second row in
+// flight under the divisions of its first, measured slower: M=4096, K=8192 31 against 28 us.)
+constexpr int kRowsPerWave = 1;
+
 template <int XDT, bool TO_INT8>
 __global__ __launch_bounds__(256) void per_token_kernel(const void* __restrict__ x, int64_t xsm, int M, int K,
                                                         uint8_t* __restrict__ y, float* __restrict__ scales) {
     constexpr int RC = row_cache<XDT>();
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= M) return;
-    const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * kRowsPerWave;
+    if (row0 >= M) return;
     const int chunks = K / 8;  // K % 8 == 0 enforced by the launcher
 
-    Raw8<XDT> cache[RC];
-    float amax = 0.0f;
+    Raw8<XDT> cache[kRowsPerWave][RC];
 #pragma unroll
-    for (int ci = 0; ci < RC; ++ci) {
-        const int c = lane + ci * kWave;
-        if (c < chunks) cache[ci] = load_raw8<XDT>(xrow, c * 8);
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        // a row past the end repeats the last one (loaded, never reduced or stored)
+        const int row = row0 + r < M ? row0 + r : M - 1;
+        const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+#pragma unroll
+        for (int ci = 0; ci < RC; ++ci) {
+            const int c = lane + ci * kWave;
+            if (c < chunks) cache[r][ci] = load_raw8<XDT>(xrow, c * 8);
+        }
     }
 #pragma unroll
-    for (int ci = 0; ci < RC; ++ci) {
-        const int c = lane + ci * kWave;
-        if (c < chunks) {
+    for (int r = 0; r < kRowsPerWave; ++r) {
+        const int row = row0 + r;
+        if (row >= M) break;
+        const char* xrow = (const char*)x + (int64_t)row * xsm * (XDT == GLA_DT_FP32 ? 4 : 2);
+        float amax = 0.0f;
+#pragma unroll
+        for (int ci = 0; ci < RC; ++ci) {
+            const int c = lane + ci * kWave;
+            if (c < chunks) {
+                float v[8];
+                decode_raw8<XDT>(cache[r][ci], v);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+            }
+        }
+        for (int c = lane + RC * kWave; c < chunks; c += kWave) {
             float v[8];
-            decode_raw8<XDT>(cache[ci], v);
+            decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
 #pragma unroll
             for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
         }
-    }
-    for (int c = lane + RC * kWave; c < chunks; c += kWave) {
-        float v[8];
-        decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-    }
-    amax = wave_max(amax);
-    const float qmax = TO_INT8 ? 127.0f : 448.0f;
-    const float s = fmaxf(amax / qmax, 1e-6f);
-    if (lane == 0) scales[row] = s;
+        amax = wave_max(amax);
+        const float qmax = TO_INT8 ? 127.0f : 448.0f;
+        const float s = fmaxf(amax / qmax, 1e-6f);
+        if (lane == 0) scales[row] = s;
 
-    uint8_t* yrow = y + (int64_t)row * K;
+        uint8_t* yrow = y + (int64_t)row * K;
 #pragma unroll
-    for (int ci = 0; ci < RC; ++ci) {
-        const int c = lane + ci * kWave;
-        if (c < chunks) {
+        for (int ci = 0; ci < RC; ++ci) {
+            const int c = lane + ci * kWave;
+            if (c < chunks) {
+                float v[8];
+                decode_raw8<XDT>(cache[r][ci], v);
+                *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
+            }
+        }
+        for (int c = lane + RC * kWave; c < chunks; c += kWave) {
             float v[8];
-            decode_raw8<XDT>(cache[ci], v);
+            decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
             *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
         }
-    }
-    for (int c = lane + RC * kWave; c < chunks; c += kWave) {
-        float v[8];
-        decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
-        *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
     }
 }
 
@@ -251,11 +265,18 @@ __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, 
         amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
         amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
 
-        const uint32_t bits = __builtin_bit_cast(uint32_t, amax / (FP8OUT ? 448.0f : 6.0f));
-        uint32_t e = (bits >> 23) & 0xffu;
-        e += (bits & 0x7fffffu) ? 1u : 0u;
-        e = e > 254u ? 254u : e;
-        e = e < 97u ? 97u : e;
+        // e8m0 of amax / qmax = biased exponent of the quotient, plus one unless the quotient is a power of two
+        // (reference: the exponent of the scale is rounded up).  qmax = 1.5 * 2^2 (6) or 1.75 * 2^8 (448), so
+        // the quotient's exponent and whether its mantissa is zero follow from amax's own fields without a
+        // division: significand above qmax's -> exponent(amax) - log2 part + 1, equal or below -> one less
+        // (equal: an exact power of two; below: the quotient drops a binade and is never a power of two).
+        const uint32_t abits = __builtin_bit_cast(uint32_t, amax);
+        const int ea = (int)(abits >> 23), ma = (int)(abits & 0x7fffffu);
+        int ei = ea - (FP8OUT ? 8 : 2) + (ma > (FP8OUT ? 0x600000 : 0x400000) ? 1 : 0);
+        if (ea == 255) ei = 254;  // an infinite amax: inf / qmax has exponent 255, clamped below
+        ei = ei > 254 ? 254 : ei;
+        ei = ei < 97 ? 97 : ei;
+        const uint32_t e = (uint32_t)ei;
 
         if (!active) continue;
         // the scale is a power of two, so v / s is an exact exponent shift: ldexp gives the same value (signed
@@ -278,17 +299,32 @@ __global__ __launch_bounds__(256) void mxfp4_kernel(const void* __restrict__ x, 
             // 3.5 times the scale: those go one ulp toward zero first) and at -0.0 (x + 0.0 is +0.0 for both
             // zeros and x otherwise).  An input that is not a number takes the reference's route.
             const float sc = __builtin_bit_cast(float, e << 23);
-            const uint32_t shift = (e - 127u) << 23;
-            const uint32_t t1 = 0x3f400000u + shift, t2 = 0x3fe00000u + shift, t3 = 0x40600000u + shift;
             bool odd = false;
             float w[8];
+            if constexpr (XDT == GLA_DT_FP32) {
+                const uint32_t shift = (e - 127u) << 23;
+                const uint32_t t1 = 0x3f400000u + shift, t2 = 0x3fe00000u + shift, t3 = 0x40600000u + shift;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float z = v[j] + 0.0f;
-                const uint32_t zb = __builtin_bit_cast(uint32_t, z), mag = zb & 0x7fffffffu;
-                const bool tie = mag == t1 || mag == t2 || mag == t3;
-                w[j] = __builtin_bit_cast(float, zb - (tie ? 1u : 0u));
-                odd |= mag > 0x7f800000u;
+                for (int j = 0; j < 8; ++j) {
+                    const float z = v[j] + 0.0f;
+                    const uint32_t zb = __builtin_bit_cast(uint32_t, z), mag = zb & 0x7fffffffu;
+                    const bool tie = mag == t1 || mag == t2 || mag == t3;
+                    w[j] = __builtin_bit_cast(float, zb - (tie ? 1u : 0u));
+                    odd |= mag > 0x7f800000u;
+                }
+            } else {
+                // 16-bit inputs have at most 11 significant bits, so a value that is not exactly on a tie is at
+                // least 2^-12 of itself away from it: scaling everything by 1 - 2^-16 moves the ties below
+                // their midpoint (they round toward zero, as the reference has them) and nothing else across
+                // one.  The fused add of +0.0 turns -0.0 into +0.0.  Not-a-number and infinite inputs make the
+                // second sum a NaN and take the reference's route.
+                float chk = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    w[j] = __builtin_fmaf(v[j], 0.9999847412109375f, 0.0f);
+                    chk = __builtin_fmaf(v[j], 0.0f, chk);
+                }
+                odd = chk != chk;
             }
             uint32_t packed = 0;
             if (__builtin_expect(!odd, 1)) {
@@ -323,7 +359,7 @@ int launch_act_per_token(const void* x, int x_dtype, int64_t x_stride_m, int M, 
         return GLA_ERR_UNSUPPORTED_DTYPE;
     }
     if (M == 0) return GLA_OK;
-    dim3 grid(ceil_div(M, 4)), block(256);
+    dim3 grid(ceil_div(M, 4 * kRowsPerWave)), block(256);
     const bool i8 = (y_dtype == GLA_DT_INT8);
 #define GLA_PT(XDT)                                                                                         \
     do {                                                                                                    \
