@@ -111,13 +111,27 @@ __device__ __forceinline__ void decode_raw8(const Raw8<XDT>& r, float (&v)[8]) {
     }
 }
 
-template <bool TO_INT8>
+// v / s, correctly rounded, for v that came from a 16-bit float and s = max(amax / qmax, 1e-6) of such values:
+// q = v * r with r the correctly rounded 1 / s, one residual e = v - q s (exact in the fused multiply-add)
+// and q + e r.  That this equals the IEEE quotient bit for bit for every such pair (65536 x 32768 per input
+// type and qmax; quotients below 2^-20, which become the code 0 either way, only have to stay that small)
+// is checked exhaustively on the CPU by tests/test_division.py; the sign is copied from v because the
+// correction step turns a quotient of -0 into +0.  One division per row instead of one per element.
+__device__ __forceinline__ float div_by_row_scale(float v, float s, float r) {
+    const float q = v * r;
+    const float e = __builtin_fmaf(-q, s, v);
+    const float c = __builtin_fmaf(e, r, q);
+    return __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, c) & 0x7fffffffu) | (__builtin_bit_cast(uint32_t, v) & 0x80000000u));
+}
+
+template <bool TO_INT8, bool FROM16>
 __device__ __forceinline__ uint2 quantise8(float (&v)[8], float s) {
     const float qmax = TO_INT8 ? 127.0f : 448.0f;
     const float qmin = TO_INT8 ? -128.0f : -448.0f;
     uint32_t lo = 0, hi = 0;
+    const float r = 1.0f / s;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = fminf(fmaxf(v[j] / s, qmin), qmax);
+    for (int j = 0; j < 8; ++j) v[j] = fminf(fmaxf(FROM16 ? div_by_row_scale(v[j], s, r) : v[j] / s, qmin), qmax);
     if constexpr (TO_INT8) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -196,13 +210,13 @@ __global__ __launch_bounds__(256) void per_token_kernel(const void* __restrict__
             if (c < chunks) {
                 float v[8];
                 decode_raw8<XDT>(cache[r][ci], v);
-                *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
+                *(uint2*)(yrow + c * 8) = quantise8<TO_INT8, XDT != GLA_DT_FP32>(v, s);
             }
         }
         for (int c = lane + RC * kWave; c < chunks; c += kWave) {
             float v[8];
             decode_raw8<XDT>(load_raw8_cached<XDT>(xrow, c * 8), v);
-            *(uint2*)(yrow + c * 8) = quantise8<TO_INT8>(v, s);
+            *(uint2*)(yrow + c * 8) = quantise8<TO_INT8, XDT != GLA_DT_FP32>(v, s);
         }
     }
 }

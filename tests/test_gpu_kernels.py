@@ -107,6 +107,50 @@ def test_mxfp4_quant_bit_exact(device, dtype, shape):
     assert np.array_equal(y.cpu().numpy(), y_ref)
 
 
+@pytest.mark.parametrize("w_dtype", [torch.int8, torch.float8_e4m3fn])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_per_token_quant_every_16_bit_value(device, dtype, w_dtype):
+    """Rows that hold every finite value of the input type up to a row maximum (both zeros, subnormals), for row
+    maxima across the type's range: codes and scales equal the oracle's bit for bit.  (The kernel divides
+    through a reciprocal and one correction step; tests/test_division.py proves the quotients equal over all
+    pairs on the CPU, this runs the kernel itself over 28 rows of them.)"""
+    allv = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    allv = allv[torch.isfinite(allv.float())]
+    g = torch.Generator().manual_seed(5)
+    tops = [allv.float().abs().max().item(), 1.0, 448.0, 127.0, 3.0e-5, 1.0e-7, 0.3333] + \
+        (torch.rand(21, generator=g) * 16 - 12).exp2().tolist()
+    rows = []
+    for top in tops:
+        top = torch.tensor(top).to(dtype)
+        row = torch.where(allv.float().abs() <= top.float(), allv, torch.zeros_like(allv))
+        rows.append(torch.cat([top.view(1), row, torch.zeros((-row.numel() - 1) % 8, dtype=dtype)]))
+    x = torch.stack(rows)
+    to_int8 = w_dtype == torch.int8
+    y, sc = gemlite_amd.scale_activations_per_token(x.to(device), w_dtype)
+    q_ref, s_ref = orc.scale_activations_per_token(to_np(x), to_int8)
+    assert np.array_equal(sc.cpu().numpy(), s_ref)
+    got = y.cpu().numpy() if to_int8 else y.cpu().view(torch.uint8).numpy()
+    assert np.array_equal(got, q_ref if to_int8 else q_ref.view(np.uint8))
+
+
+@pytest.mark.parametrize("amax_exp", [-9, -3, 0, 4, 12])
+def test_mxfp4_quant_every_bf16_value(device, amax_exp):
+    """The same for bf16 inputs (8 significant bits, the exponent range of fp32)."""
+    top = 6.0 * 2.0 ** amax_exp
+    allv = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    allv = allv[torch.isfinite(allv.float()) & (allv.float().abs() <= top)]
+    pad = (-allv.numel()) % 31
+    allv = torch.cat([allv, torch.zeros(pad, dtype=torch.bfloat16)])
+    groups = allv.view(-1, 31)
+    x = torch.cat([torch.full((groups.shape[0], 1), top, dtype=torch.bfloat16), groups], dim=1).reshape(1, -1)
+    cols = 32 * 128
+    x = torch.cat([x, torch.zeros((1, (-x.shape[1]) % cols), dtype=torch.bfloat16)], dim=1).view(-1, cols)
+    y, s = gemlite_amd.scale_activations_mxfp4(x.to(device))
+    y_ref, s_ref = orc.scale_activations_mxfp4(to_np(x))
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(y.cpu().numpy(), y_ref)
+
+
 @pytest.mark.parametrize("amax_exp", [-9, -3, 0, 4, 12])
 def test_mxfp4_quant_every_fp16_value(device, amax_exp):
     """Every finite fp16 value (both zeros, subnormals, every exact tie) up to the block maximum, under a block
