@@ -196,7 +196,7 @@ Family choose(const gla_matmul_args& p, int type) {
     if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)  // validated as eligible for the streaming kernel
     {
         // 1-2 rows: the streaming kernel; up to 16 rows the weights still go straight into registers, to the
-        // matrix cores (16384^2 MXFP4, 8 rows: 51 against 62 us of the tiled GEMM); above that the tiled GEMM
+        // matrix cores (16384^2 MXFP4, 8 rows: 48 against 62 us of the tiled GEMM); above that the tiled GEMM
         if (p.M > 2 && p.M <= 16 && p.tile_config < 1000 && mx_skinny_eligible(p)) return F_MX_SKINNY;
         return gemm_kbytes_mx_eligible(p) ? F_GEMM_KBYTES_MX : F_MX_STREAM;
     }

@@ -15,8 +15,10 @@
 //    of a 16-bit MFMA operand: the operand is the dequantised weight.  v_mfma_f32_16x16x32 multiplies
 //    it with the activations of up to 16 rows, which a lane loads (through the vector cache, they are
 //    small) for the same K positions once per step for all RT tiles.
-//  * The 8 waves of a workgroup take the steps of K in turn and add their accumulators through LDS in
-//    wave order; no workspace, no second kernel, deterministic.
+//  * The 8 waves of a workgroup take the steps of K in turn, two adjacent steps at a time, and add their
+//    accumulators through LDS in wave order; no workspace, no second kernel, deterministic.
+//  * 16384^2 MXFP4: 45 us at 3 rows, 51 at 16 (a pure read in this access pattern: 30-34 us; the tiled GEMM:
+//    52-62 us); MXFP8: 73-79 us.
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(kWavesS * 64) void mx_skinny_kernel(MxSkArgs a) {
         int n = n0 + 16 * t + r16;
         if (n > a.N - 1) n = a.N - 1;  // rows past the end repeat the last one; never stored
         wrow[t] = a.w + (int64_t)n * a.wsn + 16 * kq;
-        srow[t] = a.scales + (int64_t)n * a.msn + (W4 ? kq : kq / 2);
+        srow[t] = a.scales + (int64_t)n * a.msn;
     }
     f32x4s acc[RT];
 #pragma unroll
@@ -122,13 +124,16 @@ __global__ __launch_bounds__(kWavesS * 64) void mx_skinny_kernel(MxSkArgs a) {
     const int chunks = (a.K + KC - 1) / KC;
 
     // staging: piece id = i * 512 + tid -> (row, piece of the row)
+    // only the M rows that exist are staged (lanes of further rows read row M - 1; their results are not stored)
     const uint16_t* xsrc[XS];
     int xcol[XS], xdst[XS];
+    bool xlive[XS];
 #pragma unroll
     for (int i = 0; i < XS; ++i) {
         const int id = i * (kWavesS * 64) + tid;
         const int row = id / PIECES, col = id % PIECES;
-        xsrc[i] = a.x + (int64_t)(row < a.M ? row : a.M - 1) * a.xsm;
+        xlive[i] = row < a.M;
+        xsrc[i] = a.x + (int64_t)(xlive[i] ? row : 0) * a.xsm;
         xcol[i] = col * 8;
         xdst[i] = row * ROWB + col * 16;
     }
@@ -138,45 +143,56 @@ __global__ __launch_bounds__(kWavesS * 64) void mx_skinny_kernel(MxSkArgs a) {
         for (int i = 0; i < XS; ++i) {
             int k = c * KC + xcol[i];
             if (k > a.K - 8) k = a.K - 8;  // pieces past the end of K repeat the last one; never multiplied
-            xs[i] = *(const u32x4s*)(xsrc[i] + k);
+            if (xlive[i]) xs[i] = *(const u32x4s*)(xsrc[i] + k);
         }
     };
     auto x_store = [&](int c) __attribute__((always_inline)) {
         unsigned char* base = xbuf + (c & 1) * (16 * ROWB);
 #pragma unroll
-        for (int i = 0; i < XS; ++i) *(u32x4s*)(base + xdst[i]) = xs[i];
+        for (int i = 0; i < XS; ++i)
+            if (xlive[i]) *(u32x4s*)(base + xdst[i]) = xs[i];
     };
+    // A wave takes two adjacent steps of a chunk (2 wave, 2 wave + 1): the scale bytes of both are then 8 (W4)
+    // or 4 (W8) consecutive bytes of the row, one load per tile and chunk.  (One byte load per tile and step
+    // made the kernel a fifth slower: the CU's load unit spends as long on a byte per lane as on 16.)
     struct Batch {
         u32x4s wv[UN][RT];
-        uint32_t sc[UN][RT];
+        uint32_t sc[RT][W4 ? 2 : 1];
     };
     auto w_load = [&](Batch& b, int c) __attribute__((always_inline)) {
+        // chunks have whole pairs of steps (K is a multiple of two steps); pairs past the end re-read the first
+        int s0 = c * (UN * kWavesS) + UN * wave;
+        if (s0 > steps - UN) s0 = 0;
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            // steps past the end re-read the wave's first one and are not multiplied
-            int s = c * (UN * kWavesS) + u * kWavesS + wave;
-            if (s > steps - 1) s = wave < steps ? wave : 0;
+        for (int t = 0; t < RT; ++t) {
 #pragma unroll
-            for (int t = 0; t < RT; ++t) {
-                const uint4 q = load_streaming_u4(wrow[t] + (int64_t)s * kStepB);
+            for (int u = 0; u < UN; ++u) {
+                const uint4 q = load_streaming_u4(wrow[t] + (int64_t)(s0 + u) * kStepB);
                 b.wv[u][t] = u32x4s{q.x, q.y, q.z, q.w};
-                b.sc[u][t] = srow[t][s * (W4 ? 4 : 2)];
+            }
+            if constexpr (W4) {
+                const uint2 w = *(const uint2*)(srow[t] + s0 * 4);
+                b.sc[t][0] = w.x; b.sc[t][1] = w.y;
+            } else {
+                b.sc[t][0] = *(const uint32_t*)(srow[t] + s0 * 2);
             }
         }
     };
-    const int xoff = r16 * ROWB + kq * (STEPK / 2);  // this lane's bytes of a step's activations inside an LDS row
+    const int xoff = (r16 < a.M ? r16 : a.M - 1) * ROWB + kq * (STEPK / 2);  // this lane's bytes of a step's activations inside an LDS row
     auto multiply = [&](const Batch& b, int c) __attribute__((always_inline)) {
         const unsigned char* base = xbuf + (c & 1) * (16 * ROWB) + xoff;
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int sl = u * kWavesS + wave;  // step inside the chunk
+            const int sl = UN * wave + u;  // step inside the chunk
             if (c * (UN * kWavesS) + sl < steps) {
                 u32x4s xv[XV];
 #pragma unroll
                 for (int j = 0; j < XV; ++j) xv[j] = *(const u32x4s*)(base + sl * (STEPK * 2) + 16 * j);
 #pragma unroll
                 for (int t = 0; t < RT; ++t) {
-                    const float scale = __builtin_bit_cast(float, b.sc[u][t] << 23);
+                    // this lane's block: W4 byte kq of the step's word, W8 byte 2 u + kq / 2 of the pair's
+                    const uint32_t e8 = W4 ? (b.sc[t][u] >> (8 * kq)) & 0xffu : (b.sc[t][0] >> (8 * (2 * u + kq / 2))) & 0xffu;
+                    const float scale = __builtin_bit_cast(float, e8 << 23);
 #pragma unroll
                     for (int j = 0; j < XV; ++j) {
                         u32x4s op;
@@ -266,7 +282,8 @@ bool mx_skinny_eligible(const gla_matmul_args& p) {
     const bool w4 = p.W_nbits == 4 && p.elements_per_sample == 2;
     const bool w8 = p.W_nbits == 8 && p.elements_per_sample == 1;
     if (!w4 && !w8) return false;
-    if (p.K % (w4 ? 128 : 64) != 0) return false;
+    if (p.K % (w4 ? 256 : 128) != 0) return false;  // whole pairs of steps
+    if (p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3)) return false;  // a pair's scale bytes are read as 32-bit words
     if (p.x_stride_k != 1 || p.w_stride_k != 1 || p.out_stride_n != 1 || p.meta_stride_g != 1) return false;
     if (p.x_stride_m % 8 != 0 || p.w_stride_n % 16 != 0 || ((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
     switch (p.output_dtype) {
@@ -279,7 +296,7 @@ bool mx_skinny_eligible(const gla_matmul_args& p) {
 int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream) {
     if (!mx_skinny_eligible(p)) {
         set_error("mx_skinny: weight-only MX operands, K-contiguous with 16-byte aligned rows, up to 16 rows, "
-                  "K a multiple of 128 (MXFP4) or 64 (MXFP8)");
+                  "K a multiple of 256 (MXFP4) or 128 (MXFP8)");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     MxSkArgs a;

@@ -621,8 +621,8 @@ def test_weight_only_mxfp_layers(device, dtype, W_nbits):
 @pytest.mark.parametrize("W_nbits", [8, 4])
 def test_weight_only_mxfp_skinny_kernel_on_wide_layers(device, W_nbits):
     """3..16 rows on layers wide enough for two and four 16-row tiles per wave (N = 16400 leaves the last
-    workgroup a ragged tile; K = 2432 = 19 steps of 128 ends inside the second chunk of activations)."""
-    N, K = 16400, 2432
+    workgroup a ragged tile; K = 2560 ends inside the second chunk of activations)."""
+    N, K = 16400, 2560
     dtype = torch.bfloat16
     lin = torch.nn.Linear(K, N, bias=True, dtype=dtype)
     lin.weight.data = gen_x(N, K, torch.bfloat16, seed=57, std=0.03)
