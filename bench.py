@@ -374,13 +374,14 @@ def run_point(name, lib, device, T):
     """One GEMM point alone, a few launches: the workload of the per-kernel counter profiles under profiles/."""
     from gemlite_amd import helper
     g = torch.Generator(device="cpu").manual_seed(7)
-    if name in ("gemm_a8w8_fp8", "gemm_a8w8_int8"):
+    if name in ("gemm_a8w8_fp8", "gemm_a8w8_int8", "gemm_a8w8_fp8_block_quant", "gemm_a8w8_int8_block_quant"):
         M, N, K = 4096, 8192, 8192
         W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16).to(device)
         x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
-        fp8 = name.endswith("fp8")
-        layer = (helper.A8W8_FP8_dynamic if fp8 else helper.A8W8_INT8_dynamic)(device=device).from_weights(W)
-        xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn if fp8 else torch.int8)
+        fp8, blockq = "fp8" in name, name.endswith("block_quant")
+        layer = (helper.A8W8_FP8_dynamic if fp8 else helper.A8W8_INT8_dynamic)(device=device, block_quant=blockq).from_weights(W)
+        quant = gemlite_amd.scale_activations_per_block if blockq else gemlite_amd.scale_activations_per_token
+        xq, sx = quant(x, torch.float8_e4m3fn if fp8 else torch.int8)
         peak = 5000.0
     elif name in ("gemm_a4w4_mxfp4", "gemm_a4w4_mxfp4_M8192"):
         M, N, K = (8192 if name.endswith("8192") else 4096), 16384, 16384
@@ -471,7 +472,7 @@ def main():
     ap.add_argument("--quick-extra", action="store_true", help="a subset of the secondary points")
     ap.add_argument("--point", default=None,
                     help="run one GEMM point alone (gemm_a8w8_fp8, gemm_a8w8_int8, gemm_a4w4_mxfp4, gemm_a4w4_mxfp4_M8192, "
-                         "gemm_a16w4_gs128_fp16) for a profiler, print its line and exit")
+                         "gemm_a16w4_gs128_fp16, gemm_a8w8_fp8_block_quant, gemm_a8w8_int8_block_quant) for a profiler, print its line and exit")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 256 MiB device copy (a kernel of known traffic, to scale profiler byte counters)")
     a = ap.parse_args()
