@@ -212,6 +212,32 @@ def test_a16w4_benchmark_shapes(device, M, shape):
     assert rel_frob(to_np(y), y_hqq) <= FROB_TOL
 
 
+def test_split_k_hand_off_repeats_bit_for_bit(device):
+    """The split-K hand-off of the packed-code GEMV (tagged slots, ticket counters that the last arriver resets) over
+    many column tiles and slabs, launched 150 times in a row, two layers and several batch sizes taking turns on
+    one stream and one workspace: every launch must reproduce the layer's first result bit for bit, and that
+    result must match the oracle.  A counter or slot left dirty by one launch shows up in a later one."""
+    layers = []
+    for (N, K, seed) in ((4096, 14336, 3), (1024, 8192, 4)):   # 64 tiles x 4 slabs; 16 tiles with more slabs
+        W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16, seed=seed)
+        layers.append(GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device)))
+    cases = []
+    for li, layer in enumerate(layers):
+        for M in (1, 3, 16):
+            x = gen_x(M, layer.in_features, torch.float16, seed=10 * li + M)
+            first = layer(x.to(device))
+            torch.cuda.synchronize()
+            assert rel_frob(to_np(first), oracle_forward(layer, x)) <= TIGHT[torch.float16]
+            cases.append((layer, x.to(device), first.clone()))
+    outs = []
+    for it in range(150):
+        layer, x, _ = cases[(7 * it) % len(cases)]
+        outs.append(((7 * it) % len(cases), layer(x)))
+    torch.cuda.synchronize()
+    for ci, y in outs:
+        assert torch.equal(y, cases[ci][2]), ci
+
+
 @pytest.mark.parametrize("nbits,gs", [(2, 64), (1, 64), (4, 32), (4, 64), (8, 128), (2, 32), (4, 16)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
