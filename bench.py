@@ -264,7 +264,25 @@ def extra_points(lib, device, T, quick):
         run = Launch(lib, layer, xq, y, device, scales_x=sx)
         us = T.eager_us(run, 40)
         us_e2e = T.eager_us(lambda: layer(x), 20)
-        gemm_point(f"gemm_a8w8_{name}", M, N, K, us, 5000.0, name, zeroed(run, xq, layer.W_q.data), us_e2e)
+        # the vendor library on the same operands in the same run, for what this box's power limit lets a tuned
+        # GEMM reach (not part of the product path): torch._scaled_mm (hipBLASLt, row-wise fp32 scales -> bf16) and
+        # torch._int_mm (int32 output, no scales).  Absent or failing entry points are skipped.
+        vendor = {}
+        try:
+            if name == "fp8":
+                sb = layer.scales.float().reshape(1, N).contiguous()
+                vfn = lambda: torch._scaled_mm(xq, layer.W_q, scale_a=sx.float().reshape(M, 1), scale_b=sb, out_dtype=torch.bfloat16)  # noqa: E731
+            else:
+                vfn = lambda: torch._int_mm(xq, layer.W_q)  # noqa: E731
+            vendor["us"] = round(T.eager_us(vfn, 20), 1)
+        except Exception as e:  # noqa: BLE001
+            vendor = {"skipped": str(e)[:120]}
+        us_zero = zeroed(run, xq, layer.W_q.data)
+        if "us" in vendor:
+            vendor["us_zero_operands"] = round(T.eager_us(vfn, 20), 1)
+        gemm_point(f"gemm_a8w8_{name}", M, N, K, us, 5000.0, name, us_zero, us_e2e)
+        out[f"gemm_a8w8_{name}"]["vendor_library_same_operands"] = dict(
+            vendor, entry="torch._scaled_mm (row-wise scales)" if name == "fp8" else "torch._int_mm")
         # the quantiser alone, reading a different activation matrix every launch
         xq_o, sx_o = torch.empty_like(xq), torch.empty_like(sx)
         fns = [(lambda xi=xi: _ext.scale_activations_per_token(xi, xq_o, sx_o)) for xi in xs]
