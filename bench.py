@@ -348,10 +348,26 @@ def extra_points(lib, device, T, quick):
         us = T.eager_us(run, 12)
         us_e2e = T.eager_us(lambda: layer(xm), 8)
         us_zero = None
+        vendor = None
         if M == 4096:
+            # the vendor library on the same codes and block scales (torch._scaled_mm with e2m1 pairs and e8m0
+            # scales; timing only, its scale layout conventions are not checked), as for fp8 above
+            try:
+                a4, b4 = xq.view(torch.float4_e2m1fn_x2), layer.W_q.data.view(torch.float4_e2m1fn_x2)
+                sa8 = sx[:M].contiguous().view(torch.float8_e8m0fnu)
+                sb8 = layer.scales.data.contiguous().view(torch.float8_e8m0fnu)
+                vfn = lambda: torch._scaled_mm(a4, b4, scale_a=sa8, scale_b=sb8, out_dtype=torch.bfloat16)  # noqa: E731
+                vendor = {"us": round(T.eager_us(vfn, 8), 1), "entry": "torch._scaled_mm (e2m1 x e2m1, e8m0 block scales)"}
+            except Exception as e:  # noqa: BLE001
+                vendor = {"skipped": str(e)[:120]}
             us_zero = zeroed(run, xq, layer.W_q.data)
+            if "us" in vendor:
+                vendor["us_zero_operands"] = round(T.eager_us(vfn, 8), 1)
             layer.W_q.data.copy_(w_saved)
-        gemm_point(f"gemm_a4w4_mxfp4_M{M}" if M != 4096 else "gemm_a4w4_mxfp4", M, N, K, us, 10100.0, "mxfp4", us_zero, us_e2e)
+        name = f"gemm_a4w4_mxfp4_M{M}" if M != 4096 else "gemm_a4w4_mxfp4"
+        gemm_point(name, M, N, K, us, 10100.0, "mxfp4", us_zero, us_e2e)
+        if vendor is not None:
+            out[name]["vendor_library_same_operands"] = vendor
         if M == 4096:
             xs = [xm] + [torch.randn((M, K), device=device).to(torch.bfloat16) for _ in range(copies_for(M * K * 2.5) - 1)]
             xq_o, sx_o = torch.empty_like(xq), torch.empty_like(sx)
