@@ -69,11 +69,18 @@ struct GemvArgs {
     int waves;  // waves per workgroup (4, 8 or 16)
     int nfb;      // direct variant: flush blocks per batch of loads
     int fl_log2;  // log2(FL)
+    int srww;     // direct variant: super rows per wave = RW / LW / waves, divided on the host
+    int gr_shift; // log2(gr) when gr is a power of two, else -1 (the kernels then divide)
     int wgm, csm, meta_dt, z_dt, z_scalar, out_dt, sx_dt;
     int64_t wsk, xsm, osm, msg, sxm;
     const void* bias;  // [N] or NULL: added to the result rounded to the output type
     int bias_dt;
 };
+
+// word row -> quantisation group: a shift for the usual power-of-two groups
+__device__ __forceinline__ int div_group(const GemvArgs& a, int word_row) {
+    return a.gr_shift >= 0 ? word_row >> a.gr_shift : word_row / a.gr;
+}
 
 template <bool BF16>
 struct Magic;
@@ -340,8 +347,10 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int cg = lane & 15, kb = lane >> 4;
-    const int tile = blockIdx.x % a.tiles;
-    const int split = blockIdx.x / a.tiles;
+    // grid (column tiles, row tiles, K slabs): nothing in front of the first load is divided at run time
+    // (the wave's share of the slab and the group size as a shift come from the host)
+    const int tile = blockIdx.x;
+    const int split = blockIdx.z;
     const int m0 = blockIdx.y * RT;
     const int n0 = tile * kTileN;
     const int r0 = split * a.RW;
@@ -365,7 +374,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
 #pragma unroll
         for (int t = 0; t < T; ++t) xraw[t] = src[t];
     }
-    const int g0 = r0 / a.gr;
+    const int g0 = div_group(a, r0);
     const bool fast_meta = (a.meta_dt == GLA_DT_FP16 || a.meta_dt == GLA_DT_BF16) && !a.z_scalar &&
                            (a.z_dt == a.meta_dt) && a.wgm >= GLA_WGM_SHIFT_SCALE;
     uint2 sraw = make_uint2(0, 0), zraw = make_uint2(0, 0);
@@ -534,7 +543,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
             }
             if (((it + 1) & fl_mask) == 0) {
                 // group of this iteration: the four quarters' super rows lie in one group
-                int gl = (r0 + (wv * SRWW + 4 * it) * LW) / a.gr - g0;
+                int gl = div_group(a, r0 + (wv * SRWW + 4 * it) * LW) - g0;
                 if (gl > a.GW - 1) gl = a.GW - 1;
                 const float4* mrow = (const float4*)(mt + gl * kTileN + cg * 4);
                 const float4 m01 = mrow[0], m23 = mrow[1];
@@ -587,15 +596,17 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     const int tid = threadIdx.x;
     const int lane = tid & 63, wv = tid >> 6;
     const int cg = lane & 15, kb = lane >> 4;
-    const int tile = blockIdx.x % a.tiles;
-    const int split = blockIdx.x / a.tiles;
+    // grid (column tiles, row tiles, K slabs): nothing in front of the first load is divided at run time
+    // (the wave's share of the slab and the group size as a shift come from the host)
+    const int tile = blockIdx.x;
+    const int split = blockIdx.z;
     const int m0 = blockIdx.y * RT;
     const int n0 = tile * kTileN;
     const int r0 = split * a.RW;
-    const int SRWW = a.RW / LW / waves;  // super rows per wave
-    const int nit = SRWW / 4;            // wave iterations
+    const int SRWW = a.srww;   // super rows per wave
+    const int nit = SRWW / 4;  // wave iterations
     const int lsr0 = wv * SRWW + kb;
-    const int g0w = (r0 + wv * SRWW * LW) / a.gr;  // first group this wave touches
+    const int g0w = div_group(a, r0 + wv * SRWW * LW);  // first group this wave touches
 
     int col = n0 + cg * 4;
     if (col > a.N - 4) col = a.N - 4;  // clamped lanes are never stored
@@ -616,12 +627,31 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     // group (relative to g0w) whose fold closes flush block `fbl` of the batch starting at iteration ib
     auto block_group = [&](int ib, int fbl) {
         const int it_f = (a.FL <= IPB) ? (ib + (fbl + 1) * a.FL - 1) : (ib + IPB - 1);
-        int g = (r0 + (wv * SRWW + 4 * it_f) * LW) / a.gr;
+        int g = div_group(a, r0 + (wv * SRWW + 4 * it_f) * LW);
         if (g > a.G - 1) g = a.G - 1;
         return g;
     };
 
+    // Order of a batch's requests: the first iteration's activation chunk and weight words, then the
+    // scales / zero points, then the other iterations, each activation chunk right ahead of its weight
+    // words.  The first weight request of a wave leaves after a handful of instructions (what stands in
+    // front of it is added to the kernel's duration), and every iteration's operands are complete when its
+    // weight words arrive.
     auto issue = [&](int ib, Batch& b) {
+        b.xvalid = 0;
+        auto pair = [&](int u) __attribute__((always_inline)) {
+            int row = r0 + (lsr0 + 4 * (ib + u)) * LW;
+            if (row <= a.R - LW) b.xvalid |= 1u << u;
+            else row = a.R - LW;  // loads stay in bounds; the activations are zeroed when they are used
+#pragma unroll
+            for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xbase + (int64_t)row * E + 8 * t);
+#pragma unroll
+            for (int v = 0; v < LW; ++v) {
+                int wrow = r0 + (lsr0 + 4 * (ib + u)) * LW + v;
+                if (wrow > a.R - 1) wrow = a.R - 1;
+                b.wr[u * LW + v] = load_streaming_u4(wbase + (int64_t)wrow * a.wsk);
+            }
+        };
         if (fast_meta) {
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
@@ -637,21 +667,8 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
                 }
             }
         }
-        b.xvalid = 0;
 #pragma unroll
-        for (int u = 0; u < IPB; ++u) {
-            int row = r0 + (lsr0 + 4 * (ib + u)) * LW;
-            if (row <= a.R - LW) b.xvalid |= 1u << u;
-            else row = a.R - LW;  // loads stay in bounds; the activations are zeroed when they are used
-#pragma unroll
-            for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xbase + (int64_t)row * E + 8 * t);
-        }
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            int row = r0 + (lsr0 + 4 * (ib + u / LW)) * LW + (u % LW);
-            if (row > a.R - 1) row = a.R - 1;
-            b.wr[u] = load_streaming_u4(wbase + (int64_t)row * a.wsk);
-        }
+        for (int u = 0; u < IPB; ++u) pair(u);
     };
 
     float acc[4][RI];
@@ -908,7 +925,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
 
 template <int BITS, bool BF16, int RT>
 void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
-    dim3 grid(g.tiles * g.S, g.mchunks);
+    dim3 grid(g.tiles, g.mchunks, g.S);
     if constexpr (BITS == 2 || BITS == 4 || BITS == 8) {
         if (g.direct) {
             if (g.nb > 1)
@@ -1048,6 +1065,8 @@ int launch_gemv_packed(const gla_matmul_args& p, hipStream_t stream) {
     }
     a.M = p.M; a.N = p.N; a.K = p.K; a.R = g.R; a.RW = g.RW; a.S = g.S; a.tiles = g.tiles; a.Mp = g.Mp;
     a.gr = g.gr; a.G = g.G; a.GW = g.GW; a.FL = g.FL; a.waves = g.waves; a.nfb = g.nfb;
+    a.srww = g.RW / g.LW / g.waves;
+    a.gr_shift = (g.gr & (g.gr - 1)) == 0 ? __builtin_ctz((unsigned)g.gr) : -1;
     a.fl_log2 = 0;
     while ((1 << a.fl_log2) < g.FL) ++a.fl_log2;
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
