@@ -590,11 +590,12 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     extern __shared__ __align__(16) unsigned char smem[];
     const int nfb = a.nfb;                                        // flush blocks per batch
     const int waves = kWaves ? kWaves : (int)(blockDim.x >> 6);
-    float2* mtw = (float2*)smem + (size_t)(threadIdx.x >> 6) * nfb * kTileN;  // [nfb][64], this wave's
+    const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // wave-uniform, kept in an SGPR
+    float2* mtw = (float2*)smem + (size_t)wv * nfb * kTileN;                  // [nfb][64], this wave's
     float* red = (float*)((float2*)smem + (size_t)waves * nfb * kTileN);      // [waves][RT][64]
     __shared__ unsigned ticket;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wv = tid >> 6;
+    const int lane = tid & 63;
     const int cg = lane & 15, kb = lane >> 4;
     // grid (column tiles, row tiles, K slabs): nothing in front of the first load is divided at run time
     // (the wave's share of the slab and the group size as a shift come from the host)
@@ -605,15 +606,29 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     const int r0 = split * a.RW;
     const int SRWW = a.srww;   // super rows per wave
     const int nit = SRWW / 4;  // wave iterations
-    const int lsr0 = wv * SRWW + kb;
-    const int g0w = div_group(a, r0 + wv * SRWW * LW);  // first group this wave touches
+    const int wrow0 = r0 + wv * SRWW * LW;  // first word row of this wave
+    int g0w = div_group(a, wrow0);          // first group this wave touches
+    if (g0w > a.G - 1) g0w = a.G - 1;
 
     int col = n0 + cg * 4;
     if (col > a.N - 4) col = a.N - 4;  // clamped lanes are never stored
-    const uint32_t* wbase = a.w + col;
     int mrow = m0 + (RT == 16 ? cg : (cg & (RT - 1)));  // rows >= RT of the A operand may hold anything
     if (mrow > a.M - 1) mrow = a.M - 1;
-    const uint16_t* xbase = (const uint16_t*)a.x + (int64_t)mrow * a.xsm;
+    // Every address of the stream is a wave-uniform 64-bit base (scalar arithmetic) plus a 32-bit lane
+    // offset (the host has checked that a wave's span fits): one add and one clamp per load.  With 64-bit
+    // products per load, the address arithmetic of the four waves of a SIMD stood in front of the later
+    // loads of each for several hundred cycles.
+    const uint32_t sb = (uint32_t)a.wsk * 4u;  // bytes between word rows
+    const char* ws_base = (const char*)a.w + (int64_t)(wrow0 < a.R - 1 ? wrow0 : a.R - 1) * a.wsk * 4;
+    const uint32_t w_lane = (uint32_t)col * 4u + (uint32_t)(kb * LW) * sb;
+    const uint32_t w_lim = (uint32_t)col * 4u + (uint32_t)(wrow0 < a.R - 1 ? a.R - 1 - wrow0 : 0) * sb;
+    const int x_rel_max = a.R - LW - wrow0;  // rows this wave may still multiply (negative: none)
+    const char* xs_base = (const char*)a.x + (int64_t)(x_rel_max > 0 ? wrow0 : a.R - LW) * (E * 2);
+    const uint32_t x_lane0 = (uint32_t)mrow * (uint32_t)a.xsm * 2u;
+    const uint32_t x_lane = x_lane0 + (uint32_t)(kb * LW * E * 2);
+    const uint32_t x_lim = x_lane0 + (uint32_t)(x_rel_max > 0 ? x_rel_max : 0) * (uint32_t)(E * 2);
+    const char* ss_base = (const char*)a.scales + (int64_t)g0w * a.msg * 2;
+    const char* zs_base = (const char*)a.zeros + (int64_t)g0w * a.msg * 2;
     const bool fast_meta = (a.meta_dt == GLA_DT_FP16 || a.meta_dt == GLA_DT_BF16) && !a.z_scalar &&
                            (a.z_dt == a.meta_dt) && a.wgm >= GLA_WGM_SHIFT_SCALE;
 
@@ -627,7 +642,7 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     // group (relative to g0w) whose fold closes flush block `fbl` of the batch starting at iteration ib
     auto block_group = [&](int ib, int fbl) {
         const int it_f = (a.FL <= IPB) ? (ib + (fbl + 1) * a.FL - 1) : (ib + IPB - 1);
-        int g = div_group(a, r0 + (wv * SRWW + 4 * it_f) * LW);
+        int g = div_group(a, wrow0 + 4 * it_f * LW);
         if (g > a.G - 1) g = a.G - 1;
         return g;
     };
@@ -640,16 +655,16 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     auto issue = [&](int ib, Batch& b) {
         b.xvalid = 0;
         auto pair = [&](int u) __attribute__((always_inline)) {
-            int row = r0 + (lsr0 + 4 * (ib + u)) * LW;
-            if (row <= a.R - LW) b.xvalid |= 1u << u;
-            else row = a.R - LW;  // loads stay in bounds; the activations are zeroed when they are used
+            uint32_t xo = x_lane + (uint32_t)(4 * (ib + u) * LW * E * 2);
+            if (x_rel_max >= 0 && xo <= x_lim) b.xvalid |= 1u << u;
+            else xo = x_lim;  // loads stay in bounds; the activations are zeroed when they are used
 #pragma unroll
-            for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xbase + (int64_t)row * E + 8 * t);
+            for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xs_base + xo + 16 * t);
 #pragma unroll
             for (int v = 0; v < LW; ++v) {
-                int wrow = r0 + (lsr0 + 4 * (ib + u)) * LW + v;
-                if (wrow > a.R - 1) wrow = a.R - 1;
-                b.wr[u * LW + v] = load_streaming_u4(wbase + (int64_t)wrow * a.wsk);
+                uint32_t wo = w_lane + (uint32_t)(4 * (ib + u) * LW + v) * sb;
+                if (wo > w_lim) wo = w_lim;
+                b.wr[u * LW + v] = load_streaming_u4((const uint32_t*)(ws_base + wo));
             }
         };
         if (fast_meta) {
@@ -662,8 +677,9 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
                 int n = n0 + (item & 15) * 4;
                 if (n > a.N - 4) n = a.N - 4;
                 if (p == 0 || nfb > 4) {
-                    b.sr[p] = load_streaming_u2((const uint16_t*)a.scales + (int64_t)g * a.msg + n);
-                    b.zr[p] = load_streaming_u2((const uint16_t*)a.zeros + (int64_t)g * a.msg + n);
+                    const uint32_t mo = (uint32_t)(g - g0w) * ((uint32_t)a.msg * 2u) + (uint32_t)n * 2u;
+                    b.sr[p] = load_streaming_u2((const uint16_t*)(ss_base + mo));
+                    b.zr[p] = load_streaming_u2((const uint16_t*)(zs_base + mo));
                 }
             }
         }
@@ -915,6 +931,15 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
         }
     }
     g.S = ceil_div(g.R, g.RW);
+    if (g.direct) {
+        // the direct variant addresses with a 64-bit base per wave plus 32-bit lane offsets
+        const int64_t lim = (int64_t)1 << 31;
+        const int64_t w_span = (int64_t)p.w_stride_k * 4 * (g.RW / g.waves) + (int64_t)p.N * 4;
+        const int64_t x_span = (int64_t)p.x_stride_m * 2 * 16 + (int64_t)p.K * 2;
+        const int64_t m_span = (int64_t)p.meta_stride_g * 2 * g.GW + (int64_t)p.N * 2;
+        if (p.w_stride_k < 0 || p.x_stride_m < 0 || p.meta_stride_g < 0 || w_span >= lim || x_span >= lim || m_span >= lim)
+            return geometry(p, g, false);
+    }
     // 8-bit codes with bf16 activations exist only in the direct variant (nibble-split MFMAs)
     const bool split8 = p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16;
     if (split8 && !g.direct) return false;
