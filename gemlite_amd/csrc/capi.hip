@@ -208,6 +208,17 @@ Family choose(const gla_matmul_args& p, int type) {
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
     }
+    // Above 16 rows the streaming GEMV still runs, as row chunks of 16 that each stream the weights again (the later
+    // chunks mostly from L2).  It is the only fast kernel for packed layers the tiled GEMM does not take (1-bit codes,
+    // groups of 32, K not a multiple of 64), and up to 64 rows it beats the tiled GEMM on small and medium layers,
+    // where that one cannot fill the chip without a deep K split (4096^2 4-bit at 32 rows: 9 against 17 us; 8192^2:
+    // 22 against 26 us; 16384^2: 69 against 56 us, so large layers stay with the GEMM).
+    if (p.M > 16 && gemv_packed_eligible(p)) {
+        if (!gemm_wn_eligible(p)) return F_GEMV_PACKED;
+        const int64_t chunks = (p.M + 15) / 16;
+        const int64_t restreamed = chunks * (int64_t)p.N * p.K * (p.W_nbits < 4 ? 4 : p.W_nbits) / 8;  // 2-bit codes cost what 4-bit ones do
+        if (p.tile_config <= 0 && chunks <= 4 && restreamed <= (chunks == 4 ? 48 : 96) * (int64_t)1000000) return F_GEMV_PACKED;
+    }
     if (gemm_wn_eligible(p)) return F_GEMM_WN;
     if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // also streams K-major 8-bit operands at small M (split-K)
     if (gemm_kbytes_eligible(p)) return F_GEMM_KBYTES;

@@ -66,7 +66,7 @@ def test_streaming_split_k_twice(device):
 
 def test_gemm_split_k_twice(device):
     """Packed-code MFMA GEMM at a batch small enough that K is split over workgroups (fp32 partials)."""
-    for (N, K, M, seed) in ((4096, 4096, 40, 3), (2048, 2048, 20, 4)):
+    for (N, K, M, seed) in ((4096, 4096, 100, 3), (2048, 2048, 70, 4)):   # above 64 rows: the tiled GEMM
         print(f"case: static scratch, gemm_wn N={N} K={K} M={M}", flush=True)
         W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16, seed=seed)
         layer = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
