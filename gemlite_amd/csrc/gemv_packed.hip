@@ -844,7 +844,7 @@ struct Geometry {
 };
 
 // tile_config encoding: (waves per workgroup) * 1000 + (batches of kBatch loads per wave).
-bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
+bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true, int rt_cap = 16) {
     g.E = 32 / p.W_nbits;
     g.LW = g.E < 8 ? 8 / g.E : 1;
     g.KPS = g.E * g.LW;
@@ -852,6 +852,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
     g.R = p.K / g.E;
     g.tiles = ceil_div(p.N, kTileN);
     g.RT = row_tile(p.M);
+    if (g.RT > rt_cap) g.RT = rt_cap;
     g.mchunks = ceil_div(p.M, g.RT);
     g.Mp = g.mchunks * g.RT;
     const bool grouped = p.W_group_mode >= GLA_WGM_SCALE || (p.W_group_mode == GLA_WGM_SHIFT && !p.zero_is_scalar);
@@ -929,6 +930,9 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
         } else if (waves > 4) {
             waves = waves > 8 ? 8 : 4;
         } else {
+            // the staged 16-row tile of 1-bit codes does not fit the LDS at any wave count (its activation
+            // chunk alone is 1 KiB per super row): more rows than 4 then run as chunks of 4
+            if (g.RT == 16) return geometry(p, g, allow_direct, 4);
             return false;
         }
     }
@@ -940,7 +944,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true) {
         const int64_t x_span = (int64_t)p.x_stride_m * 2 * 16 + (int64_t)p.K * 2;
         const int64_t m_span = (int64_t)p.meta_stride_g * 2 * g.GW + (int64_t)p.N * 2;
         if (p.w_stride_k < 0 || p.x_stride_m < 0 || p.meta_stride_g < 0 || w_span >= lim || x_span >= lim || m_span >= lim)
-            return geometry(p, g, false);
+            return geometry(p, g, false, rt_cap);
     }
     // 8-bit codes with bf16 activations exist only in the direct variant (nibble-split MFMAs)
     const bool split8 = p.W_nbits == 8 && p.input_dtype == GLA_DT_BF16;
