@@ -183,14 +183,17 @@ int validate(const gla_matmul_args* p) {
 Family choose(const gla_matmul_args& p, int type) {
     if (p.input_dtype == GLA_DT_MXFP4) {
         // decode sizes: the streaming kernel (weights read once, straight into registers) beats the split-K matrix-core
-        // path, whose tiles are at least 64 rows tall
-        if (p.M <= kMxStreamRows && p.tile_config < 1000 && mx_stream_eligible(p)) return F_MX_STREAM;
+        // path, whose tiles are at least 64 rows tall: up to 2 rows everywhere, up to 4 on layers of 40 MB or less
+        // (4096^2 at 4 rows: 10.7 against 14.4 us; 8192^2: 20.2 against 20.5; 16384^2: 54 against 40)
+        const int rows = (int64_t)p.N * p.K / 2 <= 40000000 ? 4 : kMxStreamRows;
+        if (p.M <= rows && p.tile_config < 1000 && mx_stream_eligible(p)) return F_MX_STREAM;
         return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
     }
     if (p.input_dtype == GLA_DT_MXFP8) {  // validated: eligible for one of the two at least
-        // MXFP4 weights under fp8 activations: up to 2 rows the streaming kernel is the faster one (16384^2, M=2: 33
-        // against 42 us; M=3: 47 against 42 us)
-        if (p.elements_per_sample == 2 && p.M <= 2 && mx_stream_eligible(p)) return F_MX_STREAM;
+        // fp8 activations on MXFP8 or MXFP4 weights: up to 4 rows the streaming kernel is the faster one at every size
+        // (MXFP8 weights, one row: 4096^2 7.9 against 25 us, 16384^2 59 against 84; 4 rows: 13.4 against 25, 79 against
+        // 83.  MXFP4 weights, 4 rows: 4096^2 10.4 against 19.8, 16384^2 52 against 54; 6 rows: 85 against 54)
+        if (p.M <= 4 && p.tile_config < 1000 && mx_stream_eligible(p)) return F_MX_STREAM;
         return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;
     }
     if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)  // validated as eligible for the streaming kernel

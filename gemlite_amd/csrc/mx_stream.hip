@@ -20,10 +20,10 @@
 // dot instruction; the block's partial sum is then scaled once by the product of its two block
 // scales, as the scaled matrix instruction does.  A shuffle tree sums the lanes.
 //
-// This is the decode path of every micro-scaled layer: MXFP4 x MXFP4, weight-only MX layers and fp8
-// activations x MXFP4 weights up to 2 rows (above that the matrix-core kernels are faster: the
-// conversions and dot products here cost vector-unit time per row), fp8 x MXFP8 never;
-// and the path at any batch size for a K that the matrix-core kernels do not take (not tuned above
+// This is the decode path of every micro-scaled layer: weight-only MX layers up to 2 rows, MXFP4 x
+// MXFP4 up to 2 rows (4 on layers of 40 MB or less), fp8 activations on MXFP4 or MXFP8 weights up to
+// 4 rows (above that the matrix-core kernels are faster: the conversions and dot products here cost
+// vector-unit time per row); and the path at any batch size for a K that the matrix-core kernels do not take (not tuned above
 // a few rows: every group of eight activation rows streams the weights again).
 #include "common.hpp"
 #include "dispatch.hpp"
