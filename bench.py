@@ -288,7 +288,14 @@ def extra_points(lib, device, T, quick):
         fns = [(lambda xi=xi: _ext.scale_activations_per_token(xi, xq_o, sx_o)) for xi in xs]
         us = T.graph_us(fns, 6)
         out[f"actquant_per_token_{name}"] = bw_point(us, M * K * 3 + M * 4, M=M, K=K, copies=len(xs))
-        del layer, xq, sx, run
+        # decode: one row through the K-major streaming kernel (8-bit activations), weights rotated
+        wbytes = N * K + N * 4
+        layers = [layer] + [clone_layer(layer) for _ in range(copies_for(wbytes) - 1)]
+        xq1, sx1 = gemlite_amd.scale_activations_per_token(x[:1].contiguous(), wdt)
+        y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
+        us = T.graph_us([Launch(lib, l, xq1, y1, device, scales_x=sx1) for l in layers], 6)
+        out[f"gemv_a8w8_{name}_M1"] = bw_point(us, wbytes + K + 4 + N * 2, N=N, K=K, copies=len(layers))
+        del layer, layers, xq, sx, run, xq1, sx1
     # MXFP8 weights, fp8 activations quantised per token (the reference processor's default)
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
     lin.weight.data = W

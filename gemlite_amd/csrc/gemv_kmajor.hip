@@ -1,7 +1,9 @@
 // Streaming GEMV / skinny GEMM (1..16 rows) for fp16/bf16 activations x unpacked 8-bit weights kept
 // as the [K, N] view of an [N, K] array (K contiguous): int8, uint8 or fp8-e4m3 codes with
 // per-channel scales (and optionally a zero point).  The decode path of weight-only A16W8 layers
-// whose weights are not packed into 32-bit words.
+// whose weights are not packed into 32-bit words.  The vector variant also takes fp8 x fp8 and int8 x int8
+// operands (dynamically quantised A8W8 layers, per-token times per-channel scales) up to 4 rows, where
+// the matrix-core GEMM with its split-K finishing launch costs twice the time on small layers.
 //
 // Takes the place of the reference's split-K GEMV for one element per sample (reference:
 // gemlite/triton_kernels/gemv_splitK_kernels.py:257-542; dequant gemlite/triton_kernels/utils.py:73-105;
@@ -34,6 +36,7 @@ constexpr int kRowsK = 4;    // weight rows per workgroup
 constexpr int kWavesK = 4;   // waves per workgroup, interleaved over K
 constexpr int kLaneK = 16;   // K-values per lane and iteration
 constexpr int kIterK = 64 * kLaneK;
+constexpr int kRows8 = 4;    // rows up to which 8-bit activations are taken (vector variant)
 
 struct GemvKArgs {
     const uint16_t* x;
@@ -74,6 +77,9 @@ __device__ __forceinline__ void codes_to_float(const u32x4k& v, float (&f)[16]) 
     }
 }
 
+// activation kinds of the vector variant
+constexpr int kXF16 = 0, kXBF16 = 1, kXFP8 = 2, kXI8 = 3;
+
 template <bool BF16>
 __device__ __forceinline__ void acts_to_float(const u32x4k& a, const u32x4k& b, float (&f)[16]) {
 #pragma unroll
@@ -94,10 +100,18 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
 }
+__device__ __forceinline__ int wave_sum_int(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
 
-// MT: rows of x handled (power of two >= M)
-template <int WDT, bool BF16, int MT>
+// MT: rows of x handled (power of two >= M).  XK: activation kind.  int8 x int8 sums exactly: a lane's fp32
+// sums stay below 2^24 (the host bounds K), the sums over lanes and waves are taken in int32.
+template <int WDT, int XK, int MT>
 __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) {
+    constexpr bool X8 = XK == kXFP8 || XK == kXI8;
+    constexpr bool EXACT = XK == kXI8;
     __shared__ float red[kWavesK][kRowsK * MT + MT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * kRowsK;
@@ -107,9 +121,9 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
         const int n = n0 + r < a.N ? n0 + r : a.N - 1;  // rows past the end repeat the last one; never stored
         wrow[r] = a.w + (int64_t)n * a.wsn;
     }
-    const uint16_t* xrow[MT];
+    const uint8_t* xrow[MT];  // x_stride_m counts stored elements
 #pragma unroll
-    for (int m = 0; m < MT; ++m) xrow[m] = a.x + (int64_t)(m < a.M ? m : a.M - 1) * a.xsm;
+    for (int m = 0; m < MT; ++m) xrow[m] = (const uint8_t*)a.x + (int64_t)(m < a.M ? m : a.M - 1) * a.xsm * (X8 ? 1 : 2);
 
     float acc[kRowsK][MT], sumx[MT];
 #pragma unroll
@@ -128,9 +142,17 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
         for (int r = 0; r < kRowsK; ++r) codes_to_float<WDT>(wv[r], wf[r]);
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const u32x4k xa = *(const u32x4k*)(xrow[m] + k), xb = *(const u32x4k*)(xrow[m] + k + 8);
             float xf[16];
-            acts_to_float<BF16>(xa, xb, xf);
+            if constexpr (XK == kXFP8) {
+                codes_to_float<GLA_DT_FP8>(*(const u32x4k*)(xrow[m] + k), xf);
+            } else if constexpr (XK == kXI8) {
+                codes_to_float<GLA_DT_INT8>(*(const u32x4k*)(xrow[m] + k), xf);  // biased by +128
+#pragma unroll
+                for (int q = 0; q < 16; ++q) xf[q] -= 128.0f;
+            } else {
+                const u32x4k xa = *(const u32x4k*)(xrow[m] + 2 * k), xb = *(const u32x4k*)(xrow[m] + 2 * k + 16);
+                acts_to_float<XK == kXBF16>(xa, xb, xf);
+            }
 #pragma unroll
             for (int q = 0; q < 16; ++q) {
                 sumx[m] += xf[q];
@@ -143,12 +165,22 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     // sums over the lanes of the wave, then over the waves in fixed order
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        const float sx = wave_sum(sumx[m]);
-        if (lane == 0) red[wave][kRowsK * MT + m] = sx;
+        if constexpr (EXACT) {
+            const int sx = wave_sum_int((int)sumx[m]);
+            if (lane == 0) red[wave][kRowsK * MT + m] = __builtin_bit_cast(float, sx);
 #pragma unroll
-        for (int r = 0; r < kRowsK; ++r) {
-            const float d = wave_sum(acc[r][m]);
-            if (lane == 0) red[wave][r * MT + m] = d;
+            for (int r = 0; r < kRowsK; ++r) {
+                const int d = wave_sum_int((int)acc[r][m]);
+                if (lane == 0) red[wave][r * MT + m] = __builtin_bit_cast(float, d);
+            }
+        } else {
+            const float sx = wave_sum(sumx[m]);
+            if (lane == 0) red[wave][kRowsK * MT + m] = sx;
+#pragma unroll
+            for (int r = 0; r < kRowsK; ++r) {
+                const float d = wave_sum(acc[r][m]);
+                if (lane == 0) red[wave][r * MT + m] = d;
+            }
         }
     }
     __syncthreads();
@@ -157,12 +189,24 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     const int r = t / MT, m = t % MT, n = n0 + r;
     if (n >= a.N || m >= a.M) return;
     float D = 0.0f, X = 0.0f;
+    if constexpr (EXACT) {
+        int Di = 0, Xi = 0;
 #pragma unroll
-    for (int w = 0; w < kWavesK; ++w) {
-        D += red[w][r * MT + m];
-        X += red[w][kRowsK * MT + m];
+        for (int w = 0; w < kWavesK; ++w) {
+            Di += __builtin_bit_cast(int, red[w][r * MT + m]);
+            Xi += __builtin_bit_cast(int, red[w][kRowsK * MT + m]);
+        }
+        if (WDT == GLA_DT_INT8) Di -= 128 * Xi;  // undo the bias of the byte conversion
+        D = (float)Di;                            // the int32 accumulator of the reference, converted once
+        X = (float)Xi;
+    } else {
+#pragma unroll
+        for (int w = 0; w < kWavesK; ++w) {
+            D += red[w][r * MT + m];
+            X += red[w][kRowsK * MT + m];
+        }
+        if (WDT == GLA_DT_INT8) D = __builtin_fmaf(-128.0f, X, D);  // undo the bias of the byte conversion
     }
-    if (WDT == GLA_DT_INT8) D = __builtin_fmaf(-128.0f, X, D);  // undo the bias of the byte conversion
     const bool uses_s = a.wgm >= GLA_WGM_SCALE;
     const bool uses_z = a.wgm == GLA_WGM_SHIFT || a.wgm >= GLA_WGM_SHIFT_SCALE;
     const float s = uses_s ? load_as_float(a.scales, a.meta_dt, (int64_t)n * a.msn) : 1.0f;
@@ -340,12 +384,23 @@ int launch_k(const GemvKArgs& a, hipStream_t stream) {
             hipLaunchKernelGGL((gemv_kmajor_mfma_kernel<WDT, BF16, 1>), dim3(ceil_div(a.N, 16)), dim3(kWavesKM * 64), 0, stream, a);
         return check_hip(hipGetLastError(), "gemv_kmajor launch");
     }
+    constexpr int XK = BF16 ? kXBF16 : kXF16;
     const dim3 grid(ceil_div(a.N, kRowsK)), block(kWavesK * 64);
-    if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, BF16, 1>), grid, block, 0, stream, a);
-    else if (a.M == 2) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, BF16, 2>), grid, block, 0, stream, a);
-    else if (a.M <= 4) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, BF16, 4>), grid, block, 0, stream, a);
-    else if (a.M <= 8) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, BF16, 8>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, BF16, 16>), grid, block, 0, stream, a);
+    if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 1>), grid, block, 0, stream, a);
+    else if (a.M == 2) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 2>), grid, block, 0, stream, a);
+    else if (a.M <= 4) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 4>), grid, block, 0, stream, a);
+    else if (a.M <= 8) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 8>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 16>), grid, block, 0, stream, a);
+    return check_hip(hipGetLastError(), "gemv_kmajor launch");
+}
+
+// 8-bit activations of the weights' own type (fp8 x fp8, int8 x int8), up to 4 rows
+template <int WDT, int XK>
+int launch_k8(const GemvKArgs& a, hipStream_t stream) {
+    const dim3 grid(ceil_div(a.N, kRowsK)), block(kWavesK * 64);
+    if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 1>), grid, block, 0, stream, a);
+    else if (a.M == 2) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 2>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 4>), grid, block, 0, stream, a);
     return check_hip(hipGetLastError(), "gemv_kmajor launch");
 }
 
@@ -355,12 +410,25 @@ bool gemv_kmajor_eligible(const gla_matmul_args& p) {
     if (p.M < 1 || p.M > 16) return false;
     if (p.W_nbits != 8 || p.elements_per_sample != 1) return false;
     if (!(p.w_dtype == GLA_DT_INT8 || p.w_dtype == GLA_DT_UINT8 || p.w_dtype == GLA_DT_FP8)) return false;
-    if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16) || p.acc_dtype != GLA_DT_FP32) return false;
+    const bool x8 = (p.input_dtype == GLA_DT_FP8 && p.w_dtype == GLA_DT_FP8 && p.acc_dtype == GLA_DT_FP32) ||
+                    (p.input_dtype == GLA_DT_INT8 && p.w_dtype == GLA_DT_INT8 &&
+                     (p.acc_dtype == GLA_DT_INT32 || p.acc_dtype == GLA_DT_FP32));
+    if (x8) {
+        // the vector variant only; a lane's fp32 sum of |x| <= 128 times a biased code <= 255 over K / 256 values
+        // must stay below 2^24 for the int8 sums to be exact
+        if (p.M > kRows8 || p.K > 131072 || p.x_stride_m % 16 != 0) return false;
+        // 3 and 4 rows only on layers of 20 MB or less (4096^2: 13 against 15 us for the matrix-core GEMM and its
+        // finishing launch; 8192^2: 29 against 21); 1 and 2 rows everywhere (4096^2 6.7 against 14.7, 8192^2 15.6
+        // against 21.6 us)
+        if (p.M > 2 && (int64_t)p.N * p.K > 20000000) return false;
+    } else if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16) || p.acc_dtype != GLA_DT_FP32) {
+        return false;
+    }
     if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
     if (p.W_group_mode < GLA_WGM_NONE || p.W_group_mode > GLA_WGM_FMA) return false;
     if (p.channel_scale_mode < GLA_CSM_NONE || p.channel_scale_mode > GLA_CSM_BOTH) return false;
     if (p.w_stride_k != 1 || p.x_stride_k != 1 || p.out_stride_n != 1) return false;
-    if (p.K % kLaneK != 0 || p.w_stride_n % 16 != 0 || p.x_stride_m % 8 != 0) return false;
+    if (p.K % kLaneK != 0 || p.w_stride_n % 16 != 0 || (!x8 && p.x_stride_m % 8 != 0)) return false;
     if (((uintptr_t)p.w & 15) || ((uintptr_t)p.x & 15)) return false;
     const bool uses_s = p.W_group_mode >= GLA_WGM_SCALE;
     const bool uses_z = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
@@ -381,6 +449,8 @@ int launch_gemv_kmajor(const gla_matmul_args& p, hipStream_t stream) {
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.z_scalar = p.zero_is_scalar; a.out_dt = p.output_dtype; a.sx_dt = p.sx_dtype;
     a.bias = p.bias; a.bias_dt = p.bias_dtype;
+    if (p.input_dtype == GLA_DT_FP8) return launch_k8<GLA_DT_FP8, kXFP8>(a, stream);
+    if (p.input_dtype == GLA_DT_INT8) return launch_k8<GLA_DT_INT8, kXI8>(a, stream);
     const bool bf16 = p.input_dtype == GLA_DT_BF16;
     switch (p.w_dtype) {
         case GLA_DT_INT8: return bf16 ? launch_k<GLA_DT_INT8, true>(a, stream) : launch_k<GLA_DT_INT8, false>(a, stream);

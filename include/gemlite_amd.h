@@ -162,7 +162,7 @@ int gla_select_config(const gla_matmul_args* args);
  * gemlite/core.py:57-67); here several families serve one type, and tests and tuners ask which. */
 #define GLA_FAMILY_GENERIC 0      /* layout-agnostic kernel, any mode and stride */
 #define GLA_FAMILY_GEMV_PACKED 1  /* streaming kernels for 32-bit packed codes: up to 16 rows, up to 64 on small layers */
-#define GLA_FAMILY_GEMV_KMAJOR 2
+#define GLA_FAMILY_GEMV_KMAJOR 2  /* streaming kernels for K-major weight bytes: 16-bit activations up to 16 rows, fp8 / int8 ones up to 4 */
 #define GLA_FAMILY_GEMM_WN 3      /* fused-dequant MFMA GEMM for packed 2/4/8-bit codes */
 #define GLA_FAMILY_GEMM_8BIT 4    /* fp8 / int8 MFMA GEMM on K-major operands */
 #define GLA_FAMILY_GEMM_MXFP4 5   /* block-scaled FP4 MFMA GEMM */

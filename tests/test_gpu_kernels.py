@@ -336,6 +336,53 @@ def test_a8w8_dynamic(device, fp8):
         check_layer(layer, gen_x(M, K, torch.bfloat16, seed=M).to(device), torch.bfloat16)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_a8w8_dynamic_streams_the_first_rows(device, fp8):
+    """Dynamically quantised A8W8 layers at 1-2 rows (3-4 on small layers) take the K-major streaming kernel with
+    8-bit activations, the matrix-core GEMM above.  Ragged N (last workgroup has 2 of 4 columns), K that does not
+    fill the waves' last sweep, and the exact int32 sums of int8 x int8 against an int64 reference."""
+    import ctypes
+    from gemlite_amd import _ext
+    N, K = 1030, 4160
+    W = gen_x(N, K, torch.bfloat16, seed=15, std=0.02)
+    proc = helper.A8W8_FP8_dynamic(device=device) if fp8 else helper.A8W8_INT8_dynamic(device=device)
+    W_q_cpu, s_cpu = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+    proc.dtype = torch.bfloat16
+    layer = proc.from_weights(W_q_cpu, scales=s_cpu)
+    for M, fam in ((1, "GEMV_KMAJOR"), (2, "GEMV_KMAJOR"), (3, "GEMV_KMAJOR"), (4, "GEMV_KMAJOR"), (5, "GEMM_8BIT")):
+        x = gen_x(M, K, torch.bfloat16, seed=20 + M).to(device)
+        xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn if fp8 else torch.int8)
+        m = layer.get_meta_args()
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+        a = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, out, W_nbits=m[1], group_size=m[2],
+                                   unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                   acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                   data_contiguous=m[11])
+        assert _ext.matmul_family(a) == fam
+        check_layer(layer, x, torch.bfloat16)
+        if not fp8 and M <= 4:
+            # fp32 output: every element is float(int32 sum) * (s_w * s_x), the sum exact
+            y32 = torch.empty(M, N, dtype=torch.float32, device=device)
+            a32 = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, y32, W_nbits=m[1], group_size=m[2],
+                                         unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=DType.FP32.value,
+                                         acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                         data_contiguous=m[11])
+            assert _ext.matmul_family(a32) == "GEMV_KMAJOR"
+            rc = _ext.load_library().gla_matmul(ctypes.byref(a32), torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+            torch.cuda.synchronize()
+            acc = xq.cpu().to(torch.int64) @ layer.W_q.t().contiguous().cpu().to(torch.int64).t()
+            want = acc.to(torch.float32) * (layer.scales.cpu().reshape(1, N).float() * sx.cpu().reshape(M, 1).float())
+            assert torch.equal(y32.cpu(), want)
+    # a larger layer hands over at 3 rows
+    N2, K2 = 5120, 4096
+    W2 = gen_x(N2, K2, torch.bfloat16, seed=16, std=0.02)
+    l2 = proc.from_weights(*gemlite_amd.quantize_weights_per_channel(W2, torch.float8_e4m3fn if fp8 else torch.int8)[:1],
+                           scales=gemlite_amd.quantize_weights_per_channel(W2, torch.float8_e4m3fn if fp8 else torch.int8)[1])
+    for M in (2, 3):
+        check_layer(l2, gen_x(M, K2, torch.bfloat16, seed=30 + M).to(device), torch.bfloat16)
+
+
 def test_int8_activations_packed_weights(device):
     # int8 x 4-bit with an integer zero and channel-wise scales (reference: tests/test_int.py:146-171)
     N, K = 400, 1024

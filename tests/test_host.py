@@ -343,9 +343,9 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
     Wb = torch.randn(N, K, generator=g).bfloat16() * 0.02
     for proc, dt in ((gemlite_amd.helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), (gemlite_amd.helper.A8W8_INT8_dynamic, torch.int8)):
         la = proc(device="cpu").from_weights(Wb)
-        for M in (1, 4096):
+        for M, fam in ((1, "GEMV_KMAJOR"), (4, "GEMV_KMAJOR"), (5, "GEMM_8BIT"), (4096, "GEMM_8BIT")):  # streaming up to 4 rows
             xq = torch.zeros(M, K, dtype=dt)
-            assert _family(la, M, None, scales_x=torch.ones(M, 1), x=xq) == "GEMM_8BIT"
+            assert _family(la, M, None, scales_x=torch.ones(M, 1), x=xq) == fam
     # MXFP4
     codes = torch.randint(0, 16, (N, K), generator=g).to(torch.uint8)
     e8 = torch.randint(110, 130, (N, K // 32), generator=g).to(torch.uint8)
