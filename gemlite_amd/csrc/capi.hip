@@ -232,6 +232,53 @@ int resolve_type(const gla_matmul_args& p) {
     return p.matmul_type == GLA_MATMUL_AUTO ? matmul_type_for(p.M, p.W_nbits, is_mx(p.input_dtype)) : p.matmul_type;
 }
 
+int64_t family_workspace(Family f, const gla_matmul_args& a) {
+    switch (f) {
+        case F_GEMV_PACKED: return gemv_packed_workspace_bytes(a);
+        case F_GEMM_WN: return gemm_wn_workspace_bytes(a);
+        case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(a);
+        case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(a);
+        case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(a);
+        case F_GEMM_BLOCKQ: return gemm_blockq_workspace_bytes(a);
+        case F_GEMM_KBYTES_MX: return gemm_kbytes_mx_workspace_bytes(a);
+        default: return 0;
+    }
+}
+
+// fp8 / int8 activations on 32-bit packed codes (the reference's A8Wn_HQQ_INT_dynamic and A8W158_INT_dynamic
+// processors): no kernel of their own.  Both types convert to fp16 exactly, so the activations are widened into
+// the workspace by a small launch and the 16-bit kernels run on them, per-token scales in their epilogue.  An int32
+// accumulator asked for stays exact: the tiled GEMM's fp32 sums of integer products are exact below 2^24, and the
+// streaming kernel folds its offset sums every 64 K-values for such a call (gemv_packed.hip::geometry).
+struct Widened {
+    gla_matmul_args q;   // the call the 16-bit kernel sees (x and workspace filled in at launch)
+    Family f;
+    int64_t x_off;       // where the fp16 activations go in the workspace
+    int64_t x_stride;    // their row stride in elements
+    int64_t total;       // workspace bytes of the whole call
+};
+
+bool widen(const gla_matmul_args& p, Widened& w) {
+    if (!(p.input_dtype == GLA_DT_FP8 || p.input_dtype == GLA_DT_INT8) || p.w_dtype != GLA_DT_INT32) return false;
+    if (p.x_stride_k != 1 || !(p.acc_dtype == GLA_DT_FP32 || p.acc_dtype == GLA_DT_INT32)) return false;
+    if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
+    w.q = p;
+    w.q.input_dtype = GLA_DT_FP16;
+    w.x_stride = (p.K + 7) / 8 * 8;
+    w.q.x_stride_m = w.x_stride;
+    w.q.x = (const void*)(uintptr_t)256;  // stands for an aligned pointer while the kernels' rules are asked
+    w.q.workspace = nullptr;
+    w.q.workspace_bytes = 0;
+    w.f = choose(w.q, resolve_type(w.q));
+    if (!(w.f == F_GEMV_PACKED || w.f == F_GEMM_WN)) return false;
+    const int64_t inner = family_workspace(w.f, w.q);
+    if (inner < 0) return false;
+    // the first kWsPrivateBytes hold the streaming kernels' ticket counters and slots, whoever runs
+    w.x_off = ((inner > kWsPrivateBytes ? inner : kWsPrivateBytes) + 255) / 256 * 256;
+    w.total = w.x_off + (int64_t)p.M * w.x_stride * 2;
+    return true;
+}
+
 }  // namespace
 }  // namespace gla
 
@@ -252,6 +299,8 @@ int gla_select_config(const gla_matmul_args* args) {
     if (rc != GLA_OK) return rc;
     const Family f = choose(*args, resolve_type(*args));
     if (f == F_GEMV_PACKED) return gemv_packed_default_config(*args);
+    Widened w;
+    if (f == F_GENERIC && widen(*args, w) && w.f == F_GEMV_PACKED) return gemv_packed_default_config(w.q);
     return 0;
 }
 
@@ -266,23 +315,20 @@ int gla_probe_read(const void* buf, int64_t bytes, void* sink, void* stream) {
 int gla_matmul_family(const gla_matmul_args* args) {
     const int rc = validate(args);
     if (rc != GLA_OK) return rc;
-    return (int)choose(*args, resolve_type(*args));
+    const Family f = choose(*args, resolve_type(*args));
+    Widened w;
+    if (f == F_GENERIC && widen(*args, w)) return (int)w.f;  // the kernel that runs on the widened activations
+    return (int)f;
 }
 
 int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
     const int rc = validate(args);
     if (rc != GLA_OK) return rc;
     if (args->M == 0) return 0;
-    switch (choose(*args, resolve_type(*args))) {
-        case F_GEMV_PACKED: return gemv_packed_workspace_bytes(*args);
-        case F_GEMM_WN: return gemm_wn_workspace_bytes(*args);
-        case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(*args);
-        case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(*args);
-        case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(*args);
-        case F_GEMM_BLOCKQ: return gemm_blockq_workspace_bytes(*args);
-        case F_GEMM_KBYTES_MX: return gemm_kbytes_mx_workspace_bytes(*args);
-        default: return 0;
-    }
+    const Family f = choose(*args, resolve_type(*args));
+    Widened w;
+    if (f == F_GENERIC && widen(*args, w)) return w.total;
+    return family_workspace(f, *args);
 }
 
 int gla_matmul(const gla_matmul_args* args, void* stream) {
@@ -290,7 +336,22 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
     if (rc != GLA_OK) return rc;
     if (args->M == 0) return GLA_OK;
     hipStream_t s = (hipStream_t)stream;
-    const Family f = choose(*args, resolve_type(*args));
+    Family f = choose(*args, resolve_type(*args));
+    Widened w;
+    if (f == F_GENERIC && widen(*args, w)) {
+        if (args->workspace == nullptr || (int64_t)args->workspace_bytes < w.total) {
+            set_error("matmul: workspace of %lld bytes required (8-bit activations are widened into it), %llu given",
+                      (long long)w.total, (unsigned long long)args->workspace_bytes);
+            return GLA_ERR_WORKSPACE_TOO_SMALL;
+        }
+        void* x16 = (char*)args->workspace + w.x_off;
+        const int rcw = launch_widen_x8(args->x, args->x_stride_m, args->M, args->K, args->input_dtype, x16, w.x_stride, s);
+        if (rcw != GLA_OK) return rcw;
+        w.q.x = x16;
+        w.q.workspace = args->workspace;
+        w.q.workspace_bytes = (uint64_t)w.x_off;
+        return w.f == F_GEMV_PACKED ? launch_gemv_packed(w.q, s) : launch_gemm_wn(w.q, s);
+    }
     int rc2;
     switch (f) {
         // Every family adds the bias in its epilogue or split-K finishing kernel (the `return`s) except the byte-weight

@@ -9,6 +9,8 @@ namespace gla {
 int launch_generic(const gla_matmul_args& p, hipStream_t stream);
 // out += bias on the finished output, for the families that do not add the bias in their epilogue
 int launch_bias_add(const gla_matmul_args& p, hipStream_t stream);
+// fp8-e4m3 / int8 activations [M, K] (row stride in bytes) -> fp16 rows of out_stride_m elements; both convert exactly
+int launch_widen_x8(const void* x, int64_t x_stride_m, int M, int K, int input_dtype, void* out_f16, int64_t out_stride_m, hipStream_t stream);
 
 // ---- streaming GEMV on 32-bit packed words, N fastest (gemv_packed.hip) ----
 // tile_config (when >= 1000) = waves per workgroup * 1000 + load batches per wave.

@@ -698,7 +698,9 @@ bool gemm_wn_eligible(const gla_matmul_args& p) {
     if (!(p.W_nbits == 2 || p.W_nbits == 4 || p.W_nbits == 8)) return false;
     if (p.elements_per_sample * p.W_nbits != 32) return false;
     if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16)) return false;
-    if (p.acc_dtype != GLA_DT_FP32) return false;
+    // (an int32 accumulator with 16-bit activations is the library's own call for widened int8 activations: the fp32
+    // sums of integer products are exact below 2^24)
+    if (!(p.acc_dtype == GLA_DT_FP32 || p.acc_dtype == GLA_DT_INT32)) return false;
     if (p.W_group_mode < 0 || p.W_group_mode > GLA_WGM_FMA) return false;
     if (p.channel_scale_mode < 0 || p.channel_scale_mode > GLA_CSM_BOTH) return false;
     if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;

@@ -915,7 +915,10 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true, i
         // iterations per flush: whole groups, at most 1024 K-values between folds
         const int nit = g.RW / g.LW / waves / 4;
         int fl = 1;
-        while (fl * 2 * k_per_iter <= 1024 && it_per_group % (fl * 2) == 0 && nit % (fl * 2) == 0) fl *= 2;
+        // ... at most 64 when an int32 accumulator was asked for (integer-valued activations, widened from int8):
+        // |x| <= 127 times 1024 + q over 64 K-values (128 for 1-bit codes) stays below 2^24, so every fp32 sum is exact
+        const int fold_k = p.acc_dtype == GLA_DT_INT32 ? 64 : 1024;
+        while (fl * 2 * k_per_iter <= fold_k && it_per_group % (fl * 2) == 0 && nit % (fl * 2) == 0) fl *= 2;
         g.FL = fl;
         const int ipb = kBatch / g.LW;
         g.nfb = fl >= ipb ? 1 : ipb / fl;
@@ -1024,7 +1027,8 @@ bool gemv_packed_eligible(const gla_matmul_args& p) {
     if (!(p.W_nbits == 1 || p.W_nbits == 2 || p.W_nbits == 4 || p.W_nbits == 8)) return false;
     if (p.elements_per_sample * p.W_nbits != 32) return false;
     if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16)) return false;
-    if (p.acc_dtype != GLA_DT_FP32) return false;
+    // (an int32 accumulator with 16-bit activations is the library's own call for widened int8 activations)
+    if (!(p.acc_dtype == GLA_DT_FP32 || p.acc_dtype == GLA_DT_INT32)) return false;
     if (p.W_group_mode < 0 || p.W_group_mode > GLA_WGM_FMA) return false;
     if (p.channel_scale_mode < 0 || p.channel_scale_mode > GLA_CSM_BOTH) return false;
     if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32))

@@ -187,7 +187,30 @@ __global__ __launch_bounds__(256) void bias_add_kernel(void* out, const void* bi
     store_from_float(out, out_dt, o, load_as_float(out, out_dt, o) + load_as_float(bias, bias_dt, n));
 }
 
+// fp8-e4m3 / int8 activations -> dense fp16 rows (both convert exactly): 8 values per thread
+__global__ __launch_bounds__(256) void widen_x8_kernel(const uint8_t* x, int64_t xsm, int M, int K, int in_dt, uint16_t* out, int64_t osm) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int per_row = (K + 7) / 8;
+    if (t >= (int64_t)M * per_row) return;
+    const int m = (int)(t / per_row), k0 = (int)(t % per_row) * 8;
+    const uint8_t* src = x + (int64_t)m * xsm + k0;
+    uint16_t* dst = out + (int64_t)m * osm + k0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        if (k0 + i >= K) break;
+        const float v = in_dt == GLA_DT_INT8 ? (float)(int8_t)src[i] : load_as_float(src, GLA_DT_FP8, i);
+        dst[i] = float_to_half_bits(v);
+    }
+}
+
 }  // namespace
+
+int launch_widen_x8(const void* x, int64_t x_stride_m, int M, int K, int input_dtype, void* out_f16, int64_t out_stride_m, hipStream_t stream) {
+    const int64_t items = (int64_t)M * ((K + 7) / 8);
+    hipLaunchKernelGGL(widen_x8_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, (const uint8_t*)x, x_stride_m, M,
+                       K, input_dtype, (uint16_t*)out_f16, out_stride_m);
+    return check_hip(hipGetLastError(), "activation widening launch");
+}
 
 int launch_bias_add(const gla_matmul_args& p, hipStream_t stream) {
     const int out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);

@@ -840,6 +840,21 @@ def test_ternary_weight_layers(device, dtype):
     torch.cuda.synchronize()
     want = xi.double() @ W.double().T
     assert np.array_equal(to_np(y).astype(np.float64), want.numpy())
+    # the same at the extremes (every activation 127, long K) through each kernel the int8 activations are widened
+    # for: the streaming kernel at 1, 5 and 20 rows (it folds its offset sums every 64 K-values for an int32
+    # accumulator, so that no fp32 sum passes 2^24) and the tiled GEMM at 100 rows
+    K2 = 8192
+    W2 = torch.randint(-1, 2, (N, K2), generator=g).to(dtype)
+    W2[:8] = 1.0
+    unit2 = helper.A8W158_INT_dynamic(device=device).from_weights(W2, torch.tensor(1.0))
+    unit2.output_dtype = DType.FP32
+    for M in (1, 5, 20, 100):
+        xa = torch.randint(-127, 128, (M, K2), generator=g).to(dtype)
+        xa[0] = 127.0
+        xa[:, 0] = 127.0
+        y2 = unit2(xa.to(device))
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(y2).astype(np.float64), (xa.double() @ W2.double().T).numpy()), M
 
 
 @pytest.mark.gpu
