@@ -829,7 +829,12 @@ static Plan8 plan_blockq(const gla_matmul_args& p) {
 }
 
 bool gemm_blockq_eligible(const gla_matmul_args& p) {
-    if (!blockq_stream_eligible(p) || p.M <= 1 || p.out_stride_n != 1) return false;
+    // The streaming kernel keeps the first rows: 2 everywhere (4096^2 11 against 15 us, 16384^2 63-65 against 74;
+    // within 7 % either way on 8192^2 and 4096 x 14336), 3 on layers of 20 MB or less and of 200 MB or more (4096^2
+    // 13-14.5 against 15-16; 16384^2 62-68 against 74; 8192^2 24-27 against 22)
+    const int64_t wbytes = (int64_t)p.N * p.K;
+    const int stream_rows = (wbytes <= 20000000 || wbytes >= 200000000) ? 3 : 2;
+    if (!blockq_stream_eligible(p) || p.M <= stream_rows || p.out_stride_n != 1) return false;
     if (p.meta_stride_n < 0 || p.meta_stride_g < 0 || p.sx_stride_m < 0 || p.sx_stride_g < 0) return false;
     if ((int64_t)p.M * p.x_stride_m >= (1ll << 31) || (int64_t)p.N * p.w_stride_n >= (1ll << 31)) return false;
     if ((int64_t)p.M * p.sx_stride_m * 4 >= (1ll << 31) || (int64_t)(p.N / 128 + 1) * p.meta_stride_n * 4 >= (1ll << 31)) return false;

@@ -170,7 +170,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_MXFP8 7   /* MXFP8 weights x fp8 activations, MFMA GEMM */
 #define GLA_FAMILY_MX_STREAM 8    /* streaming kernel: weight-only MX layers, MXFP8 x MXFP4 */
 #define GLA_FAMILY_BLOCKQ_STREAM 9 /* streaming kernel: 128 x 128 block-quantised int8 / fp8 */
-#define GLA_FAMILY_GEMM_BLOCKQ 10  /* the same from 2 rows up: MFMA GEMM with a second, scaled accumulator */
+#define GLA_FAMILY_GEMM_BLOCKQ 10  /* the same above 2-3 rows: MFMA GEMM with a second, scaled accumulator */
 #define GLA_FAMILY_GEMM_KBYTES_MX 11 /* weight-only MX layers above 16 rows: MFMA GEMM, block scale applied on conversion */
 #define GLA_FAMILY_MX_SKINNY 12     /* weight-only MX layers at 3..16 rows: weights read once into registers, MFMA */
 int gla_matmul_family(const gla_matmul_args* args);

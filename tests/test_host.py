@@ -489,7 +489,8 @@ def test_block_quant_processor_packs_like_the_reference():
         l2 = proc(device="cpu", dtype=torch.bfloat16, block_quant=True).from_weights(
             l.W_q.t().contiguous(), scales=l.scales.t().contiguous())
         assert torch.equal(l2.W_q.view(torch.uint8), l.W_q.view(torch.uint8)) and torch.equal(l2.scales, l.scales)
-        for M, fam in ((1, "BLOCKQ_STREAM"), (2, "GEMM_BLOCKQ"), (5, "GEMM_BLOCKQ"), (300, "GEMM_BLOCKQ")):
+        # (a layer this small streams its first 3 rows)
+        for M, fam in ((1, "BLOCKQ_STREAM"), (3, "BLOCKQ_STREAM"), (4, "GEMM_BLOCKQ"), (5, "GEMM_BLOCKQ"), (300, "GEMM_BLOCKQ")):
             xq = torch.zeros(M, K, dtype=wdt)
             assert _family(l, M, None, scales_x=torch.ones(M, K // 128), x=xq) == fam
 
