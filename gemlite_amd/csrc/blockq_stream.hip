@@ -124,6 +124,13 @@ constexpr int kColsQ = 4;
 
 template <bool FP8>
 void launch_rows_q(const BqArgs& a, int rm, dim3 grid, hipStream_t s) {
+    // narrow layers (fewer than 512 workgroups at 4 columns per wave: 4 waves per CU or less): 2 columns per wave
+    if (rm <= 2 && ceil_div(a.N, 4 * kColsQ) < 512) {
+        const dim3 g2(ceil_div(a.N, 4 * 2), grid.y);
+        if (rm == 1) hipLaunchKernelGGL((blockq_stream_kernel<FP8, 1, 2>), g2, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((blockq_stream_kernel<FP8, 2, 2>), g2, dim3(256), 0, s, a);
+        return;
+    }
     if (rm == 1) hipLaunchKernelGGL((blockq_stream_kernel<FP8, 1, kColsQ>), grid, dim3(256), 0, s, a);
     else if (rm == 2) hipLaunchKernelGGL((blockq_stream_kernel<FP8, 2, kColsQ>), grid, dim3(256), 0, s, a);
     else if (rm == 4) hipLaunchKernelGGL((blockq_stream_kernel<FP8, 4, kColsQ>), grid, dim3(256), 0, s, a);
