@@ -9,6 +9,42 @@ namespace gla {
 int launch_generic(const gla_matmul_args& p, hipStream_t stream);
 // out += bias on the finished output, for the families that do not add the bias in their epilogue
 int launch_bias_add(const gla_matmul_args& p, hipStream_t stream);
+// Tile height and K split of a tiled MFMA GEMM from a small cost model (host only).  A workgroup's time is its
+// pipeline stages times a per-stage cost that grows with the tile height (taller tiles do more per stage and are
+// the more efficient ones, but only when there are enough of them); workgroups run in rounds of one per CU; a split
+// K pays a finishing launch and the fp32 partials' round trip through memory.  The constants come from timing every
+// (tile, split) pair on 4096^2, 14336 x 4096 and 4096 x 14336 layers at 64..2048 rows; before, the tallest tile was
+// taken above 128 rows whatever the layer, which left small layers with a quarter of the chip busy or with deep
+// splits (fp8 4096^2 at 1024 rows: 63 us, 31 with 64-row tiles and no split).
+struct TilePick {
+    int bm, S;
+};
+inline TilePick pick_tile_and_split(int M, int N, int bn, int steps, int min_steps_per_split, int max_splits, const int* bms,
+                                    const float* stage_cost_us, int n_bms, int bm_fixed, int s_fixed) {
+    TilePick best{bms[0], 1};
+    double best_t = 1e30;
+    const int tiles_n = (N + bn - 1) / bn;
+    for (int i = 0; i < n_bms; ++i) {
+        const int bm = bms[i];
+        if (bm_fixed > 0 ? bm != bm_fixed : (i > 0 && bm >= 2 * M)) continue;  // no tile more than twice as tall as the batch
+        const int tiles = ((M + bm - 1) / bm) * tiles_n;
+        for (int want = 1; want <= max_splits; ++want) {
+            if (s_fixed > 0 ? want != s_fixed : (want > 1 && steps / want < min_steps_per_split)) continue;
+            const int sps = (steps + want - 1) / want, S = (steps + sps - 1) / sps;
+            if (s_fixed <= 0 && S != want) continue;  // the same split under another name
+            const double wgs = (double)tiles * S, rounds = (double)((int64_t)(wgs + 255) / 256);
+            const double fill = wgs < 256.0 ? wgs / 256.0 : 1.0;
+            double t = rounds * sps * stage_cost_us[i] * (0.8 + 0.2 * fill);  // a half-empty chip runs each workgroup a little faster
+            if (S > 1) t += 2.0 + 2.0e-6 * (double)M * N * S;                 // finishing launch; 8 bytes per partial at ~4 TB/s
+            if (t < best_t) {
+                best_t = t;
+                best = TilePick{bm, S};
+            }
+        }
+    }
+    return best;
+}
+
 // fp8-e4m3 / int8 activations [M, K] (row stride in bytes) -> fp16 rows of out_stride_m elements; both convert exactly
 int launch_widen_x8(const void* x, int64_t x_stride_m, int M, int K, int input_dtype, void* out_f16, int64_t out_stride_m, hipStream_t stream);
 

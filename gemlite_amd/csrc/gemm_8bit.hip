@@ -742,20 +742,17 @@ constexpr int64_t kWsReserved8 = kWsPrivateBytes;  // the start of the workspace
 Plan8 plan8(int M, int N, int Kb, int tile_config) {
     Plan8 g;
     const int cfg = tile_config > 0 ? tile_config : 0;
-    g.bm = cfg % 1000;
-    if (g.bm != 64 && g.bm != 128 && g.bm != 256) g.bm = M > 128 ? 256 : (M > 64 ? 128 : 64);
+    const int bm_asked = cfg % 1000;
+    const int total_steps = ceil_div(Kb, kRowB8);
+    // per-stage cost of a workgroup (64 bytes of K) by tile height, us, the chip full
+    static const int bms[3] = {64, 128, 256};
+    static const float cost[3] = {0.53f, 0.66f, 0.85f};
+    const TilePick pick = pick_tile_and_split(M, N, kBN, total_steps, 8, 16, bms, cost, 3,
+                                              (bm_asked == 64 || bm_asked == 128 || bm_asked == 256) ? bm_asked : 0, cfg / 1000);
+    g.bm = pick.bm;
     g.tiles_m = ceil_div(M, g.bm);
     g.tiles_n = ceil_div(N, kBN);
-    const int total_steps = ceil_div(Kb, kRowB8);
-    int want = cfg / 1000;
-    if (want <= 0) {
-        // one workgroup per CU at least, but no split shorter than 16 stages and at most 16 splits
-        const int tiles = g.tiles_m * g.tiles_n;
-        want = tiles * 2 > 256 ? 1 : ceil_div(256, tiles);
-        const int max_s = total_steps / 16 > 0 ? total_steps / 16 : 1;
-        if (want > max_s) want = max_s;
-        if (want > 16) want = 16;
-    }
+    int want = pick.S;
     if (want > total_steps) want = total_steps;
     if (want < 1) want = 1;
     g.sps = ceil_div(total_steps, want);

@@ -529,20 +529,18 @@ struct KbPlan {
 KbPlan kb_plan(const gla_matmul_args& p) {
     KbPlan g;
     const int cfg = p.tile_config > 0 ? p.tile_config : 0;
-    g.bm = cfg % 1000;
-    if (!(g.bm == 64 || g.bm == 128 || g.bm == 256)) g.bm = p.M > 128 ? 256 : (p.M > 64 ? 128 : 64);
+    const int bm_asked = cfg % 1000;
+    const int total_steps = p.K / kBKb;
+    // per-stage cost of a workgroup (64 K-values) by tile height, us, the chip full: the byte -> 16-bit conversion
+    // makes the short tiles cheaper per stage than their share of the MFMA work
+    static const int bms[3] = {64, 128, 256};
+    static const float cost[3] = {0.95f, 1.48f, 1.8f};
+    const TilePick pick = pick_tile_and_split(p.M, p.N, kBNb, total_steps, 8, 32, bms, cost, 3,
+                                              (bm_asked == 64 || bm_asked == 128 || bm_asked == 256) ? bm_asked : 0, cfg / 1000);
+    g.bm = pick.bm;
     g.tiles_m = ceil_div(p.M, g.bm);
     g.tiles_n = ceil_div(p.N, kBNb);
-    const int total_steps = p.K / kBKb;
-    int want = cfg / 1000;
-    if (want <= 0) {
-        // enough workgroups for 256 CUs, but no split shorter than 8 stages and at most 32 splits
-        const int tiles = g.tiles_m * g.tiles_n;
-        want = tiles * 2 > 256 ? 1 : ceil_div(256, tiles);
-        const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
-        if (want > max_s) want = max_s;
-        if (want > 32) want = 32;
-    }
+    int want = pick.S;
     if (want > total_steps) want = total_steps;
     if (want < 1) want = 1;
     g.sps = ceil_div(total_steps, want);

@@ -668,8 +668,12 @@ WnPlan wn_plan(const gla_matmul_args& p) {
         // them the fp32 partials, at the same number of workgroups (8192^2 4-bit, M=256: 55-58
         // against 61-64 us)
         g.bm = p.M > 256 ? 256 : (p.M > 64 ? 128 : (p.M > 32 ? 64 : 32));
-    g.tiles_m = ceil_div(p.M, g.bm);
     g.tiles_n = ceil_div(p.N, kBNw);
+    // ... and above 256 rows too while 256-row tiles would not give every CU one: the 128-row tile then fills the
+    // chip with half the K splits or none (4096^2 4-bit, weights rotated: M=512 64 -> 38 us, M=1024 85 -> 57, M=2048
+    // 101 -> 85; 14336 x 4096 M=512 119 -> 82)
+    if (g.bm == 256 && cfg % 1000 != 256 && ceil_div(p.M, 256) * g.tiles_n < 256) g.bm = 128;
+    g.tiles_m = ceil_div(p.M, g.bm);
     const int total_steps = p.K / kBKw;
     int want = cfg / 1000;
     if (want <= 0) {
@@ -679,7 +683,9 @@ WnPlan wn_plan(const gla_matmul_args& p) {
         // short tiles (4 waves) are bound by unpacking on one wave per SIMD: two workgroups per CU
         // (16384^2, 2-bit, M=64: 72 against 90 us; 4-bit, M=32: 47 against 56 us)
         const int target = g.bm <= 64 ? 512 : 256;
-        want = tiles * 2 > target ? 1 : ceil_div(target, tiles);
+        // (rounded down: 56 column tiles x 5 splits are 280 workgroups, a second round for 24 of them - 14336 x 4096 at
+        // 128 rows took 47 us that way and 36 with 4 splits)
+        want = tiles * 2 > target ? 1 : target / tiles;
         const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
         if (want > max_s) want = max_s;
         if (want > 32) want = 32;
