@@ -950,14 +950,16 @@ bool gemm_mxfp8_eligible(const gla_matmul_args& p) {
 
 // with block scales on both sides the 256-row tile has no registers for the scale words next to two
 // fragment buffers of 8-register operands
-// Left to choose, 64 rows or fewer take the 128-row tile too: it reads the scales regrouped by stage, the
-// 64-row tile reads them where the caller keeps them (16384^2, M=8: MXFP4 weights 42 against 54 us, MXFP8
-// weights 59 against 66 us).
+// Left to choose, short batches on very large MXFP4 layers take the 128-row tile too: it reads the scales regrouped
+// by stage (a launch of its own), the 64-row tile reads them where the caller keeps them (weights rotated, M=8:
+// 16384^2 MXFP4 weights 54 against 64 us, MXFP8 weights 87 against 84; 8192^2 28 against 24 and 33 against 27;
+// 4096^2 20 against 15.5 and 20 against 15).
 static Plan8 plan_mxfp8(const gla_matmul_args& p) {
     Plan8 g = plan8(p.M, p.N, p.K, p.tile_config);
     const int asked = p.tile_config > 0 ? p.tile_config % 1000 : 0;
     const bool chosen_here = !(asked == 64 || asked == 128 || asked == 256);
-    if ((g.bm == 256 && p.channel_scale_mode == GLA_CSM_MX) || (g.bm == 64 && chosen_here)) {
+    const bool large_fp4 = p.elements_per_sample == 2 && (int64_t)p.N * p.K >= 100000000;
+    if ((g.bm == 256 && p.channel_scale_mode == GLA_CSM_MX) || (g.bm == 64 && chosen_here && large_fp4)) {
         const int cfg = (p.tile_config > 0 ? p.tile_config / 1000 : 0) * 1000 + 128;
         g = plan8(p.M, p.N, p.K, cfg);
     }
