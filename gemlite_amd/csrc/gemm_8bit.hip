@@ -815,9 +815,12 @@ static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 // number of stages) and their partials are the scaled fp32 sums, which the reduction kernel only adds.
 static Plan8 plan_blockq(const gla_matmul_args& p) {
     const int cfg = p.tile_config > 0 ? p.tile_config : 0;
-    int bm = cfg % 1000;
-    if (bm != 64 && bm != 128) bm = p.M > 64 ? 128 : 64;
-    Plan8 g = plan8(p.M, p.N, p.K, (cfg / 1000) * 1000 + bm);
+    const int bm_asked = (cfg % 1000 == 64 || cfg % 1000 == 128) ? cfg % 1000 : 0;
+    // the same cost model as plan8() over the two tile heights there are (the fold makes a stage dearer)
+    static const int bms[2] = {64, 128};
+    static const float cost[2] = {0.77f, 0.96f};
+    const TilePick pick = pick_tile_and_split(p.M, p.N, kBN, ceil_div(p.K, kRowB8), 8, 16, bms, cost, 2, bm_asked, cfg / 1000);
+    Plan8 g = plan8(p.M, p.N, p.K, pick.S * 1000 + pick.bm);
     if (g.S > 1 && (g.sps & 1)) {
         g.sps += 1;
         g.S = ceil_div(ceil_div(p.K, kRowB8), g.sps);
