@@ -66,6 +66,32 @@ def test_a8w8_dynamic_4096x8192x8192(device, fp8):
     assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("shape", [(4096, 4096), (14336, 4096), (4096, 14336)])
+def test_a8w8_dynamic_medium_batches_on_small_layers(device, fp8, shape):
+    """Layers of a 4096-wide model at prefill chunks of a few hundred to a few thousand rows: the tile height and K
+    split are chosen per layer size there (64- and 128-row tiles, with and without a split), and the first rows go
+    through the streaming kernel.  Sampled output columns against exact sums of the GPU quantiser's own codes."""
+    N, K = shape
+    W = gen_x(N, K, torch.bfloat16, seed=13, std=0.02)
+    wq, sw = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+    proc = (helper.A8W8_FP8_dynamic if fp8 else helper.A8W8_INT8_dynamic)(device=device)
+    proc.dtype = torch.bfloat16
+    layer = proc.from_weights(wq, scales=sw)
+    cols = sample_cols(N, seed=17)
+    wsub = wq.view(torch.uint8).numpy()[cols] if fp8 else wq.numpy()[cols]
+    b = (orc.e4m3fn_decode(wsub) if fp8 else wsub).astype(np.float64)
+    swc = to_np(sw).astype(np.float64).reshape(-1)[cols][None, :]
+    for M in (2, 40, 300, 1024, 2048):
+        x = gen_x(M, K, torch.bfloat16, seed=M)
+        y = to_np(layer(x.to(device)))
+        xq, sx = gemlite_amd.scale_activations_per_token(x.to(device), torch.float8_e4m3fn if fp8 else torch.int8)
+        a = orc.e4m3fn_decode(xq.view(torch.uint8).cpu().numpy()) if fp8 else xq.cpu().numpy()
+        want = (a.astype(np.float64) @ b.T) * sx.cpu().numpy().astype(np.float64) * swc
+        assert rel_frob(y[:, cols], want.astype(np.float32)) <= TIGHT_BF16, M
+        assert elementwise_excess(y[:, cols], want, "bf16") <= 1.0, M
+
+
 def test_int8_x_int8_int32_exact_4096x8192x8192(device):
     """INT8 x INT8 -> INT32 at M = 4096, N = K = 8192 with the accumulators as the output: sampled
     columns, all rows, bit for bit against exact sums (|sum| <= 8192 * 2^14 < 2^53, so float64 BLAS is
@@ -139,6 +165,26 @@ def test_a16w4_prefill_4096_cubed(device):
     err = rel_frob(y[:, cols], want)
     assert err <= FROB_TOL and err <= TIGHT_FP16, err
     assert elementwise_excess(y[:, cols], want, "fp16") <= 1.0
+
+
+@pytest.mark.parametrize("nbits,gs", [(4, 128), (8, 4096), (2, 64), (1, 128)])
+@pytest.mark.parametrize("shape", [(4096, 4096), (11008, 4096)])
+def test_a16wn_medium_batches_on_small_layers(device, nbits, gs, shape):
+    """Packed-code layers of a 4096-wide model between decode and prefill: row chunks of 16 through the streaming
+    kernel up to 64 rows (1-bit codes: chunks of 4 at any row count), the tiled GEMM with 128-row tiles above."""
+    N, K = shape
+    W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.float16, seed=37 + nbits)
+    layer = GemLiteLinear(nbits, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    cols = sample_cols(N, seed=3)
+    gpn = K // gs
+    idx = (cols[:, None] * gpn + np.arange(gpn)[None, :]).reshape(-1)
+    for M in (5, 20, 48, 64, 100, 300, 1024):
+        x = gen_x(M, K, torch.float16, seed=M)
+        y = to_np(layer(x.to(device)))
+        want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], gs)
+        err = rel_frob(y[:, cols], want)
+        assert err <= FROB_TOL and err <= TIGHT_FP16, (M, err)
+        assert elementwise_excess(y[:, cols], want, "fp16") <= 1.0, M
 
 
 @pytest.mark.parametrize("to_int8", [True, False])
