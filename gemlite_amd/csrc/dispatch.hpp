@@ -28,10 +28,12 @@ inline TilePick pick_tile_and_split(int M, int N, int bn, int steps, int min_ste
         const int bm = bms[i];
         if (bm_fixed > 0 ? bm != bm_fixed : (i > 0 && bm >= 2 * M)) continue;  // no tile more than twice as tall as the batch
         const int tiles = ((M + bm - 1) / bm) * tiles_n;
-        for (int want = 1; want <= max_splits; ++want) {
+        const int top = s_fixed > max_splits ? s_fixed : max_splits;  // a split asked for is taken as asked
+        for (int want = 1; want <= top; ++want) {
             if (s_fixed > 0 ? want != s_fixed : (want > 1 && steps / want < min_steps_per_split)) continue;
             const int sps = (steps + want - 1) / want, S = (steps + sps - 1) / sps;
             if (s_fixed <= 0 && S != want) continue;  // the same split under another name
+            if (s_fixed > 0 && bm_fixed > 0) return TilePick{bm, S};
             const double wgs = (double)tiles * S, rounds = (double)((int64_t)(wgs + 255) / 256);
             const double fill = wgs < 256.0 ? wgs / 256.0 : 1.0;
             double t = rounds * sps * stage_cost_us[i] * (0.8 + 0.2 * fill);  // a half-empty chip runs each workgroup a little faster
