@@ -508,6 +508,24 @@ def test_ternary_processors_pack_like_the_reference():
     d = gemlite_amd.helper.A8W158_INT_dynamic(device="cpu").from_weights(W, torch.tensor(0.037))
     assert (d.W_group_mode, d.channel_scale_mode, d.input_dtype, d.acc_dtype) == (1, 3, DType.INT8, DType.INT32)
     assert d.scaled_activations and d.output_dtype == DType.FP16
+    # int8 activations on packed codes have no kernel of their own: the library widens them to fp16 in the workspace
+    # and runs the packed-code kernels, so the call reports those families, asks for the room, and refuses to run
+    # without it before anything is launched
+    import ctypes
+    lib = _ext.load_library()
+    for M, fam in ((1, "GEMV_PACKED"), (40, "GEMV_PACKED"), (300, "GEMM_WN")):
+        xq = torch.zeros(M, K, dtype=torch.int8)
+        m = d.get_meta_args()
+        out = torch.zeros(M, N, dtype=torch.float16)
+        a = _ext.build_matmul_args(xq, d.W_q, d.scales, d.zeros, torch.ones(M, 1), out, W_nbits=m[1], group_size=m[2],
+                                   unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                   acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                   data_contiguous=m[11])
+        assert _ext.matmul_family(a) == fam
+        need = lib.gla_matmul_workspace_bytes(ctypes.byref(a))
+        assert need >= (4 << 20) + M * K * 2
+        assert lib.gla_matmul(ctypes.byref(a), None) == -5   # GLA_ERR_WORKSPACE_TOO_SMALL: no workspace given
+        assert b"widened" in lib.gla_last_error()
 
 
 # ------------------------------------------------------------------ workspace keyed by (device, stream)
