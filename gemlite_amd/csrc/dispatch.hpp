@@ -19,8 +19,16 @@ int launch_bias_add(const gla_matmul_args& p, hipStream_t stream);
 struct TilePick {
     int bm, S;
 };
+struct TileModel {
+    double underfill = 0.8;       // per-stage cost of a workgroup on an almost empty chip, relative to the full one
+    double split_fixed_us = 2.0;  // finishing launch
+    double split_us_per_elem = 2.0e-6;  // 8 bytes per partial, written and read
+    int pair_up_to = 0;           // tiles this tall or shorter run two workgroups per CU ...
+    double pair_cost = 1.65;      // ... each at this multiple of its stage cost
+};
 inline TilePick pick_tile_and_split(int M, int N, int bn, int steps, int min_steps_per_split, int max_splits, const int* bms,
-                                    const float* stage_cost_us, int n_bms, int bm_fixed, int s_fixed) {
+                                    const float* stage_cost_us, int n_bms, int bm_fixed, int s_fixed,
+                                    const TileModel& model = TileModel()) {
     TilePick best{bms[0], 1};
     double best_t = 1e30;
     const int tiles_n = (N + bn - 1) / bn;
@@ -34,10 +42,13 @@ inline TilePick pick_tile_and_split(int M, int N, int bn, int steps, int min_ste
             const int sps = (steps + want - 1) / want, S = (steps + sps - 1) / sps;
             if (s_fixed <= 0 && S != want) continue;  // the same split under another name
             if (s_fixed > 0 && bm_fixed > 0) return TilePick{bm, S};
-            const double wgs = (double)tiles * S, rounds = (double)((int64_t)(wgs + 255) / 256);
+            const double wgs = (double)tiles * S;
+            const bool paired = bm <= model.pair_up_to && wgs > 256.0;
+            const double per_round = paired ? 512.0 : 256.0;
+            const double rounds = (double)((int64_t)((wgs + per_round - 1) / per_round));
             const double fill = wgs < 256.0 ? wgs / 256.0 : 1.0;
-            double t = rounds * sps * stage_cost_us[i] * (0.8 + 0.2 * fill);  // a half-empty chip runs each workgroup a little faster
-            if (S > 1) t += 2.0 + 2.0e-6 * (double)M * N * S;                 // finishing launch; 8 bytes per partial at ~4 TB/s
+            double t = rounds * sps * stage_cost_us[i] * (model.underfill + (1.0 - model.underfill) * fill) * (paired ? model.pair_cost : 1.0);
+            if (S > 1) t += model.split_fixed_us + model.split_us_per_elem * (double)M * N * S;
             if (t < best_t) {
                 best_t = t;
                 best = TilePick{bm, S};

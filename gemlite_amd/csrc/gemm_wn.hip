@@ -662,34 +662,35 @@ struct WnPlan {
 WnPlan wn_plan(const gla_matmul_args& p) {
     WnPlan g;
     const int cfg = p.tile_config > 0 ? p.tile_config : 0;
-    g.bm = cfg % 1000;
-    if (!(g.bm == 32 || g.bm == 64 || g.bm == 128 || g.bm == 256))
-        // Up to 256 rows the 128-row tile: against the 256-row one it halves the K splits, and with
-        // them the fp32 partials, at the same number of workgroups (8192^2 4-bit, M=256: 55-58
-        // against 61-64 us)
-        g.bm = p.M > 256 ? 256 : (p.M > 64 ? 128 : (p.M > 32 ? 64 : 32));
-    g.tiles_n = ceil_div(p.N, kBNw);
-    // ... and above 256 rows too while 256-row tiles would not give every CU one: the 128-row tile then fills the
-    // chip with half the K splits or none (4096^2 4-bit, weights rotated: M=512 64 -> 38 us, M=1024 85 -> 57, M=2048
-    // 101 -> 85; 14336 x 4096 M=512 119 -> 82)
-    if (g.bm == 256 && cfg % 1000 != 256 && ceil_div(p.M, 256) * g.tiles_n < 256) g.bm = 128;
-    g.tiles_m = ceil_div(p.M, g.bm);
+    const int bm_asked = cfg % 1000;
     const int total_steps = p.K / kBKw;
-    int want = cfg / 1000;
-    if (want <= 0) {
-        // enough workgroups for 256 CUs, but no split shorter than 8 stages (512 K-values) and at
-        // most 32 splits
-        const int tiles = g.tiles_m * g.tiles_n;
-        // short tiles (4 waves) are bound by unpacking on one wave per SIMD: two workgroups per CU
-        // (16384^2, 2-bit, M=64: 72 against 90 us; 4-bit, M=32: 47 against 56 us)
-        const int target = g.bm <= 64 ? 512 : 256;
-        // (rounded down: 56 column tiles x 5 splits are 280 workgroups, a second round for 24 of them - 14336 x 4096 at
-        // 128 rows took 47 us that way and 36 with 4 splits)
-        want = tiles * 2 > target ? 1 : target / tiles;
-        const int max_s = total_steps / 8 > 0 ? total_steps / 8 : 1;
-        if (want > max_s) want = max_s;
-        if (want > 32) want = 32;
-    }
+    // Tile height and K split from the cost model of dispatch.hpp, fitted to timings of every (tile, split) pair on
+    // 4096^2 .. 16384^2 layers at 32..1024 rows.  What it reproduces for 2- and 4-bit codes: the 128-row tile up to
+    // 256 rows (half the splits and partials of the 256-row one); above that the 128-row tile while 256-row ones would
+    // leave CUs idle, unless K is long enough that a split of the 256-row tile costs less than it saves (16384^2 at 512
+    // rows: 256-row tiles with 2 splits 295 us, 128-row tiles unsplit 316; 4096^2 at 2048 rows the other way round,
+    // 105 and 85); tiles of up to 128 rows (4 waves) two to a CU on large layers (16384^2 at 64 rows: 8 splits 65 us,
+    // 4 splits 69; 4096 x 14336 at 1024 rows: 128-row tiles with 4 splits 142 us, 256-row ones 158) and one to a CU on
+    // medium ones (14336 x 4096 at 64 rows: 4 splits 26 us, 8 splits 30); whole rounds of workgroups.
+    // 8-bit codes gain nothing from a second workgroup on the CU (4096^2 at 1024 rows, 32-row tiles: 512 workgroups
+    // 117 us, 256 of them at 512 rows 60 us), so they count one to a CU: then the 256-row tile with splits wins from
+    // 256 rows on 16384^2 (4 splits 166 us, 128-row tiles with 2 splits 185) and short tiles cost more per stage.
+    static const int bms[4] = {32, 64, 128, 256};
+    static const float cost_4[4] = {0.62f, 0.92f, 1.23f, 2.08f};  // us per 64-K stage, the chip full
+    static const float cost_8[4] = {0.86f, 0.98f, 1.27f, 2.19f};
+    const bool w8 = p.W_nbits == 8;
+    const float* cost = w8 ? cost_8 : cost_4;
+    TileModel model;
+    model.underfill = w8 ? 0.9 : 0.78;
+    model.split_us_per_elem = 1.4e-6;
+    model.pair_up_to = w8 ? 0 : 128;  // one wave row: 4 waves, two workgroups fit a CU
+    const TilePick pick = pick_tile_and_split(p.M, p.N, kBNw, total_steps, 8, 32, bms, cost, 4,
+                                              (bm_asked == 32 || bm_asked == 64 || bm_asked == 128 || bm_asked == 256) ? bm_asked : 0,
+                                              cfg / 1000, model);
+    g.bm = pick.bm;
+    g.tiles_m = ceil_div(p.M, g.bm);
+    g.tiles_n = ceil_div(p.N, kBNw);
+    int want = pick.S;
     if (want > total_steps) want = total_steps;
     if (want < 1) want = 1;
     g.sps = ceil_div(total_steps, want);
