@@ -676,7 +676,7 @@ WnPlan wn_plan(const gla_matmul_args& p) {
     // 117 us, 256 of them at 512 rows 60 us), so they count one to a CU: then the 256-row tile with splits wins from
     // 256 rows on 16384^2 (4 splits 166 us, 128-row tiles with 2 splits 185) and short tiles cost more per stage.
     static const int bms[4] = {32, 64, 128, 256};
-    static const float cost_4[4] = {0.62f, 0.92f, 1.23f, 2.08f};  // us per 64-K stage, the chip full
+    static const float cost_4[4] = {0.62f, 0.92f, 1.23f, 2.15f};  // us per 64-K stage, the chip full
     static const float cost_8[4] = {0.86f, 0.98f, 1.27f, 2.19f};
     const bool w8 = p.W_nbits == 8;
     const float* cost = w8 ? cost_8 : cost_4;
@@ -684,6 +684,7 @@ WnPlan wn_plan(const gla_matmul_args& p) {
     model.underfill = w8 ? 0.9 : 0.78;
     model.split_us_per_elem = 1.4e-6;
     model.pair_up_to = w8 ? 0 : 128;  // one wave row: 4 waves, two workgroups fit a CU
+    model.pair_cost = 1.7;
     const TilePick pick = pick_tile_and_split(p.M, p.N, kBNw, total_steps, 8, 32, bms, cost, 4,
                                               (bm_asked == 32 || bm_asked == 64 || bm_asked == 128 || bm_asked == 256) ? bm_asked : 0,
                                               cfg / 1000, model);
