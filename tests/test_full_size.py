@@ -20,10 +20,11 @@ def sample_cols(N, count=48, seed=0):
     return cols
 
 
-@pytest.mark.parametrize("nbits,gs,M", [(8, 16384, 1), (8, 16384, 16), (8, 16384, 64), (8, 16384, 512),
-                                        (2, 64, 1), (2, 64, 16), (2, 64, 64), (2, 64, 512)])
+@pytest.mark.parametrize("nbits,gs,M", [(8, 16384, 1), (8, 16384, 16), (8, 16384, 64), (8, 16384, 256), (8, 16384, 512),
+                                        (2, 64, 1), (2, 64, 16), (2, 64, 64), (2, 64, 256), (2, 64, 512)])
 def test_a16wn_bf16_16384_square(device, nbits, gs, M):
-    """bf16 activations x 8-bit channel-wise / 2-bit group-64 weights, N = K = 16384."""
+    """bf16 activations x 8-bit channel-wise / 2-bit group-64 weights, N = K = 16384 (at 256 and 512 rows the tiled
+    GEMM splits K under 256-row tiles for 8-bit codes and runs 128-row tiles two to a CU for 2-bit ones)."""
     N = K = 16384
     W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.bfloat16, seed=nbits, scale_std=0.01)
     layer = helper.A16Wn(device=device, post_scale=True).from_weights(W_q, scales, zeros, nbits, gs)
@@ -171,14 +172,16 @@ def test_a16w4_prefill_4096_cubed(device):
 @pytest.mark.parametrize("shape", [(4096, 4096), (11008, 4096)])
 def test_a16wn_medium_batches_on_small_layers(device, nbits, gs, shape):
     """Packed-code layers of a 4096-wide model between decode and prefill: row chunks of 16 through the streaming
-    kernel up to 64 rows (1-bit codes: chunks of 4 at any row count), the tiled GEMM with 128-row tiles above."""
+    kernel up to 64 rows (1-bit codes: chunks of 4 at any row count), the tiled GEMM above with the tile height and
+    K split its cost model picks (32- and 64-row tiles with 4 to 8 splits, some ragged, up to 128 rows; 128-row tiles
+    two to a CU at 1024)."""
     N, K = shape
     W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.float16, seed=37 + nbits)
     layer = GemLiteLinear(nbits, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
     cols = sample_cols(N, seed=3)
     gpn = K // gs
     idx = (cols[:, None] * gpn + np.arange(gpn)[None, :]).reshape(-1)
-    for M in (5, 20, 48, 64, 100, 300, 1024):
+    for M in (5, 20, 48, 64, 65, 100, 128, 300, 1024):
         x = gen_x(M, K, torch.float16, seed=M)
         y = to_np(layer(x.to(device)))
         want = orc.hqq_dequant_matmul(to_np(x), W_q.numpy()[cols], to_np(scales)[idx], to_np(zeros)[idx], gs)
