@@ -136,6 +136,157 @@ __global__ __launch_bounds__(64) void generic_int_kernel(GenericArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Packed int32 words x fp16 / bf16 activations, any group size that is a whole number of words: the arithmetic of
+// generic_int_kernel for the packings whose groups are shorter than one step of the tuned kernels (1-bit codes in
+// groups of 32 or 64, 2-bit codes in groups of 16 or 32, ...).  One lane per output column as there, but the K range
+// is split over the 16 waves of a workgroup, every word is loaded once, the activations of a word come as 128-bit
+// loads, and the group's scale and zero are applied to the two sums of a group segment (sum x q, sum x) instead of
+// to every code; the waves' partial sums meet in LDS and are added in wave order.
+constexpr int kPackedWaves = 16;
+
+template <int NBITS, bool BF16, int RP>
+__global__ __launch_bounds__(64 * kPackedWaves) void generic_packed_kernel(GenericArgs a) {
+    constexpr int E = 32 / NBITS;            // codes per word
+    constexpr int CH = E < 8 ? E : 8;        // activations per load (4 for byte codes)
+    constexpr uint32_t MASK = (1u << NBITS) - 1u;
+    __shared__ float red[kPackedWaves][RP][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n_raw = blockIdx.x * 64 + lane;
+    const int n = n_raw < a.N ? n_raw : a.N - 1;  // lanes past N repeat the last column and store nothing
+    const int m0 = blockIdx.y * RP;
+    const int R = a.K / E;                         // word rows
+    const int gw = a.wgm == GLA_WGM_NONE ? R : a.gs / E;  // word rows per group
+    const int rpw = (R + kPackedWaves - 1) / kPackedWaves;
+    int r = wv * rpw;
+    const int r_end = r + rpw < R ? r + rpw : R;
+    const bool has_scale = (a.wgm == GLA_WGM_SCALE || a.wgm == GLA_WGM_SHIFT_SCALE || a.wgm == GLA_WGM_FMA);
+    const bool has_zero = (a.wgm == GLA_WGM_SHIFT || a.wgm == GLA_WGM_SHIFT_SCALE || a.wgm == GLA_WGM_FMA);
+    const uint16_t* xrow[RP];
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) {
+        const int m = m0 + rr < a.M ? m0 + rr : a.M - 1;
+        xrow[rr] = (const uint16_t*)a.x + (int64_t)m * a.xsm;
+    }
+    const uint32_t* wcol = (const uint32_t*)a.w + n;
+    float tot[RP];
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) tot[rr] = 0.0f;
+    while (r < r_end) {
+        const int g = r / gw;
+        int seg_end = (g + 1) * gw;
+        if (seg_end > r_end) seg_end = r_end;
+        float s = 1.0f, z = 0.0f;
+        if (has_scale) s = load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + (int64_t)n * a.msn);
+        if (has_zero)
+            z = a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0)
+                           : load_as_float(a.zeros, a.z_dt, (int64_t)g * a.msg + (int64_t)n * a.msn);
+        float acc[RP], xs[RP];
+#pragma unroll
+        for (int rr = 0; rr < RP; ++rr) acc[rr] = xs[rr] = 0.0f;
+        for (; r < seg_end; ++r) {
+            const uint32_t word = wcol[(int64_t)r * a.wsk];
+#pragma unroll
+            for (int c = 0; c < E / CH; ++c) {
+                uint32_t xw[RP][CH / 2];
+#pragma unroll
+                for (int rr = 0; rr < RP; ++rr) {
+                    const uint16_t* src = xrow[rr] + (int64_t)r * E + c * CH;
+                    if constexpr (CH == 8) {
+                        const uint4 v = *(const uint4*)src;
+                        xw[rr][0] = v.x; xw[rr][1] = v.y; xw[rr][2] = v.z; xw[rr][3] = v.w;
+                    } else {
+                        const uint2 v = *(const uint2*)src;
+                        xw[rr][0] = v.x; xw[rr][1] = v.y;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < CH; ++j) {
+                    const float qf = (float)((word >> ((c * CH + j) * NBITS)) & MASK);
+#pragma unroll
+                    for (int rr = 0; rr < RP; ++rr) {
+                        const uint16_t bits = (uint16_t)(xw[rr][j / 2] >> ((j % 2) * 16));
+                        const float xv = BF16 ? bf16_bits_to_float(bits) : half_bits_to_float(bits);
+                        acc[rr] = __builtin_fmaf(xv, qf, acc[rr]);
+                        xs[rr] += xv;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int rr = 0; rr < RP; ++rr) {
+            float v;
+            switch (a.wgm) {
+                case GLA_WGM_SHIFT: v = __builtin_fmaf(-z, xs[rr], acc[rr]); break;
+                case GLA_WGM_SCALE: v = s * acc[rr]; break;
+                case GLA_WGM_SHIFT_SCALE: v = s * __builtin_fmaf(-z, xs[rr], acc[rr]); break;
+                case GLA_WGM_FMA: v = __builtin_fmaf(s, acc[rr], z * xs[rr]); break;
+                default: v = acc[rr]; break;
+            }
+            tot[rr] += v;
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) red[wv][rr][lane] = tot[rr];
+    __syncthreads();
+    if (wv != 0 || n_raw >= a.N) return;
+    float sb = 1.0f;
+    if (a.csm == GLA_CSM_WEIGHT || a.csm == GLA_CSM_BOTH) sb = load_as_float(a.scales, a.meta_dt, n);
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) {
+        const int m = m0 + rr;
+        if (m >= a.M) continue;
+        float v = 0.0f;
+        for (int w = 0; w < kPackedWaves; ++w) v += red[w][rr][lane];
+        float sa = 1.0f;
+        if (a.csm == GLA_CSM_ACTIVATION || a.csm == GLA_CSM_BOTH) sa = load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
+        if (a.csm == GLA_CSM_WEIGHT) v *= sb;
+        else if (a.csm == GLA_CSM_ACTIVATION) v *= sa;
+        else if (a.csm == GLA_CSM_BOTH) v *= (sa * sb);
+        store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, v);
+    }
+}
+
+// what generic_packed_kernel assumes of a call
+bool packed_words_ok(const gla_matmul_args& p) {
+    if (p.w_dtype != GLA_DT_INT32 || p.w == nullptr || p.x == nullptr) return false;
+    if (!(p.W_nbits == 1 || p.W_nbits == 2 || p.W_nbits == 4 || p.W_nbits == 8)) return false;
+    const int E = 32 / p.W_nbits;
+    if (p.elements_per_sample != E || p.unpack_mask != (1 << p.W_nbits) - 1) return false;
+    if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16) || p.acc_dtype != GLA_DT_FP32) return false;
+    if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
+    if (p.channel_scale_mode < GLA_CSM_NONE || p.channel_scale_mode > GLA_CSM_BOTH) return false;
+    if (p.W_group_mode < GLA_WGM_NONE || p.W_group_mode > GLA_WGM_FMA) return false;
+    if (p.M < 1 || p.N < 1 || p.K < E || p.K % E != 0 || p.K % 8 != 0) return false;
+    if (p.x_stride_k != 1 || p.w_stride_n != 1 || p.x_stride_m % 8 != 0 || ((uintptr_t)p.x & 15)) return false;
+    if (p.W_group_mode != GLA_WGM_NONE && (p.group_size < E || p.group_size % E != 0 || p.K % p.group_size != 0)) return false;
+    const bool has_scale = p.W_group_mode == GLA_WGM_SCALE || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
+    const bool has_zero = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
+    if ((has_scale || (p.channel_scale_mode & 1)) && p.scales == nullptr) return false;
+    if (has_zero && p.zeros == nullptr) return false;
+    if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
+    return true;
+}
+
+template <int NBITS, bool BF16>
+void launch_packed_rows(const GenericArgs& a, hipStream_t stream) {
+    const int rp = a.M >= 3 ? 4 : a.M;
+    const dim3 grid(ceil_div(a.N, 64), ceil_div(a.M, rp)), block(64 * kPackedWaves);
+    if (rp == 4) hipLaunchKernelGGL((generic_packed_kernel<NBITS, BF16, 4>), grid, block, 0, stream, a);
+    else if (rp == 2) hipLaunchKernelGGL((generic_packed_kernel<NBITS, BF16, 2>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((generic_packed_kernel<NBITS, BF16, 1>), grid, block, 0, stream, a);
+}
+
+template <bool BF16>
+void launch_packed_bits(const GenericArgs& a, hipStream_t stream) {
+    switch (a.nbits) {
+        case 1: return launch_packed_rows<1, BF16>(a, stream);
+        case 2: return launch_packed_rows<2, BF16>(a, stream);
+        case 4: return launch_packed_rows<4, BF16>(a, stream);
+        default: return launch_packed_rows<8, BF16>(a, stream);
+    }
+}
+
 // e2m1 x e2m1 with e8m0 block scales on both operands (block = 32 along K).
 __global__ __launch_bounds__(64) void generic_mxfp4_kernel(GenericArgs a) {
     const int n = blockIdx.x * 64 + threadIdx.x;
@@ -239,6 +390,9 @@ int launch_generic(const gla_matmul_args& p, hipStream_t stream) {
             return GLA_ERR_UNSUPPORTED_MODE;
         }
         hipLaunchKernelGGL(generic_mxfp4_kernel, grid, dim3(64), 0, stream, a);
+    } else if (packed_words_ok(p)) {
+        if (p.input_dtype == GLA_DT_BF16) launch_packed_bits<true>(a, stream);
+        else launch_packed_bits<false>(a, stream);
     } else {
         hipLaunchKernelGGL(generic_int_kernel, grid, dim3(64), 0, stream, a);
     }

@@ -160,7 +160,7 @@ int gla_select_config(const gla_matmul_args* args);
 /* Which kernel family gla_matmul would run for a problem: one of GLA_FAMILY_*, or a negative
  * status.  No counterpart in the reference (its registry maps a matmul type to one Triton class,
  * gemlite/core.py:57-67); here several families serve one type, and tests and tuners ask which. */
-#define GLA_FAMILY_GENERIC 0      /* layout-agnostic kernel, any mode and stride */
+#define GLA_FAMILY_GENERIC 0      /* layout-agnostic kernels, any mode and stride (packed codes in short groups: K split over waves) */
 #define GLA_FAMILY_GEMV_PACKED 1  /* streaming kernels for 32-bit packed codes: up to 16 rows, up to 64 on small layers */
 #define GLA_FAMILY_GEMV_KMAJOR 2  /* streaming kernels for K-major weight bytes: 16-bit activations up to 16 rows, fp8 / int8 ones up to 4 */
 #define GLA_FAMILY_GEMM_WN 3      /* fused-dequant MFMA GEMM for packed 2/4/8-bit codes */

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import gemlite_amd
-from gemlite_amd import DType, GemLiteLinear, helper
+from gemlite_amd import DType, GemLiteLinear, _ext, helper
 from gemlite_amd.bitpack import pack_weights_over_cols_hip, unpack_over_cols_hip
 from oracle import oracle as orc
 from parity import (FROB_TOL, elementwise_excess, gen_int_case, gen_x, kind_of, oracle_forward, rel_frob, round_like,
@@ -247,6 +247,35 @@ def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
     layer = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device))
     for M in (1, 4, 7, 24, 64, 100, 200):   # above 16 rows: every tile height of the MFMA GEMM
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
+
+
+@pytest.mark.parametrize("nbits,gs", [(1, 32), (1, 64), (2, 16), (2, 32), (4, 16), (8, 16)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_packed_codes_in_short_groups(device, nbits, gs, dtype):
+    """Groups shorter than a step of the tuned kernels: the generic family's K-split packed-word kernel.  N is not a
+    multiple of 64 (lanes past N), K gives some waves no word row (1-bit: 10 word rows for 16 waves) or splits groups
+    between waves, rows 1 / 2 / 4 per lane and a ragged last block; scale-only, shift-only and scalar-zero modes."""
+    dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
+    for N, K in ((200, 320), (1000, 2112)):
+        W_q, scales, zeros = gen_int_case(N, K, nbits, gs, dtype, seed=nbits * 100 + gs)
+        layer = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device))
+        x1 = gen_x(1, K, dtype, seed=1).to(device)
+        a = _ext.build_matmul_args(x1, layer.W_q, layer.scales, layer.zeros, None, torch.empty(1, N, dtype=dtype, device=device),
+                                   **dict(zip(("W_nbits", "group_size", "unpack_mask", "elements_per_sample", "input_dtype", "output_dtype",
+                                               "acc_dtype", "meta_dtype", "channel_scale_mode", "W_group_mode", "data_contiguous"),
+                                              layer.get_meta_args()[1:12])))
+        assert _ext.matmul_family(a) == "GENERIC"
+        for M in (1, 2, 3, 4, 9, 21):
+            check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype, types=())
+    N, K = 328, 1088
+    W_q, scales, _ = gen_int_case(N, K, nbits, gs, dtype, seed=5)
+    l2 = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), None)                 # scales only
+    l3 = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), 1 if nbits < 4 else 3)  # one integer zero
+    l1 = GemLiteLinear(nbits, gs, K, N, dt, DType.FP32).pack(W_q.to(device), None, 1)                          # shift only
+    assert (l2.W_group_mode, l3.W_group_mode, l1.W_group_mode) == (2, 3, 1)
+    for layer, tol in ((l2, dtype), (l3, dtype), (l1, torch.float32)):
+        for M in (1, 6):
+            check_layer(layer, (gen_x(M, K, dtype, seed=M) / 10).to(device), tol, types=())
 
 
 @pytest.mark.parametrize("post_scale", [True, False])
