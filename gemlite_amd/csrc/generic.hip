@@ -287,6 +287,173 @@ void launch_packed_bits(const GenericArgs& a, hipStream_t stream) {
     }
 }
 
+// 16-bit weights [K, N] (no codes, no groups) x 16-bit activations: the same K split over 16 waves, 8 K-values per
+// step with their 8 weight loads in flight together.
+template <bool WBF16, bool XBF16, int RP>
+__global__ __launch_bounds__(64 * kPackedWaves) void generic_w16_kernel(GenericArgs a) {
+    __shared__ float red[kPackedWaves][RP][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n_raw = blockIdx.x * 64 + lane;
+    const int n = n_raw < a.N ? n_raw : a.N - 1;
+    const int m0 = blockIdx.y * RP;
+    const int steps = a.K / 8;
+    const int spw = (steps + kPackedWaves - 1) / kPackedWaves;
+    const int s_end = (wv + 1) * spw < steps ? (wv + 1) * spw : steps;
+    const uint16_t* xrow[RP];
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) {
+        const int m = m0 + rr < a.M ? m0 + rr : a.M - 1;
+        xrow[rr] = (const uint16_t*)a.x + (int64_t)m * a.xsm;
+    }
+    const uint16_t* wcol = (const uint16_t*)a.w + n;
+    float acc[RP];
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) acc[rr] = 0.0f;
+    for (int st = wv * spw; st < s_end; ++st) {
+        uint16_t wb[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) wb[j] = wcol[(int64_t)(st * 8 + j) * a.wsk];
+        uint32_t xw[RP][4];
+#pragma unroll
+        for (int rr = 0; rr < RP; ++rr) {
+            const uint4 v = *(const uint4*)(xrow[rr] + (int64_t)st * 8);
+            xw[rr][0] = v.x; xw[rr][1] = v.y; xw[rr][2] = v.z; xw[rr][3] = v.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float wf = WBF16 ? bf16_bits_to_float(wb[j]) : half_bits_to_float(wb[j]);
+#pragma unroll
+            for (int rr = 0; rr < RP; ++rr) {
+                const uint16_t bits = (uint16_t)(xw[rr][j / 2] >> ((j % 2) * 16));
+                acc[rr] = __builtin_fmaf(XBF16 ? bf16_bits_to_float(bits) : half_bits_to_float(bits), wf, acc[rr]);
+            }
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) red[wv][rr][lane] = acc[rr];
+    __syncthreads();
+    if (wv != 0 || n_raw >= a.N) return;
+    float sb = 1.0f;
+    if (a.csm == GLA_CSM_WEIGHT || a.csm == GLA_CSM_BOTH) sb = load_as_float(a.scales, a.meta_dt, n);
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) {
+        const int m = m0 + rr;
+        if (m >= a.M) continue;
+        float v = 0.0f;
+        for (int w = 0; w < kPackedWaves; ++w) v += red[w][rr][lane];
+        float sa = 1.0f;
+        if (a.csm == GLA_CSM_ACTIVATION || a.csm == GLA_CSM_BOTH) sa = load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
+        if (a.csm == GLA_CSM_WEIGHT) v *= sb;
+        else if (a.csm == GLA_CSM_ACTIVATION) v *= sa;
+        else if (a.csm == GLA_CSM_BOTH) v *= (sa * sb);
+        store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, v);
+    }
+}
+
+// what generic_w16_kernel assumes of a call
+bool w16_ok(const gla_matmul_args& p) {
+    if (!(p.w_dtype == GLA_DT_FP16 || p.w_dtype == GLA_DT_BF16) || p.w == nullptr || p.x == nullptr) return false;
+    if (p.elements_per_sample != 1 || p.W_group_mode != GLA_WGM_NONE) return false;
+    if (!(p.input_dtype == GLA_DT_FP16 || p.input_dtype == GLA_DT_BF16) || p.acc_dtype != GLA_DT_FP32) return false;
+    if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
+    if (p.channel_scale_mode < GLA_CSM_NONE || p.channel_scale_mode > GLA_CSM_BOTH) return false;
+    if (p.M < 1 || p.N < 1 || p.K < 8 || p.K % 8 != 0) return false;
+    if (p.x_stride_k != 1 || p.x_stride_m % 8 != 0 || ((uintptr_t)p.x & 15)) return false;
+    // N contiguous, or K contiguous with rows that 128-bit loads can read
+    const bool kmajor = p.w_stride_k == 1 && p.w_stride_n % 8 == 0 && !((uintptr_t)p.w & 15);
+    if (p.w_stride_n != 1 && !kmajor) return false;
+    if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
+    if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
+    return true;
+}
+
+template <bool WBF16, bool XBF16>
+void launch_w16_rows(const GenericArgs& a, hipStream_t stream) {
+    const int rp = a.M >= 3 ? 4 : a.M;
+    const dim3 grid(ceil_div(a.N, 64), ceil_div(a.M, rp)), block(64 * kPackedWaves);
+    if (rp == 4) hipLaunchKernelGGL((generic_w16_kernel<WBF16, XBF16, 4>), grid, block, 0, stream, a);
+    else if (rp == 2) hipLaunchKernelGGL((generic_w16_kernel<WBF16, XBF16, 2>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((generic_w16_kernel<WBF16, XBF16, 1>), grid, block, 0, stream, a);
+}
+
+// 16-bit weights as the layer classes keep them, [N, K] with K contiguous: one wave per two output columns, the
+// lanes along K with 128-bit loads, a butterfly sum over the wave at the end.
+template <bool WBF16, bool XBF16, int RP>
+__global__ __launch_bounds__(256) void generic_w16_kmajor_kernel(GenericArgs a) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n0 = (blockIdx.x * 4 + wv) * 2;
+    if (n0 >= a.N) return;  // (no barrier below)
+    const bool two = n0 + 1 < a.N;
+    const int m0 = blockIdx.y * RP;
+    const uint16_t* wrow[2] = {(const uint16_t*)a.w + (int64_t)n0 * a.wsn, (const uint16_t*)a.w + (int64_t)(two ? n0 + 1 : n0) * a.wsn};
+    const uint16_t* xrow[RP];
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) {
+        const int m = m0 + rr < a.M ? m0 + rr : a.M - 1;
+        xrow[rr] = (const uint16_t*)a.x + (int64_t)m * a.xsm;
+    }
+    float acc[RP][2];
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr) acc[rr][0] = acc[rr][1] = 0.0f;
+    for (int k = lane * 8; k < a.K; k += 512) {
+        uint32_t ww[2][4];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint4 v = *(const uint4*)(wrow[c] + k);
+            ww[c][0] = v.x; ww[c][1] = v.y; ww[c][2] = v.z; ww[c][3] = v.w;
+        }
+#pragma unroll
+        for (int rr = 0; rr < RP; ++rr) {
+            const uint4 v = *(const uint4*)(xrow[rr] + k);
+            const uint32_t xw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint16_t xb = (uint16_t)(xw[j / 2] >> ((j % 2) * 16));
+                const float xf = XBF16 ? bf16_bits_to_float(xb) : half_bits_to_float(xb);
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const uint16_t wb = (uint16_t)(ww[c][j / 2] >> ((j % 2) * 16));
+                    acc[rr][c] = __builtin_fmaf(xf, WBF16 ? bf16_bits_to_float(wb) : half_bits_to_float(wb), acc[rr][c]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < RP; ++rr)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) acc[rr][c] += __shfl_xor(acc[rr][c], off, 64);
+    if (lane != 0) return;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        if (c == 1 && !two) break;
+        const int n = n0 + c;
+        float sb = 1.0f;
+        if (a.csm == GLA_CSM_WEIGHT || a.csm == GLA_CSM_BOTH) sb = load_as_float(a.scales, a.meta_dt, n);
+#pragma unroll
+        for (int rr = 0; rr < RP; ++rr) {
+            const int m = m0 + rr;
+            if (m >= a.M) continue;
+            float v = acc[rr][c], sa = 1.0f;
+            if (a.csm == GLA_CSM_ACTIVATION || a.csm == GLA_CSM_BOTH) sa = load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
+            if (a.csm == GLA_CSM_WEIGHT) v *= sb;
+            else if (a.csm == GLA_CSM_ACTIVATION) v *= sa;
+            else if (a.csm == GLA_CSM_BOTH) v *= (sa * sb);
+            store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, v);
+        }
+    }
+}
+
+template <bool WBF16, bool XBF16>
+void launch_w16_kmajor_rows(const GenericArgs& a, hipStream_t stream) {
+    const int rp = a.M >= 3 ? 4 : a.M;
+    const dim3 grid(ceil_div(a.N, 8), ceil_div(a.M, rp)), block(256);
+    if (rp == 4) hipLaunchKernelGGL((generic_w16_kmajor_kernel<WBF16, XBF16, 4>), grid, block, 0, stream, a);
+    else if (rp == 2) hipLaunchKernelGGL((generic_w16_kmajor_kernel<WBF16, XBF16, 2>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((generic_w16_kmajor_kernel<WBF16, XBF16, 1>), grid, block, 0, stream, a);
+}
+
 // e2m1 x e2m1 with e8m0 block scales on both operands (block = 32 along K).
 __global__ __launch_bounds__(64) void generic_mxfp4_kernel(GenericArgs a) {
     const int n = blockIdx.x * 64 + threadIdx.x;
@@ -390,6 +557,17 @@ int launch_generic(const gla_matmul_args& p, hipStream_t stream) {
             return GLA_ERR_UNSUPPORTED_MODE;
         }
         hipLaunchKernelGGL(generic_mxfp4_kernel, grid, dim3(64), 0, stream, a);
+    } else if (w16_ok(p)) {
+        const bool wb = p.w_dtype == GLA_DT_BF16, xb = p.input_dtype == GLA_DT_BF16;
+        if (p.w_stride_n != 1) {
+            if (wb && xb) launch_w16_kmajor_rows<true, true>(a, stream);
+            else if (wb) launch_w16_kmajor_rows<true, false>(a, stream);
+            else if (xb) launch_w16_kmajor_rows<false, true>(a, stream);
+            else launch_w16_kmajor_rows<false, false>(a, stream);
+        } else if (wb && xb) launch_w16_rows<true, true>(a, stream);
+        else if (wb) launch_w16_rows<true, false>(a, stream);
+        else if (xb) launch_w16_rows<false, true>(a, stream);
+        else launch_w16_rows<false, false>(a, stream);
     } else if (packed_words_ok(p)) {
         if (p.input_dtype == GLA_DT_BF16) launch_packed_bits<true>(a, stream);
         else launch_packed_bits<false>(a, stream);

@@ -320,6 +320,22 @@ def test_unpacked_fp16_weights_and_bias(device):
     assert y.shape == (2, 3, N)
 
 
+@pytest.mark.parametrize("contiguous", [None, True])
+@pytest.mark.parametrize("w_dtype,x_dtype", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float16), (torch.float16, torch.bfloat16)])
+def test_unpacked_16_bit_weights_both_layouts(device, contiguous, w_dtype, x_dtype):
+    """16-bit weights as the layer keeps them ([N, K], K contiguous: a wave per two columns, lanes along K) and as
+    pack(contiguous=True) makes them ([K, N]: a lane per column, K split over the waves); N odd or not a multiple of
+    64, K not a multiple of the 512 values a wave covers per step, 1 / 2 / 4 rows per lane and a ragged last block."""
+    xdt = gemlite_amd.TORCH_TO_DTYPE[x_dtype]
+    for N, K in ((1000, 2048), (77, 224), (4096, 4128)):
+        W = gen_x(N, K, w_dtype, seed=N, std=0.05)
+        layer = GemLiteLinear(16, None, K, N, xdt, xdt).pack(W.to(device), None, None, contiguous=contiguous)
+        assert layer.data_contiguous == bool(contiguous) and layer.W_q.stride(1) == (1 if contiguous else K)
+        for M in (1, 2, 3, 4, 9, 18):
+            check_layer(layer, gen_x(M, K, x_dtype, seed=M).to(device), x_dtype, types=())
+
+
 @pytest.mark.parametrize("width", [8, 16, 64])
 def test_other_packing_widths(device, width):
     N, K, gs = 256, 512, 64
