@@ -179,6 +179,28 @@ def extra_points(lib, device, T, quick):
         us, nbytes, copies=len(layers), frac_of_read_ceiling=round(nbytes / us / 1e3 / ceil["9MB"]["GB/s"], 4))
     del layers
 
+    # ---- the generic family's vector kernels at M = 1: 1-bit codes in groups of 64 (shorter than a step of the
+    # streaming kernel) and 16-bit weights, both 4096 -> 14336
+    Ng, Kg = 14336, 4096
+    W1 = torch.randint(0, 2, (Ng, Kg), generator=g, dtype=torch.int32).to(torch.uint8)
+    s1 = (torch.randn((Ng * Kg // 64, 1), generator=g) * 0.02).abs().to(torch.float16)
+    z1 = torch.rand((Ng * Kg // 64, 1), generator=g).to(torch.float16)
+    base1 = GemLiteLinear(1, 64, Kg, Ng, DType.FP16, DType.FP16).pack(W1.to(device), s1.to(device), z1.to(device))
+    nbytes = algorithmic_bytes(Ng, Kg, nbits=1, gs=64)
+    layers = [base1] + [clone_layer(base1) for _ in range(copies_for(nbytes) - 1)]
+    yg = torch.empty((1, Ng), dtype=torch.float16, device=device)
+    us = T.graph_us([Launch(lib, l, x1, yg, device) for l in layers], 10)
+    out["gemv_a16w1_gs64_M1"] = bw_point(us, nbytes, copies=len(layers), N=Ng, K=Kg)
+    del layers, base1, W1, s1, z1
+    W16 = (torch.randn((Ng, Kg), generator=g) * 0.02).to(torch.float16)
+    nbytes = Ng * Kg * 2 + Kg * 2 + Ng * 2
+    layers = [GemLiteLinear(16, None, Kg, Ng, DType.FP16, DType.FP16).pack(W16.to(device), None, None)
+              for _ in range(copies_for(nbytes))]
+    us = T.graph_us([Launch(lib, l, x1, yg, device) for l in layers], 10)
+    out["gemv_a16w16_fp16_M1"] = bw_point(us, nbytes, copies=len(layers), N=Ng, K=Kg)
+    del layers, W16
+    torch.cuda.empty_cache()
+
     # Sustained matrix rate of this board: a register-only MFMA loop (no memory traffic) with zero and
     # with random operand bits.  With random bits the power limit lowers the clock; that rate, not the
     # datasheet one, is what a GEMM on real data can at most reach here.
