@@ -43,8 +43,6 @@ constexpr int kCounterStride = 32;  // words between the counters of two column 
                                     // one line, the 256 tickets of a launch queued up there for ~2 us
 constexpr int64_t kSlotBytes = kWsPrivateBytes - kWsCounterBytes;  // tagged partial slots, private to this family
 constexpr uint32_t kSlotValid = 0x7fc5a11du;  // tag of a published slot; a consumed slot is all zeros
-constexpr int kSpinLimit = 1 << 22;           // polls of a slot whose store is in flight (it has been issued)
-constexpr int kSpec = 8;                      // slots read ahead of the ticket
 
 struct GemvArgs {
     const uint32_t* w;
@@ -175,9 +173,11 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
     // loaded before the reduction, so that its latency is not the kernel's tail
     const float bias = (a.bias != nullptr && col_ok) ? load_as_float(a.bias, a.bias_dt, n_out) : 0.0f;
     float total[NT];
+    bool alive[NT];  // this thread still owes the output element of row t
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int m = wv + t * waves;
+        alive[t] = true;
         float v = 0.0f;
         if (m < RT) {
             for (int w2 = 0; w2 < waves; ++w2) v += red[((size_t)w2 * RT + m) * kTileN + lane];
@@ -186,81 +186,40 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
     }
 
     if (a.S > 1 && a.slots != nullptr) {
-        // ---- tagged protocol.  Publish (value, tag) slots, then ticket and read-ahead together.
+        // ---- exchange tree.  The slabs of a column tile are the leaves of a binary tree; at every level the
+        // two children of a node meet in one 64-bit slot: each swaps (value, tag) into it with one atomic
+        // exchange.  The child that finds the slot empty has left its partial there and is done; the one that
+        // finds the other's partial adds it to its own (a sum of two floats does not depend on who came first),
+        // empties the slot for the next launch and climbs.  The root stores the output.  Every thread decides for
+        // its own output element: no ticket, no barrier, no polling, and the last arriver is log2(S) atomic
+        // round trips from the end.  The sum order is the tree's, whatever the order of arrival.
         const size_t stride = (size_t)a.Mp * a.N;
-        unsigned long long* mine[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int m = wv + t * waves;
-            mine[t] = a.slots + (size_t)(m0 + (m < RT ? m : 0)) * a.N + (col_ok ? n_out : 0);
-            if (m < RT && col_ok)
-                __hip_atomic_store(mine[t] + (size_t)split * stride,
-                                   ((unsigned long long)kSlotValid << 32) | __builtin_bit_cast(uint32_t, total[t]),
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads();  // every wave of this workgroup has issued its slot stores
-        // The ticket is issued here and awaited below, after the read-ahead loads have been issued
-        // too: written as __hip_atomic_fetch_add the compiler waits for the returned value on the
-        // spot (it funnels the one-lane add through a wave-wide reduction), which would put the
-        // ticket's round trip in front of the loads' instead of beside it.  Same instruction and
-        // cache policy as the compiler emits for an agent-scope relaxed fetch-add.
-        unsigned tk = 0;
-        if (tid == 0) {
-            unsigned* cnt = a.counters + (size_t)(blockIdx.y * a.tiles + tile) * kCounterStride;
-            const unsigned one = 1u;
-            asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(tk) : "v"(cnt), "v"(one) : "memory");
-        }
-        // Read ahead the first kSpec slabs' slots while the ticket is on its way (one output row per
-        // thread only: more rows would cost more registers than the round trip is worth).
-        unsigned long long ahead[kSpec];
-        if constexpr (NT == 1) {
-            const bool live = (wv < RT) && col_ok;
-#pragma unroll
-            for (int u = 0; u < kSpec; ++u) {
-                ahead[u] = 0ull;
-                if (live && u < a.S && u != split)
-                    ahead[u] = __hip_atomic_load(mine[0] + (size_t)u * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(tk) : : "memory");  // ticket and read-ahead have returned
-        if (tid == 0) ticket = tk;
-        __syncthreads();
-        if (ticket != (unsigned)(a.S - 1)) return;
-        // ---- last arriver: every other slab's stores were issued before its ticket, so a slot that is
-        // not valid yet is in flight and a bounded poll gets it.  Sum in slab order.
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const int m = wv + t * waves;
-            if (!(m < RT && col_ok)) continue;
-            float v = 0.0f;
-            for (int sl = 0; sl < a.S; ++sl) {
-                if (sl == split) {
-                    v += total[t];
-                    continue;
-                }
-                unsigned long long q = 0ull;
-                if constexpr (NT == 1) {
-                    if (sl < kSpec) {
-#pragma unroll
-                        for (int u = 0; u < kSpec; ++u)
-                            if (u == sl) q = ahead[u];
+            alive[t] = m < RT && col_ok;
+            if (!alive[t]) continue;
+            unsigned long long* lvl = a.slots + (size_t)(m0 + m) * a.N + n_out;
+            float v = total[t];
+            int node = split;
+            for (int nodes = a.S; nodes > 1; nodes = (nodes + 1) >> 1) {
+                const int pair = node >> 1;
+                if ((node ^ 1) < nodes) {  // an odd node out climbs without meeting anybody
+                    unsigned long long* slot = lvl + (size_t)pair * stride;
+                    const unsigned long long mine = ((unsigned long long)kSlotValid << 32) | __builtin_bit_cast(uint32_t, v);
+                    const unsigned long long was = __hip_atomic_exchange(slot, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if ((uint32_t)(was >> 32) != kSlotValid) {
+                        alive[t] = false;
+                        break;
                     }
+                    v += __builtin_bit_cast(float, (uint32_t)was);
+                    __hip_atomic_store(slot, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
-                unsigned long long* src = mine[t] + (size_t)sl * stride;
-                for (int tries = 0; (uint32_t)(q >> 32) != kSlotValid && tries < kSpinLimit; ++tries)
-                    q = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                // a slot that never turned valid cannot happen with a healthy memory system; make it loud
-                v += (uint32_t)(q >> 32) == kSlotValid ? __builtin_bit_cast(float, (uint32_t)q)
-                                                       : __builtin_bit_cast(float, 0x7fc00000u);
+                lvl += (size_t)((nodes + 1) >> 1) * stride;
+                node = pair;
             }
             total[t] = v;
-            // leave the slots invalid and the counter at zero for the next launch
-            for (int sl = 0; sl < a.S; ++sl)
-                __hip_atomic_store(mine[t] + (size_t)sl * stride, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (tid == 0)
-            __hip_atomic_store(a.counters + (size_t)(blockIdx.y * a.tiles + tile) * kCounterStride, 0u, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
     } else if (a.S > 1) {
         // ---- plain protocol (partials too large for the slot region): publish this slab's partial, wait
         // for it to land, then take a ticket; the last slab to arrive sums all
@@ -312,7 +271,7 @@ __device__ __forceinline__ void wg_finish(const GemvArgs& a, float (&acc)[4][RI]
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int m = wv + t * waves;
-        if (m >= RT || !col_ok || (m0 + m) >= a.M) continue;
+        if (m >= RT || !col_ok || (m0 + m) >= a.M || !alive[t]) continue;
         float v = total[t];
         if (a.csm == GLA_CSM_WEIGHT) {
             v *= load_as_float(a.scales, a.meta_dt, n_out);
