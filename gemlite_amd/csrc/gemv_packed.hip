@@ -140,6 +140,37 @@ __device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t m
     return (w & mask) | magic;
 }
 
+// Lane l of every row of 16 lanes receives the value of lane l + n of the same row (lanes past the row's end: zero).
+// n is a constant after unrolling.
+template <int N>
+__device__ __forceinline__ uint32_t row_down_c(uint32_t v) {
+    if constexpr (N == 0) return v;
+    else return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x100 + N, 0xf, 0xf, true);  // row_shl:N
+}
+__device__ __forceinline__ uint32_t row_down(uint32_t v, int n) {
+    switch (n) {
+        case 1: return row_down_c<1>(v);
+        case 2: return row_down_c<2>(v);
+        case 3: return row_down_c<3>(v);
+        case 4: return row_down_c<4>(v);
+        case 5: return row_down_c<5>(v);
+        case 6: return row_down_c<6>(v);
+        case 7: return row_down_c<7>(v);
+        case 8: return row_down_c<8>(v);
+        case 9: return row_down_c<9>(v);
+        case 10: return row_down_c<10>(v);
+        case 11: return row_down_c<11>(v);
+        case 12: return row_down_c<12>(v);
+        case 13: return row_down_c<13>(v);
+        case 14: return row_down_c<14>(v);
+        case 15: return row_down_c<15>(v);
+        default: return v;
+    }
+}
+__device__ __forceinline__ uint4 row_down(const uint4& v, int n) {
+    return make_uint4(row_down(v.x, n), row_down(v.y, n), row_down(v.z, n), row_down(v.w, n));
+}
+
 __device__ __forceinline__ uint32_t pick(const uint4& v, int j) {
     return j == 0 ? v.x : (j == 1 ? v.y : (j == 2 ? v.z : v.w));
 }
@@ -532,13 +563,23 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_packed_kernel(GemvArgs a) {
 // ---------------------------------------------------------------------------------------------
 // kWaves = 0: the wave count is blockDim.x / 64, any number from 4 to 16 (row tiles up to 4), so that
 // the K slabs of a column tile can be cut equal: 56 wave-batches are 4 slabs of 14 waves, not 16/16/16/8.
-template <int BITS, bool BF16, int RT, int kWaves, bool LOOP>
+// FLC: wave iterations per fold when the host knows them to be 4 (the usual group of 128), else 0 (a.FL decides):
+// with the folds at fixed places of the unrolled batch, the accumulators of a group start from the MFMA's zero
+// operand instead of being cleared, and no branch stands between the iterations.
+template <int BITS, bool BF16, int RT, int kWaves, bool LOOP, int FLC = 0>
 __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kernel(GemvArgs a) {
     using SH = Shape<BITS>;
     constexpr int E = SH::E, LW = SH::LW, T = SH::T;  // T MFMA K-steps per super row (2 for 2-bit codes)
     static_assert(BITS == 2 || BITS == 4 || BITS == 8, "direct variant: 2-, 4- and 8-bit codes");
     constexpr int RI = RT < 4 ? RT : 4;  // accumulator rows a lane folds
     constexpr int IPB = kBatch / LW;  // wave iterations per batch
+    // Up to 4 rows the 16 rows of the MFMA's A operand are mostly idle, so one activation load serves several
+    // iterations: lane (quarter q, i) loads the chunk of iteration i / RT for row i % RT, and iteration u takes
+    // its A operand from the lanes RT * u further up the row of 16 (a DPP move per register instead of a load
+    // per iteration: an eighth of the activation requests at one row).
+    constexpr bool XS = RT <= 4 && T == 1;
+    constexpr int IPL = XS ? ((16 / RT) < IPB ? (16 / RT) : IPB) : 1;  // iterations per activation load
+    constexpr int NXL = XS ? IPB / IPL : IPB * T;                       // activation loads per batch
     // 8-bit codes with bf16 activations: 128 + q is exact in bf16 only up to q = 127, so a code is fed as
     // two nibbles, q = lo + 16 hi: one MFMA multiplies x by 128 + lo, a second 16 x by 128 + hi, both into
     // the same accumulator, which then holds sum x q + 128 * 17 * sum x.
@@ -583,8 +624,12 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     const uint32_t w_lim = (uint32_t)col * 4u + (uint32_t)(wrow0 < a.R - 1 ? a.R - 1 - wrow0 : 0) * sb;
     const int x_rel_max = a.R - LW - wrow0;  // rows this wave may still multiply (negative: none)
     const char* xs_base = (const char*)a.x + (int64_t)(x_rel_max > 0 ? wrow0 : a.R - LW) * (E * 2);
+    if constexpr (XS) {  // lane (kb, cg): row cg % RT of iteration cg / RT (lanes past the last iteration repeat)
+        mrow = m0 + (cg % RT);
+        if (mrow > a.M - 1) mrow = a.M - 1;
+    }
     const uint32_t x_lane0 = (uint32_t)mrow * (uint32_t)a.xsm * 2u;
-    const uint32_t x_lane = x_lane0 + (uint32_t)(kb * LW * E * 2);
+    const uint32_t x_lane = x_lane0 + (uint32_t)((XS ? 4 * ((cg / RT) % IPL) + kb : kb) * LW * E * 2);
     const uint32_t x_lim = x_lane0 + (uint32_t)(x_rel_max > 0 ? x_rel_max : 0) * (uint32_t)(E * 2);
     const char* ss_base = (const char*)a.scales + (int64_t)g0w * a.msg * 2;
     const char* zs_base = (const char*)a.zeros + (int64_t)g0w * a.msg * 2;
@@ -593,9 +638,9 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
 
     struct Batch {
         uint2 sr[2], zr[2];
-        uint4 xr[IPB * T];
+        uint4 xr[NXL];
         uint4 wr[kBatch];
-        unsigned xvalid;  // bit u: iteration u of the batch lies inside K (a ragged last slab runs past it)
+        unsigned xvalid;  // bit u: activation load u of the batch lies inside K (a ragged last slab runs past it)
     };
 
     // group (relative to g0w) whose fold closes flush block `fbl` of the batch starting at iteration ib
@@ -613,12 +658,23 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
     // weight words arrive.
     auto issue = [&](int ib, Batch& b) {
         b.xvalid = 0;
-        auto pair = [&](int u) __attribute__((always_inline)) {
-            uint32_t xo = x_lane + (uint32_t)(4 * (ib + u) * LW * E * 2);
-            if (x_rel_max >= 0 && xo <= x_lim) b.xvalid |= 1u << u;
-            else xo = x_lim;  // loads stay in bounds; the activations are zeroed when they are used
+        if constexpr (XS) {
 #pragma unroll
-            for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xs_base + xo + 16 * t);
+            for (int xl = 0; xl < NXL; ++xl) {
+                uint32_t xo = x_lane + (uint32_t)(4 * (ib + xl * IPL) * LW * E * 2);
+                if (x_rel_max >= 0 && xo <= x_lim) b.xvalid |= 1u << xl;
+                else xo = x_lim;  // loads stay in bounds; the chunk is zeroed when it is used
+                b.xr[xl] = *(const uint4*)(xs_base + xo);
+            }
+        }
+        auto pair = [&](int u) __attribute__((always_inline)) {
+            if constexpr (!XS) {
+                uint32_t xo = x_lane + (uint32_t)(4 * (ib + u) * LW * E * 2);
+                if (x_rel_max >= 0 && xo <= x_lim) b.xvalid |= 1u << u;
+                else xo = x_lim;  // loads stay in bounds; the activations are zeroed when they are used
+#pragma unroll
+                for (int t = 0; t < T; ++t) b.xr[u * T + t] = *(const uint4*)(xs_base + xo + 16 * t);
+            }
 #pragma unroll
             for (int v = 0; v < LW; ++v) {
                 uint32_t wo = w_lane + (uint32_t)(4 * (ib + u) * LW + v) * sb;
@@ -655,7 +711,9 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
         for (int i = 0; i < RI; ++i) acc[j][i] = 0.0f;
     }
     csx = float4_t{0.f, 0.f, 0.f, 0.f};
-    const uint4 ones = make_uint4(Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones);
+    uint4 ones = make_uint4(Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones, Magic<BF16>::ones);
+    // four registers that stay put: left to itself the compiler builds the operand anew before every use
+    asm volatile("" : "+v"(ones.x), "+v"(ones.y), "+v"(ones.z), "+v"(ones.w));
     uint32_t pair_mask = kPairMask, magic = Magic<BF16>::bits;
     asm volatile("" : "+s"(pair_mask), "+v"(magic));  // keep both in registers, not literals
     const int fl_mask = a.FL - 1;                      // FL is a power of two
@@ -696,48 +754,67 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
         __builtin_amdgcn_wave_barrier();
     };
 
+    // chunk of 8 activations as loaded -> the pair order of the code extraction (one K-step)
+    auto pair_order = [&](const uint4& xr) {
+        uint4 av;
+        if constexpr (E == 8) {  // pairs (j, j + 4)
+            av.x = __builtin_amdgcn_perm(xr.z, xr.x, 0x05040100u);
+            av.y = __builtin_amdgcn_perm(xr.z, xr.x, 0x07060302u);
+            av.z = __builtin_amdgcn_perm(xr.w, xr.y, 0x05040100u);
+            av.w = __builtin_amdgcn_perm(xr.w, xr.y, 0x07060302u);
+        } else {  // two words of 4 codes: pairs (j, j + 2) inside each word
+            av.x = __builtin_amdgcn_perm(xr.y, xr.x, 0x05040100u);
+            av.y = __builtin_amdgcn_perm(xr.y, xr.x, 0x07060302u);
+            av.z = __builtin_amdgcn_perm(xr.w, xr.z, 0x05040100u);
+            av.w = __builtin_amdgcn_perm(xr.w, xr.z, 0x07060302u);
+        }
+        return av;
+    };
+    // 16 x: add 4 to the exponent of every non-zero bf16 half (zeros and denormals stay)
+    auto times16 = [](uint32_t v) {
+        const uint32_t lo_nz = (v & 0x00007f80u) ? 0x00000200u : 0u;
+        const uint32_t hi_nz = (v & 0x7f800000u) ? 0x02000000u : 0u;
+        return v + (lo_nz | hi_nz);
+    };
+
     auto process = [&](int ib, const Batch& b) {
         stage_meta(ib, b);
+        const uint4 zero4 = make_uint4(0, 0, 0, 0);
+        // shared activation loads: zero what lies past K, order the pairs once per load
+        uint4 xp[XS ? NXL : 1], xp16[XS ? NXL : 1];
+        if constexpr (XS) {
+#pragma unroll
+            for (int xl = 0; xl < NXL; ++xl) {
+                xp[xl] = pair_order(((b.xvalid >> xl) & 1u) ? b.xr[xl] : zero4);
+                if constexpr (SPLIT8)
+                    xp16[xl] = make_uint4(times16(xp[xl].x), times16(xp[xl].y), times16(xp[xl].z), times16(xp[xl].w));
+            }
+        }
 #pragma unroll
         for (int ii = 0; ii < IPB; ++ii) {
             const int it = ib + ii;
+            // first iteration after a fold: the accumulators start from zero (FLC: known at compile time)
 #pragma unroll
             for (int t = 0; t < T; ++t) {
-                // activation chunk -> the pair order of the code extraction
-                uint4 av;
-                const bool xok = (b.xvalid >> ii) & 1u;
-                const uint4 zero4 = make_uint4(0, 0, 0, 0);
-                if constexpr (E == 16) {  // 16 codes per word: K-step t pairs (4t + r, 4t + r + 8)
-                    const uint4 lo = xok ? b.xr[ii * T] : zero4, hi = xok ? b.xr[ii * T + 1] : zero4;
-                    const uint32_t l0 = t ? lo.z : lo.x, l1 = t ? lo.w : lo.y, h0 = t ? hi.z : hi.x, h1 = t ? hi.w : hi.y;
-                    av.x = __builtin_amdgcn_perm(h0, l0, 0x05040100u);
-                    av.y = __builtin_amdgcn_perm(h0, l0, 0x07060302u);
-                    av.z = __builtin_amdgcn_perm(h1, l1, 0x05040100u);
-                    av.w = __builtin_amdgcn_perm(h1, l1, 0x07060302u);
-                } else if constexpr (E == 8) {  // pairs (j, j + 4)
-                    const uint4 xr = xok ? b.xr[ii] : zero4;
-                    av.x = __builtin_amdgcn_perm(xr.z, xr.x, 0x05040100u);
-                    av.y = __builtin_amdgcn_perm(xr.z, xr.x, 0x07060302u);
-                    av.z = __builtin_amdgcn_perm(xr.w, xr.y, 0x05040100u);
-                    av.w = __builtin_amdgcn_perm(xr.w, xr.y, 0x07060302u);
-                } else {  // two words of 4 codes: pairs (j, j + 2) inside each word
-                    const uint4 xr = xok ? b.xr[ii] : zero4;
-                    av.x = __builtin_amdgcn_perm(xr.y, xr.x, 0x05040100u);
-                    av.y = __builtin_amdgcn_perm(xr.y, xr.x, 0x07060302u);
-                    av.z = __builtin_amdgcn_perm(xr.w, xr.z, 0x05040100u);
-                    av.w = __builtin_amdgcn_perm(xr.w, xr.z, 0x07060302u);
+                uint4 av, av16;
+                if constexpr (XS) {
+                    av = row_down(xp[ii / IPL], RT * (ii % IPL));
+                    if constexpr (SPLIT8) av16 = row_down(xp16[ii / IPL], RT * (ii % IPL));
+                } else {
+                    const bool xok = (b.xvalid >> ii) & 1u;
+                    if constexpr (E == 16) {  // 16 codes per word: K-step t pairs (4t + r, 4t + r + 8)
+                        const uint4 lo = xok ? b.xr[ii * T] : zero4, hi = xok ? b.xr[ii * T + 1] : zero4;
+                        const uint32_t l0 = t ? lo.z : lo.x, l1 = t ? lo.w : lo.y, h0 = t ? hi.z : hi.x, h1 = t ? hi.w : hi.y;
+                        av.x = __builtin_amdgcn_perm(h0, l0, 0x05040100u);
+                        av.y = __builtin_amdgcn_perm(h0, l0, 0x07060302u);
+                        av.z = __builtin_amdgcn_perm(h1, l1, 0x05040100u);
+                        av.w = __builtin_amdgcn_perm(h1, l1, 0x07060302u);
+                    } else {
+                        av = pair_order(xok ? b.xr[ii] : zero4);
+                    }
+                    if constexpr (SPLIT8) av16 = make_uint4(times16(av.x), times16(av.y), times16(av.z), times16(av.w));
                 }
                 csx = mfma16<BF16>(av, ones, csx);
-                uint4 av16 = av;
-                if constexpr (SPLIT8) {
-                    // 16 x: add 4 to the exponent of every non-zero bf16 half (zeros and denormals stay)
-                    auto times16 = [](uint32_t v) {
-                        const uint32_t lo_nz = (v & 0x00007f80u) ? 0x00000200u : 0u;
-                        const uint32_t hi_nz = (v & 0x7f800000u) ? 0x02000000u : 0u;
-                        return v + (lo_nz | hi_nz);
-                    };
-                    av16 = make_uint4(times16(av.x), times16(av.y), times16(av.z), times16(av.w));
-                }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     uint32_t bq[4], bh[4];
@@ -755,8 +832,9 @@ __global__ __launch_bounds__(kWaves ? kWaves * 64 : 1024) void gemv_direct_kerne
                     if constexpr (SPLIT8) c[j] = mfma16<BF16>(av16, make_uint4(bh[0], bh[1], bh[2], bh[3]), c[j]);
                 }
             }
-            if (((it + 1) & fl_mask) == 0) {
-                const int fbl = (a.FL <= IPB) ? (((ii + 1) >> a.fl_log2) - 1) : 0;
+            const bool fold_now = FLC ? ((ii + 1) % (FLC ? FLC : 1) == 0) : (((it + 1) & fl_mask) == 0);
+            if (fold_now) {
+                const int fbl = FLC ? ((ii + 1) / (FLC ? FLC : 1) - 1) : ((a.FL <= IPB) ? (((ii + 1) >> a.fl_log2) - 1) : 0);
                 const float4* mrow = (const float4*)(mtw + fbl * kTileN + cg * 4);
                 const float4 m01 = mrow[0], m23 = mrow[1];
                 const float sj[4] = {m01.x, m01.z, m23.x, m23.z};
@@ -916,34 +994,48 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true, i
     return true;
 }
 
+// The single-batch direct kernel at the wave count the geometry chose.
+template <int BITS, bool BF16, int RT, int FLC>
+void launch_direct(const GemvArgs& a, const Geometry& g, dim3 grid, hipStream_t stream) {
+    if (g.waves == 16) {
+        if constexpr (RT == 16) {  // its cross-wave buffer alone is 64 KiB
+            static DeviceOnce once;
+            if (once.first())
+                (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 16, false, FLC>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
+        }
+        hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false, FLC>), grid, dim3(1024), g.smem, stream, a);
+    } else if (g.waves == 8) {
+        hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 8, false, FLC>), grid, dim3(512), g.smem, stream, a);
+    } else if (g.waves == 4) {
+        hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, false, FLC>), grid, dim3(256), g.smem, stream, a);
+    } else {
+        if constexpr (RT == 16) {  // a cross-wave buffer of up to 60 KiB
+            static DeviceOnce once;
+            if (once.first())
+                (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 0, false, FLC>,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
+        }
+        hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 0, false, FLC>), grid, dim3(g.waves * 64), g.smem, stream, a);
+    }
+}
+
 template <int BITS, bool BF16, int RT>
 void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
     dim3 grid(g.tiles, g.mchunks, g.S);
     if constexpr (BITS == 2 || BITS == 4 || BITS == 8) {
         if (g.direct) {
-            if (g.nb > 1)
+            if (g.nb > 1) {
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
-            else if (g.waves == 16) {
-                if constexpr (RT == 16) {  // its cross-wave buffer alone is 64 KiB
-                    static DeviceOnce once;
-                    if (once.first())
-                        (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 16, false>,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
-                }
-                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 16, false>), grid, dim3(1024), g.smem, stream, a);
-            } else if (g.waves == 8)
-                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 8, false>), grid, dim3(512), g.smem, stream, a);
-            else if (g.waves == 4)
-                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, false>), grid, dim3(256), g.smem, stream, a);
-            else {
-                if constexpr (RT == 16) {  // a cross-wave buffer of up to 60 KiB
-                    static DeviceOnce once;
-                    if (once.first())
-                        (void)hipFuncSetAttribute((const void*)gemv_direct_kernel<BITS, BF16, RT, 0, false>,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 100 * 1024);
-                }
-                hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 0, false>), grid, dim3(g.waves * 64), g.smem, stream, a);
+                return;
             }
+            if constexpr (RT <= 4 && (BITS == 4 || BITS == 8)) {
+                if (g.FL == 4) {  // groups of 128 (and channel-wise 8-bit codes): folds at fixed places of the batch
+                    launch_direct<BITS, BF16, RT, 4>(a, g, grid, stream);
+                    return;
+                }
+            }
+            launch_direct<BITS, BF16, RT, 0>(a, g, grid, stream);
             return;
         }
     }
