@@ -156,15 +156,26 @@ def extra_points(lib, device, T, quick):
         n = copies_for(nbytes)
         bufs = [torch.full((nbytes // 4,), 0x01010101, dtype=torch.int32, device=device) for _ in range(n)]
 
-        def reader(b):
+        def reader(b, shape):
             def run():
-                if lib.gla_probe_read(b.data_ptr(), b.numel() * 4, sink.data_ptr(), stream()) != 0:
+                rc = (lib.gla_probe_read(b.data_ptr(), b.numel() * 4, sink.data_ptr(), stream()) if shape is None else
+                      lib.gla_probe_read_cfg(b.data_ptr(), b.numel() * 4, sink.data_ptr(), *shape, stream()))
+                if rc != 0:
                     raise RuntimeError(lib.gla_last_error().decode())
             return run
-        us = T.graph_us([reader(b) for b in bufs], 4 if nbytes > 1e8 else 10)
-        ceil[label] = bw_point(us, nbytes, copies=n)
+        # a few launch shapes (workgroups, threads, 128-bit loads in flight per lane); the best one is the ceiling
+        best = None
+        for shape in (None, (256, 1024, 8), (224, 1024, 8), (256, 1024, 16), (512, 512, 8), (512, 1024, 4), (1024, 256, 16),
+                      (2048, 256, 8), (256, 512, 16)):
+            us = T.graph_us([reader(b, shape) for b in bufs], 4 if nbytes > 1e8 else 10)
+            if best is None or us < best[0]:
+                best = (us, shape)
+        ceil[label] = bw_point(best[0], nbytes, copies=n,
+                               launch_shape="default" if best[1] is None else
+                               f"{best[1][0]} workgroups x {best[1][1]} threads x {best[1][2]} loads in flight")
         del bufs
-    out["read_ceiling"] = {"kernel": "gla_probe_read (contiguous chunks, 128-bit non-temporal loads, nothing stored)", **ceil}
+    out["read_ceiling"] = {"kernel": "gla_probe_read / gla_probe_read_cfg (contiguous chunks, 128-bit non-temporal loads, nothing "
+                                     "stored), best of nine launch shapes", **ceil}
     torch.cuda.empty_cache()
 
     # ---- C1: A16W4 gs128 fp16, K = N = 4096, M = 1 (and the same layer at M = 4096 below)
@@ -317,7 +328,15 @@ def extra_points(lib, device, T, quick):
         y1 = torch.empty((1, N), dtype=torch.bfloat16, device=device)
         us = T.graph_us([Launch(lib, l, xq1, y1, device, scales_x=sx1) for l in layers], 6)
         out[f"gemv_a8w8_{name}_M1"] = bw_point(us, wbytes + K + 4 + N * 2, N=N, K=K, copies=len(layers))
-        del layer, layers, xq, sx, run, xq1, sx1
+        # ... and end to end: the per-token quantiser of the bf16 row and the GEMV on its codes, both in the graph
+        x1b = x[:1].contiguous()
+        fns = []
+        for l in layers:
+            fns.append(lambda: _ext.scale_activations_per_token(x1b, xq1, sx1))
+            fns.append(Launch(lib, l, xq1, y1, device, scales_x=sx1))
+        us_pair = T.graph_us(fns, 6) * 2
+        out[f"gemv_a8w8_{name}_M1"]["us_with_activation_quantiser"] = round(us_pair, 2)
+        del layer, layers, xq, sx, run, xq1, sx1, fns
     # MXFP8 weights, fp8 activations quantised per token (the reference processor's default)
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
     lin.weight.data = W
@@ -366,6 +385,12 @@ def extra_points(lib, device, T, quick):
         ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
         us = T.graph_us([Launch(lib, l, xq, ym, device, scales_x=sx) for l in layers], 6)
         out[f"gemv_a4w4_mxfp4_16384sq_M{M}"] = bw_point(us, wbytes + M * K // 2 + M * K // 32 + M * N * 2, copies=len(layers))
+        fns = []
+        for l in layers:   # end to end: MXFP4 quantiser of the bf16 rows + GEMV, both in the graph
+            fns.append(lambda: _ext.scale_activations_mxfp4(xm, xq, sx))
+            fns.append(Launch(lib, l, xq, ym, device, scales_x=sx))
+        out[f"gemv_a4w4_mxfp4_16384sq_M{M}"]["us_with_activation_quantiser"] = round(T.graph_us(fns, 6) * 2, 2)
+        del fns
     w_saved = layer.W_q.data.clone()
     for M in (1024, 4096, 8192):
         if quick and M == 1024:
@@ -431,6 +456,43 @@ def extra_points(lib, device, T, quick):
         us = T.eager_us(Launch(lib, a84, xq, ym, device, scales_x=sx), 10)
         gemm_point("gemm_a8w4_mxfp", 4096, N, K, us, 5000.0, "fp8")
     return out
+
+
+def prefetch_experiment(lib, sets, launches, side, n_steps):
+    """Microseconds per decode step when every launch runs beside a gla_prefetch of the next launch's weights,
+    captured as a forked and re-joined branch of the same graph."""
+    seq = []
+    for i in range(n_steps):
+        s, (up, down) = sets[i % len(sets)], launches[i % len(launches)]
+        seq += [(up, s[0]), (down, s[1])]
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=side):
+            for i, (launch, _) in enumerate(seq):
+                nxt = seq[i + 1][1] if i + 1 < len(seq) else None
+                if nxt is not None:
+                    fork = torch.cuda.Event()
+                    fork.record(side)
+                    other.wait_event(fork)
+                    for t in (nxt.W_q, nxt.scales, nxt.zeros):
+                        if lib.gla_prefetch(t.data_ptr(), t.numel() * t.element_size(), 0, other.cuda_stream) != 0:
+                            raise RuntimeError(lib.gla_last_error().decode())
+                launch()
+                if nxt is not None:
+                    join = torch.cuda.Event()
+                    join.record(other)
+                    side.wait_event(join)
+        gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(side)
+        for _ in range(4):
+            gr.replay()
+        e1.record(side)
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (4 * n_steps)
 
 
 def run_point(name, lib, device, T):
@@ -593,18 +655,31 @@ def main():
             gr.replay()
         torch.cuda.synchronize()
 
-        # ---- timed region: exactly a.steps steps
+        # ---- timed region: exactly a.steps steps, bracketed by synchronisations; the device time between two events
+        # on the launch stream is what `value` is computed from, the host clock around the same region is reported
+        # beside it (at a few hundred microseconds of work it mostly measures the host's launch and wake-up latency)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
+        e0.record(side)
         if full:
             for _ in range(full):
                 graphs[0].replay()
         if rem:
             graphs[-1].replay()
+        e1.record(side)
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
+        elapsed_host = time.perf_counter() - t0
+        elapsed = e0.elapsed_time(e1) * 1e-3
     ms_per_step = elapsed * 1e3 / a.steps
     value = step_bytes / (elapsed / a.steps) / 1e9
     y_gpu = y.float().cpu().numpy()
+
+    # ---- the same steps with the next launch's weights pulled into the 256 MB memory-side cache by gla_prefetch on
+    # a forked branch of the graph while the current launch runs (an experiment, not the metric: reported as it is)
+    prefetch_us = None
+    if not a.no_extra:
+        prefetch_us = prefetch_experiment(lib, sets, launches, side, min(a.steps, 64))
 
     # ---- launch duration of each of the two kernels of a step: HIP events on the launch stream around a
     # graph that holds only that kernel, one launch per weight copy
@@ -655,6 +730,7 @@ def main():
             "bytes_per_step": step_bytes,
             "weight_copies": copies,
             "launch": "HIP graph replay of prepared gla_matmul calls",
+            "timer": "HIP events on the launch stream around the replays, device synchronised before and after",
             "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         },
         "roofline": {
@@ -669,6 +745,8 @@ def main():
             "traffic": None,
         },
         "extra": {
+            "host_clock_GBps": round(step_bytes / (elapsed_host / a.steps) / 1e9, 1),
+            "host_clock_ms_per_step": round(elapsed_host * 1e3 / a.steps, 6),
             "up_proj_avg_launch_us": round(up_avg, 3),
             "up_proj_GBps": round(kbytes[0] / (up_avg * 1e-6) / 1e9, 1),
             "down_proj_avg_launch_us": round(down_avg, 3),
@@ -677,11 +755,21 @@ def main():
         },
     }
 
-    # traffic per launch of that kernel as read from the HBM byte counters, when a profile holds it
+    # traffic per launch of that kernel as read from the HBM byte counters, when a profile holds it (counters are
+    # collected by separate rocprofv3 --pmc runs of this script, not in this run)
     traffic_file = os.path.join(ROOT, "profiles", "gemv_direct_a16w4_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file) as f:
-            out["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch_down" if heavy else "hbm_bytes_per_launch")
+            prof = json.load(f)
+        out["roofline"]["traffic"] = prof.get("hbm_bytes_per_launch_down" if heavy else "hbm_bytes_per_launch")
+        out["roofline"]["traffic_source"] = (f"profiles/gemv_direct_a16w4_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                                             f"taken at commit {prof.get('commit', 'unrecorded')})")
+    if prefetch_us is not None:
+        out["extra"]["decode_step_with_prefetch_on_forked_graph_branch"] = {
+            "us_per_step": round(prefetch_us, 2), "GB/s": round(step_bytes / prefetch_us / 1e3, 1),
+            "us_per_step_without": round(ms_per_step * 1e3, 2),
+            "note": "gla_prefetch of launch i+1's W_q, scales and zeros on a second captured stream, forked before and joined "
+                    "after launch i; the fork and join cost more than the cache-fed launch saves"}
 
     if not a.no_extra:
         del launches, sets, base

@@ -94,6 +94,9 @@ SYMBOLS = {
     "gla_probe_mfma": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                       ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]),
     "gla_probe_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "gla_probe_read_cfg": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                          ctypes.c_int, ctypes.c_void_p]),
+    "gla_prefetch": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "gla_matmul_workspace_bytes": (ctypes.c_int64, [ctypes.POINTER(MatmulArgs)]),
     "gla_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),
     "gla_matmul_static": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_void_p]),

@@ -271,6 +271,10 @@ bool widen(const gla_matmul_args& p, Widened& w) {
     w.q.workspace_bytes = 0;
     w.f = choose(w.q, resolve_type(w.q));
     if (!(w.f == F_GEMV_PACKED || w.f == F_GEMM_WN)) return false;
+    // An int32 accumulator was asked for: the 16-bit kernels sum in fp32, which is the same number as long as every
+    // partial sum of |x| (<= 128) times |q - z| (below 2^W_nbits for a zero point inside the code range) over K stays
+    // below 2^24.  Longer sums go to the generic kernel, which adds integers.
+    if (p.acc_dtype == GLA_DT_INT32 && (int64_t)p.K * 128 * ((1 << p.W_nbits) - 1) >= ((int64_t)1 << 24)) return false;
     const int64_t inner = family_workspace(w.f, w.q);
     if (inner < 0) return false;
     // the first kWsPrivateBytes hold the streaming kernels' ticket counters and slots, whoever runs
@@ -310,6 +314,14 @@ int gla_probe_mfma(int dtype, int random_operands, int iters, void* sink, double
 
 int gla_probe_read(const void* buf, int64_t bytes, void* sink, void* stream) {
     return gla::launch_probe_read(buf, bytes, sink, (hipStream_t)stream);
+}
+
+int gla_probe_read_cfg(const void* buf, int64_t bytes, void* sink, int workgroups, int threads, int loads, void* stream) {
+    return gla::launch_probe_read_cfg(buf, bytes, sink, workgroups, threads, loads, (hipStream_t)stream);
+}
+
+int gla_prefetch(const void* buf, int64_t bytes, int workgroups, void* stream) {
+    return gla::launch_prefetch(buf, bytes, workgroups, (hipStream_t)stream);
 }
 
 int gla_matmul_family(const gla_matmul_args* args) {
@@ -354,19 +366,19 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
     }
     int rc2;
     switch (f) {
-        // Every family adds the bias in its epilogue or split-K finishing kernel (the `return`s) except the byte-weight
-        // MFMA GEMM and the generic kernel, which are followed by the elementwise launch below.
+        // Every family adds the bias in its epilogue or split-K finishing kernel (the `return`s) except the generic
+        // kernel, which is followed by the elementwise launch below.
         case F_GEMV_PACKED: return launch_gemv_packed(*args, s);
         case F_GEMV_KMAJOR: return launch_gemv_kmajor(*args, s);
         case F_GEMM_WN: return launch_gemm_wn(*args, s);
         case F_GEMM_8BIT: return launch_gemm_8bit(*args, s);
         case F_GEMM_MXFP4: return launch_gemm_mxfp4(*args, s);
-        case F_GEMM_KBYTES: rc2 = launch_gemm_kbytes(*args, s); break;
+        case F_GEMM_KBYTES: return args->bias != nullptr ? launch_gemm_kbytes_bias(*args, s) : launch_gemm_kbytes(*args, s);
         case F_GEMM_MXFP8: return launch_gemm_mxfp8(*args, s);
         case F_MX_STREAM: return launch_mx_stream(*args, s);
         case F_BLOCKQ_STREAM: return launch_blockq_stream(*args, s);
         case F_GEMM_BLOCKQ: return launch_gemm_blockq(*args, s);
-        case F_GEMM_KBYTES_MX: rc2 = launch_gemm_kbytes_mx(*args, s); break;
+        case F_GEMM_KBYTES_MX: return args->bias != nullptr ? launch_gemm_kbytes_mx_bias(*args, s) : launch_gemm_kbytes_mx(*args, s);
         case F_MX_SKINNY: return launch_mx_skinny(*args, s);
         default: rc2 = launch_generic(*args, s); break;
     }
@@ -387,18 +399,12 @@ namespace {
 static __device__ __align__(256) unsigned char scratch[GLA_STATIC_SCRATCH_BYTES];
 
 constexpr int kMaxDevices = 64;
-constexpr size_t kCounterRegionBytes = (size_t)kWsPrivateBytes;  // ticket counters and partial slots of the streaming kernels: must start at zero
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-__global__ void clear_words_kernel(uint32_t* p, size_t n) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
-}
-
-// Address of this device's copy of `scratch`; the first call on a device looks it up and clears the
-// counter region with a kernel on `stream` (a fill kernel, not a memset: the call may be recorded
-// into a graph).  Every later kernel that takes tickets leaves its counters at zero again.
-int static_scratch(hipStream_t stream, void** out) {
+// Address of this device's copy of `scratch`, looked up on the first call on a device.  Nothing is cleared: a
+// device array without an initialiser is zero-filled when the code object is loaded, and every kernel that keeps
+// counters or slots there leaves them at zero again, so the first call may as well be recorded into a graph.
+int static_scratch(void** out) {
     int dev = 0;
     int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
     if (rc != GLA_OK) return rc;
@@ -419,11 +425,6 @@ int static_scratch(hipStream_t stream, void** out) {
                 set_error("gla_matmul_static: the device array has no address on device %d", dev);
                 return GLA_ERR_LAUNCH_FAILED;
             }
-            const size_t words = kCounterRegionBytes / 4;
-            hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream,
-                               (uint32_t*)ptr, words);
-            rc = check_hip(hipGetLastError(), "gla_matmul_static: clearing the ticket counters");
-            if (rc != GLA_OK) return rc;
             g_scratch_ptr[dev].store(ptr, std::memory_order_release);
         }
     }
@@ -451,7 +452,7 @@ int gla_matmul_static(const gla_matmul_args* args, void* stream) {
     a.workspace_bytes = 0;
     if (need > 0) {
         void* ptr = nullptr;
-        const int rc = static_scratch((hipStream_t)stream, &ptr);
+        const int rc = static_scratch(&ptr);
         if (rc != GLA_OK) return rc;
         a.workspace = ptr;
         a.workspace_bytes = (uint64_t)GLA_STATIC_SCRATCH_BYTES;

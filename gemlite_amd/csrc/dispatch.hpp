@@ -122,6 +122,8 @@ int launch_unpack_over_cols(const void* packed, uint8_t* out, int64_t rows, int6
 // ---- MFMA GEMM for 16-bit activations x K-contiguous weight bytes (gemm_kbytes.hip)
 bool gemm_kbytes_eligible(const gla_matmul_args& p);
 int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream);
+int launch_gemm_kbytes_bias(const gla_matmul_args& p, hipStream_t stream);      // the same with p.bias added in the epilogue
+int launch_gemm_kbytes_mx_bias(const gla_matmul_args& p, hipStream_t stream);
 int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p);
 
 // ---- weight-only MX layers above 2 rows: the same MFMA GEMM with micro-scaled weights (gemm_kbytes.hip)
@@ -136,5 +138,7 @@ int64_t gemm_kbytes_mx_workspace_bytes(const gla_matmul_args& p);
 int launch_probe_mfma(int dtype, int random_operands, int iters, void* sink, double* flops, hipStream_t stream);
 // ---- diagnostic: streaming-read ceiling (probe.hip) --------------------------
 int launch_probe_read(const void* buf, int64_t bytes, void* sink, hipStream_t stream);
+int launch_probe_read_cfg(const void* buf, int64_t bytes, void* sink, int workgroups, int threads, int loads, hipStream_t stream);
+int launch_prefetch(const void* buf, int64_t bytes, int workgroups, hipStream_t stream);
 
 }  // namespace gla

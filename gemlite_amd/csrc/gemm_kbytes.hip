@@ -32,9 +32,19 @@
 #include "common.hpp"
 #include "dispatch.hpp"
 
+// This file is compiled twice: as it is, and from gemm_kbytes_bias.hip with GLA_KB_BIAS set, which gives the same
+// kernels with the bias added in the epilogue under other entry-point names.  A layer without a bias runs the
+// epilogue without the extra loads, rounding and registers (a run-time test inside one kernel cost such layers 4-6 %),
+// and the two halves compile side by side.
+#ifndef GLA_KB_BIAS
+#define GLA_KB_BIAS 0
+#endif
+
 namespace gla {
 
 namespace {
+
+constexpr bool kWithBias = GLA_KB_BIAS != 0;
 
 typedef unsigned int u32x4b __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2b __attribute__((ext_vector_type(2)));
@@ -70,6 +80,8 @@ struct GemmKbArgs {
     float* partials;
     const uint8_t* bscales;  // micro-scaled weights: e8m0 block scales [N, K/32], K contiguous
     int64_t bsn;             // ... bytes from one row's scales to the next
+    const void* bias;        // [N] or NULL: added to the result rounded to the output type
+    int bias_dt;
 };
 
 __device__ __forceinline__ void tile_coords_kb(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -451,6 +463,11 @@ __global__ __launch_bounds__(WAVES_M * kWavesNb * 64) __attribute__((amdgpu_wave
                     float v[4];
 #pragma unroll
                     for (int t = 0; t < 4; ++t) v[t] = acc[i][j][4 * g + t] * (sa * sb[j][4 * g + t]);
+                    if constexpr (kWithBias) {  // `out += bias` on the output already rounded to its type
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (n + t < p.N) v[t] = round_to_dtype(DT, v[t]) + load_as_float(p.bias, p.bias_dt, n + t);
+                    }
                     if (wide && n + 3 < p.N) {
                         if constexpr (DT == GLA_DT_FP32) {
                             *(float4_t*)((float*)p.out + o) = float4_t{v[0], v[1], v[2], v[3]};
@@ -487,7 +504,9 @@ __global__ __launch_bounds__(256) void splitk_finish_kb_kernel(GemmKbArgs p) {
         const float s = load_as_float(p.scales, p.meta_dt, (int64_t)n * p.msn);
         sc *= p.col_scale == 2 ? s * s : s;
     }
-    store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n, v * sc);
+    v *= sc;
+    if (p.bias != nullptr) v = round_to_dtype(p.out_dt, v) + load_as_float(p.bias, p.bias_dt, n);
+    store_from_float(p.out, p.out_dt, (int64_t)m * p.osm + n, v);
 }
 
 template <int WDT, bool BF16, int WAVES_M, int TI>
@@ -550,6 +569,7 @@ KbPlan kb_plan(const gla_matmul_args& p) {
 
 }  // namespace
 
+#if !GLA_KB_BIAS
 bool gemm_kbytes_eligible(const gla_matmul_args& p) {
     if (p.W_nbits != 8 || p.elements_per_sample != 1) return false;
     if (!(p.w_dtype == GLA_DT_INT8 || p.w_dtype == GLA_DT_UINT8 || p.w_dtype == GLA_DT_FP8)) return false;
@@ -597,8 +617,13 @@ bool gemm_kbytes_mx_eligible(const gla_matmul_args& p) {
 }
 
 int64_t gemm_kbytes_mx_workspace_bytes(const gla_matmul_args& p) { return gemm_kbytes_workspace_bytes(p); }
+#endif
 
+#if GLA_KB_BIAS
+int launch_gemm_kbytes_mx_bias(const gla_matmul_args& p, hipStream_t stream) {
+#else
 int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream) {
+#endif
     if (!gemm_kbytes_mx_eligible(p)) {
         set_error("gemm_kbytes_mx: operands not eligible (K-contiguous MXFP8 / MXFP4 weights, K %% 128 == 0, more than 2 rows)");
         return GLA_ERR_UNSUPPORTED_MODE;
@@ -609,6 +634,11 @@ int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream) {
     a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = 0; a.sxm = 0;
     a.col_scale = 0; a.row_scale = 0;
     a.bscales = (const uint8_t*)p.scales; a.bsn = p.meta_stride_n;
+    a.bias = kWithBias ? p.bias : nullptr; a.bias_dt = p.bias_dtype;
+    if (kWithBias && p.bias == nullptr) {
+        set_error("gemm_kbytes_mx: the bias variant was called without a bias");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
     a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
     a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
     const KbPlan g = kb_plan(p);
@@ -629,7 +659,11 @@ int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream) {
     return bf16 ? launch_kb_m<kWMX8, true>(a, g.bm, stream) : launch_kb_m<kWMX8, false>(a, g.bm, stream);
 }
 
+#if GLA_KB_BIAS
+int launch_gemm_kbytes_bias(const gla_matmul_args& p, hipStream_t stream) {
+#else
 int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream) {
+#endif
     GemmKbArgs a;
     a.x = (const uint16_t*)p.x; a.w = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.K = p.K;
@@ -638,6 +672,11 @@ int launch_gemm_kbytes(const gla_matmul_args& p, hipStream_t stream) {
     a.row_scale = (p.channel_scale_mode & 2) ? 1 : 0;
     a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
     a.bscales = nullptr; a.bsn = 0;
+    a.bias = kWithBias ? p.bias : nullptr; a.bias_dt = p.bias_dtype;
+    if (kWithBias && p.bias == nullptr) {
+        set_error("gemm_kbytes: the bias variant was called without a bias");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
     const KbPlan g = kb_plan(p);
     a.tiles_m = g.tiles_m; a.tiles_n = g.tiles_n; a.S = g.S; a.sps = g.sps;
     a.partials = nullptr;

@@ -154,7 +154,6 @@ __global__ __launch_bounds__(64 * kPackedWaves) void generic_packed_kernel(Gener
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int n_raw = blockIdx.x * 64 + lane;
     const int n = n_raw < a.N ? n_raw : a.N - 1;  // lanes past N repeat the last column and store nothing
-    const int m0 = blockIdx.y * RP;
     const int R = a.K / E;                         // word rows
     const int gw = a.wgm == GLA_WGM_NONE ? R : a.gs / E;  // word rows per group
     const int rpw = (R + kPackedWaves - 1) / kPackedWaves;
@@ -162,6 +161,9 @@ __global__ __launch_bounds__(64 * kPackedWaves) void generic_packed_kernel(Gener
     const int r_end = r + rpw < R ? r + rpw : R;
     const bool has_scale = (a.wgm == GLA_WGM_SCALE || a.wgm == GLA_WGM_SHIFT_SCALE || a.wgm == GLA_WGM_FMA);
     const bool has_zero = (a.wgm == GLA_WGM_SHIFT || a.wgm == GLA_WGM_SHIFT_SCALE || a.wgm == GLA_WGM_FMA);
+    // row blocks of RP rows: the grid's second dimension strides over them (it is capped at 65535 blocks)
+    for (int m0 = blockIdx.y * RP; m0 < a.M; m0 += gridDim.y * RP) {
+    r = wv * rpw;
     const uint16_t* xrow[RP];
 #pragma unroll
     for (int rr = 0; rr < RP; ++rr) {
@@ -229,7 +231,7 @@ __global__ __launch_bounds__(64 * kPackedWaves) void generic_packed_kernel(Gener
 #pragma unroll
     for (int rr = 0; rr < RP; ++rr) red[wv][rr][lane] = tot[rr];
     __syncthreads();
-    if (wv != 0 || n_raw >= a.N) return;
+    if (wv == 0 && n_raw < a.N) {
     float sb = 1.0f;
     if (a.csm == GLA_CSM_WEIGHT || a.csm == GLA_CSM_BOTH) sb = load_as_float(a.scales, a.meta_dt, n);
 #pragma unroll
@@ -244,6 +246,9 @@ __global__ __launch_bounds__(64 * kPackedWaves) void generic_packed_kernel(Gener
         else if (a.csm == GLA_CSM_ACTIVATION) v *= sa;
         else if (a.csm == GLA_CSM_BOTH) v *= (sa * sb);
         store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + (int64_t)n * a.osn, v);
+    }
+    }
+    __syncthreads();  // the next row block reuses the reduction buffer
     }
 }
 
@@ -271,7 +276,8 @@ bool packed_words_ok(const gla_matmul_args& p) {
 template <int NBITS, bool BF16>
 void launch_packed_rows(const GenericArgs& a, hipStream_t stream) {
     const int rp = a.M >= 3 ? 4 : a.M;
-    const dim3 grid(ceil_div(a.N, 64), ceil_div(a.M, rp)), block(64 * kPackedWaves);
+    const int row_blocks = ceil_div(a.M, rp);
+    const dim3 grid(ceil_div(a.N, 64), row_blocks < 65535 ? row_blocks : 65535), block(64 * kPackedWaves);
     if (rp == 4) hipLaunchKernelGGL((generic_packed_kernel<NBITS, BF16, 4>), grid, block, 0, stream, a);
     else if (rp == 2) hipLaunchKernelGGL((generic_packed_kernel<NBITS, BF16, 2>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((generic_packed_kernel<NBITS, BF16, 1>), grid, block, 0, stream, a);
@@ -539,6 +545,26 @@ int launch_bias_add(const gla_matmul_args& p, hipStream_t stream) {
 }
 
 int launch_generic(const gla_matmul_args& p, hipStream_t stream) {
+    // the kernels below put blocks of 1-4 rows on the grid's second dimension (at most 65535 blocks): very tall
+    // problems run as slices of rows
+    constexpr int kSliceRows = 65532;
+    if (p.M > kSliceRows) {
+        if (p.input_dtype == GLA_DT_MXFP4) {
+            set_error("generic matmul: more than %d rows of MXFP4 activations are not sliced (two codes per byte)", kSliceRows);
+            return GLA_ERR_MISALIGNED_SHAPE;
+        }
+        for (int m0 = 0; m0 < p.M; m0 += kSliceRows) {
+            gla_matmul_args q = p;
+            q.M = p.M - m0 < kSliceRows ? p.M - m0 : kSliceRows;
+            auto bytes_of = [](int dt) { return (dt == GLA_DT_MXFP16 || dt == GLA_DT_MXBF16) ? 2 : dtype_size(dt); };
+            q.x = (const char*)p.x + (int64_t)m0 * p.x_stride_m * bytes_of(p.input_dtype);
+            q.out = (char*)p.out + (int64_t)m0 * p.out_stride_m * bytes_of(p.output_dtype);
+            if (p.scales_x != nullptr) q.scales_x = (const char*)p.scales_x + (int64_t)m0 * p.sx_stride_m * dtype_size(p.sx_dtype);
+            const int rc = launch_generic(q, stream);
+            if (rc != GLA_OK) return rc;
+        }
+        return GLA_OK;
+    }
     GenericArgs a;
     a.x = p.x; a.w = p.w; a.scales = p.scales; a.zeros = p.zeros; a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.K = p.K;

@@ -89,7 +89,88 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
     if (acc == 0x12345678u) sink[0] = 1.0f;  // keeps the loads alive; the buffers the callers use never fold to this
 }
 
+// The same chunked read with the grid, the workgroup size and the loads in flight chosen by the caller
+// (U = 4, 8 or 16 loads of 16 bytes per lane).
+template <int U>
+__global__ __launch_bounds__(1024) void probe_read_cfg_kernel(const uint4* __restrict__ p, size_t n16, float* sink) {
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t lo = per * blockIdx.x;
+    size_t hi = lo + per;
+    if (hi > n16) hi = n16;
+    unsigned acc = 0;
+    for (size_t i = lo + threadIdx.x; i < hi; i += (size_t)blockDim.x * U) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            size_t j = i + (size_t)u * blockDim.x;
+            if (j >= hi) j = hi - 1;
+            v[u] = load_streaming_u4(p + j);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (acc == 0x12345678u) sink[0] = 1.0f;
+}
+
+// Cache warm-up: plain (cacheable, not streaming) loads of a whole buffer, nothing stored.  What it reads stays
+// in the memory-side cache for the kernel that uses the buffer next.  The never-true store keeps the loads alive.
+__device__ unsigned g_prefetch_sink;
+__global__ __launch_bounds__(256) void prefetch_kernel(const uint4* __restrict__ p, size_t n16) {
+    constexpr int U = 4;
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t lo = per * blockIdx.x;
+    size_t hi = lo + per;
+    if (hi > n16) hi = n16;
+    unsigned acc = 0;
+    for (size_t i = lo + threadIdx.x; i < hi; i += (size_t)256 * U) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            size_t j = i + (size_t)u * 256;
+            if (j >= hi) j = hi - 1;
+            v[u] = p[j];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (acc == 0x9e3779b9u && n16 == 1) g_prefetch_sink = acc;
+}
+
 }  // namespace
+
+int launch_prefetch(const void* buf, int64_t bytes, int workgroups, hipStream_t stream) {
+    if (buf == nullptr || bytes < 0) {
+        set_error("gla_prefetch: a device buffer and a non-negative size are required");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    // whole 16-byte pieces inside [buf, buf + bytes)
+    const uintptr_t lo = ((uintptr_t)buf + 15) & ~(uintptr_t)15, hi = ((uintptr_t)buf + (uintptr_t)bytes) & ~(uintptr_t)15;
+    if (hi <= lo) return GLA_OK;
+    const size_t n16 = (hi - lo) / 16;
+    int grid = workgroups > 0 ? workgroups : 256;
+    if (grid > 4096) grid = 4096;
+    if ((size_t)grid > (n16 + 255) / 256) grid = (int)((n16 + 255) / 256);
+    hipLaunchKernelGGL(prefetch_kernel, dim3(grid), dim3(256), 0, stream, (const uint4*)lo, n16);
+    return check_hip(hipGetLastError(), "gla_prefetch launch");
+}
+
+int launch_probe_read_cfg(const void* buf, int64_t bytes, void* sink, int workgroups, int threads, int loads, hipStream_t stream) {
+    if (buf == nullptr || sink == nullptr || bytes < 16 || (bytes & 15) || ((uintptr_t)buf & 15)) {
+        set_error("gla_probe_read_cfg: a 16-byte aligned device buffer of a multiple of 16 bytes and a 4-byte sink are required");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    if (workgroups < 1 || workgroups > 65535 || threads < 64 || threads > 1024 || (threads & 63) ||
+        !(loads == 4 || loads == 8 || loads == 16)) {
+        set_error("gla_probe_read_cfg: 1..65535 workgroups of 64..1024 threads (a multiple of 64) and 4, 8 or 16 loads per lane");
+        return GLA_ERR_INVALID_ARGUMENT;
+    }
+    const uint4* p = (const uint4*)buf;
+    const size_t n16 = (size_t)(bytes / 16);
+    if (loads == 4) hipLaunchKernelGGL(probe_read_cfg_kernel<4>, dim3(workgroups), dim3(threads), 0, stream, p, n16, (float*)sink);
+    else if (loads == 8) hipLaunchKernelGGL(probe_read_cfg_kernel<8>, dim3(workgroups), dim3(threads), 0, stream, p, n16, (float*)sink);
+    else hipLaunchKernelGGL(probe_read_cfg_kernel<16>, dim3(workgroups), dim3(threads), 0, stream, p, n16, (float*)sink);
+    return check_hip(hipGetLastError(), "gla_probe_read_cfg launch");
+}
 
 int launch_probe_read(const void* buf, int64_t bytes, void* sink, hipStream_t stream) {
     if (buf == nullptr || sink == nullptr || bytes < 16 || (bytes & 15) || ((uintptr_t)buf & 15)) {

@@ -193,6 +193,21 @@ int gla_probe_mfma(int dtype, int random_operands, int iters, void* sink, double
  * of 16; sink: 4 bytes of device memory (never written in practice). */
 int gla_probe_read(const void* buf, int64_t bytes, void* sink, void* stream);
 
+/* Diagnostic, no counterpart in the reference: gla_probe_read with the launch shape chosen by the
+ * caller: `workgroups` workgroups of `threads` threads (a multiple of 64, at most 1024), `loads`
+ * (4, 8 or 16) 128-bit loads in flight per lane.  A caller that sweeps a few shapes and keeps the
+ * best gets the read ceiling of the device for a footprint rather than that of one launch shape. */
+int gla_probe_read_cfg(const void* buf, int64_t bytes, void* sink, int workgroups, int threads, int loads, void* stream);
+
+/* No counterpart in the reference (its kernels rely on the hardware caches as they are).  Reads
+ * [buf, buf + bytes) once with cacheable loads and stores nothing, so that the bytes sit in the
+ * device's memory-side cache (256 MB on MI355X) when the next kernel asks for them.  Meant for a
+ * decode loop that knows which layer runs next: launched on a second stream (or a forked branch of a
+ * captured graph) while layer L runs, it streams the weights of layer L+1 during L's launch gap,
+ * ramp and tail, when the memory system is otherwise idle.  workgroups: grid size, 0 for the default
+ * (256); never allocates, never synchronises. */
+int gla_prefetch(const void* buf, int64_t bytes, int workgroups, void* stream);
+
 /* Scratch bytes gla_matmul needs for these arguments (0 if none).  The scratch
  * must be zero-filled once when it is allocated; the library leaves it zeroed
  * where it needs zeros.  (Plays the role of the reference's pre-zeroed output

@@ -278,6 +278,38 @@ def test_packed_codes_in_short_groups(device, nbits, gs, dtype):
             check_layer(layer, (gen_x(M, K, dtype, seed=M) / 10).to(device), tol, types=())
 
 
+@pytest.mark.parametrize("nbits,gs", [(1, 32), (2, 16)])
+def test_short_group_codes_at_prefill_size(device, nbits, gs):
+    """1024 rows on packings no matrix-core kernel takes (the generic family's packed-word kernel walks the row
+    blocks, four rows at a time)."""
+    N, K, M = 256, 1024, 1024
+    W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.float16, seed=nbits + gs)
+    layer = GemLiteLinear(nbits, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    check_layer(layer, gen_x(M, K, torch.float16, seed=M).to(device), torch.float16, types=())
+
+
+def test_int32_accumulator_on_4_bit_codes_stays_exact(device):
+    """int8 activations x shift-only 4-bit codes with an int32 accumulator (reference: tests/test_int.py:173-199),
+    every activation 127 and every code at the top of its range: the sums of 127 * 8 over K are exact integers at
+    K = 8192, where the widened 16-bit kernels run them in fp32 (K * 128 * 15 < 2^24), and at K = 16384, which is
+    past that bound and goes to the integer loop of the generic kernel."""
+    N = 256
+    for K in (8192, 16384):
+        W_q = torch.full((N, K), 15, dtype=torch.uint8)
+        W_q[::2, ::3] = 3
+        layer = GemLiteLinear(4, 128, K, N, DType.INT8, DType.FP32, scaled_activations=True).pack(W_q.to(device), None, 7)
+        layer.meta_dtype = DType.FP32
+        assert (layer.W_group_mode, layer.channel_scale_mode, layer.acc_dtype) == (1, 2, DType.INT32)
+        for M in (1, 20, 100):
+            x = torch.full((M, K), 127.0, dtype=torch.float16)
+            x[:, 1::2] = -127.0
+            x[:, ::5] = 127.0
+            y = layer(x.to(device))
+            torch.cuda.synchronize()
+            want = x.double() @ (W_q.double() - 7.0).T
+            assert np.array_equal(to_np(y).astype(np.float64), want.numpy()), (K, M)
+
+
 @pytest.mark.parametrize("post_scale", [True, False])
 @pytest.mark.parametrize("nbits", [8, 4])
 def test_a16wn_channelwise(device, nbits, post_scale):

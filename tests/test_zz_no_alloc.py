@@ -51,6 +51,41 @@ def _same(a, b):
                        b.view(torch.int16 if b.element_size() == 2 else torch.int32))
 
 
+def test_static_entry_point_captured_into_a_graph(device):
+    """A split-K GEMV and a split-K GEMM through gla_matmul_static, recorded into one HIP graph and replayed with new
+    activations: every replay equals gla_matmul bit for bit.  When this file runs on its own, the capture holds the
+    very first static call of the process on the device (the scratch address is looked up while capturing; nothing
+    is cleared or allocated then)."""
+    lib = _ext.load_library()
+    W_q, scales, zeros = gen_int_case(1024, 8192, 4, 128, torch.float16, seed=21)
+    layer = GemLiteLinear(4, 128, 8192, 1024, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    xs = {M: gen_x(M, 8192, torch.float16, seed=30 + M).to(device) for M in (1, 70)}   # GEMV with K slabs; split-K GEMM
+    outs = {M: torch.full((M, 1024), float("nan"), dtype=torch.float16, device=device) for M in xs}
+    args = {M: _args(layer, xs[M], None, outs[M]) for M in xs}
+    for M in xs:
+        assert _ext.matmul_workspace_need(args[M]) > 0, "the case is meant to use scratch"
+        args[M].workspace, args[M].workspace_bytes = None, 0
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for M in xs:
+                rc = lib.gla_matmul_static(ctypes.byref(args[M]), torch.cuda.current_stream().cuda_stream)
+                assert rc == 0, lib.gla_last_error().decode()
+    for rep in range(4):
+        for M in xs:
+            xs[M].copy_(gen_x(M, 8192, torch.float16, seed=100 * rep + M).to(device))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for M in xs:
+            want = torch.empty_like(outs[M])
+            _ext.matmul(_args(layer, xs[M], None, want), device)   # eager work between the replays
+            torch.cuda.synchronize()
+            assert _same(outs[M], want), (M, rep)
+            assert rel_frob(to_np(outs[M]), oracle_forward(layer, xs[M])) <= 1.5e-3
+
+
 def test_streaming_split_k_twice(device):
     """A16W4 group 128 decode shapes whose K is cut into slabs (fp32 partials + ticket counters)."""
     for (N, K, M, seed) in ((4096, 14336, 1, 1), (1024, 4096, 3, 2)):
