@@ -63,11 +63,14 @@ def clone_layer(layer):
 class Launch:
     """A prepared `gla_matmul` call: argument struct built once, launched on the current stream."""
 
-    def __init__(self, lib, layer, x, out, device, scales_x=None):
+    def __init__(self, lib, layer, x, out, device, scales_x=None, quantise_inside=False):
+        """quantise_inside: x holds fp16 / bf16 rows and the kernel quantises them to the layer's input type itself."""
         m = layer.get_meta_args()
         self.lib = lib
         in_dt = m[5]
-        if scales_x is None and not gemlite_amd.dtypes.is_mx_dtype(in_dt):
+        if quantise_inside:
+            pass
+        elif scales_x is None and not gemlite_amd.dtypes.is_mx_dtype(in_dt):
             in_dt = gemlite_amd.TORCH_TO_DTYPE[x.dtype].value  # the kernels read x as the type it has
         elif scales_x is None:  # weight-only MX layer
             in_dt = DType.MXFP16.value if x.dtype == torch.float16 else DType.MXBF16.value
@@ -76,6 +79,7 @@ class Launch:
             W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=in_dt,
             output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
             data_contiguous=m[11],  # matmul type left to the dispatcher
+            x_quant_from=gemlite_amd.TORCH_TO_DTYPE[x.dtype].value if quantise_inside else 0,
         )
         need = lib.gla_matmul_workspace_bytes(ctypes.byref(self.args))
         if need < 0:
@@ -336,6 +340,9 @@ def extra_points(lib, device, T, quick):
             fns.append(Launch(lib, l, xq1, y1, device, scales_x=sx1))
         us_pair = T.graph_us(fns, 6) * 2
         out[f"gemv_a8w8_{name}_M1"]["us_with_activation_quantiser"] = round(us_pair, 2)
+        # ... and with the row quantised inside the GEMV (one launch; what forward() runs at decode sizes)
+        us_in = T.graph_us([Launch(lib, l, x1b, y1, device, quantise_inside=True) for l in layers], 6)
+        out[f"gemv_a8w8_{name}_M1"]["us_quantised_inside_the_matmul"] = round(us_in, 2)
         del layer, layers, xq, sx, run, xq1, sx1, fns
     # MXFP8 weights, fp8 activations quantised per token (the reference processor's default)
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
@@ -390,6 +397,9 @@ def extra_points(lib, device, T, quick):
             fns.append(lambda: _ext.scale_activations_mxfp4(xm, xq, sx))
             fns.append(Launch(lib, l, xq, ym, device, scales_x=sx))
         out[f"gemv_a4w4_mxfp4_16384sq_M{M}"]["us_with_activation_quantiser"] = round(T.graph_us(fns, 6) * 2, 2)
+        if M == 1:  # the rows the streaming kernel takes: quantised inside it (one launch; what forward() runs)
+            us_in = T.graph_us([Launch(lib, l, xm, ym, device, quantise_inside=True) for l in layers], 6)
+            out[f"gemv_a4w4_mxfp4_16384sq_M{M}"]["us_quantised_inside_the_matmul"] = round(us_in, 2)
         del fns
     w_saved = layer.W_q.data.clone()
     for M in (1024, 4096, 8192):

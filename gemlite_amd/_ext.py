@@ -76,7 +76,7 @@ class MatmulArgs(ctypes.Structure):
         ("tile_config", ctypes.c_int32),
         ("bias", ctypes.c_void_p),
         ("bias_dtype", ctypes.c_int32),
-        ("reserved0", ctypes.c_int32),
+        ("x_quant_from", ctypes.c_int32),
     ]
 
 
@@ -272,8 +272,10 @@ def build_matmul_args(
     x, W_q, scales, zeros, scales_x, out, *,
     W_nbits, group_size, unpack_mask, elements_per_sample, input_dtype, output_dtype, acc_dtype, meta_dtype,
     channel_scale_mode, W_group_mode, data_contiguous, matmul_type=MATMUL_AUTO, tile_config=-1, bias=None,
+    x_quant_from=0,
 ) -> MatmulArgs:
-    """Fill a ``gla_matmul_args`` from tensors and the reference's meta ints."""
+    """Fill a ``gla_matmul_args`` from tensors and the reference's meta ints.  ``x_quant_from``: the DType value of
+    the 16-bit rows in ``x`` when the kernel is to quantise them to ``input_dtype`` itself (``scales_x`` is then None)."""
     a = MatmulArgs()
     a.struct_size = ctypes.sizeof(MatmulArgs)
     a.matmul_type = int(matmul_type)
@@ -322,6 +324,7 @@ def build_matmul_args(
     a.zero_is_scalar = int(has_zeros and zeros.numel() == 1)
     a.sx_dtype = _dt(scales_x, DType.FP32.value)
     a.tile_config = int(tile_config)
+    a.x_quant_from = int(x_quant_from)
     if bias is not None:
         if bias.numel() < N or bias.stride(-1) != 1:
             raise ValueError(f"bias: need {N} contiguous elements, got shape {tuple(bias.shape)} strides {bias.stride()}")
@@ -353,7 +356,7 @@ def _check_operand_bounds(a, x, W_q, scales, zeros, scales_x, out, mx):
             )
 
     M, N, K, e = a.M, a.N, a.K, a.elements_per_sample
-    kx = K // 2 if a.input_dtype == DType.MXFP4.value else K
+    kx = K // 2 if (a.input_dtype == DType.MXFP4.value and not a.x_quant_from) else K
     check("x", x, need((M, a.x_stride_m), (kx, a.x_stride_k)))
     check("W_q", W_q, need((K // e, a.w_stride_k), (N, a.w_stride_n)))
     check("out", out, need((M, a.out_stride_m), (N, a.out_stride_n)))
@@ -417,6 +420,11 @@ def matmul_workspace_need(args: MatmulArgs) -> int:
     if need < 0:
         _check(int(need), "gla_matmul_workspace_bytes")
     return int(need)
+
+
+def matmul_is_supported(args: MatmulArgs) -> bool:
+    """Whether the library has a kernel for ``args`` as they are (host logic only; no exception, no launch)."""
+    return load_library().gla_matmul_family(ctypes.byref(args)) >= 0
 
 
 FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM", "BLOCKQ_STREAM", "GEMM_BLOCKQ", "GEMM_KBYTES_MX", "MX_SKINNY"]

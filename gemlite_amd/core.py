@@ -128,6 +128,15 @@ def _cached_tile_config(matmul_type: str, key: str) -> int:
     return int(entry)
 
 
+# rows up to which forward() asks the matmul to quantise the activations itself (the library may still decline)
+_FUSED_QUANT_ROWS = 4
+
+
+def _bias_is_fusable(bias, output_dtype, x2d):
+    return bias is not None and bias.dtype in _BIAS_DTYPES and DTYPE_TO_TORCH[output_dtype] in _BIAS_DTYPES \
+        and bias.dim() == 1 and bias.is_contiguous() and bias.device == x2d.device
+
+
 # ---------------------------------------------------------------------------
 # functional forward
 # ---------------------------------------------------------------------------
@@ -159,6 +168,25 @@ def forward_functional(
 
     scales_x = None
     kernel_input_dtype = input_dtype
+    if scaled_activations and x2d.shape[0] <= _FUSED_QUANT_ROWS and x2d.dtype in (torch.float16, torch.bfloat16):
+        # decode sizes: the streaming kernels quantise the rows themselves (same codes and scales as the quantiser
+        # launch, one launch less); the library says whether the call at hand is one they take
+        in_dt = DType(input_dtype)
+        if (in_dt in FP8_INT8_DTYPES and channel_scale_mode in (2, 3)) or (in_dt == DType.MXFP4 and channel_scale_mode == 4):
+            fused_bias = _bias_is_fusable(bias, output_dtype, x2d)
+            type_str = GEMLITE_MATMUL_TYPES[matmul_type] if matmul_type >= 0 else get_matmul_type(
+                x2d.shape[0], W_nbits, is_mx_dtype(input_dtype))
+            out = _KERNEL_FORWARD[type_str](
+                x2d, W_q, scales, zeros, None, W_nbits, group_size, unpack_mask, elements_per_sample,
+                input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
+                data_contiguous, get_type_id(input_dtype, W_nbits), bias=bias if fused_bias else None,
+                x_quant_from=TORCH_TO_DTYPE[x2d.dtype].value,
+            )
+            if out is not None:
+                out = out.view(out_shape)
+                if bias is not None and not fused_bias:
+                    out += bias
+                return out
     if scaled_activations:
         in_dt = DType(input_dtype)
         if in_dt in FP8_INT8_DTYPES and channel_scale_mode == 5:  # 128 x 128 block quantisation
@@ -196,8 +224,7 @@ def forward_functional(
 
     # the library adds a floating-point bias itself (in the GEMV epilogue, or with one small launch after
     # the other kernels); anything else is added here like the reference does (gemlite/core.py:271-272)
-    fused_bias = bias is not None and bias.dtype in _BIAS_DTYPES and DTYPE_TO_TORCH[output_dtype] in _BIAS_DTYPES \
-        and bias.dim() == 1 and bias.is_contiguous() and bias.device == x2d.device
+    fused_bias = _bias_is_fusable(bias, output_dtype, x2d)
     out = _KERNEL_FORWARD[matmul_type_str](
         x2d, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
         kernel_input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
@@ -223,6 +250,7 @@ def forward_functional(
 # Entries are per thread: the struct is rewritten in place on every call.
 _PREPARED = {}
 _PREPARED_LIMIT = 8192
+_DECLINED = object()  # cached answer: the library has no kernel for this (optional) form of the call
 _thread_id = threading.get_ident
 
 
@@ -231,7 +259,9 @@ def _kernel_forward(matmul_type_str):
 
     def forward(x, W_q, scales, zeros, scales_x, W_nbits, group_size, unpack_mask, elements_per_sample,
                 input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode, W_group_mode,
-                data_contiguous, type_id, meta_scale=0.0, bias=None):
+                data_contiguous, type_id, meta_scale=0.0, bias=None, x_quant_from=0):
+        """``x_quant_from``: DType value of the 16-bit rows in ``x`` that the kernel is to quantise to ``input_dtype``
+        itself; returns None when the library has no kernel that does so for this call."""
         M, K, N = x.shape[0], W_q.shape[0] * elements_per_sample, W_q.shape[1]
         out = torch.empty((M, N), dtype=DTYPE_TO_TORCH[int(output_dtype)], device=x.device)
         if M == 0:
@@ -244,8 +274,10 @@ def _kernel_forward(matmul_type_str):
         key = (id(W_q), W_q.shape, W_q.stride(), _thread_id(), matmul_type_id, x.shape, x.stride(), x.dtype, sx_key,
                x.device.index, W_nbits, group_size,
                unpack_mask, elements_per_sample, input_dtype, output_dtype, acc_dtype, meta_dtype, channel_scale_mode,
-               W_group_mode, data_contiguous, tile, None if bias is None else (bias.data_ptr(), bias.dtype))
+               W_group_mode, data_contiguous, tile, None if bias is None else (bias.data_ptr(), bias.dtype), x_quant_from)
         hit = _PREPARED.get(key)
+        if hit is _DECLINED:
+            return None
         if hit is not None:
             args, need, w_ptr, s_ptr, z_ptr = hit
             if (W_q.data_ptr() == w_ptr and (scales is None or scales.data_ptr() == s_ptr)
@@ -259,8 +291,13 @@ def _kernel_forward(matmul_type_str):
             elements_per_sample=elements_per_sample, input_dtype=input_dtype, output_dtype=output_dtype,
             acc_dtype=acc_dtype, meta_dtype=meta_dtype, channel_scale_mode=channel_scale_mode,
             W_group_mode=W_group_mode, data_contiguous=data_contiguous,
-            matmul_type=matmul_type_id, tile_config=tile, bias=bias,
+            matmul_type=matmul_type_id, tile_config=tile, bias=bias, x_quant_from=x_quant_from,
         )
+        if x_quant_from and not _ext.matmul_is_supported(args):
+            if len(_PREPARED) >= _PREPARED_LIMIT:
+                _PREPARED.clear()
+            _PREPARED[key] = _DECLINED
+            return None
         need = _ext.matmul_workspace_need(args)
         _ext.matmul_prepared(args, need, args.x, args.out, args.scales_x, x.device)
         if len(_PREPARED) >= _PREPARED_LIMIT:

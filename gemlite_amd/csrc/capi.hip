@@ -55,7 +55,7 @@ constexpr int kMxStreamRows = 2;  // MXFP4 x MXFP4: rows up to which the streami
 
 enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY };
 
-int validate(const gla_matmul_args* p) {
+int validate_operands(const gla_matmul_args* p) {
     if (p == nullptr) {
         set_error("matmul: args is NULL");
         return GLA_ERR_INVALID_ARGUMENT;
@@ -166,7 +166,7 @@ int validate(const gla_matmul_args* p) {
     const bool need_s = p->W_group_mode >= GLA_WGM_SCALE || (p->channel_scale_mode & 1);
     const bool need_z = p->W_group_mode == GLA_WGM_SHIFT || p->W_group_mode >= GLA_WGM_SHIFT_SCALE;
     if ((need_s && p->scales == nullptr) || (need_z && p->zeros == nullptr) ||
-        ((p->channel_scale_mode & 2) && p->scales_x == nullptr)) {
+        ((p->channel_scale_mode & 2) && p->scales_x == nullptr && !p->x_quant_from)) {
         set_error("matmul: mode (W_group_mode=%d, channel_scale_mode=%d) needs a tensor that is NULL",
                   p->W_group_mode, p->channel_scale_mode);
         return GLA_ERR_INVALID_ARGUMENT;
@@ -176,6 +176,42 @@ int validate(const gla_matmul_args* p) {
             set_error("matmul: K=%d not divisible by group_size=%d", p->K, p->group_size);
             return GLA_ERR_MISALIGNED_SHAPE;
         }
+    }
+    return GLA_OK;
+}
+
+Family choose(const gla_matmul_args& p, int type);
+int resolve_type(const gla_matmul_args& p);
+
+// Operand checks, then: a call that asks for its activations to be quantised inside the matmul must land on a kernel
+// that does it (the others would read the 16-bit rows as codes).
+int validate(const gla_matmul_args* p) {
+    const int rc = validate_operands(p);
+    if (rc != GLA_OK || p->x_quant_from == 0 || p->M == 0) return rc;
+    if (!(p->x_quant_from == GLA_DT_FP16 || p->x_quant_from == GLA_DT_BF16)) {
+        set_error("matmul: x_quant_from %d: activations are quantised on the fly from fp16 or bf16 rows only", p->x_quant_from);
+        return GLA_ERR_UNSUPPORTED_DTYPE;
+    }
+    const Family f = choose(*p, resolve_type(*p));
+    const bool per_token = f == F_GEMV_KMAJOR && (p->input_dtype == GLA_DT_FP8 || p->input_dtype == GLA_DT_INT8);
+    const bool mxfp4 = f == F_MX_STREAM && p->input_dtype == GLA_DT_MXFP4 && mx_stream_quantises(*p);
+    // ... and only where the same call on ready-made codes would take that kernel too: a batch the matrix-core GEMM
+    // serves better is not kept on the streaming kernel for the sake of the quantiser
+    gla_matmul_args q = *p;
+    q.x_quant_from = 0;
+    q.x = (const void*)(uintptr_t)256;         // stand-ins for aligned code and scale arrays
+    q.scales_x = (const void*)(uintptr_t)256;
+    const bool mx = p->input_dtype == GLA_DT_MXFP4;
+    q.x_stride_m = mx ? (p->K / 2 + 15) / 16 * 16 : (p->K + 15) / 16 * 16;
+    q.sx_dtype = mx ? GLA_DT_UINT8 : GLA_DT_FP32;
+    q.sx_stride_m = mx ? p->K / 32 : 1;
+    q.sx_stride_g = 1;
+    const bool same = choose(q, resolve_type(q)) == f;
+    if (!((per_token || mxfp4) && same)) {
+        set_error("matmul: no kernel quantises the activations inside the matmul for this call (M=%d N=%d K=%d, input type %d, "
+                  "channel_scale_mode %d): the streaming kernels do, for the first rows of per-token fp8 / int8 and MXFP4 layers; "
+                  "run the quantiser launch first", p->M, p->N, p->K, p->input_dtype, p->channel_scale_mode);
+        return GLA_ERR_UNSUPPORTED_MODE;
     }
     return GLA_OK;
 }

@@ -94,6 +94,7 @@ int64_t gemm_mxfp8_workspace_bytes(const gla_matmul_args& p);
 // ---- streaming kernel for K-contiguous micro-scaled operands (mx_stream.hip): weight-only MX
 // layers (fp16/bf16 x MXFP8/MXFP4 weights), MXFP8 activations x MXFP4 weights
 bool mx_stream_eligible(const gla_matmul_args& p);
+bool mx_stream_quantises(const gla_matmul_args& p);  // the call asks for MXFP4 activations made inside the kernel, and it makes them
 int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream);
 
 // ---- 128 x 128 block-quantised int8 / fp8 above 4 rows: MFMA GEMM (gemm_8bit.hip)

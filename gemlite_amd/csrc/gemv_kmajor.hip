@@ -24,6 +24,7 @@
 
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "actquant_device.hpp"
 
 namespace gla {
 
@@ -108,11 +109,19 @@ __device__ __forceinline__ int wave_sum_int(int v) {
 
 // MT: rows of x handled (power of two >= M).  XK: activation kind.  int8 x int8 sums exactly: a lane's fp32
 // sums stay below 2^24 (the host bounds K), the sums over lanes and waves are taken in int32.
-template <int WDT, int XK, int MT>
+// QF (8-bit activation kinds only): 0 = x holds the codes; kXF16 + 1 / kXBF16 + 1 = x holds fp16 / bf16 rows and the
+// workgroup quantises them per token itself (the quantiser launch in front of a decode matmul costs a third of the
+// matmul's time): every workgroup takes the row's amax (the row is a few KB and sits in L2), forms the scale
+// max(amax / qmax, 1e-6) and turns the 16 activations a lane multiplies into the quantiser's codes, with the
+// quantiser's own arithmetic, before it multiplies them, so the result equals quantiser + matmul bit for bit.
+template <int WDT, int XK, int MT, int QF = 0>
 __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) {
     constexpr bool X8 = XK == kXFP8 || XK == kXI8;
     constexpr bool EXACT = XK == kXI8;
+    constexpr bool FUSED = QF != 0;
+    static_assert(!FUSED || X8, "on-the-fly quantisation makes 8-bit codes");
     __shared__ float red[kWavesK][kRowsK * MT + MT];
+    __shared__ float amax_sh[kWavesK][MT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * kRowsK;
     const uint8_t* wrow[kRowsK];
@@ -123,7 +132,43 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     }
     const uint8_t* xrow[MT];  // x_stride_m counts stored elements
 #pragma unroll
-    for (int m = 0; m < MT; ++m) xrow[m] = (const uint8_t*)a.x + (int64_t)(m < a.M ? m : a.M - 1) * a.xsm * (X8 ? 1 : 2);
+    for (int m = 0; m < MT; ++m) xrow[m] = (const uint8_t*)a.x + (int64_t)(m < a.M ? m : a.M - 1) * a.xsm * ((X8 && !FUSED) ? 1 : 2);
+
+    // per-token scales of the rows, as gla_scale_activations_per_token computes them
+    float xs_s[MT], xs_r[MT];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float am = 0.0f;
+            for (int c = threadIdx.x; c < a.K / 8; c += kWavesK * 64) {
+                const u32x4k raw = *(const u32x4k*)(xrow[m] + 16 * c);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float lo, hi;
+                    if constexpr (QF == kXBF16 + 1) {
+                        lo = __builtin_bit_cast(float, raw[q] << 16);
+                        hi = __builtin_bit_cast(float, raw[q] & 0xffff0000u);
+                    } else {
+                        lo = half_bits_to_float((uint16_t)(raw[q] & 0xffffu));
+                        hi = half_bits_to_float((uint16_t)(raw[q] >> 16));
+                    }
+                    am = fmaxf(am, fmaxf(fabsf(lo), fabsf(hi)));
+                }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
+            if (lane == 0) amax_sh[wave][m] = am;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            float am = amax_sh[0][m];
+#pragma unroll
+            for (int w = 1; w < kWavesK; ++w) am = fmaxf(am, amax_sh[w][m]);
+            xs_s[m] = fmaxf(am / (XK == kXI8 ? 127.0f : 448.0f), 1e-6f);
+            xs_r[m] = 1.0f / xs_s[m];
+        }
+    }
 
     float acc[kRowsK][MT], sumx[MT];
 #pragma unroll
@@ -143,7 +188,24 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             float xf[16];
-            if constexpr (XK == kXFP8) {
+            if constexpr (FUSED) {
+                const u32x4k xa = *(const u32x4k*)(xrow[m] + 2 * k), xb = *(const u32x4k*)(xrow[m] + 2 * k + 16);
+                acts_to_float<QF == kXBF16 + 1>(xa, xb, xf);
+                const float qmax = XK == kXI8 ? 127.0f : 448.0f, qmin = XK == kXI8 ? -128.0f : -448.0f;
+#pragma unroll
+                for (int q = 0; q < 16; ++q) xf[q] = fminf(fmaxf(div_by_row_scale(xf[q], xs_s[m], xs_r[m]), qmin), qmax);
+                if constexpr (XK == kXI8) {
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) xf[q] = floorf(xf[q] + 0.5f);  // the code itself, as a float
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 16; q += 2) {  // to e4m3 and back: the value the stored code would give
+                        const f32x2k back = __builtin_amdgcn_cvt_pk_f32_fp8((int)f32_to_fp8_pair(xf[q], xf[q + 1]), false);
+                        xf[q] = back.x;
+                        xf[q + 1] = back.y;
+                    }
+                }
+            } else if constexpr (XK == kXFP8) {
                 codes_to_float<GLA_DT_FP8>(*(const u32x4k*)(xrow[m] + k), xf);
             } else if constexpr (XK == kXI8) {
                 codes_to_float<GLA_DT_INT8>(*(const u32x4k*)(xrow[m] + k), xf);  // biased by +128
@@ -221,7 +283,16 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     }
     float post = 1.0f;
     if (a.csm & 1) post *= load_as_float(a.scales, a.meta_dt, (int64_t)n * a.msn);
-    if (a.csm & 2) post *= load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
+    if (a.csm & 2) {
+        if constexpr (FUSED) {
+            float sx = xs_s[0];
+#pragma unroll
+            for (int mm = 1; mm < MT; ++mm) sx = m == mm ? xs_s[mm] : sx;
+            post *= sx;
+        } else {
+            post *= load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm);
+        }
+    }
     store_result(a, m, n, v * post);
 }
 
@@ -394,13 +465,13 @@ int launch_k(const GemvKArgs& a, hipStream_t stream) {
     return check_hip(hipGetLastError(), "gemv_kmajor launch");
 }
 
-// 8-bit activations of the weights' own type (fp8 x fp8, int8 x int8), up to 4 rows
-template <int WDT, int XK>
+// 8-bit activations of the weights' own type (fp8 x fp8, int8 x int8), up to 4 rows; QF: see the kernel
+template <int WDT, int XK, int QF = 0>
 int launch_k8(const GemvKArgs& a, hipStream_t stream) {
     const dim3 grid(ceil_div(a.N, kRowsK)), block(kWavesK * 64);
-    if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 1>), grid, block, 0, stream, a);
-    else if (a.M == 2) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 2>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 4>), grid, block, 0, stream, a);
+    if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 1, QF>), grid, block, 0, stream, a);
+    else if (a.M == 2) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 2, QF>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 4, QF>), grid, block, 0, stream, a);
     return check_hip(hipGetLastError(), "gemv_kmajor launch");
 }
 
@@ -416,7 +487,10 @@ bool gemv_kmajor_eligible(const gla_matmul_args& p) {
     if (x8) {
         // the vector variant only; a lane's fp32 sum of |x| <= 128 times a biased code <= 255 over K / 256 values
         // must stay below 2^24 for the int8 sums to be exact
-        if (p.M > kRows8 || p.K > 131072 || p.x_stride_m % 16 != 0) return false;
+        if (p.M > kRows8 || p.K > 131072 || p.x_stride_m % (p.x_quant_from ? 8 : 16) != 0) return false;
+        // quantised on the fly from fp16 / bf16 rows: per-token scales only, and they come from the kernel
+        if (p.x_quant_from && !(p.x_quant_from == GLA_DT_FP16 || p.x_quant_from == GLA_DT_BF16)) return false;
+        if (p.x_quant_from && !(p.channel_scale_mode & 2)) return false;
         // 3 and 4 rows only on layers of 20 MB or less (4096^2: 13 against 15 us for the matrix-core GEMM and its
         // finishing launch; 8192^2: 29 against 21); 1 and 2 rows everywhere (4096^2 6.7 against 14.7, 8192^2 15.6
         // against 21.6 us)
@@ -437,7 +511,8 @@ bool gemv_kmajor_eligible(const gla_matmul_args& p) {
     if (uses_s && p.scales == nullptr) return false;
     if (uses_z && p.zeros == nullptr) return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
-    if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
+    if ((p.channel_scale_mode & 2) && p.scales_x == nullptr && !(x8 && p.x_quant_from)) return false;
+    if (!x8 && p.x_quant_from) return false;
     return true;
 }
 
@@ -449,6 +524,14 @@ int launch_gemv_kmajor(const gla_matmul_args& p, hipStream_t stream) {
     a.wgm = p.W_group_mode; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.z_scalar = p.zero_is_scalar; a.out_dt = p.output_dtype; a.sx_dt = p.sx_dtype;
     a.bias = p.bias; a.bias_dt = p.bias_dtype;
+    if (p.x_quant_from == GLA_DT_FP16) {
+        return p.input_dtype == GLA_DT_FP8 ? launch_k8<GLA_DT_FP8, kXFP8, kXF16 + 1>(a, stream)
+                                           : launch_k8<GLA_DT_INT8, kXI8, kXF16 + 1>(a, stream);
+    }
+    if (p.x_quant_from == GLA_DT_BF16) {
+        return p.input_dtype == GLA_DT_FP8 ? launch_k8<GLA_DT_FP8, kXFP8, kXBF16 + 1>(a, stream)
+                                           : launch_k8<GLA_DT_INT8, kXI8, kXBF16 + 1>(a, stream);
+    }
     if (p.input_dtype == GLA_DT_FP8) return launch_k8<GLA_DT_FP8, kXFP8>(a, stream);
     if (p.input_dtype == GLA_DT_INT8) return launch_k8<GLA_DT_INT8, kXI8>(a, stream);
     const bool bf16 = p.input_dtype == GLA_DT_BF16;

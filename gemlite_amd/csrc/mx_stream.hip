@@ -27,12 +27,15 @@
 // a few rows: every group of eight activation rows streams the weights again).
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "actquant_device.hpp"
 
 namespace gla {
 
 namespace {
 
-enum { A_F16 = 0, A_BF16 = 1, A_FP8 = 2, A_FP4 = 3 };
+// A_Q4F16 / A_Q4BF16: fp16 / bf16 rows that the kernel quantises to MXFP4 itself, block by block, with the
+// arithmetic of the activation quantiser (same codes, same e8m0 bytes), in place of a quantiser launch in front
+enum { A_F16 = 0, A_BF16 = 1, A_FP8 = 2, A_FP4 = 3, A_Q4F16 = 4, A_Q4BF16 = 5 };
 enum { B_FP8 = 0, B_FP4 = 1 };
 
 struct MxArgs {
@@ -115,10 +118,37 @@ __device__ __forceinline__ void block_from_16bit(const u32x4 (&raw)[4], typename
     }
 }
 
+// One 32-block of 16-bit activations -> its MXFP4 codes (16 bytes, as the quantiser stores them) and e8m0 byte.
+template <bool XBF>
+__device__ __forceinline__ u32x4 quantise_block_mxfp4(const u32x4 (&raw)[4], uint32_t& e) {
+    float v[4][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t w = raw[d][j];
+            if constexpr (XBF) {
+                v[d][2 * j] = __builtin_bit_cast(float, w << 16);
+                v[d][2 * j + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
+            } else {
+                v[d][2 * j] = half_bits_to_float((uint16_t)(w & 0xffffu));
+                v[d][2 * j + 1] = half_bits_to_float((uint16_t)(w >> 16));
+            }
+            amax = fmaxf(amax, fmaxf(fabsf(v[d][2 * j]), fabsf(v[d][2 * j + 1])));
+        }
+    e = e8m0_of_amax<false>(amax);
+    u32x4 codes;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) codes[d] = mxfp4_pack8<true>(v[d], e);
+    return codes;
+}
+
 // NC output columns per wave, RM activation rows per workgroup row.
 template <int AK, int BK, int RM, int NC>
 __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
     constexpr bool BF = (AK == A_BF16);
+    constexpr bool QUANT = AK == A_Q4F16 || AK == A_Q4BF16;
     using pair_t = typename Pair<BF>::type;
     constexpr int kABytes = AK == A_FP4 ? 16 : (AK == A_FP8 ? 32 : 64);
     constexpr int kBBytes = BK == B_FP4 ? 16 : 32;
@@ -174,12 +204,15 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
                 const uint8_t* xp = a.x + (int64_t)m * a.xsm_bytes + (int64_t)b * kABytes;
 #pragma unroll
                 for (int q = 0; q < AQ; ++q) st.x[r][q] = *(const u32x4*)(xp + 16 * q);
-                st.sa[r] = a.csm == GLA_CSM_MX ? ((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)b * a.sxg] : (uint8_t)127;
+                if constexpr (!QUANT)
+                    st.sa[r] = a.csm == GLA_CSM_MX ? ((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)b * a.sxg] : (uint8_t)127;
             }
         }
     };
-    auto to_pairs_a = [&](const u32x4 (&raw)[AQ], pair_t (&xv)[16]) __attribute__((always_inline)) {
-        if constexpr (AK == A_FP4) block_from_fp4<BF>(raw[0], xv);
+    // (quantised on the fly: `e` receives the block's e8m0 byte)
+    auto to_pairs_a = [&](const u32x4 (&raw)[AQ], pair_t (&xv)[16], uint32_t& e) __attribute__((always_inline)) {
+        if constexpr (QUANT) block_from_fp4<BF>(quantise_block_mxfp4<AK == A_Q4BF16>(raw, e), xv);
+        else if constexpr (AK == A_FP4) block_from_fp4<BF>(raw[0], xv);
         else if constexpr (AK == A_FP8) block_from_fp8<BF>(raw[0], raw[1], xv);
         else block_from_16bit<BF>(raw, xv);
     };
@@ -199,16 +232,19 @@ __global__ __launch_bounds__(256) void mx_stream_kernel(MxArgs a) {
             if (m < a.M) {
                 pair_t xv[16];
                 float sa = 1.0f;
+                uint32_t eq = 127;
                 if constexpr (XPRE) {
-                    to_pairs_a(st.x[r], xv);
-                    if (a.csm == GLA_CSM_MX) sa = e8m0_to_float(st.sa[r]);
+                    to_pairs_a(st.x[r], xv, eq);
+                    if constexpr (QUANT) sa = e8m0_to_float((uint8_t)eq);
+                    else if (a.csm == GLA_CSM_MX) sa = e8m0_to_float(st.sa[r]);
                 } else {
                     const uint8_t* xp = a.x + (int64_t)m * a.xsm_bytes + (int64_t)blk * kABytes;
                     u32x4 raw[AQ];
 #pragma unroll
                     for (int q = 0; q < AQ; ++q) raw[q] = *(const u32x4*)(xp + 16 * q);
-                    to_pairs_a(raw, xv);
-                    if (a.csm == GLA_CSM_MX)
+                    to_pairs_a(raw, xv, eq);
+                    if constexpr (QUANT) sa = e8m0_to_float((uint8_t)eq);
+                    else if (a.csm == GLA_CSM_MX)
                         sa = e8m0_to_float(((const uint8_t*)a.scales_x)[(int64_t)m * a.sxm + (int64_t)blk * a.sxg]);
                 }
 #pragma unroll
@@ -259,7 +295,8 @@ int a_kind(const gla_matmul_args& p) {
         case GLA_DT_MXFP16: return A_F16;
         case GLA_DT_MXBF16: return A_BF16;
         case GLA_DT_MXFP8: return A_FP8;
-        case GLA_DT_MXFP4: return A_FP4;
+        case GLA_DT_MXFP4:
+            return p.x_quant_from == GLA_DT_FP16 ? A_Q4F16 : (p.x_quant_from == GLA_DT_BF16 ? A_Q4BF16 : A_FP4);
         default: return -1;
     }
 }
@@ -274,7 +311,7 @@ void launch_rows(const MxArgs& a, int rm, dim3 grid, hipStream_t s) {
     // loads of a CU in flight.  1-2 rows then take 2 columns per wave (2048 x 8192: MXFP4 x MXFP4 7.1 -> 5.8 us, fp8 x
     // MXFP8 8.7 -> 6.3; 4096^2 7-15 % faster).  16-bit activations, which weigh as much as two columns of MXFP4
     // weights, only up to K = 8192 (4096 x 14336 was 6-9 % slower with them read twice as often).
-    if (rm <= 2 && ceil_div(a.N, 4 * kCols) < 512 && (AK > A_BF16 || a.KB <= 8192 / 32)) {
+    if (rm <= 2 && ceil_div(a.N, 4 * kCols) < 512 && (AK == A_FP8 || AK == A_FP4 || a.KB <= 8192 / 32)) {
         const dim3 g2(ceil_div(a.N, 4 * 2), grid.y);
         if (rm == 1) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 1, 2>), g2, dim3(256), 0, s, a);
         else hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 2, 2>), g2, dim3(256), 0, s, a);
@@ -301,7 +338,11 @@ bool mx_stream_eligible(const gla_matmul_args& p) {
     if (p.W_nbits != (p.elements_per_sample == 2 ? 4 : 8)) return false;
     if (p.scales == nullptr || p.x_stride_k != 1 || p.w_stride_k != 1) return false;
     // x_stride_m counts stored elements (bytes for the 8- and 4-bit kinds, 16-bit words otherwise)
-    const int64_t xsm_bytes = p.x_stride_m * (ak <= A_BF16 ? 2 : 1);
+    const int64_t xsm_bytes = p.x_stride_m * ((ak <= A_BF16 || ak >= A_Q4F16) ? 2 : 1);
+    if (p.x_quant_from && ak < A_Q4F16) return false;  // only MXFP4 activations are made here
+    if (ak >= A_Q4F16) return p.channel_scale_mode == GLA_CSM_MX && p.elements_per_sample == 2 && xsm_bytes % 16 == 0 &&
+                              p.w_stride_n % 16 == 0 && aligned16(p.x) && aligned16(p.w) &&
+                              (p.output_dtype == GLA_DT_FP32 || p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16);
     if (xsm_bytes % 16 != 0 || p.w_stride_n % 16 != 0 || !aligned16(p.x) || !aligned16(p.w)) return false;
     switch (p.output_dtype) {
         case GLA_DT_FP32: case GLA_DT_FP16: case GLA_DT_BF16: case GLA_DT_MXFP16: case GLA_DT_MXBF16: break;
@@ -312,6 +353,8 @@ bool mx_stream_eligible(const gla_matmul_args& p) {
     if (csm == GLA_CSM_ACTIVATION) return p.scales_x != nullptr && p.sx_dtype == GLA_DT_FP32;
     return csm == GLA_CSM_NONE;
 }
+
+bool mx_stream_quantises(const gla_matmul_args& p) { return a_kind(p) >= A_Q4F16 && mx_stream_eligible(p); }
 
 int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream) {
     if (!mx_stream_eligible(p)) {
@@ -324,7 +367,7 @@ int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream) {
     a.x = (const uint8_t*)p.x; a.w = (const uint8_t*)p.w; a.scales = (const uint8_t*)p.scales;
     a.scales_x = p.scales_x; a.out = p.out;
     a.M = p.M; a.N = p.N; a.KB = p.K / 32;
-    a.xsm_bytes = p.x_stride_m * (ak <= A_BF16 ? 2 : 1);
+    a.xsm_bytes = p.x_stride_m * ((ak <= A_BF16 || ak >= A_Q4F16) ? 2 : 1);
     a.wsn_bytes = p.w_stride_n;
     a.osm = p.out_stride_m; a.osn = p.out_stride_n;
     a.msg = p.meta_stride_g; a.msn = p.meta_stride_n; a.sxm = p.sx_stride_m; a.sxg = p.sx_stride_g;
@@ -338,6 +381,8 @@ int launch_mx_stream(const gla_matmul_args& p, hipStream_t stream) {
         case A_F16: launch_b<A_F16>(a, bk, rm, grid, stream); break;
         case A_BF16: launch_b<A_BF16>(a, bk, rm, grid, stream); break;
         case A_FP8: launch_b<A_FP8>(a, bk, rm, grid, stream); break;
+        case A_Q4F16: launch_rows<A_Q4F16, B_FP4>(a, rm, grid, stream); break;
+        case A_Q4BF16: launch_rows<A_Q4BF16, B_FP4>(a, rm, grid, stream); break;
         default: launch_b<A_FP4>(a, bk, rm, grid, stream); break;
     }
     return check_hip(hipGetLastError(), "mx_stream launch");

@@ -138,7 +138,15 @@ typedef struct gla_matmul_args {
      * on the same stream. */
     const void* bias;
     int32_t bias_dtype;
-    int32_t reserved0;
+
+    /* Activation quantisation inside the matmul, for decode sizes (replaces the quantiser launch in front of it;
+     * reference: gemlite/core.py:220-250).  0: x holds input_dtype.  GLA_DT_FP16 / GLA_DT_BF16: x holds rows of that
+     * 16-bit type ([M, K], x_stride_* in its elements) and the kernel quantises them itself to input_dtype, exactly as
+     * gla_scale_activations_per_token (input_dtype FP8 or INT8, channel_scale_mode 2 or 3) or
+     * gla_scale_activations_mxfp4 (input_dtype MXFP4, channel_scale_mode 4) would: same codes, same scales, same
+     * result as the two launches.  scales_x is not read.  Only the streaming kernels do this (up to 4 rows, fewer on
+     * large layers); gla_matmul_family returns GLA_ERR_UNSUPPORTED_MODE for a call they do not take. */
+    int32_t x_quant_from;
 } gla_matmul_args;
 
 /* Library identification.  No reference counterpart. */

@@ -479,6 +479,92 @@ def test_int8_activations_packed_weights(device):
         check_layer(layer, (gen_x(M, K, torch.float16, seed=M) / 20).to(device), torch.float32)
 
 
+def _forward_both_ways(layer, x):
+    """(forward with the activations quantised inside the matmul, forward with the quantiser launch in front)."""
+    from gemlite_amd import core
+    y_fused = layer(x)
+    rows = core._FUSED_QUANT_ROWS
+    core._FUSED_QUANT_ROWS = 0
+    try:
+        y_two = layer(x)
+    finally:
+        core._FUSED_QUANT_ROWS = rows
+    torch.cuda.synchronize()
+    return y_fused, y_two
+
+
+def _fused_family(layer, x):
+    """Kernel family the library picks when asked to quantise `x` inside the matmul, or None if it declines."""
+    m = layer.get_meta_args()
+    out = torch.empty(x.shape[0], layer.out_features, dtype=gemlite_amd.DTYPE_TO_TORCH[m[6]], device=x.device)
+    a = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                               unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                               acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                               data_contiguous=m[11], x_quant_from=gemlite_amd.TORCH_TO_DTYPE[x.dtype].value)
+    return _ext.matmul_family(a) if _ext.matmul_is_supported(a) else None
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_a8w8_decode_rows_are_quantised_inside_the_matmul(device, fp8, dtype):
+    """Up to 4 rows (2 on large layers) the K-major streaming kernel takes the 16-bit rows and quantises them per
+    token itself (reference: the quantiser call in front of the matmul, gemlite/core.py:220-250): the output must
+    equal the quantiser launch followed by the matmul bit for bit, rows of very different magnitudes, an all-zero
+    row (scale 1e-6) and a ragged K included; above those rows the library declines and forward() runs two launches."""
+    for (N, K) in ((1030, 4160), (512, 8192)):
+        W = gen_x(N, K, torch.bfloat16, seed=15, std=0.02)
+        proc = helper.A8W8_FP8_dynamic(device=device) if fp8 else helper.A8W8_INT8_dynamic(device=device)
+        W_q_cpu, s_cpu = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+        proc.dtype = dtype
+        layer = proc.from_weights(W_q_cpu, scales=s_cpu)
+        for M in (1, 2, 3, 4, 5):
+            x = gen_x(M, K, dtype, seed=40 + M)
+            x[0] *= 37.0
+            if M > 1:
+                x[1] = 0.0
+            if M > 2:
+                x[2] *= 1e-3
+            x = x.to(device)
+            assert _fused_family(layer, x) == ("GEMV_KMAJOR" if M <= 4 else None), M
+            y_fused, y_two = _forward_both_ways(layer, x)
+            assert torch.equal(y_fused, y_two), (N, K, M)
+            check_layer(layer, x, dtype)
+    # a large layer keeps the streaming kernel, and with it the quantiser inside, for 2 rows only
+    big = helper.A8W8_INT8_dynamic(device=device)
+    big.dtype = torch.bfloat16
+    Wb = gen_x(8192, 4096, torch.bfloat16, seed=3, std=0.02)
+    Wq_b, s_b = gemlite_amd.quantize_weights_per_channel(Wb, torch.int8)
+    layer = big.from_weights(Wq_b, scales=s_b)
+    for M, fam in ((2, "GEMV_KMAJOR"), (3, None)):
+        x = gen_x(M, 4096, torch.bfloat16, seed=M).to(device)
+        assert _fused_family(layer, x) == fam
+        y_fused, y_two = _forward_both_ways(layer, x)
+        assert torch.equal(y_fused, y_two), M
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_a4w4_decode_rows_are_quantised_inside_the_matmul(device, dtype):
+    """MXFP4 x MXFP4 at the rows the streaming kernel takes: the kernel makes the e2m1 codes and e8m0 bytes of its
+    activation blocks itself; same output as the quantiser launch + matmul bit for bit (blocks of all zeros, of
+    tiny and of huge values, ties of the e2m1 grid included)."""
+    for (N, K) in ((520, 4224), (512, 4096)):   # K of the reference's MX tests (streams at any row count); a K the matrix cores take
+        W = gen_x(N, K, torch.bfloat16, seed=7, std=0.02)
+        codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+        layer = helper.A4W4_MXFP_dynamic(device=device, dtype=dtype).from_weights(torch.from_numpy(codes), scales=torch.from_numpy(e8))
+        for M in (1, 2, 3, 4, 5):
+            x = gen_x(M, K, dtype, seed=60 + M)
+            x[0, :32] = 0.0
+            x[0, 32:64] = torch.tensor([0.75, 1.75, 3.5, -0.75, -1.75, -3.5, 0.25, 6.0] * 4).to(dtype)  # ties at scale 1
+            x[0, 64:96] *= 1e-4
+            x[0, 96:128] *= 3e3
+            x = x.to(device)
+            if K % 128 == 0:
+                assert _fused_family(layer, x) == ("MX_STREAM" if M <= 4 else None), M
+            y_fused, y_two = _forward_both_ways(layer, x)
+            assert torch.equal(y_fused, y_two), (K, M)
+            check_layer(layer, x, dtype)
+
+
 # ------------------------------------------------------------------ MXFP4
 @pytest.mark.parametrize("M", [1, 3, 32, 100, 128])
 def test_a4w4_mxfp4(device, M):
