@@ -114,19 +114,21 @@ __device__ __forceinline__ int wave_sum_int(int v) {
 // matmul's time): every workgroup takes the row's amax (the row is a few KB and sits in L2), forms the scale
 // max(amax / qmax, 1e-6) and turns the 16 activations a lane multiplies into the quantiser's codes, with the
 // quantiser's own arithmetic, before it multiplies them, so the result equals quantiser + matmul bit for bit.
-template <int WDT, int XK, int MT, int QF = 0>
+// RK: weight rows per workgroup: 4; 8 when the rows are quantised here, so that the quantisation of a K-chunk is
+// shared by twice the columns (every workgroup quantises the whole row).
+template <int WDT, int XK, int MT, int QF = 0, int RK = kRowsK>
 __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) {
     constexpr bool X8 = XK == kXFP8 || XK == kXI8;
     constexpr bool EXACT = XK == kXI8;
     constexpr bool FUSED = QF != 0;
     static_assert(!FUSED || X8, "on-the-fly quantisation makes 8-bit codes");
-    __shared__ float red[kWavesK][kRowsK * MT + MT];
+    __shared__ float red[kWavesK][RK * MT + MT];
     __shared__ float amax_sh[kWavesK][MT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kRowsK;
-    const uint8_t* wrow[kRowsK];
+    const int n0 = blockIdx.x * RK;
+    const uint8_t* wrow[RK];
 #pragma unroll
-    for (int r = 0; r < kRowsK; ++r) {
+    for (int r = 0; r < RK; ++r) {
         const int n = n0 + r < a.N ? n0 + r : a.N - 1;  // rows past the end repeat the last one; never stored
         wrow[r] = a.w + (int64_t)n * a.wsn;
     }
@@ -170,21 +172,23 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
         }
     }
 
-    float acc[kRowsK][MT], sumx[MT];
+    float acc[RK][MT], sumx[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         sumx[m] = 0.0f;
 #pragma unroll
-        for (int r = 0; r < kRowsK; ++r) acc[r][m] = 0.0f;
+        for (int r = 0; r < RK; ++r) acc[r][m] = 0.0f;
     }
 
     for (int k = wave * kIterK + lane * kLaneK; k < a.K; k += kWavesK * kIterK) {  // K % 16 == 0
-        u32x4k wv[kRowsK];
+        u32x4k wv[RK];
 #pragma unroll
-        for (int r = 0; r < kRowsK; ++r) wv[r] = *(const u32x4k*)(wrow[r] + k);
-        float wf[kRowsK][16];
+        for (int r = 0; r < RK; ++r) wv[r] = *(const u32x4k*)(wrow[r] + k);
+        float wf[RK <= 4 ? RK : 1][16];
+        if constexpr (RK <= 4) {
 #pragma unroll
-        for (int r = 0; r < kRowsK; ++r) codes_to_float<WDT>(wv[r], wf[r]);
+            for (int r = 0; r < RK; ++r) codes_to_float<WDT>(wv[r], wf[r]);
+        }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             float xf[16];
@@ -215,11 +219,22 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
                 const u32x4k xa = *(const u32x4k*)(xrow[m] + 2 * k), xb = *(const u32x4k*)(xrow[m] + 2 * k + 16);
                 acts_to_float<XK == kXBF16>(xa, xb, xf);
             }
+            if constexpr (RK <= 4) {
 #pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                sumx[m] += xf[q];
+                for (int q = 0; q < 16; ++q) {
+                    sumx[m] += xf[q];
 #pragma unroll
-                for (int r = 0; r < kRowsK; ++r) acc[r][m] = __builtin_fmaf(xf[q], wf[r][q], acc[r][m]);
+                    for (int r = 0; r < RK; ++r) acc[r][m] = __builtin_fmaf(xf[q], wf[r][q], acc[r][m]);
+                }
+            } else {  // more rows than registers for all their floats: one weight row at a time
+#pragma unroll
+                for (int q = 0; q < 16; ++q) sumx[m] += xf[q];
+#pragma unroll
+                for (int r = 0; r < RK; ++r) {
+                    codes_to_float<WDT>(wv[r], wf[0]);
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) acc[r][m] = __builtin_fmaf(xf[q], wf[0][q], acc[r][m]);
+                }
             }
         }
     }
@@ -229,17 +244,17 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     for (int m = 0; m < MT; ++m) {
         if constexpr (EXACT) {
             const int sx = wave_sum_int((int)sumx[m]);
-            if (lane == 0) red[wave][kRowsK * MT + m] = __builtin_bit_cast(float, sx);
+            if (lane == 0) red[wave][RK * MT + m] = __builtin_bit_cast(float, sx);
 #pragma unroll
-            for (int r = 0; r < kRowsK; ++r) {
+            for (int r = 0; r < RK; ++r) {
                 const int d = wave_sum_int((int)acc[r][m]);
                 if (lane == 0) red[wave][r * MT + m] = __builtin_bit_cast(float, d);
             }
         } else {
             const float sx = wave_sum(sumx[m]);
-            if (lane == 0) red[wave][kRowsK * MT + m] = sx;
+            if (lane == 0) red[wave][RK * MT + m] = sx;
 #pragma unroll
-            for (int r = 0; r < kRowsK; ++r) {
+            for (int r = 0; r < RK; ++r) {
                 const float d = wave_sum(acc[r][m]);
                 if (lane == 0) red[wave][r * MT + m] = d;
             }
@@ -247,7 +262,7 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
     }
     __syncthreads();
     const int t = threadIdx.x;
-    if (t >= kRowsK * MT) return;
+    if (t >= RK * MT) return;
     const int r = t / MT, m = t % MT, n = n0 + r;
     if (n >= a.N || m >= a.M) return;
     float D = 0.0f, X = 0.0f;
@@ -256,7 +271,7 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
 #pragma unroll
         for (int w = 0; w < kWavesK; ++w) {
             Di += __builtin_bit_cast(int, red[w][r * MT + m]);
-            Xi += __builtin_bit_cast(int, red[w][kRowsK * MT + m]);
+            Xi += __builtin_bit_cast(int, red[w][RK * MT + m]);
         }
         if (WDT == GLA_DT_INT8) Di -= 128 * Xi;  // undo the bias of the byte conversion
         D = (float)Di;                            // the int32 accumulator of the reference, converted once
@@ -265,7 +280,7 @@ __global__ __launch_bounds__(kWavesK * 64) void gemv_kmajor_kernel(GemvKArgs a) 
 #pragma unroll
         for (int w = 0; w < kWavesK; ++w) {
             D += red[w][r * MT + m];
-            X += red[w][kRowsK * MT + m];
+            X += red[w][RK * MT + m];
         }
         if (WDT == GLA_DT_INT8) D = __builtin_fmaf(-128.0f, X, D);  // undo the bias of the byte conversion
     }
@@ -468,6 +483,15 @@ int launch_k(const GemvKArgs& a, hipStream_t stream) {
 // 8-bit activations of the weights' own type (fp8 x fp8, int8 x int8), up to 4 rows; QF: see the kernel
 template <int WDT, int XK, int QF = 0>
 int launch_k8(const GemvKArgs& a, hipStream_t stream) {
+    if constexpr (QF != 0) {
+        // one and two rows on layers wide enough to give every CU four workgroups of 8 columns
+        if (a.M <= 2 && a.N >= 8 * 1024) {
+            const dim3 grid8(ceil_div(a.N, 8)), block8(kWavesK * 64);
+            if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 1, QF, 8>), grid8, block8, 0, stream, a);
+            else hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 2, QF, 8>), grid8, block8, 0, stream, a);
+            return check_hip(hipGetLastError(), "gemv_kmajor launch");
+        }
+    }
     const dim3 grid(ceil_div(a.N, kRowsK)), block(kWavesK * 64);
     if (a.M == 1) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 1, QF>), grid, block, 0, stream, a);
     else if (a.M == 2) hipLaunchKernelGGL((gemv_kmajor_kernel<WDT, XK, 2, QF>), grid, block, 0, stream, a);

@@ -311,6 +311,8 @@ void launch_rows(const MxArgs& a, int rm, dim3 grid, hipStream_t s) {
     // loads of a CU in flight.  1-2 rows then take 2 columns per wave (2048 x 8192: MXFP4 x MXFP4 7.1 -> 5.8 us, fp8 x
     // MXFP8 8.7 -> 6.3; 4096^2 7-15 % faster).  16-bit activations, which weigh as much as two columns of MXFP4
     // weights, only up to K = 8192 (4096 x 14336 was 6-9 % slower with them read twice as often).
+    // (Rows quantised in the kernel: 8 columns per wave, which would halve the quantising work per column, measured
+    // slower than 4: 16384^2 at one row 40.5 against 35.9 us.)
     if (rm <= 2 && ceil_div(a.N, 4 * kCols) < 512 && (AK == A_FP8 || AK == A_FP4 || a.KB <= 8192 / 32)) {
         const dim3 g2(ceil_div(a.N, 4 * 2), grid.y);
         if (rm == 1) hipLaunchKernelGGL((mx_stream_kernel<AK, BK, 1, 2>), g2, dim3(256), 0, s, a);
