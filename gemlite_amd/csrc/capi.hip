@@ -217,32 +217,42 @@ int validate(const gla_matmul_args* p) {
 }
 
 Family choose(const gla_matmul_args& p, int type) {
+    // what the caller (or the tuner's cache) prefers where a streaming kernel and a matrix-core GEMM both take the call
+    const bool want_stream = p.tile_config == GLA_TILE_PREFER_STREAMING, want_matrix = p.tile_config == GLA_TILE_PREFER_MATRIX;
     if (p.input_dtype == GLA_DT_MXFP4) {
         // decode sizes: the streaming kernel (weights read once, straight into registers) beats the split-K matrix-core
         // path, whose tiles are at least 64 rows tall: up to 2 rows everywhere, up to 4 on layers of 40 MB or less
         // (4096^2 at 4 rows: 10.7 against 14.4 us; 8192^2: 20.2 against 20.5; 16384^2: 54 against 40)
         const int rows = (int64_t)p.N * p.K / 2 <= 40000000 ? 4 : kMxStreamRows;
-        if (p.M <= rows && p.tile_config < 1000 && mx_stream_eligible(p)) return F_MX_STREAM;
-        return gemm_mxfp4_eligible(p) ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
+        const bool stream_ok = p.tile_config < 1000 && mx_stream_eligible(p), matrix_ok = gemm_mxfp4_eligible(p);
+        if (want_stream && stream_ok) return F_MX_STREAM;
+        if (want_matrix && matrix_ok) return F_GEMM_MXFP4;
+        if (p.M <= rows && stream_ok) return F_MX_STREAM;
+        return matrix_ok ? F_GEMM_MXFP4 : (mx_stream_eligible(p) ? F_MX_STREAM : F_GENERIC);
     }
     if (p.input_dtype == GLA_DT_MXFP8) {  // validated: eligible for one of the two at least
         // fp8 activations on MXFP8 or MXFP4 weights: up to 4 rows the streaming kernel is the faster one at every size
         // (MXFP8 weights, one row: 4096^2 7.9 against 25 us, 16384^2 59 against 84; 4 rows: 13.4 against 25, 79 against
         // 83.  MXFP4 weights, 4 rows: 4096^2 10.4 against 19.8, 16384^2 52 against 54; 6 rows: 85 against 54)
-        if (p.M <= 4 && p.tile_config < 1000 && mx_stream_eligible(p)) return F_MX_STREAM;
-        return gemm_mxfp8_eligible(p) ? F_GEMM_MXFP8 : F_MX_STREAM;
+        const bool stream_ok = p.tile_config < 1000 && mx_stream_eligible(p), matrix_ok = gemm_mxfp8_eligible(p);
+        if (want_stream && stream_ok) return F_MX_STREAM;
+        if (want_matrix && matrix_ok) return F_GEMM_MXFP8;
+        if (p.M <= 4 && stream_ok) return F_MX_STREAM;
+        return matrix_ok ? F_GEMM_MXFP8 : F_MX_STREAM;
     }
     if (p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)  // validated as eligible for the streaming kernel
     {
         // 1-2 rows: the streaming kernel; up to 16 rows the weights still go straight into registers, to the
         // matrix cores (16384^2 MXFP4, 8 rows: 48 against 62 us of the tiled GEMM); above that the tiled GEMM
+        if (want_stream) return F_MX_STREAM;
+        if (want_matrix && gemm_kbytes_mx_eligible(p)) return F_GEMM_KBYTES_MX;
         if (p.M > 2 && p.M <= 16 && p.tile_config < 1000 && mx_skinny_eligible(p)) return F_MX_SKINNY;
         return gemm_kbytes_mx_eligible(p) ? F_GEMM_KBYTES_MX : F_MX_STREAM;
     }
     if (p.channel_scale_mode == GLA_CSM_BLOCK)  // validated as eligible for the streaming kernel at least
-        return gemm_blockq_eligible(p) ? F_GEMM_BLOCKQ : F_BLOCKQ_STREAM;
+        return (gemm_blockq_eligible(p) && !want_stream) ? F_GEMM_BLOCKQ : F_BLOCKQ_STREAM;
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
-    const bool small = type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16;
+    const bool small = !want_matrix && (type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16 || want_stream);
     if (small) {
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
@@ -256,11 +266,15 @@ Family choose(const gla_matmul_args& p, int type) {
         if (!gemm_wn_eligible(p)) return F_GEMV_PACKED;
         const int64_t chunks = (p.M + 15) / 16;
         const int64_t restreamed = chunks * (int64_t)p.N * p.K * (p.W_nbits < 4 ? 4 : p.W_nbits) / 8;  // 2-bit codes cost what 4-bit ones do
-        if (p.tile_config <= 0 && chunks <= 4 && restreamed <= (chunks == 4 ? 48 : 96) * (int64_t)1000000) return F_GEMV_PACKED;
+        if (!want_matrix && p.tile_config <= 0 && chunks <= 4 && restreamed <= (chunks == 4 ? 48 : 96) * (int64_t)1000000) return F_GEMV_PACKED;
     }
     if (gemm_wn_eligible(p)) return F_GEMM_WN;
     if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // also streams K-major 8-bit operands at small M (split-K)
     if (gemm_kbytes_eligible(p)) return F_GEMM_KBYTES;
+    if (want_matrix) {  // no matrix-core kernel takes the call: the streaming ones after all
+        if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
+        if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
+    }
     return F_GENERIC;
 }
 

@@ -26,6 +26,10 @@ from .quant_utils import (scale_activations_mxfp4, scale_activations_mxfp8, scal
                           scale_activations_per_token)
 
 
+PREFER_STREAMING, PREFER_MATRIX = -2, -3   # GLA_TILE_PREFER_STREAMING / GLA_TILE_PREFER_MATRIX of the C header
+HAND_OFF_ROWS = 128                        # batch sizes up to which both kinds of kernel are timed
+
+
 def candidate_configs(family: str, M: int, K: int) -> List[int]:
     """``tile_config`` ids worth timing for a kernel family (-1, the built-in heuristic, comes first)."""
     if family == "GEMV_PACKED":      # waves per workgroup * 1000 + batches of loads per wave
@@ -98,7 +102,12 @@ def tune_layer(layer: GemLiteLinear, batch_sizes: Iterable[int], reps: int = 20,
         family = _ext.matmul_family(build(-1))
         stream = torch.cuda.current_stream(device).cuda_stream
         runnable = []
-        for tile in candidate_configs(family, M, layer.in_features):
+        candidates = candidate_configs(family, M, layer.in_features)
+        if M <= HAND_OFF_ROWS:
+            # around the hand-off between the streaming kernels and the matrix-core GEMMs the other side is timed too;
+            # the library's thresholds there were fitted on one machine
+            candidates += [t for t in (PREFER_STREAMING, PREFER_MATRIX) if _ext.matmul_family(build(t)) != family]
+        for tile in candidates:
             args = build(tile)
             need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))
             if need < 0:

@@ -76,6 +76,13 @@ extern "C" {
 #define GLA_CSM_BLOCK 5      /* fp32 scales per 128 x 128 weight block and per (row, 128) of x;
                                 scales: [K/128, ceil(N/128)], scales_x: [M, K/128] */
 
+/* tile_config values that leave the tile to the library and say which kind of kernel to take where both a streaming
+ * (decode) kernel and a matrix-core GEMM could run the call.  The library's own hand-off between the two is a set of
+ * thresholds on rows and layer size measured on one machine; the offline tuner times both sides of it for a layer
+ * and batch size and stores the winner under the reference's config-cache key (reference: gemlite/core.py:838-906). */
+#define GLA_TILE_PREFER_STREAMING (-2)
+#define GLA_TILE_PREFER_MATRIX (-3)
+
 /*
  * Arguments of one quantized matmul  out[M,N] = x[M,K] * dequant(w)[K,N].
  *
@@ -129,7 +136,8 @@ typedef struct gla_matmul_args {
     int32_t zeros_dtype;    /* element type of zeros */
     int32_t zero_is_scalar; /* zeros holds a single element */
     int32_t sx_dtype;       /* element type of scales_x (FP32 or UINT8/E8M0) */
-    int32_t tile_config;    /* -1 = library heuristic, else an id from gla_select_config */
+    int32_t tile_config;    /* -1 = library heuristic; an id from gla_select_config or the offline tuner; or one of
+                             * GLA_TILE_PREFER_* below */
 
     /* Optional bias [N] (fp16, bf16 or fp32), or NULL: out = cast(cast(acc ...) + bias[n]), i.e. added to the
      * result already rounded to the output type, as the reference's `out += bias` does

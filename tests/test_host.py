@@ -356,6 +356,39 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
         assert _family(lm, M, None, scales_x=sx, x=xq) == ("MX_STREAM" if M <= 2 else "GEMM_MXFP4")
 
 
+def test_tile_config_can_state_a_preference_between_streaming_and_matrix_kernels():
+    """GLA_TILE_PREFER_STREAMING (-2) / GLA_TILE_PREFER_MATRIX (-3): where both kinds of kernel take a call, the
+    preference decides; where only one does, it runs; -1 keeps the library's own hand-off."""
+    g = torch.Generator().manual_seed(0)
+    N, K = 512, 1024
+    W_q = torch.randint(0, 16, (N, K), generator=g).to(torch.uint8)
+    s, z = torch.rand(N * K // 128, 1).half(), torch.rand(N * K // 128, 1).half()
+    l = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q, s, z)
+    m = l.get_meta_args()
+
+    def fam(M, tile):
+        x = torch.zeros(M, K, dtype=torch.float16)
+        out = torch.zeros(M, N, dtype=torch.float16)
+        a = _ext.build_matmul_args(x, l.W_q, l.scales, l.zeros, None, out, W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+                                   elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7],
+                                   meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11],
+                                   tile_config=tile)
+        return _ext.matmul_family(a)
+    assert [fam(M, -1) for M in (8, 32, 100)] == ["GEMV_PACKED", "GEMV_PACKED", "GEMM_WN"]
+    assert [fam(M, -3) for M in (8, 32, 100)] == ["GEMM_WN"] * 3
+    assert [fam(M, -2) for M in (8, 32, 100)] == ["GEMV_PACKED"] * 3
+    # 1-bit codes have no matrix-core kernel: the streaming one runs whatever the preference
+    W1 = torch.randint(0, 2, (N, K), generator=g).to(torch.uint8)
+    l1 = GemLiteLinear(1, 128, K, N, DType.FP16, DType.FP16).pack(W1, torch.rand(N * K // 128, 1).half(), torch.rand(N * K // 128, 1).half())
+    m1 = l1.get_meta_args()
+    x = torch.zeros(40, K, dtype=torch.float16)
+    a = _ext.build_matmul_args(x, l1.W_q, l1.scales, l1.zeros, None, torch.zeros(40, N, dtype=torch.float16), W_nbits=m1[1],
+                               group_size=m1[2], unpack_mask=m1[3], elements_per_sample=m1[4], input_dtype=m1[5],
+                               output_dtype=m1[6], acc_dtype=m1[7], meta_dtype=m1[8], channel_scale_mode=m1[9],
+                               W_group_mode=m1[10], data_contiguous=m1[11], tile_config=-3)
+    assert _ext.matmul_family(a) == "GEMV_PACKED"
+
+
 def test_tuner_candidates_and_cache_file_round_trip(tmp_path):
     from gemlite_amd import tune
     assert tune.candidate_configs("GEMV_PACKED", 1, 4096)[0] == -1
