@@ -401,6 +401,24 @@ def extra_points(lib, device, T, quick):
             us_in = T.graph_us([Launch(lib, l, xm, ym, device, quantise_inside=True) for l in layers], 6)
             out[f"gemv_a4w4_mxfp4_16384sq_M{M}"]["us_quantised_inside_the_matmul"] = round(us_in, 2)
         del fns
+    # the same format on an 8192^2 layer at decode batches: weights straight from registers into the scaled MFMA
+    N8 = K8 = 8192
+    lin = torch.nn.Linear(K8, N8, bias=False, dtype=torch.bfloat16)
+    lin.weight.data = (torch.randn((N8, K8), generator=g) * 0.02).to(torch.bfloat16)
+    layer8 = helper.A4W4_MXFP_dynamic(device=device, dtype=torch.bfloat16).from_linear(lin.to(device))
+    del lin
+    wbytes8 = N8 * K8 // 2 + N8 * K8 // 32
+    layers8 = [layer8] + [clone_layer(layer8) for _ in range(copies_for(wbytes8) - 1)]
+    for M in (8, 32):
+        xm = torch.randn((M, K8), device=device).to(torch.bfloat16)
+        xq, sx = gemlite_amd.scale_activations_mxfp4(xm)
+        ym = torch.empty((M, N8), dtype=torch.bfloat16, device=device)
+        ls = [Launch(lib, l, xq, ym, device, scales_x=sx) for l in layers8]
+        us = T.graph_us(ls, 6)
+        out[f"gemv_a4w4_mxfp4_8192sq_M{M}"] = bw_point(us, wbytes8 + M * K8 // 2 + M * K8 // 32 + M * N8 * 2, copies=len(layers8),
+                                                       family=_ext.matmul_family(ls[0].args))
+        del ls
+    del layers8, layer8
     w_saved = layer.W_q.data.clone()
     for M in (1024, 4096, 8192):
         if quick and M == 1024:

@@ -19,6 +19,8 @@
 //    accumulators through LDS in wave order; no workspace, no second kernel, deterministic.
 //  * 16384^2 MXFP4: 45 us at 3 rows, 51 at 16 (a pure read in this access pattern: 30-34 us; the tiled GEMM:
 //    52-62 us); MXFP8: 73-79 us.
+// The second kernel of the file takes MXFP4 activations (codes + e8m0 bytes) on the same weights, 3..32 rows, and
+// feeds both sides to the block-scaled MFMA unconverted.
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -249,6 +251,226 @@ __global__ __launch_bounds__(kWavesS * 64) void mx_skinny_kernel(MxSkArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// MXFP4 x MXFP4 at 3..32 rows: the same walk over the weights, but nothing is converted.  A lane's 16 weight
+// bytes (32 e2m1 codes of one 32-block) ARE its share of the A operand of v_mfma_scale_f32_16x16x128_f8f6f4,
+// the block's e8m0 byte its scale; the B operand is the same 32-block of 16 activation rows (codes and e8m0
+// bytes staged through LDS like the 16-bit activations above), so one instruction multiplies 16 weight rows
+// with 16 activation rows over 128 K-values and applies both block scales (reference:
+// gemlite/triton_kernels/gemm_splitK_kernels.py:536-770, `tl.dot_scaled` on e2m1 operands).  XT = 1 or 2 tiles of
+// 16 activation rows.  Between the vector-unit streaming kernel (1-2 rows, 4 on small layers) and the tiled
+// GEMM (64-row tiles through LDS, split K, a finishing launch and a scale-regrouping launch in front).
+//  * 8 / 32 rows: 4096^2 5.1 / 6.5 us (tiled GEMM 14.1 / 15.3), 8192^2 13.0 / 16.0 (17.8 / 19.9), 14336 x 4096
+//    11.3 / 14.5 (16.1 / 18.6), 16384^2 42.7 / 48.0 (41.0 / 44.4: the dispatcher keeps the GEMM there).
+//  * The bound is the access pattern the [N, K/2] layout forces on an MFMA operand: a wave instruction reads 16
+//    rows x 64 bytes.  The same kernel reading 1 KiB contiguous per instruction (weights regrouped by operand;
+//    timing only, not built) took 28 / 35 us at 1 / 16 rows on 16384^2 and 9.5 / 11.1 on 8192^2.  Loading the
+//    activations per lane from global memory instead of through LDS (no barrier in the K loop) gave the same
+//    times up to 16 rows and 10-20 % worse ones at 32.
+struct Mx4SkArgs {
+    const uint8_t* x;         // [M, K/2] e2m1 pairs
+    const uint8_t* sx;        // [ceil32(M), K/32] e8m0
+    const uint8_t* w;         // [N, K/2]
+    const uint8_t* scales;    // [N, K/32]
+    void* out;
+    int M, N, K;
+    int64_t xsm, sxm, wsn, osm, msn;   // bytes (osm: elements)
+    int out_dt;
+    const void* bias;
+    int bias_dt;
+};
+
+typedef int i32x8s __attribute__((ext_vector_type(8)));
+
+template <int RT, int XT>
+__global__ __launch_bounds__(kWavesS * 64) void mx4_skinny_kernel(Mx4SkArgs a) {
+    constexpr int STEPK = 128, UN = 2;
+    constexpr int KC = STEPK * UN * kWavesS;   // 2048 K-values per chunk
+    constexpr int ROWB = KC / 2 + 16;          // LDS row of codes: 1 KiB + padding (the 16 rows of a quarter-wave in different banks)
+    constexpr int SROW = KC / 32 + 4;          // LDS row of scale bytes: 64 + padding
+    constexpr int ROWS = 16 * XT;
+    constexpr int PIECES = KC / 2 / 16;        // 16-byte pieces per row and chunk: 64
+    constexpr int XS = ROWS * PIECES / (kWavesS * 64);  // code pieces a thread stages per chunk: 2 XT
+    extern __shared__ __align__(16) unsigned char xbuf[];  // [2][ROWS][ROWB] codes, then [2][ROWS][SROW] scales
+    unsigned char* sbuf = xbuf + 2 * ROWS * ROWB;
+    __shared__ f32x4s red[kWavesS][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.x * 16 * RT;
+    const uint8_t* wrow[RT];
+    const uint8_t* srow[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        int n = n0 + 16 * t + r16;
+        if (n > a.N - 1) n = a.N - 1;  // rows past the end repeat the last one; never stored
+        wrow[t] = a.w + (int64_t)n * a.wsn + 16 * kq;
+        srow[t] = a.scales + (int64_t)n * a.msn;
+    }
+    f32x4s acc[RT][XT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt) acc[t][xt] = f32x4s{0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps = a.K / STEPK;
+    const int chunks = (a.K + KC - 1) / KC;
+
+    // staging of a chunk: code pieces id = i * 512 + tid -> (row, piece); the scale bytes of a row are 4 pieces,
+    // taken by the first 4 ROWS threads.  Rows past M repeat row M - 1 (their results are not stored).
+    const uint8_t* xsrc[XS];
+    int xcol[XS], xdst[XS];
+#pragma unroll
+    for (int i = 0; i < XS; ++i) {
+        const int id = i * (kWavesS * 64) + tid;
+        const int row = id / PIECES, col = id % PIECES;
+        xsrc[i] = a.x + (int64_t)(row < a.M ? row : a.M - 1) * a.xsm;
+        xcol[i] = col * 16;
+        xdst[i] = row * ROWB + col * 16;
+    }
+    const bool s_stager = tid < 4 * ROWS;
+    const int s_row = tid >> 2, s_col = (tid & 3) * 16;
+    const uint8_t* ssrc = a.sx + (int64_t)(s_stager && s_row < a.M ? s_row : a.M - 1) * a.sxm;
+    u32x4s xs[XS], ss;
+    auto x_load = [&](int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            int kb = c * (KC / 2) + xcol[i];
+            if (kb > a.K / 2 - 16) kb = a.K / 2 - 16;  // pieces past the end of K repeat the last one; never multiplied
+            xs[i] = *(const u32x4s*)(xsrc[i] + kb);
+        }
+        if (s_stager) {
+            // 16 scale bytes as four dwords (rows are only 4-byte aligned in general, and K/32 is a multiple of 8,
+            // not of 16: a piece can end inside the row).  Dwords past the end repeat the last one; never multiplied.
+            const int sb = c * (KC / 32) + s_col, last = a.K / 32 - 4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int o = sb + 4 * j;
+                ss[j] = *(const uint32_t*)(ssrc + (o < last ? o : last));
+            }
+        }
+    };
+    auto x_store = [&](int c) __attribute__((always_inline)) {
+        unsigned char* base = xbuf + (c & 1) * (ROWS * ROWB);
+#pragma unroll
+        for (int i = 0; i < XS; ++i) *(u32x4s*)(base + xdst[i]) = xs[i];
+        if (s_stager) {
+            uint32_t* d = (uint32_t*)(sbuf + (c & 1) * (ROWS * SROW) + s_row * SROW + s_col);
+            d[0] = ss[0]; d[1] = ss[1]; d[2] = ss[2]; d[3] = ss[3];
+        }
+    };
+    struct Batch {
+        u32x4s wv[UN][RT];
+        uint32_t sc[RT][2];
+    };
+    auto w_load = [&](Batch& b, int c) __attribute__((always_inline)) {
+        int s0 = c * (UN * kWavesS) + UN * wave;
+        if (s0 > steps - UN) s0 = 0;  // pairs past the end re-read the first; never multiplied
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const uint4 q = load_streaming_u4(wrow[t] + (int64_t)(s0 + u) * kStepB);
+                b.wv[u][t] = u32x4s{q.x, q.y, q.z, q.w};
+            }
+            const uint32_t* sp = (const uint32_t*)(srow[t] + s0 * 4);  // rows are 4-byte aligned in general
+            b.sc[t][0] = sp[0]; b.sc[t][1] = sp[1];
+        }
+    };
+    auto multiply = [&](const Batch& b, int c) __attribute__((always_inline)) {
+        const unsigned char* cbase = xbuf + (c & 1) * (ROWS * ROWB) + r16 * ROWB + kq * 16;
+        const unsigned char* sbase = sbuf + (c & 1) * (ROWS * SROW) + r16 * SROW;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int sl = UN * wave + u;  // step inside the chunk
+            if (c * (UN * kWavesS) + sl < steps) {
+#pragma unroll
+                for (int xt = 0; xt < XT; ++xt) {
+                    const u32x4s xv = *(const u32x4s*)(cbase + xt * 16 * ROWB + sl * (STEPK / 2));
+                    const uint32_t sxw = *(const uint32_t*)(sbase + xt * 16 * SROW + sl * 4);
+                    const int ex = (int)((sxw >> (8 * kq)) & 0xffu);
+                    const i32x8s b8 = {(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3], 0, 0, 0, 0};
+#pragma unroll
+                    for (int t = 0; t < RT; ++t) {
+                        const int ew = (int)((b.sc[t][u] >> (8 * kq)) & 0xffu);
+                        const u32x4s wv = b.wv[u][t];
+                        const i32x8s a8 = {(int)wv[0], (int)wv[1], (int)wv[2], (int)wv[3], 0, 0, 0, 0};
+                        acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 4, 0, ew, 0, ex);
+                    }
+                }
+            }
+        }
+    };
+    Batch b0, b1;
+    x_load(0);
+    w_load(b0, 0);
+    x_store(0);
+    if (chunks > 1) x_load(1);
+    for (int c = 0; c < chunks; c += 2) {
+        __syncthreads();  // chunk c is in LDS; everybody is done with the buffer chunk c + 1 goes to
+        if (c + 1 < chunks) {
+            x_store(c + 1);
+            w_load(b1, c + 1);
+        }
+        if (c + 2 < chunks) x_load(c + 2);
+        multiply(b0, c);
+        if (c + 1 < chunks) {
+            __syncthreads();
+            if (c + 2 < chunks) {
+                x_store(c + 2);
+                w_load(b0, c + 2);
+            }
+            if (c + 3 < chunks) x_load(c + 3);
+            multiply(b1, c + 1);
+        }
+    }
+    // lane holds D[n0 + 16 t + 4 kq + e][m = 16 xt + r16]; the waves' sums are added in wave order, one tile at a time
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt) {
+            if (t || xt) __syncthreads();
+            red[wave][lane] = acc[t][xt];
+            __syncthreads();
+            const int m = 16 * xt + r16;
+            if (wave != 0 || m >= a.M) continue;
+            f32x4s D = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int w = 0; w < kWavesS; ++w) D += red[w][lane];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n0 + 16 * t + 4 * kq + e;
+                if (n >= a.N) continue;
+                float v = D[e];
+                if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + load_as_float(a.bias, a.bias_dt, n);
+                store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + n, v);
+            }
+        }
+    }
+}
+
+template <int RT, int XT>
+int launch_variant4(const Mx4SkArgs& a, hipStream_t stream) {
+    constexpr int KC = 128 * 2 * kWavesS;
+    const size_t smem = 2 * 16 * XT * (size_t)(KC / 2 + 16) + 2 * 16 * XT * (size_t)(KC / 32 + 4);
+    static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
+    auto kern = mx4_skinny_kernel<RT, XT>;
+    if (once.first()) {
+        const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
+                                 "mx4_skinny: raising the dynamic LDS limit");
+        if (rc != GLA_OK) return rc;
+    }
+    hipLaunchKernelGGL(kern, dim3(ceil_div(ceil_div(a.N, 16), RT)), dim3(kWavesS * 64), smem, stream, a);
+    return check_hip(hipGetLastError(), "mx4_skinny launch");
+}
+
+template <int XT>
+int launch_sk4(const Mx4SkArgs& a, hipStream_t stream) {
+    // as many row tiles per wave as still leave every CU a workgroup
+    const int tiles = ceil_div(a.N, 16);
+    if (tiles >= 4 * 256) return launch_variant4<4, XT>(a, stream);
+    if (tiles >= 2 * 256) return launch_variant4<2, XT>(a, stream);
+    return launch_variant4<1, XT>(a, stream);
+}
+
 template <bool W4, bool BF16, int RT>
 int launch_variant(const MxSkArgs& a, hipStream_t stream) {
     constexpr int KC = (W4 ? 128 : 64) * 2 * kWavesS;
@@ -276,7 +498,21 @@ int launch_sk(const MxSkArgs& a, hipStream_t stream) {
 
 }  // namespace
 
+// MXFP4 x MXFP4 (codes and e8m0 bytes on both sides), up to 32 rows
+static bool mx4_skinny_ok(const gla_matmul_args& p) {
+    if (p.input_dtype != GLA_DT_MXFP4 || p.x_quant_from != 0) return false;
+    if (p.M < 1 || p.M > 32 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_MX) return false;
+    if (p.scales == nullptr || p.scales_x == nullptr || p.sx_dtype != GLA_DT_UINT8) return false;
+    if (!(p.W_nbits == 4 && p.elements_per_sample == 2)) return false;
+    if (p.K % 256 != 0) return false;  // whole pairs of steps
+    if (p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3) || p.sx_stride_m % 4 != 0 || ((uintptr_t)p.scales_x & 3)) return false;
+    if (p.x_stride_k != 1 || p.w_stride_k != 1 || p.out_stride_n != 1 || p.meta_stride_g != 1 || p.sx_stride_g != 1) return false;
+    if (p.x_stride_m % 16 != 0 || p.w_stride_n % 16 != 0 || ((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
+    return p.output_dtype == GLA_DT_FP32 || p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16;
+}
+
 bool mx_skinny_eligible(const gla_matmul_args& p) {
+    if (p.input_dtype == GLA_DT_MXFP4) return mx4_skinny_ok(p);
     if (!(p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)) return false;
     if (p.M < 1 || p.M > 16 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_NONE || p.scales == nullptr) return false;
     const bool w4 = p.W_nbits == 4 && p.elements_per_sample == 2;
@@ -294,6 +530,14 @@ bool mx_skinny_eligible(const gla_matmul_args& p) {
 }
 
 int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream) {
+    if (p.input_dtype == GLA_DT_MXFP4 && mx4_skinny_ok(p)) {
+        Mx4SkArgs a;
+        a.x = (const uint8_t*)p.x; a.sx = (const uint8_t*)p.scales_x; a.w = (const uint8_t*)p.w; a.scales = (const uint8_t*)p.scales;
+        a.out = p.out; a.M = p.M; a.N = p.N; a.K = p.K;
+        a.xsm = p.x_stride_m; a.sxm = p.sx_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = p.meta_stride_n;
+        a.out_dt = p.output_dtype; a.bias = p.bias; a.bias_dt = p.bias_dtype;
+        return p.M <= 16 ? launch_sk4<1>(a, stream) : launch_sk4<2>(a, stream);
+    }
     if (!mx_skinny_eligible(p)) {
         set_error("mx_skinny: weight-only MX operands, K-contiguous with 16-byte aligned rows, up to 16 rows, "
                   "K a multiple of 256 (MXFP4) or 128 (MXFP8)");

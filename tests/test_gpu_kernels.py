@@ -547,7 +547,7 @@ def test_a4w4_decode_rows_are_quantised_inside_the_matmul(device, dtype):
     """MXFP4 x MXFP4 at the rows the streaming kernel takes: the kernel makes the e2m1 codes and e8m0 bytes of its
     activation blocks itself; same output as the quantiser launch + matmul bit for bit (blocks of all zeros, of
     tiny and of huge values, ties of the e2m1 grid included)."""
-    for (N, K) in ((520, 4224), (512, 4096)):   # K of the reference's MX tests (streams at any row count); a K the matrix cores take
+    for (N, K) in ((520, 4224), (512, 4096)):   # K of the reference's MX tests (streams up to 4 rows); a K the matrix cores take
         W = gen_x(N, K, torch.bfloat16, seed=7, std=0.02)
         codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
         layer = helper.A4W4_MXFP_dynamic(device=device, dtype=dtype).from_weights(torch.from_numpy(codes), scales=torch.from_numpy(e8))
@@ -558,10 +558,36 @@ def test_a4w4_decode_rows_are_quantised_inside_the_matmul(device, dtype):
             x[0, 64:96] *= 1e-4
             x[0, 96:128] *= 3e3
             x = x.to(device)
-            if K % 128 == 0:
-                assert _fused_family(layer, x) == ("MX_STREAM" if M <= 4 else None), M
+            if K % 256 == 0:   # from 3 rows the scaled-MFMA kernel takes ready-made codes: the fused call is declined
+                assert _fused_family(layer, x) == ("MX_STREAM" if M <= 2 else None), M
             y_fused, y_two = _forward_both_ways(layer, x)
             assert torch.equal(y_fused, y_two), (K, M)
+            check_layer(layer, x, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_a4w4_mxfp4_skinny_rows_on_the_scaled_mfma(device, dtype):
+    """3..32 rows of MXFP4 x MXFP4 (K a multiple of 256): weight codes go from registers straight into the scaled
+    MFMA against the activation codes of 16 or 32 rows.  Ragged N (last tile of 16 columns partly past N), a K that
+    ends inside a chunk of 2048, one and two activation tiles, a bias."""
+    for (N, K) in ((1040, 4096), (520, 2304), (2056, 512), (72, 256)):
+        W = gen_x(N, K, torch.bfloat16, seed=N, std=0.02)
+        codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+        layer = helper.A4W4_MXFP_dynamic(device=device, dtype=dtype).from_weights(
+            torch.from_numpy(codes), scales=torch.from_numpy(e8), bias=gen_x(1, N, dtype, seed=1).reshape(-1) if N == 520 else None)
+        for M in (3, 5, 16, 17, 32, 33):
+            x = gen_x(M, K, dtype, seed=70 + M).to(device)
+            xq, sx = gemlite_amd.scale_activations_mxfp4(x)
+            m = layer.get_meta_args()
+            out = torch.empty(M, N, dtype=dtype, device=device)
+            a = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, out, W_nbits=m[1], group_size=m[2],
+                                       unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                       acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                       data_contiguous=m[11])
+            if M == 33:
+                assert _ext.matmul_family(a) == "GEMM_MXFP4"
+            else:
+                assert _ext.matmul_family(a) == "MX_SKINNY", (N, K, M, _ext.matmul_family(a))
             check_layer(layer, x, dtype)
 
 

@@ -353,7 +353,7 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
     for M in (1, 32, 1024):
         xq = torch.zeros(M, K // 2, dtype=torch.uint8)
         sx = torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
-        assert _family(lm, M, None, scales_x=sx, x=xq) == ("MX_STREAM" if M <= 2 else "GEMM_MXFP4")
+        assert _family(lm, M, None, scales_x=sx, x=xq) == {1: "MX_STREAM", 32: "MX_SKINNY", 1024: "GEMM_MXFP4"}[M]
 
 
 def test_tile_config_can_state_a_preference_between_streaming_and_matrix_kernels():
