@@ -221,16 +221,15 @@ Family choose(const gla_matmul_args& p, int type) {
     const bool want_stream = p.tile_config == GLA_TILE_PREFER_STREAMING, want_matrix = p.tile_config == GLA_TILE_PREFER_MATRIX;
     if (p.input_dtype == GLA_DT_MXFP4) {
         // Three kernels.  The streaming kernel (dot products on the vector unit; also the one that quantises 16-bit rows
-        // itself) for 1-2 rows.  From 3 to 32 rows the weights go straight from registers into the scaled MFMA: no LDS
-        // tile, no K split, no finishing or scale-regrouping launch (8 rows, 4096^2: 5.1 against 14.1 us of the tiled
-        // GEMM; 8192^2: 13.0 against 17.8; 3 rows: 5.2 / 13.0 against 9.9 / 18.8 of the streaming kernel).  On layers of 100 MB and more the tiled GEMM is level with it or
-        // ahead (16384^2, 8 / 32 rows: 41.0 / 44.4 against 42.7 / 48.0) and keeps the call.
+        // itself) for 1-2 rows.  From 3 to 32 rows the weights go as they are into the scaled MFMA, copied to LDS by
+        // whole 128-byte lines: no K split, no finishing or scale-regrouping launch (8 / 32 rows: 4096^2 4.7 / 6.5 us
+        // against 14.1 / 15.3 of the tiled GEMM, 16384^2 34.3 / 41.2 against 41.0 / 44.4; 3 rows on 4096^2: 4.7 against
+        // 9.9 of the streaming kernel).  Above 32 rows the tiled GEMM.
         const int64_t wbytes = (int64_t)p.N * p.K / 2;
         const bool stream_ok = p.tile_config < 1000 && mx_stream_eligible(p), matrix_ok = gemm_mxfp4_eligible(p);
         if (want_stream && stream_ok) return F_MX_STREAM;
         if (want_matrix && matrix_ok) return F_GEMM_MXFP4;
-        if (p.M >= 3 && p.M <= 32 && p.tile_config < 1000 && (wbytes < 100000000 || !matrix_ok) && mx_skinny_eligible(p))
-            return F_MX_SKINNY;
+        if (p.M >= 3 && p.M <= 32 && p.tile_config < 1000 && mx_skinny_eligible(p)) return F_MX_SKINNY;
         // K not a multiple of 256 (or operands the skinny kernel does not take): the streaming kernel up to 2 rows
         // everywhere, up to 4 on layers of 40 MB or less (4096^2 at 4 rows: 10.7 against 14.4 us of the tiled GEMM;
         // 16384^2: 54 against 40)

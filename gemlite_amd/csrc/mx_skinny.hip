@@ -254,19 +254,11 @@ __global__ __launch_bounds__(kWavesS * 64) void mx_skinny_kernel(MxSkArgs a) {
 // ---------------------------------------------------------------------------------------------------------
 // MXFP4 x MXFP4 at 3..32 rows: the same walk over the weights, but nothing is converted.  A lane's 16 weight
 // bytes (32 e2m1 codes of one 32-block) ARE its share of the A operand of v_mfma_scale_f32_16x16x128_f8f6f4,
-// the block's e8m0 byte its scale; the B operand is the same 32-block of 16 activation rows (codes and e8m0
-// bytes staged through LDS like the 16-bit activations above), so one instruction multiplies 16 weight rows
-// with 16 activation rows over 128 K-values and applies both block scales (reference:
+// the block's e8m0 byte its scale; the B operand is the same 32-block of 16 activation rows, so one instruction
+// multiplies 16 weight rows with 16 activation rows over 128 K-values and applies both block scales (reference:
 // gemlite/triton_kernels/gemm_splitK_kernels.py:536-770, `tl.dot_scaled` on e2m1 operands).  XT = 1 or 2 tiles of
-// 16 activation rows.  Between the vector-unit streaming kernel (1-2 rows, 4 on small layers) and the tiled
-// GEMM (64-row tiles through LDS, split K, a finishing launch and a scale-regrouping launch in front).
-//  * 8 / 32 rows: 4096^2 5.1 / 6.5 us (tiled GEMM 14.1 / 15.3), 8192^2 13.0 / 16.0 (17.8 / 19.9), 14336 x 4096
-//    11.3 / 14.5 (16.1 / 18.6), 16384^2 42.7 / 48.0 (41.0 / 44.4: the dispatcher keeps the GEMM there).
-//  * The bound is the access pattern the [N, K/2] layout forces on an MFMA operand: a wave instruction reads 16
-//    rows x 64 bytes.  The same kernel reading 1 KiB contiguous per instruction (weights regrouped by operand;
-//    timing only, not built) took 28 / 35 us at 1 / 16 rows on 16384^2 and 9.5 / 11.1 on 8192^2.  Loading the
-//    activations per lane from global memory instead of through LDS (no barrier in the K loop) gave the same
-//    times up to 16 rows and 10-20 % worse ones at 32.
+// 16 activation rows.  Between the vector-unit streaming kernel (1-2 rows) and the tiled GEMM (64-row tiles
+// through LDS, split K, a finishing launch and a scale-regrouping launch in front).
 struct Mx4SkArgs {
     const uint8_t* x;         // [M, K/2] e2m1 pairs
     const uint8_t* sx;        // [ceil32(M), K/32] e8m0
@@ -282,145 +274,138 @@ struct Mx4SkArgs {
 
 typedef int i32x8s __attribute__((ext_vector_type(8)));
 
-template <int RT, int XT>
-__global__ __launch_bounds__(kWavesS * 64) void mx4_skinny_kernel(Mx4SkArgs a) {
-    constexpr int STEPK = 128, UN = 2;
-    constexpr int KC = STEPK * UN * kWavesS;   // 2048 K-values per chunk
-    constexpr int ROWB = KC / 2 + 16;          // LDS row of codes: 1 KiB + padding (the 16 rows of a quarter-wave in different banks)
-    constexpr int SROW = KC / 32 + 4;          // LDS row of scale bytes: 64 + padding
-    constexpr int ROWS = 16 * XT;
-    constexpr int PIECES = KC / 2 / 16;        // 16-byte pieces per row and chunk: 64
-    constexpr int XS = ROWS * PIECES / (kWavesS * 64);  // code pieces a thread stages per chunk: 2 XT
-    extern __shared__ __align__(16) unsigned char xbuf[];  // [2][ROWS][ROWB] codes, then [2][ROWS][SROW] scales
-    unsigned char* sbuf = xbuf + 2 * ROWS * ROWB;
-    __shared__ f32x4s red[kWavesS][64];
+// s_waitcnt vmcnt(N) only: vmcnt is bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "no wait"
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_sk() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// Every operand is copied global -> LDS by the load unit (global_load_lds) into a ring that is private to the wave:
+// a copy instruction moves 8 rows x 128 contiguous bytes (the codes of a pair of steps), so rows are read in whole
+// 128-byte lines instead of the 16 x 64 bytes an MFMA operand load touches, nothing waits in registers, and there is
+// no barrier before the final sum of the waves' accumulators.  A tile (16 weight rows, or 16 activation rows) of a
+// pair is 2 KiB of codes, 16-byte slots XOR-swizzled by row >> 1 so that the operand reads (16 rows, one slot each)
+// fall in different banks, plus its 16 x 8 scale bytes.  The NW waves take the pairs of K in turn, NB pairs per wave
+// in flight.  K must be a multiple of 256.
+//  * 8 / 32 rows (us; tiled GEMM in brackets): 4096^2 4.7 / 6.5 (14.1 / 15.3), 8192^2 11.2 / 14.5 (17.8 / 19.9),
+//    4096 x 14336 9.8 / 14.3 (18.9 / 21.0), 14336 x 4096 10.8 / 14.7 (16.1 / 18.6), 16384^2 34.3 / 41.2 (41.0 / 44.4).
+//  * Two earlier forms of this kernel loaded the weights per lane in operand order (16 rows x 64 bytes per wave
+//    instruction), the activations through a shared LDS stage or per lane: 13.0-13.8 us on 8192^2 and 42.7-43.0 on
+//    16384^2 at 8 rows whatever else was varied (rows per wave, steps in flight, 8 or 16 waves, K order rotated per
+//    workgroup); the same code reading 1 KiB contiguous per instruction (timing only) took 9.5-11.1 and 28-35 us.
+//    The access pattern was the bound; copies by whole lines recover most of it without a second weight layout.
+template <int RT, int XT, int NW, int NB>
+__global__ __launch_bounds__(NW * 64) void mx4_ring_kernel(Mx4SkArgs a) {
+    constexpr int TILE = 2048 + 256;
+    constexpr int NT = RT + XT;
+    constexpr int OPS = 3 * NT;  // copy instructions per pair
+    static_assert((NB - 1) * OPS < 64, "outstanding copies must fit the vmcnt counter");
+    extern __shared__ __align__(16) unsigned char ring[];  // [NW][NB][NT][TILE]
+    __shared__ f32x4s red[NW][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.x * 16 * RT;
-    const uint8_t* wrow[RT];
-    const uint8_t* srow[RT];
+    unsigned char* mine = ring + (size_t)wave * NB * NT * TILE;
+
+    // copy plan of a pair: per tile two code instructions (rows 8j + lane / 8, slot lane % 8 <- piece slot ^ (row >> 1))
+    // and one for the scale bytes (row (lane / 2) % 16, dword lane % 2; the upper half-wave writes a duplicate)
+    const uint8_t* csrc[NT][2];
+    const uint8_t* ssrc[NT];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
-        int n = n0 + 16 * t + r16;
-        if (n > a.N - 1) n = a.N - 1;  // rows past the end repeat the last one; never stored
-        wrow[t] = a.w + (int64_t)n * a.wsn + 16 * kq;
-        srow[t] = a.scales + (int64_t)n * a.msn;
+    for (int i = 0; i < NT; ++i) {
+        const bool is_w = i < RT;
+        auto row_ptr = [&](int row, bool scale) -> const uint8_t* {
+            if (is_w) {
+                int n = n0 + 16 * i + row;
+                if (n > a.N - 1) n = a.N - 1;  // rows past the end repeat the last one; never stored
+                return scale ? a.scales + (int64_t)n * a.msn : a.w + (int64_t)n * a.wsn;
+            }
+            int m = 16 * (i - RT) + row;
+            if (m > a.M - 1) m = a.M - 1;
+            return scale ? a.sx + (int64_t)m * a.sxm : a.x + (int64_t)m * a.xsm;
+        };
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int row = 8 * j + (lane >> 3), slot = lane & 7;
+            csrc[i][j] = row_ptr(row, false) + ((slot ^ (row >> 1)) & 7) * 16;
+        }
+        ssrc[i] = row_ptr((lane >> 1) & 15, true) + (lane & 1) * 4;
     }
+    auto issue = [&](int p, int slot) __attribute__((always_inline)) {
+        unsigned char* base = mine + slot * (NT * TILE);
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(csrc[i][j] + (int64_t)p * 128),
+                                                 (__attribute__((address_space(3))) void*)(base + i * TILE + j * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ssrc[i] + (int64_t)p * 8),
+                                             (__attribute__((address_space(3))) void*)(base + i * TILE + 2048), 4, 0, 0);
+        }
+    };
     f32x4s acc[RT][XT];
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
         for (int xt = 0; xt < XT; ++xt) acc[t][xt] = f32x4s{0.0f, 0.0f, 0.0f, 0.0f};
-    const int steps = a.K / STEPK;
-    const int chunks = (a.K + KC - 1) / KC;
-
-    // staging of a chunk: code pieces id = i * 512 + tid -> (row, piece); the scale bytes of a row are 4 pieces,
-    // taken by the first 4 ROWS threads.  Rows past M repeat row M - 1 (their results are not stored).
-    const uint8_t* xsrc[XS];
-    int xcol[XS], xdst[XS];
+    const int code_off = r16 * 128, swz = r16 >> 1, scale_off = 2048 + r16 * 8;
+    auto multiply = [&](int slot) __attribute__((always_inline)) {
+        const unsigned char* base = mine + slot * (NT * TILE);
 #pragma unroll
-    for (int i = 0; i < XS; ++i) {
-        const int id = i * (kWavesS * 64) + tid;
-        const int row = id / PIECES, col = id % PIECES;
-        xsrc[i] = a.x + (int64_t)(row < a.M ? row : a.M - 1) * a.xsm;
-        xcol[i] = col * 16;
-        xdst[i] = row * ROWB + col * 16;
-    }
-    const bool s_stager = tid < 4 * ROWS;
-    const int s_row = tid >> 2, s_col = (tid & 3) * 16;
-    const uint8_t* ssrc = a.sx + (int64_t)(s_stager && s_row < a.M ? s_row : a.M - 1) * a.sxm;
-    u32x4s xs[XS], ss;
-    auto x_load = [&](int c) __attribute__((always_inline)) {
+        for (int u = 0; u < 2; ++u) {
+            const int piece = (((4 * u + kq) ^ swz) & 7) * 16;
 #pragma unroll
-        for (int i = 0; i < XS; ++i) {
-            int kb = c * (KC / 2) + xcol[i];
-            if (kb > a.K / 2 - 16) kb = a.K / 2 - 16;  // pieces past the end of K repeat the last one; never multiplied
-            xs[i] = *(const u32x4s*)(xsrc[i] + kb);
-        }
-        if (s_stager) {
-            // 16 scale bytes as four dwords (rows are only 4-byte aligned in general, and K/32 is a multiple of 8,
-            // not of 16: a piece can end inside the row).  Dwords past the end repeat the last one; never multiplied.
-            const int sb = c * (KC / 32) + s_col, last = a.K / 32 - 4;
+            for (int xt = 0; xt < XT; ++xt) {
+                const unsigned char* xb = base + (RT + xt) * TILE;
+                const u32x4s xv = *(const u32x4s*)(xb + code_off + piece);
+                const int ex = (int)((*(const uint32_t*)(xb + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
+                const i32x8s b8 = {(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3], 0, 0, 0, 0};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int o = sb + 4 * j;
-                ss[j] = *(const uint32_t*)(ssrc + (o < last ? o : last));
-            }
-        }
-    };
-    auto x_store = [&](int c) __attribute__((always_inline)) {
-        unsigned char* base = xbuf + (c & 1) * (ROWS * ROWB);
-#pragma unroll
-        for (int i = 0; i < XS; ++i) *(u32x4s*)(base + xdst[i]) = xs[i];
-        if (s_stager) {
-            uint32_t* d = (uint32_t*)(sbuf + (c & 1) * (ROWS * SROW) + s_row * SROW + s_col);
-            d[0] = ss[0]; d[1] = ss[1]; d[2] = ss[2]; d[3] = ss[3];
-        }
-    };
-    struct Batch {
-        u32x4s wv[UN][RT];
-        uint32_t sc[RT][2];
-    };
-    auto w_load = [&](Batch& b, int c) __attribute__((always_inline)) {
-        int s0 = c * (UN * kWavesS) + UN * wave;
-        if (s0 > steps - UN) s0 = 0;  // pairs past the end re-read the first; never multiplied
-#pragma unroll
-        for (int t = 0; t < RT; ++t) {
-#pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                const uint4 q = load_streaming_u4(wrow[t] + (int64_t)(s0 + u) * kStepB);
-                b.wv[u][t] = u32x4s{q.x, q.y, q.z, q.w};
-            }
-            const uint32_t* sp = (const uint32_t*)(srow[t] + s0 * 4);  // rows are 4-byte aligned in general
-            b.sc[t][0] = sp[0]; b.sc[t][1] = sp[1];
-        }
-    };
-    auto multiply = [&](const Batch& b, int c) __attribute__((always_inline)) {
-        const unsigned char* cbase = xbuf + (c & 1) * (ROWS * ROWB) + r16 * ROWB + kq * 16;
-        const unsigned char* sbase = sbuf + (c & 1) * (ROWS * SROW) + r16 * SROW;
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const int sl = UN * wave + u;  // step inside the chunk
-            if (c * (UN * kWavesS) + sl < steps) {
-#pragma unroll
-                for (int xt = 0; xt < XT; ++xt) {
-                    const u32x4s xv = *(const u32x4s*)(cbase + xt * 16 * ROWB + sl * (STEPK / 2));
-                    const uint32_t sxw = *(const uint32_t*)(sbase + xt * 16 * SROW + sl * 4);
-                    const int ex = (int)((sxw >> (8 * kq)) & 0xffu);
-                    const i32x8s b8 = {(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3], 0, 0, 0, 0};
-#pragma unroll
-                    for (int t = 0; t < RT; ++t) {
-                        const int ew = (int)((b.sc[t][u] >> (8 * kq)) & 0xffu);
-                        const u32x4s wv = b.wv[u][t];
-                        const i32x8s a8 = {(int)wv[0], (int)wv[1], (int)wv[2], (int)wv[3], 0, 0, 0, 0};
-                        acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 4, 0, ew, 0, ex);
-                    }
+                for (int t = 0; t < RT; ++t) {
+                    const unsigned char* wb = base + t * TILE;
+                    const u32x4s wv = *(const u32x4s*)(wb + code_off + piece);
+                    const int ew = (int)((*(const uint32_t*)(wb + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
+                    const i32x8s a8 = {(int)wv[0], (int)wv[1], (int)wv[2], (int)wv[3], 0, 0, 0, 0};
+                    acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 4, 0, ew, 0, ex);
                 }
             }
         }
     };
-    Batch b0, b1;
-    x_load(0);
-    w_load(b0, 0);
-    x_store(0);
-    if (chunks > 1) x_load(1);
-    for (int c = 0; c < chunks; c += 2) {
-        __syncthreads();  // chunk c is in LDS; everybody is done with the buffer chunk c + 1 goes to
-        if (c + 1 < chunks) {
-            x_store(c + 1);
-            w_load(b1, c + 1);
-        }
-        if (c + 2 < chunks) x_load(c + 2);
-        multiply(b0, c);
-        if (c + 1 < chunks) {
-            __syncthreads();
-            if (c + 2 < chunks) {
-                x_store(c + 2);
-                w_load(b0, c + 2);
+    const int pairs = a.K / 256;
+    const int iters = (pairs + NW - 1) / NW;
+    // a wave whose turn lies past the end copies the last pair again (same count of copies for everybody) and skips the multiply
+    auto pair_of = [&](int it) { const int p = it * NW + wave; return p < pairs ? p : pairs - 1; };
+#pragma unroll
+    for (int b = 0; b < NB - 1; ++b)
+        if (b < iters) issue(pair_of(b), b);
+    int slot = 0, islot = NB - 1;
+    for (int it = 0; it < iters; ++it) {
+        const int later = iters - 1 - it;  // pairs issued after this one
+        if (later >= NB - 1) {
+            issue(pair_of(it + NB - 1), islot);
+            islot = islot == NB - 1 ? 0 : islot + 1;
+            wait_vmcnt_sk<(NB - 1) * OPS>();
+        } else {
+            // the ring drains: `later` pairs are still allowed in flight
+            bool done = false;
+#pragma unroll
+            for (int k = NB - 2; k >= 1; --k) {
+                if (!done && later == k) {
+                    if (k == 1) wait_vmcnt_sk<1 * OPS < 64 ? 1 * OPS : 0>();
+                    else if (k == 2) wait_vmcnt_sk<2 * OPS < 64 ? 2 * OPS : 0>();
+                    else if (k == 3) wait_vmcnt_sk<3 * OPS < 64 ? 3 * OPS : 0>();
+                    else wait_vmcnt_sk<0>();
+                    done = true;
+                }
             }
-            if (c + 3 < chunks) x_load(c + 3);
-            multiply(b1, c + 1);
+            if (!done) wait_vmcnt_sk<0>();
         }
+        asm volatile("" ::: "memory");
+        if (it * NW + wave < pairs) multiply(slot);
+        slot = slot == NB - 1 ? 0 : slot + 1;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);  // the copies of the next turn go to the slot these reads came from
     }
     // lane holds D[n0 + 16 t + 4 kq + e][m = 16 xt + r16]; the waves' sums are added in wave order, one tile at a time
 #pragma unroll
@@ -434,7 +419,7 @@ __global__ __launch_bounds__(kWavesS * 64) void mx4_skinny_kernel(Mx4SkArgs a) {
             if (wave != 0 || m >= a.M) continue;
             f32x4s D = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int w = 0; w < kWavesS; ++w) D += red[w][lane];
+            for (int w = 0; w < NW; ++w) D += red[w][lane];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int n = n0 + 16 * t + 4 * kq + e;
@@ -447,28 +432,18 @@ __global__ __launch_bounds__(kWavesS * 64) void mx4_skinny_kernel(Mx4SkArgs a) {
     }
 }
 
-template <int RT, int XT>
-int launch_variant4(const Mx4SkArgs& a, hipStream_t stream) {
-    constexpr int KC = 128 * 2 * kWavesS;
-    const size_t smem = 2 * 16 * XT * (size_t)(KC / 2 + 16) + 2 * 16 * XT * (size_t)(KC / 32 + 4);
+template <int RT, int XT, int NW, int NB>
+int launch_ring4(const Mx4SkArgs& a, hipStream_t stream) {
+    const size_t smem = (size_t)NW * NB * (RT + XT) * (2048 + 256);
     static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
-    auto kern = mx4_skinny_kernel<RT, XT>;
+    auto kern = mx4_ring_kernel<RT, XT, NW, NB>;
     if (once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
-                                 "mx4_skinny: raising the dynamic LDS limit");
+                                 "mx4_ring: raising the dynamic LDS limit");
         if (rc != GLA_OK) return rc;
     }
-    hipLaunchKernelGGL(kern, dim3(ceil_div(ceil_div(a.N, 16), RT)), dim3(kWavesS * 64), smem, stream, a);
-    return check_hip(hipGetLastError(), "mx4_skinny launch");
-}
-
-template <int XT>
-int launch_sk4(const Mx4SkArgs& a, hipStream_t stream) {
-    // as many row tiles per wave as still leave every CU a workgroup
-    const int tiles = ceil_div(a.N, 16);
-    if (tiles >= 4 * 256) return launch_variant4<4, XT>(a, stream);
-    if (tiles >= 2 * 256) return launch_variant4<2, XT>(a, stream);
-    return launch_variant4<1, XT>(a, stream);
+    hipLaunchKernelGGL(kern, dim3(ceil_div(ceil_div(a.N, 16), RT)), dim3(NW * 64), smem, stream, a);
+    return check_hip(hipGetLastError(), "mx4_ring launch");
 }
 
 template <bool W4, bool BF16, int RT>
@@ -536,7 +511,18 @@ int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream) {
         a.out = p.out; a.M = p.M; a.N = p.N; a.K = p.K;
         a.xsm = p.x_stride_m; a.sxm = p.sx_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = p.meta_stride_n;
         a.out_dt = p.output_dtype; a.bias = p.bias; a.bias_dt = p.bias_dtype;
-        return p.M <= 16 ? launch_sk4<1>(a, stream) : launch_sk4<2>(a, stream);
+        // rows of tiles per wave so that about one workgroup per CU comes out; fewer, deeper waves where a wave has
+        // 4 weight tiles to an activation tile (16384^2 at 8 rows: 34.3 us with 4 tiles x 4 waves x 3 pairs in flight,
+        // 38.4 with 2 x 8 x 2, 35.2 with 1 x 8 x 4; 8192^2: 15.5 / 11.2 / 12.6; 4096^2: 8.9 / 6.1 / 4.7)
+        const int tiles = ceil_div(p.N, 16);
+        if (p.M <= 16) {
+            if (tiles >= 880) return launch_ring4<4, 1, 4, 3>(a, stream);
+            if (tiles >= 440) return launch_ring4<2, 1, 8, 2>(a, stream);
+            return launch_ring4<1, 1, 8, 4>(a, stream);
+        }
+        if (tiles >= 880) return launch_ring4<4, 2, 4, 2>(a, stream);
+        if (tiles >= 440) return launch_ring4<2, 2, 4, 4>(a, stream);
+        return launch_ring4<1, 2, 8, 2>(a, stream);
     }
     if (!mx_skinny_eligible(p)) {
         set_error("mx_skinny: weight-only MX operands, K-contiguous with 16-byte aligned rows, up to 16 rows, "

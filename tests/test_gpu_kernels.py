@@ -567,10 +567,11 @@ def test_a4w4_decode_rows_are_quantised_inside_the_matmul(device, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_a4w4_mxfp4_skinny_rows_on_the_scaled_mfma(device, dtype):
-    """3..32 rows of MXFP4 x MXFP4 (K a multiple of 256): weight codes go from registers straight into the scaled
-    MFMA against the activation codes of 16 or 32 rows.  Ragged N (last tile of 16 columns partly past N), a K that
-    ends inside a chunk of 2048, one and two activation tiles, a bias."""
-    for (N, K) in ((1040, 4096), (520, 2304), (2056, 512), (72, 256)):
+    """3..32 rows of MXFP4 x MXFP4 (K a multiple of 256): weight and activation codes are copied to LDS by lines and
+    go into the scaled MFMA as they are.  Ragged N (last tile of 16 columns partly past N), K with fewer pairs of steps
+    than waves and with a last turn only some waves take, one and two activation tiles, every launch shape (1, 2 and 4
+    weight tiles per wave), a bias."""
+    for (N, K) in ((1040, 4096), (520, 2304), (2056, 512), (72, 256), (7056, 768), (14096, 512)):
         W = gen_x(N, K, torch.bfloat16, seed=N, std=0.02)
         codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
         layer = helper.A4W4_MXFP_dynamic(device=device, dtype=dtype).from_weights(
