@@ -26,6 +26,8 @@
 //    the activation fragment is used as it lies in memory.  bf16 activations: codes paired (j, j+4)
 //    in the mantissa of 128.0, fp32 fma, one packed round-to-nearest-even conversion (byte codes:
 //    direct byte-to-float conversion); the activation fragment is reordered to match (v_perm).
+//    2-bit codes on bf16: the four dequantised values of a column and group are made once per group and a
+//    code pair picks its two with one byte permute (4 instructions per pair instead of 7; identical bits).
 //  * The weights are the row operand of the MFMA: an accumulator is the transposed output tile and
 //    a lane holds 4 TJ adjacent output columns of one row, stored 16 bytes at a time.
 //  * When the output has too few tiles to fill the chip (small M), K is split over gridDim.y:
@@ -102,6 +104,7 @@ struct ColMeta<false> {
 template <>
 struct ColMeta<true> {
     float s, z;  // s and z' - 128 s in fp32: the offset of the unpacking trick is folded into the constant
+    uint32_t lut01, lut23;  // 2-bit codes: the four dequantised values of the group as bf16 pairs (w0, w1), (w2, w3)
 };
 
 // OFF: the offset the unpacking leaves on the codes in the fp32 path (128, or 0 for byte codes)
@@ -313,6 +316,15 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
             const float s = (meta_bf16 ? s_b : s_h) + s_add;
             const float z = (meta_bf16 ? z_b : z_h) + z_add;
             meta[j] = make_meta<BF16, (BITS == 8 ? 0 : 128)>(s, z * __builtin_fmaf(c2, s, c1));
+            if constexpr (BF16 && BITS == 2) {
+                // a 2-bit code has four values per column and group: dequantise them once (same arithmetic as
+                // dequant_pair: (128 + q) s + (z' - 128 s) in fp32, one round-to-nearest-even conversion) ...
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                const f32x2 w01 = {__builtin_fmaf(128.0f, meta[j].s, meta[j].z), __builtin_fmaf(129.0f, meta[j].s, meta[j].z)};
+                const f32x2 w23 = {__builtin_fmaf(130.0f, meta[j].s, meta[j].z), __builtin_fmaf(131.0f, meta[j].s, meta[j].z)};
+                meta[j].lut01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(w01, bf16x2_t));
+                meta[j].lut23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(w23, bf16x2_t));
+            }
         }
     };
 
@@ -452,9 +464,16 @@ __global__ __launch_bounds__(WAVES_M * (8 / TJ) * 64) __attribute__((amdgpu_wave
                         }
                     }
                 } else {
-                    if constexpr (BITS == 4) t = ((r.w[0][j] >> (q * 4)) & pair_mask) | magic;
-                    else t = ((r.w[0][j] >> ((4 * kb + q) * 2)) & pair_mask) | magic;
-                    o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
+                    if constexpr (BITS == 4) {
+                        t = ((r.w[0][j] >> (q * 4)) & pair_mask) | magic;
+                        o.bq[j][q] = dequant_pair<BF16>(t, meta[j]);
+                    } else {
+                        // ... and pick them per code pair with one byte permute: selector bytes (2q, 2q + 1) of each
+                        // code, made from the pair (q_lo, q_hi << 16) by one 24-bit multiply-add
+                        t = (r.w[0][j] >> ((4 * kb + q) * 2)) & pair_mask;
+                        const uint32_t sel = __umul24(t, 0x0202u) + 0x01000100u;
+                        o.bq[j][q] = __builtin_amdgcn_perm(meta[j].lut23, meta[j].lut01, sel);
+                    }
                 }
             }
         }
