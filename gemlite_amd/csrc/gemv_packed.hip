@@ -19,15 +19,17 @@
 //    C = sum_k x_k (OFF + q_k) and SX = sum_k x_k (one more MFMA against a B of ones) the
 //    group adds s*C + zz*SX, where (s, zz) folds scale, zero point and -OFF*s in fp32.  All
 //    five dequant modes are a choice of (s, zz), staged per slab in LDS.
-//  * The K reduction is deterministic: k-blocks inside the MFMA, waves through LDS, slabs by
-//    fp32 partials in a workspace that the last-arriving workgroup of a column tile sums in
-//    slab order (no float atomics).  A partial travels as a 64-bit slot (value, tag) written with
-//    one atomic store, so a reader sees either the whole slot or none of it: a workgroup publishes
-//    its slots, takes a ticket and reads the other slabs' slots in the same breath, and the one
-//    whose ticket says "last" already holds every partial that had landed (it polls the few that
-//    had not).  One memory round trip ends the kernel instead of three (store-and-wait, ticket,
-//    load); measured on the 4096^2 launch the tail after the last weight load is then about 1.6 us
-//    (ticket 0.25, one re-poll 0.6, LDS reduction and store 0.75) of 6 us.
+//  * The K reduction is deterministic: k-blocks inside the MFMA, waves through LDS, slabs through a
+//    pairwise tree in the workspace (no float atomics, no second launch).  Every output element has,
+//    per tree node, one 64-bit slot (value, tag); the two children of a node each swap their partial
+//    into it with one atomic exchange.  The one that finds the slot empty is done; the one that gets
+//    its sibling's partial back adds it (the tree is fixed and a sum of two is the same either way
+//    round, so the result never depends on who arrived first), clears the slot for the next launch
+//    and goes on to the parent.  Whoever leaves
+//    the root holds the total and stores the output.  Every thread decides for its own element: no
+//    ticket, no barrier, no polling.  Problems whose slots do not fit the private region of the
+//    workspace use fp32 partials and a ticket counter per column tile instead (the last-arriving
+//    workgroup sums the slabs in order).
 #include "common.hpp"
 #include "dispatch.hpp"
 
