@@ -261,6 +261,12 @@ Family choose(const gla_matmul_args& p, int type) {
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
     const bool small = !want_matrix && (type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16 || want_stream);
     if (small) {
+        // 8-bit codes on very large layers from 6 rows: the tiled GEMM's split-K stream is ahead of the 16-row GEMV
+        // pass (16384^2 at 8 / 16 rows: 65.2 / 64.6 against 70.6 / 72.8 us; 8192^2: 27.3 against 21.5-22.3, so only
+        // from 256 M weights up)
+        const bool big8 = p.W_nbits == 8 && p.M >= 6 && !want_stream && p.tile_config <= 0 && (int64_t)p.N * p.K >= ((int64_t)1 << 28) &&
+                          type > GLA_MATMUL_GEMV_SPLITK;
+        if (big8 && gemv_packed_eligible(p) && gemm_wn_eligible(p)) return F_GEMM_WN;
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
     }
