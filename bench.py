@@ -343,7 +343,13 @@ def extra_points(lib, device, T, quick):
         # ... and with the row quantised inside the GEMV (one launch; what forward() runs at decode sizes)
         us_in = T.graph_us([Launch(lib, l, x1b, y1, device, quantise_inside=True) for l in layers], 6)
         out[f"gemv_a8w8_{name}_M1"]["us_quantised_inside_the_matmul"] = round(us_in, 2)
-        del layer, layers, xq, sx, run, xq1, sx1, fns
+        # a decode batch of 8 rows: both operands as they are into the MFMA, one launch
+        xq8, sx8 = gemlite_amd.scale_activations_per_token(x[:8].contiguous(), wdt)
+        y8 = torch.empty((8, N), dtype=torch.bfloat16, device=device)
+        ls8 = [Launch(lib, l, xq8, y8, device, scales_x=sx8) for l in layers]
+        out[f"gemv_a8w8_{name}_M8"] = bw_point(T.graph_us(ls8, 6), wbytes + 8 * (K + 4) + 8 * N * 2, N=N, K=K, copies=len(layers),
+                                               family=_ext.matmul_family(ls8[0].args))
+        del layer, layers, xq, sx, run, xq1, sx1, fns, ls8, xq8, sx8
     # MXFP8 weights, fp8 activations quantised per token (the reference processor's default)
     lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
     lin.weight.data = W
@@ -390,8 +396,11 @@ def extra_points(lib, device, T, quick):
         xm = torch.randn((M, K), device=device).to(torch.bfloat16)
         xq, sx = gemlite_amd.scale_activations_mxfp4(xm)
         ym = torch.empty((M, N), dtype=torch.bfloat16, device=device)
-        us = T.graph_us([Launch(lib, l, xq, ym, device, scales_x=sx) for l in layers], 6)
-        out[f"gemv_a4w4_mxfp4_16384sq_M{M}"] = bw_point(us, wbytes + M * K // 2 + M * K // 32 + M * N * 2, copies=len(layers))
+        ls = [Launch(lib, l, xq, ym, device, scales_x=sx) for l in layers]
+        us = T.graph_us(ls, 6)
+        out[f"gemv_a4w4_mxfp4_16384sq_M{M}"] = bw_point(us, wbytes + M * K // 2 + M * K // 32 + M * N * 2, copies=len(layers),
+                                                        family=_ext.matmul_family(ls[0].args))
+        del ls
         fns = []
         for l in layers:   # end to end: MXFP4 quantiser of the bf16 rows + GEMV, both in the graph
             fns.append(lambda: _ext.scale_activations_mxfp4(xm, xq, sx))

@@ -53,7 +53,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
 
 constexpr int kMxStreamRows = 2;  // MXFP4 x MXFP4: rows up to which the streaming kernel is chosen
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY, F_K_SKINNY };
 
 int validate_operands(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -229,7 +229,7 @@ Family choose(const gla_matmul_args& p, int type) {
         const bool stream_ok = p.tile_config < 1000 && mx_stream_eligible(p), matrix_ok = gemm_mxfp4_eligible(p);
         if (want_stream && stream_ok) return F_MX_STREAM;
         if (want_matrix && matrix_ok) return F_GEMM_MXFP4;
-        if (p.M >= 3 && p.M <= 32 && p.tile_config < 1000 && mx_skinny_eligible(p)) return F_MX_SKINNY;
+        if (p.M >= 3 && p.M <= 32 && p.tile_config < 1000 && kring_eligible(p)) return F_K_SKINNY;
         // K not a multiple of 256 (or operands the skinny kernel does not take): the streaming kernel up to 2 rows
         // everywhere, up to 4 on layers of 40 MB or less (4096^2 at 4 rows: 10.7 against 14.4 us of the tiled GEMM;
         // 16384^2: 54 against 40)
@@ -259,6 +259,14 @@ Family choose(const gla_matmul_args& p, int type) {
     if (p.channel_scale_mode == GLA_CSM_BLOCK)  // validated as eligible for the streaming kernel at least
         return (gemm_blockq_eligible(p) && !want_stream) ? F_GEMM_BLOCKQ : F_BLOCKQ_STREAM;
     // Up to 16 rows the streaming kernels win whatever type was asked for; above that the MFMA GEMMs.
+    // fp8 x fp8 and int8 x int8 at 3..32 rows: operands as they are into the MFMA, one launch (between the vector
+    // streaming kernel and the tiled GEMM with its split K and finishing launch)
+    // (4096^2 fp8 at 8 / 32 rows: 7.1 / 9.3 against 13.8 / 14.8 us; 8192^2 at 8 rows 17.3 against 21.2; 16384^2 58.6 against
+    // 74.6; 3 rows on 4096^2: 7.0 against 13.3 of the streaming kernel.  With two activation tiles, 17..32 rows, the
+    // tiled GEMM is ahead from N = 7040: 8192^2 22.2 against 23.8, 14336 x 4096 20.4 against 24.0)
+    if (p.M >= 3 && p.M <= 32 && (p.M <= 16 || p.N < 7040) && !want_matrix && p.tile_config < 1000 &&
+        !(want_stream && gemv_kmajor_eligible(p)) && kring_eligible(p))
+        return F_K_SKINNY;
     const bool small = !want_matrix && (type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16 || want_stream);
     if (small) {
         // 8-bit codes on very large layers from 6 rows: the tiled GEMM's split-K stream is ahead of the 16-row GEMV
@@ -443,6 +451,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_GEMM_BLOCKQ: return launch_gemm_blockq(*args, s);
         case F_GEMM_KBYTES_MX: return args->bias != nullptr ? launch_gemm_kbytes_mx_bias(*args, s) : launch_gemm_kbytes_mx(*args, s);
         case F_MX_SKINNY: return launch_mx_skinny(*args, s);
+        case F_K_SKINNY: return launch_kring(*args, s);
         default: rc2 = launch_generic(*args, s); break;
     }
     if (rc2 == GLA_OK && args->bias != nullptr) rc2 = launch_bias_add(*args, s);

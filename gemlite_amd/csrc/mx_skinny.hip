@@ -19,8 +19,6 @@
 //    accumulators through LDS in wave order; no workspace, no second kernel, deterministic.
 //  * 16384^2 MXFP4: 45 us at 3 rows, 51 at 16 (a pure read in this access pattern: 30-34 us; the tiled GEMM:
 //    52-62 us); MXFP8: 73-79 us.
-// The second kernel of the file takes MXFP4 activations (codes + e8m0 bytes) on the same weights, 3..32 rows, and
-// feeds both sides to the block-scaled MFMA unconverted.
 #include "common.hpp"
 #include "dispatch.hpp"
 
@@ -251,201 +249,6 @@ __global__ __launch_bounds__(kWavesS * 64) void mx_skinny_kernel(MxSkArgs a) {
     }
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// MXFP4 x MXFP4 at 3..32 rows: the same walk over the weights, but nothing is converted.  A lane's 16 weight
-// bytes (32 e2m1 codes of one 32-block) ARE its share of the A operand of v_mfma_scale_f32_16x16x128_f8f6f4,
-// the block's e8m0 byte its scale; the B operand is the same 32-block of 16 activation rows, so one instruction
-// multiplies 16 weight rows with 16 activation rows over 128 K-values and applies both block scales (reference:
-// gemlite/triton_kernels/gemm_splitK_kernels.py:536-770, `tl.dot_scaled` on e2m1 operands).  XT = 1 or 2 tiles of
-// 16 activation rows.  Between the vector-unit streaming kernel (1-2 rows) and the tiled GEMM (64-row tiles
-// through LDS, split K, a finishing launch and a scale-regrouping launch in front).
-struct Mx4SkArgs {
-    const uint8_t* x;         // [M, K/2] e2m1 pairs
-    const uint8_t* sx;        // [ceil32(M), K/32] e8m0
-    const uint8_t* w;         // [N, K/2]
-    const uint8_t* scales;    // [N, K/32]
-    void* out;
-    int M, N, K;
-    int64_t xsm, sxm, wsn, osm, msn;   // bytes (osm: elements)
-    int out_dt;
-    const void* bias;
-    int bias_dt;
-};
-
-typedef int i32x8s __attribute__((ext_vector_type(8)));
-
-// s_waitcnt vmcnt(N) only: vmcnt is bits 3:0 and 15:14, expcnt (6:4) and lgkmcnt (11:8) left at "no wait"
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_sk() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-// Every operand is copied global -> LDS by the load unit (global_load_lds) into a ring that is private to the wave:
-// a copy instruction moves 8 rows x 128 contiguous bytes (the codes of a pair of steps), so rows are read in whole
-// 128-byte lines instead of the 16 x 64 bytes an MFMA operand load touches, nothing waits in registers, and there is
-// no barrier before the final sum of the waves' accumulators.  A tile (16 weight rows, or 16 activation rows) of a
-// pair is 2 KiB of codes, 16-byte slots XOR-swizzled by row >> 1 so that the operand reads (16 rows, one slot each)
-// fall in different banks, plus its 16 x 8 scale bytes.  The NW waves take the pairs of K in turn, NB pairs per wave
-// in flight.  K must be a multiple of 256.
-//  * 8 / 32 rows (us; tiled GEMM in brackets): 4096^2 4.7 / 6.5 (14.1 / 15.3), 8192^2 11.2 / 14.5 (17.8 / 19.9),
-//    4096 x 14336 9.8 / 14.3 (18.9 / 21.0), 14336 x 4096 10.8 / 14.7 (16.1 / 18.6), 16384^2 34.3 / 41.2 (41.0 / 44.4).
-//  * Two earlier forms of this kernel loaded the weights per lane in operand order (16 rows x 64 bytes per wave
-//    instruction), the activations through a shared LDS stage or per lane: 13.0-13.8 us on 8192^2 and 42.7-43.0 on
-//    16384^2 at 8 rows whatever else was varied (rows per wave, steps in flight, 8 or 16 waves, K order rotated per
-//    workgroup); the same code reading 1 KiB contiguous per instruction (timing only) took 9.5-11.1 and 28-35 us.
-//    The access pattern was the bound; copies by whole lines recover most of it without a second weight layout.
-template <int RT, int XT, int NW, int NB>
-__global__ __launch_bounds__(NW * 64) void mx4_ring_kernel(Mx4SkArgs a) {
-    constexpr int TILE = 2048 + 256;
-    constexpr int NT = RT + XT;
-    constexpr int OPS = 3 * NT;  // copy instructions per pair
-    static_assert((NB - 1) * OPS < 64, "outstanding copies must fit the vmcnt counter");
-    extern __shared__ __align__(16) unsigned char ring[];  // [NW][NB][NT][TILE]
-    __shared__ f32x4s red[NW][64];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r16 = lane & 15, kq = lane >> 4;
-    const int n0 = blockIdx.x * 16 * RT;
-    unsigned char* mine = ring + (size_t)wave * NB * NT * TILE;
-
-    // copy plan of a pair: per tile two code instructions (rows 8j + lane / 8, slot lane % 8 <- piece slot ^ (row >> 1))
-    // and one for the scale bytes (row (lane / 2) % 16, dword lane % 2; the upper half-wave writes a duplicate)
-    const uint8_t* csrc[NT][2];
-    const uint8_t* ssrc[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
-        const bool is_w = i < RT;
-        auto row_ptr = [&](int row, bool scale) -> const uint8_t* {
-            if (is_w) {
-                int n = n0 + 16 * i + row;
-                if (n > a.N - 1) n = a.N - 1;  // rows past the end repeat the last one; never stored
-                return scale ? a.scales + (int64_t)n * a.msn : a.w + (int64_t)n * a.wsn;
-            }
-            int m = 16 * (i - RT) + row;
-            if (m > a.M - 1) m = a.M - 1;
-            return scale ? a.sx + (int64_t)m * a.sxm : a.x + (int64_t)m * a.xsm;
-        };
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int row = 8 * j + (lane >> 3), slot = lane & 7;
-            csrc[i][j] = row_ptr(row, false) + ((slot ^ (row >> 1)) & 7) * 16;
-        }
-        ssrc[i] = row_ptr((lane >> 1) & 15, true) + (lane & 1) * 4;
-    }
-    auto issue = [&](int p, int slot) __attribute__((always_inline)) {
-        unsigned char* base = mine + slot * (NT * TILE);
-#pragma unroll
-        for (int i = 0; i < NT; ++i) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(csrc[i][j] + (int64_t)p * 128),
-                                                 (__attribute__((address_space(3))) void*)(base + i * TILE + j * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ssrc[i] + (int64_t)p * 8),
-                                             (__attribute__((address_space(3))) void*)(base + i * TILE + 2048), 4, 0, 0);
-        }
-    };
-    f32x4s acc[RT][XT];
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-        for (int xt = 0; xt < XT; ++xt) acc[t][xt] = f32x4s{0.0f, 0.0f, 0.0f, 0.0f};
-    const int code_off = r16 * 128, swz = r16 >> 1, scale_off = 2048 + r16 * 8;
-    auto multiply = [&](int slot) __attribute__((always_inline)) {
-        const unsigned char* base = mine + slot * (NT * TILE);
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int piece = (((4 * u + kq) ^ swz) & 7) * 16;
-#pragma unroll
-            for (int xt = 0; xt < XT; ++xt) {
-                const unsigned char* xb = base + (RT + xt) * TILE;
-                const u32x4s xv = *(const u32x4s*)(xb + code_off + piece);
-                const int ex = (int)((*(const uint32_t*)(xb + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
-                const i32x8s b8 = {(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3], 0, 0, 0, 0};
-#pragma unroll
-                for (int t = 0; t < RT; ++t) {
-                    const unsigned char* wb = base + t * TILE;
-                    const u32x4s wv = *(const u32x4s*)(wb + code_off + piece);
-                    const int ew = (int)((*(const uint32_t*)(wb + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
-                    const i32x8s a8 = {(int)wv[0], (int)wv[1], (int)wv[2], (int)wv[3], 0, 0, 0, 0};
-                    acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 4, 0, ew, 0, ex);
-                }
-            }
-        }
-    };
-    const int pairs = a.K / 256;
-    const int iters = (pairs + NW - 1) / NW;
-    // a wave whose turn lies past the end copies the last pair again (same count of copies for everybody) and skips the multiply
-    auto pair_of = [&](int it) { const int p = it * NW + wave; return p < pairs ? p : pairs - 1; };
-#pragma unroll
-    for (int b = 0; b < NB - 1; ++b)
-        if (b < iters) issue(pair_of(b), b);
-    int slot = 0, islot = NB - 1;
-    for (int it = 0; it < iters; ++it) {
-        const int later = iters - 1 - it;  // pairs issued after this one
-        if (later >= NB - 1) {
-            issue(pair_of(it + NB - 1), islot);
-            islot = islot == NB - 1 ? 0 : islot + 1;
-            wait_vmcnt_sk<(NB - 1) * OPS>();
-        } else {
-            // the ring drains: `later` pairs are still allowed in flight
-            bool done = false;
-#pragma unroll
-            for (int k = NB - 2; k >= 1; --k) {
-                if (!done && later == k) {
-                    if (k == 1) wait_vmcnt_sk<1 * OPS < 64 ? 1 * OPS : 0>();
-                    else if (k == 2) wait_vmcnt_sk<2 * OPS < 64 ? 2 * OPS : 0>();
-                    else if (k == 3) wait_vmcnt_sk<3 * OPS < 64 ? 3 * OPS : 0>();
-                    else wait_vmcnt_sk<0>();
-                    done = true;
-                }
-            }
-            if (!done) wait_vmcnt_sk<0>();
-        }
-        asm volatile("" ::: "memory");
-        if (it * NW + wave < pairs) multiply(slot);
-        slot = slot == NB - 1 ? 0 : slot + 1;
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);  // the copies of the next turn go to the slot these reads came from
-    }
-    // lane holds D[n0 + 16 t + 4 kq + e][m = 16 xt + r16]; the waves' sums are added in wave order, one tile at a time
-#pragma unroll
-    for (int t = 0; t < RT; ++t) {
-#pragma unroll
-        for (int xt = 0; xt < XT; ++xt) {
-            if (t || xt) __syncthreads();
-            red[wave][lane] = acc[t][xt];
-            __syncthreads();
-            const int m = 16 * xt + r16;
-            if (wave != 0 || m >= a.M) continue;
-            f32x4s D = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int w = 0; w < NW; ++w) D += red[w][lane];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int n = n0 + 16 * t + 4 * kq + e;
-                if (n >= a.N) continue;
-                float v = D[e];
-                if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + load_as_float(a.bias, a.bias_dt, n);
-                store_from_float(a.out, a.out_dt, (int64_t)m * a.osm + n, v);
-            }
-        }
-    }
-}
-
-template <int RT, int XT, int NW, int NB>
-int launch_ring4(const Mx4SkArgs& a, hipStream_t stream) {
-    const size_t smem = (size_t)NW * NB * (RT + XT) * (2048 + 256);
-    static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
-    auto kern = mx4_ring_kernel<RT, XT, NW, NB>;
-    if (once.first()) {
-        const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
-                                 "mx4_ring: raising the dynamic LDS limit");
-        if (rc != GLA_OK) return rc;
-    }
-    hipLaunchKernelGGL(kern, dim3(ceil_div(ceil_div(a.N, 16), RT)), dim3(NW * 64), smem, stream, a);
-    return check_hip(hipGetLastError(), "mx4_ring launch");
-}
-
 template <bool W4, bool BF16, int RT>
 int launch_variant(const MxSkArgs& a, hipStream_t stream) {
     constexpr int KC = (W4 ? 128 : 64) * 2 * kWavesS;
@@ -473,21 +276,7 @@ int launch_sk(const MxSkArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-// MXFP4 x MXFP4 (codes and e8m0 bytes on both sides), up to 32 rows
-static bool mx4_skinny_ok(const gla_matmul_args& p) {
-    if (p.input_dtype != GLA_DT_MXFP4 || p.x_quant_from != 0) return false;
-    if (p.M < 1 || p.M > 32 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_MX) return false;
-    if (p.scales == nullptr || p.scales_x == nullptr || p.sx_dtype != GLA_DT_UINT8) return false;
-    if (!(p.W_nbits == 4 && p.elements_per_sample == 2)) return false;
-    if (p.K % 256 != 0) return false;  // whole pairs of steps
-    if (p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3) || p.sx_stride_m % 4 != 0 || ((uintptr_t)p.scales_x & 3)) return false;
-    if (p.x_stride_k != 1 || p.w_stride_k != 1 || p.out_stride_n != 1 || p.meta_stride_g != 1 || p.sx_stride_g != 1) return false;
-    if (p.x_stride_m % 16 != 0 || p.w_stride_n % 16 != 0 || ((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
-    return p.output_dtype == GLA_DT_FP32 || p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16;
-}
-
 bool mx_skinny_eligible(const gla_matmul_args& p) {
-    if (p.input_dtype == GLA_DT_MXFP4) return mx4_skinny_ok(p);
     if (!(p.input_dtype == GLA_DT_MXFP16 || p.input_dtype == GLA_DT_MXBF16)) return false;
     if (p.M < 1 || p.M > 16 || p.group_size != 32 || p.channel_scale_mode != GLA_CSM_NONE || p.scales == nullptr) return false;
     const bool w4 = p.W_nbits == 4 && p.elements_per_sample == 2;
@@ -505,25 +294,6 @@ bool mx_skinny_eligible(const gla_matmul_args& p) {
 }
 
 int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream) {
-    if (p.input_dtype == GLA_DT_MXFP4 && mx4_skinny_ok(p)) {
-        Mx4SkArgs a;
-        a.x = (const uint8_t*)p.x; a.sx = (const uint8_t*)p.scales_x; a.w = (const uint8_t*)p.w; a.scales = (const uint8_t*)p.scales;
-        a.out = p.out; a.M = p.M; a.N = p.N; a.K = p.K;
-        a.xsm = p.x_stride_m; a.sxm = p.sx_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m; a.msn = p.meta_stride_n;
-        a.out_dt = p.output_dtype; a.bias = p.bias; a.bias_dt = p.bias_dtype;
-        // rows of tiles per wave so that about one workgroup per CU comes out; fewer, deeper waves where a wave has
-        // 4 weight tiles to an activation tile (16384^2 at 8 rows: 34.3 us with 4 tiles x 4 waves x 3 pairs in flight,
-        // 38.4 with 2 x 8 x 2, 35.2 with 1 x 8 x 4; 8192^2: 15.5 / 11.2 / 12.6; 4096^2: 8.9 / 6.1 / 4.7)
-        const int tiles = ceil_div(p.N, 16);
-        if (p.M <= 16) {
-            if (tiles >= 880) return launch_ring4<4, 1, 4, 3>(a, stream);
-            if (tiles >= 440) return launch_ring4<2, 1, 8, 2>(a, stream);
-            return launch_ring4<1, 1, 8, 4>(a, stream);
-        }
-        if (tiles >= 880) return launch_ring4<4, 2, 4, 2>(a, stream);
-        if (tiles >= 440) return launch_ring4<2, 2, 4, 4>(a, stream);
-        return launch_ring4<1, 2, 8, 2>(a, stream);
-    }
     if (!mx_skinny_eligible(p)) {
         set_error("mx_skinny: weight-only MX operands, K-contiguous with 16-byte aligned rows, up to 16 rows, "
                   "K a multiple of 256 (MXFP4) or 128 (MXFP8)");

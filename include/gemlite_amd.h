@@ -189,6 +189,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_BLOCKQ 10  /* the same above 2-3 rows: MFMA GEMM with a second, scaled accumulator */
 #define GLA_FAMILY_GEMM_KBYTES_MX 11 /* weight-only MX layers above 16 rows: MFMA GEMM, block scale applied on conversion */
 #define GLA_FAMILY_MX_SKINNY 12     /* weight-only MX layers at 3..16 rows: weights read once into registers, MFMA */
+#define GLA_FAMILY_K_SKINNY 13      /* MXFP4 x MXFP4, fp8 x fp8, int8 x int8 at 3..32 rows: operands as they are into the MFMA, one launch */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of

@@ -460,6 +460,57 @@ def test_a8w8_dynamic_streams_the_first_rows(device, fp8):
         check_layer(l2, gen_x(M, K2, torch.bfloat16, seed=30 + M).to(device), torch.bfloat16)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_a8w8_decode_batches_on_the_matrix_cores_in_one_launch(device, fp8):
+    """fp8 x fp8 and int8 x int8 at 3..32 rows (K a multiple of 128): both operands are copied to LDS by lines and go
+    into the MFMA as they are.  Ragged N, K with fewer turns than waves and with a last turn only some waves take,
+    one and two activation tiles, every launch shape (1, 2 and 4 weight tiles per wave), a bias; for int8 the fp32
+    output is float(exact int32 sum) * (s_w * s_x) and the int32 output the exact sum."""
+    import ctypes
+    from gemlite_amd import _ext
+    lib = _ext.load_library()
+    wdt = torch.float8_e4m3fn if fp8 else torch.int8
+    for (N, K) in ((1040, 4096), (520, 2304), (72, 128), (7056, 768), (14096, 512)):
+        W = gen_x(N, K, torch.bfloat16, seed=N + 1, std=0.02)
+        proc = helper.A8W8_FP8_dynamic(device=device) if fp8 else helper.A8W8_INT8_dynamic(device=device)
+        proc.dtype = torch.bfloat16
+        W_q_cpu, s_cpu = gemlite_amd.quantize_weights_per_channel(W, wdt)
+        layer = proc.from_weights(W_q_cpu, scales=s_cpu, bias=gen_x(1, N, torch.bfloat16, seed=2).reshape(-1) if N == 520 else None)
+        for M in (3, 5, 16, 17, 32, 33):
+            x = gen_x(M, K, torch.bfloat16, seed=80 + M).to(device)
+            xq, sx = gemlite_amd.scale_activations_per_token(x, wdt)
+            m = layer.get_meta_args()
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+            a = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, out, W_nbits=m[1], group_size=m[2],
+                                       unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                       acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                       data_contiguous=m[11])
+            ring = M <= 16 or (M <= 32 and N < 7040)   # two activation tiles: only where N is short
+            assert _ext.matmul_family(a) == ("K_SKINNY" if ring else "GEMM_8BIT"), (N, K, M, _ext.matmul_family(a))
+            check_layer(layer, x, torch.bfloat16)
+            if not fp8 and N != 520 and ring:
+                y32 = torch.empty(M, N, dtype=torch.float32, device=device)
+                a32 = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, y32, W_nbits=m[1], group_size=m[2],
+                                             unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=DType.FP32.value,
+                                             acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                             data_contiguous=m[11])
+                assert lib.gla_matmul(ctypes.byref(a32), torch.cuda.current_stream().cuda_stream) == 0
+                torch.cuda.synchronize()
+                acc = xq.cpu().to(torch.int64) @ layer.W_q.t().contiguous().cpu().to(torch.int64).t()
+                want = acc.to(torch.float32) * (layer.scales.cpu().reshape(1, N).float() * sx.cpu().reshape(M, 1).float())
+                assert torch.equal(y32.cpu(), want), (N, K, M)
+    if not fp8:
+        # INT8 x INT8 -> INT32, no scales: the exact sums
+        g = torch.Generator().manual_seed(3)
+        N, K = 1048, 1536
+        Wi = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+        li = GemLiteLinear(8, None, K, N, DType.INT8, DType.INT32).pack(Wi.to(device), None, None)
+        for M in (3, 16, 20, 32):
+            xi = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+            y = li.forward_manual(xi.to(device), matmul_type="GEMM_SPLITK")
+            assert y.dtype == torch.int32 and np.array_equal(y.cpu().numpy(), (xi.long() @ Wi.long().t()).numpy()), M
+
+
 def test_int8_activations_packed_weights(device):
     # int8 x 4-bit with an integer zero and channel-wise scales (reference: tests/test_int.py:146-171)
     N, K = 400, 1024
@@ -507,10 +558,11 @@ def _fused_family(layer, x):
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_a8w8_decode_rows_are_quantised_inside_the_matmul(device, fp8, dtype):
-    """Up to 4 rows (2 on large layers) the K-major streaming kernel takes the 16-bit rows and quantises them per
-    token itself (reference: the quantiser call in front of the matmul, gemlite/core.py:220-250): the output must
-    equal the quantiser launch followed by the matmul bit for bit, rows of very different magnitudes, an all-zero
-    row (scale 1e-6) and a ragged K included; above those rows the library declines and forward() runs two launches."""
+    """At the rows the K-major streaming kernel takes (up to 4 when K is not a multiple of 128, else 2: from 3 rows
+    the one-launch matrix-core kernel wants ready-made codes) it takes the 16-bit rows and quantises them per token
+    itself (reference: the quantiser call in front of the matmul, gemlite/core.py:220-250): the output must equal
+    the quantiser launch followed by the matmul bit for bit, rows of very different magnitudes, an all-zero row
+    (scale 1e-6) and a ragged K included; above those rows the library declines and forward() runs two launches."""
     for (N, K) in ((1030, 4160), (512, 8192)):
         W = gen_x(N, K, torch.bfloat16, seed=15, std=0.02)
         proc = helper.A8W8_FP8_dynamic(device=device) if fp8 else helper.A8W8_INT8_dynamic(device=device)
@@ -525,7 +577,7 @@ def test_a8w8_decode_rows_are_quantised_inside_the_matmul(device, fp8, dtype):
             if M > 2:
                 x[2] *= 1e-3
             x = x.to(device)
-            assert _fused_family(layer, x) == ("GEMV_KMAJOR" if M <= 4 else None), M
+            assert _fused_family(layer, x) == ("GEMV_KMAJOR" if M <= (4 if K % 128 else 2) else None), M
             y_fused, y_two = _forward_both_ways(layer, x)
             assert torch.equal(y_fused, y_two), (N, K, M)
             check_layer(layer, x, dtype)
@@ -588,7 +640,7 @@ def test_a4w4_mxfp4_skinny_rows_on_the_scaled_mfma(device, dtype):
             if M == 33:
                 assert _ext.matmul_family(a) == "GEMM_MXFP4"
             else:
-                assert _ext.matmul_family(a) == "MX_SKINNY", (N, K, M, _ext.matmul_family(a))
+                assert _ext.matmul_family(a) == "K_SKINNY", (N, K, M, _ext.matmul_family(a))
             check_layer(layer, x, dtype)
 
 

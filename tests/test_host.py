@@ -343,7 +343,8 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
     Wb = torch.randn(N, K, generator=g).bfloat16() * 0.02
     for proc, dt in ((gemlite_amd.helper.A8W8_FP8_dynamic, torch.float8_e4m3fn), (gemlite_amd.helper.A8W8_INT8_dynamic, torch.int8)):
         la = proc(device="cpu").from_weights(Wb)
-        for M, fam in ((1, "GEMV_KMAJOR"), (4, "GEMV_KMAJOR"), (5, "GEMM_8BIT"), (4096, "GEMM_8BIT")):  # streaming up to 4 rows
+        # streaming up to 2 rows, operands as they are into the MFMA in one launch up to 32 (K = 1024 is a multiple of 128), the tiled GEMM above
+        for M, fam in ((1, "GEMV_KMAJOR"), (2, "GEMV_KMAJOR"), (3, "K_SKINNY"), (32, "K_SKINNY"), (33, "GEMM_8BIT"), (4096, "GEMM_8BIT")):
             xq = torch.zeros(M, K, dtype=dt)
             assert _family(la, M, None, scales_x=torch.ones(M, 1), x=xq) == fam
     # MXFP4
@@ -353,7 +354,7 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
     for M in (1, 32, 1024):
         xq = torch.zeros(M, K // 2, dtype=torch.uint8)
         sx = torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
-        assert _family(lm, M, None, scales_x=sx, x=xq) == {1: "MX_STREAM", 32: "MX_SKINNY", 1024: "GEMM_MXFP4"}[M]
+        assert _family(lm, M, None, scales_x=sx, x=xq) == {1: "MX_STREAM", 32: "K_SKINNY", 1024: "GEMM_MXFP4"}[M]
 
 
 def test_tile_config_can_state_a_preference_between_streaming_and_matrix_kernels():
