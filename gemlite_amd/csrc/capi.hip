@@ -244,6 +244,9 @@ Family choose(const gla_matmul_args& p, int type) {
         const bool stream_ok = p.tile_config < 1000 && mx_stream_eligible(p), matrix_ok = gemm_mxfp8_eligible(p);
         if (want_stream && stream_ok) return F_MX_STREAM;
         if (want_matrix && matrix_ok) return F_GEMM_MXFP8;
+        // from 3 rows both operands go into the scaled MFMA as they are, copied to LDS by lines, in one launch
+        // (two activation tiles, 17..32 rows: only where N is short, as for fp8 x fp8)
+        if (p.M >= 3 && p.M <= 32 && (p.M <= 16 || p.N < 7040) && p.tile_config < 1000 && kring_eligible(p)) return F_K_SKINNY;
         if (p.M <= 4 && stream_ok) return F_MX_STREAM;
         return matrix_ok ? F_GEMM_MXFP8 : F_MX_STREAM;
     }

@@ -4,6 +4,10 @@
 //                   (v_mfma_scale_f32_16x16x128_f8f6f4, both block scales applied by the instruction)
 //   fp8 x fp8       e4m3 bytes, per-token x per-channel scales in the epilogue (the same instruction, unit scales)
 //   int8 x int8     exact int32 sums (v_mfma_i32_16x16x64_i8), scaled in the epilogue or stored as int32
+//   fp8 x MXFP8      e4m3 bytes on both sides, e8m0 block scales on the weights and, by channel_scale_mode, either the
+//                   same on the activations or one fp32 scale per token in the epilogue
+//   fp8 x MXFP4      the mixed form of the instruction (A e2m1, B e4m3): 256 K-values a turn, the activations of a
+//                   turn travelling as two tiles (4096^2 at 8 rows 5.2 us against 16.2 tiled, 16384^2 35.0 against 54.9)
 //
 // The decode-batch path of dynamically quantised A8W8 and A4W4 layers, between the streaming kernels (dot products
 // on the vector unit, 1-2 rows) and the tiled GEMMs (64-row tiles, K split over workgroups, a finishing launch and,
@@ -41,17 +45,17 @@ typedef float f32x4r __attribute__((ext_vector_type(4)));
 typedef int i32x4r __attribute__((ext_vector_type(4)));
 typedef int i32x8r __attribute__((ext_vector_type(8)));
 
-enum { R_MX44 = 0, R_FP8 = 1, R_INT8 = 2 };
+enum { R_MX44 = 0, R_FP8 = 1, R_INT8 = 2, R_MX88 = 3, R_MX84 = 4 };
 
 struct KRingArgs {
-    const uint8_t* x;         // [M, K bytes or K/2 nibble pairs]
-    const uint8_t* w;         // [N, the same]
-    const uint8_t* bsx;       // MXFP4: activation block scales [ceil32(M), K/32] e8m0
-    const uint8_t* bsw;       // MXFP4: weight block scales [N, K/32]
-    const void* scales;       // 8-bit: per-channel scales [N] (channel_scale_mode bit 0)
-    const void* scales_x;     // 8-bit: per-token scales [M] (bit 1)
+    const uint8_t* x;         // [M, bytes of K]
+    const uint8_t* w;         // [N, bytes of K]
+    const uint8_t* bsx;       // block-scaled activations: [ceil32(M), K/32] e8m0
+    const uint8_t* bsw;       // block-scaled weights: [N, K/32] e8m0
+    const void* scales;       // fp8 / int8: per-channel scales [N] (channel_scale_mode bit 0)
+    const void* scales_x;     // per-token scales [M] (bit 1)
     void* out;
-    int M, N, Kb;             // Kb = operand bytes per row
+    int M, N, turns;          // turns = K / (K-values per turn)
     int64_t xsm, wsn, bsxm, bswn, sxm, osm;   // bytes (sxm, osm: elements)
     int csm, meta_dt, sx_dt, out_dt;
     const void* bias;
@@ -65,14 +69,28 @@ __device__ __forceinline__ void wait_vmcnt_r() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <int MODE, int RT, int XT, int NW, int NB>
+// What a turn of K is in each mode.  A tile is always 16 rows x 128 bytes; the fp8 activations under MXFP4 weights
+// are 256 bytes per row and turn and travel as two tiles.
+template <int MODE>
+struct RingShape {
+    static constexpr bool WBS = MODE == R_MX44 || MODE == R_MX88 || MODE == R_MX84;  // weights carry block scales
+    static constexpr int XH = MODE == R_MX84 ? 2 : 1;                                // activation tiles per 16 rows and turn
+    static constexpr int KT = (MODE == R_MX44 || MODE == R_MX84) ? 256 : 128;        // K-values per turn
+    static constexpr int SB = KT / 32;                                               // scale bytes per row and turn
+};
+
+// XBS: the activations carry block scales too (always with MXFP4 activations; MXFP8 activations by channel_scale_mode)
+template <int MODE, bool XBS, int RT, int XT, int NW, int NB>
 __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
-    constexpr bool BS = MODE == R_MX44;                 // block scales travel with the tiles
-    constexpr int TILE = 2048 + (BS ? 256 : 0);
-    constexpr int NT = RT + XT;
-    constexpr int OPS = (2 + (BS ? 1 : 0)) * NT;        // copy instructions per turn
+    using SH = RingShape<MODE>;
+    constexpr bool WBS = SH::WBS;
+    constexpr int XH = SH::XH, SB = SH::SB;
+    constexpr int TILE = 2048 + (WBS ? 256 : 0);
+    constexpr int NT = RT + XT * XH;
+    constexpr int OPS = RT * (2 + (WBS ? 1 : 0)) + XT * XH * 2 + (XBS ? XT : 0);  // copy instructions per turn
     typedef typename std::conditional<MODE == R_INT8, i32x4r, f32x4r>::type acc_t;
     static_assert((NB - 1) * OPS < 64, "outstanding copies must fit the vmcnt counter");
+    static_assert(!XBS || WBS, "block-scaled activations come with block-scaled weights");
     extern __shared__ __align__(16) unsigned char ring[];  // [NW][NB][NT][TILE]
     __shared__ acc_t red[NW][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -81,41 +99,50 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
     unsigned char* mine = ring + (size_t)wave * NB * NT * TILE;
 
     // copy plan of a turn: per tile two code instructions (rows 8j + lane / 8, slot lane % 8 <- piece slot ^ (row >> 1))
-    // and, with block scales, one for the scale bytes (row (lane / 2) % 16, dword lane % 2; the upper half-wave
-    // writes a duplicate)
+    // and, with block scales, one for the tile's scale bytes: 8 per row (row (lane / 2) % 16, dword lane % 2) or 4
+    // (row lane % 16); the rest of the wave writes duplicates behind them
     const uint8_t* csrc[NT][2];
-    const uint8_t* ssrc[BS ? NT : 1];
+    const uint8_t* ssrc[WBS ? NT : 1];
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
         const bool is_w = i < RT;
+        const int xt = is_w ? 0 : (i - RT) / XH, half = is_w ? 0 : (i - RT) % XH;
         auto row_ptr = [&](int row, bool scale) -> const uint8_t* {
             if (is_w) {
                 int n = n0 + 16 * i + row;
                 if (n > a.N - 1) n = a.N - 1;  // rows past the end repeat the last one; never stored
                 return scale ? a.bsw + (int64_t)n * a.bswn : a.w + (int64_t)n * a.wsn;
             }
-            int m = 16 * (i - RT) + row;
+            int m = 16 * xt + row;
             if (m > a.M - 1) m = a.M - 1;
-            return scale ? a.bsx + (int64_t)m * a.bsxm : a.x + (int64_t)m * a.xsm;
+            return scale ? a.bsx + (int64_t)m * a.bsxm : a.x + (int64_t)m * a.xsm + half * 128;
         };
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int row = 8 * j + (lane >> 3), slot = lane & 7;
             csrc[i][j] = row_ptr(row, false) + ((slot ^ (row >> 1)) & 7) * 16;
         }
-        if constexpr (BS) ssrc[i] = row_ptr((lane >> 1) & 15, true) + (lane & 1) * 4;
+        if constexpr (WBS) {
+            if (is_w || (XBS && half == 0))
+                ssrc[i] = SB == 8 ? row_ptr((lane >> 1) & 15, true) + (lane & 1) * 4 : row_ptr(lane & 15, true);
+            else
+                ssrc[i] = nullptr;
+        }
     }
     auto issue = [&](int p, int slot) __attribute__((always_inline)) {
         unsigned char* base = mine + slot * (NT * TILE);
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
+            const int adv = i < RT ? 128 : 128 * XH;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(csrc[i][j] + (int64_t)p * 128),
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(csrc[i][j] + (int64_t)p * adv),
                                                  (__attribute__((address_space(3))) void*)(base + i * TILE + j * 1024), 16, 0, 0);
-            if constexpr (BS)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ssrc[i] + (int64_t)p * 8),
-                                                 (__attribute__((address_space(3))) void*)(base + i * TILE + 2048), 4, 0, 0);
+            if constexpr (WBS) {
+                if (i < RT || (XBS && (i - RT) % XH == 0))
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ssrc[i] + (int64_t)p * SB),
+                                                     (__attribute__((address_space(3))) void*)(base + i * TILE + 2048), 4, 0, 0);
+            }
         }
     };
     acc_t acc[RT][XT];
@@ -123,37 +150,56 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
     for (int t = 0; t < RT; ++t)
 #pragma unroll
         for (int xt = 0; xt < XT; ++xt) acc[t][xt] = acc_t{0, 0, 0, 0};
-    const int code_off = r16 * 128, swz = r16 >> 1, scale_off = 2048 + r16 * 8;
+    const int code_off = r16 * 128, swz = r16 >> 1, scale_off = 2048 + r16 * SB;
     auto slot16 = [&](const unsigned char* tile, int piece) __attribute__((always_inline)) {
         return *(const u32x4r*)(tile + code_off + ((piece ^ swz) & 7) * 16);
     };
+    // the lane's 32 bytes of a row as an 8-register fp8 operand.  Registers 0-3 of the four lane groups together are
+    // K-values 0..63 of the instruction, registers 4-7 K-values 64..127 (slots kq and 4 + kq), while the scale byte a
+    // lane group hands in applies to 32-block kq.
+    auto slot32 = [&](const unsigned char* tile) __attribute__((always_inline)) {
+        const u32x4r lo = slot16(tile, kq), hi = slot16(tile, 4 + kq);
+        return i32x8r{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    };
+    // e8m0 byte of the lane's 32-block: byte kq of dword u of the row's scale bytes
+    auto scale_byte = [&](const unsigned char* tile, int u) __attribute__((always_inline)) {
+        return (int)((*(const uint32_t*)(tile + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
+    };
     auto multiply = [&](int slot) __attribute__((always_inline)) {
         const unsigned char* base = mine + slot * (NT * TILE);
-        if constexpr (MODE == R_FP8) {
-            // a turn is one MFMA: the lane's 32 bytes are slots 2 kq and 2 kq + 1 of its row
+        if constexpr (MODE == R_FP8 || MODE == R_MX88) {
+            // a turn is one MFMA of 128 bytes of K
 #pragma unroll
             for (int xt = 0; xt < XT; ++xt) {
                 const unsigned char* xb = base + (RT + xt) * TILE;
-                const u32x4r x0 = slot16(xb, 2 * kq), x1 = slot16(xb, 2 * kq + 1);
-                const i32x8r b8 = {(int)x0[0], (int)x0[1], (int)x0[2], (int)x0[3], (int)x1[0], (int)x1[1], (int)x1[2], (int)x1[3]};
+                const i32x8r b8 = slot32(xb);
+                int ex = 127;
+                if constexpr (XBS) ex = scale_byte(xb, 0);
 #pragma unroll
                 for (int t = 0; t < RT; ++t) {
                     const unsigned char* wb = base + t * TILE;
-                    const u32x4r w0 = slot16(wb, 2 * kq), w1 = slot16(wb, 2 * kq + 1);
-                    const i32x8r a8 = {(int)w0[0], (int)w0[1], (int)w0[2], (int)w0[3], (int)w1[0], (int)w1[1], (int)w1[2], (int)w1[3]};
-                    acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 0, 0, 0, 127, 0, 127);
+                    int ew = 127;
+                    if constexpr (WBS) ew = scale_byte(wb, 0);
+                    acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(slot32(wb), b8, acc[t][xt], 0, 0, 0, ew, 0, ex);
                 }
             }
         } else {
-            // two MFMAs a turn (MXFP4: 128 K-values each; int8: 64): the lane's 16 bytes are slot 4 u + kq
+            // two MFMAs a turn (MXFP4 weights: 128 K-values each; int8: 64): the lane's 16 bytes are slot 4 u + kq
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
                 for (int xt = 0; xt < XT; ++xt) {
-                    const unsigned char* xb = base + (RT + xt) * TILE;
-                    const u32x4r xv = slot16(xb, 4 * u + kq);
-                    int ex = 0;
-                    if constexpr (BS) ex = (int)((*(const uint32_t*)(xb + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
+                    const unsigned char* xb = base + (RT + xt * XH) * TILE;  // (first) tile of these 16 rows: holds their scales
+                    int ex = 127;
+                    if constexpr (XBS) ex = scale_byte(xb, u);
+                    u32x4r xv;
+                    i32x8r b8;
+                    if constexpr (MODE == R_MX84) {
+                        b8 = slot32(xb + u * TILE);  // fp8 activations: half u of the turn is a tile of its own
+                    } else {
+                        xv = slot16(xb, 4 * u + kq);
+                        b8 = i32x8r{(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3], 0, 0, 0, 0};
+                    }
 #pragma unroll
                     for (int t = 0; t < RT; ++t) {
                         const unsigned char* wb = base + t * TILE;
@@ -163,17 +209,20 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
                                                                                i32x4r{(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3]},
                                                                                acc[t][xt], 0, 0, 0);
                         } else {
-                            const int ew = (int)((*(const uint32_t*)(wb + scale_off + 4 * u) >> (8 * kq)) & 0xffu);
+                            const int ew = scale_byte(wb, u);
                             const i32x8r a8 = {(int)wv[0], (int)wv[1], (int)wv[2], (int)wv[3], 0, 0, 0, 0};
-                            const i32x8r b8 = {(int)xv[0], (int)xv[1], (int)xv[2], (int)xv[3], 0, 0, 0, 0};
-                            acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 4, 0, ew, 0, ex);
+                            // operand formats: 4 = e2m1, 0 = e4m3
+                            if constexpr (MODE == R_MX84)
+                                acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 0, 0, ew, 0, ex);
+                            else
+                                acc[t][xt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[t][xt], 4, 4, 0, ew, 0, ex);
                         }
                     }
                 }
             }
         }
     };
-    const int turns = a.Kb / 128;
+    const int turns = a.turns;
     const int iters = (turns + NW - 1) / NW;
     // a wave whose turn lies past the end copies the last one again (same count of copies for everybody) and skips the multiply
     auto turn_of = [&](int it) { const int p = it * NW + wave; return p < turns ? p : turns - 1; };
@@ -203,7 +252,7 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
         __builtin_amdgcn_sched_barrier(0);  // the copies of the next turn go to the slot these reads came from
     }
     // lane holds D[n0 + 16 t + 4 kq + e][m = 16 xt + r16]; the waves' sums are added in wave order, one tile at a time
-    const bool col_scale = !BS && (a.csm & 1), row_scale = !BS && (a.csm & 2);
+    const bool col_scale = a.csm <= GLA_CSM_BOTH && (a.csm & 1), row_scale = a.csm <= GLA_CSM_BOTH && (a.csm & 2);
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
 #pragma unroll
@@ -229,7 +278,7 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
                     }
                 }
                 float v = (float)D[e];
-                if constexpr (!BS) v *= sa * (col_scale ? load_as_float(a.scales, a.meta_dt, n) : 1.0f);
+                if (row_scale || col_scale) v *= sa * (col_scale ? load_as_float(a.scales, a.meta_dt, n) : 1.0f);
                 if (a.bias != nullptr) v = round_to_dtype(a.out_dt, v) + load_as_float(a.bias, a.bias_dt, n);
                 store_from_float(a.out, a.out_dt, o, v);
             }
@@ -237,11 +286,12 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
     }
 }
 
-template <int MODE, int RT, int XT, int NW, int NB>
+template <int MODE, bool XBS, int RT, int XT, int NW, int NB>
 int launch_ring(const KRingArgs& a, hipStream_t stream) {
-    const size_t smem = (size_t)NW * NB * (RT + XT) * (2048 + (MODE == R_MX44 ? 256 : 0));
+    using SH = RingShape<MODE>;
+    const size_t smem = (size_t)NW * NB * (RT + XT * SH::XH) * (2048 + (SH::WBS ? 256 : 0));
     static DeviceOnce once;  // per instantiation; the attribute is sticky per function and device
-    auto kern = kring_kernel<MODE, RT, XT, NW, NB>;
+    auto kern = kring_kernel<MODE, XBS, RT, XT, NW, NB>;
     if (once.first()) {
         const int rc = check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
                                  "kring: raising the dynamic LDS limit");
@@ -251,7 +301,7 @@ int launch_ring(const KRingArgs& a, hipStream_t stream) {
     return check_hip(hipGetLastError(), "kring launch");
 }
 
-template <int MODE>
+template <int MODE, bool XBS>
 int launch_mode_ring(const KRingArgs& a, hipStream_t stream) {
     // rows of tiles per wave so that about one workgroup per CU comes out; fewer, deeper waves where a wave has
     // 4 weight tiles to an activation tile (MXFP4, 16384^2 at 8 rows: 34.3 us with 4 tiles x 4 waves x 3 turns in
@@ -259,25 +309,35 @@ int launch_mode_ring(const KRingArgs& a, hipStream_t stream) {
     const int tiles = ceil_div(a.N, 16);
     if constexpr (MODE == R_MX44) {
         if (a.M <= 16) {
-            if (tiles >= 880) return launch_ring<MODE, 4, 1, 4, 3>(a, stream);
-            if (tiles >= 440) return launch_ring<MODE, 2, 1, 8, 2>(a, stream);
-            return launch_ring<MODE, 1, 1, 8, 4>(a, stream);
+            if (tiles >= 880) return launch_ring<MODE, XBS, 4, 1, 4, 3>(a, stream);
+            if (tiles >= 440) return launch_ring<MODE, XBS, 2, 1, 8, 2>(a, stream);
+            return launch_ring<MODE, XBS, 1, 1, 8, 4>(a, stream);
         }
-        if (tiles >= 880) return launch_ring<MODE, 4, 2, 4, 2>(a, stream);
-        if (tiles >= 440) return launch_ring<MODE, 2, 2, 4, 4>(a, stream);
-        return launch_ring<MODE, 1, 2, 8, 2>(a, stream);
+        if (tiles >= 880) return launch_ring<MODE, XBS, 4, 2, 4, 2>(a, stream);
+        if (tiles >= 440) return launch_ring<MODE, XBS, 2, 2, 4, 4>(a, stream);
+        return launch_ring<MODE, XBS, 1, 2, 8, 2>(a, stream);
+    } else if constexpr (MODE == R_MX84) {
+        // 16 activation rows are two tiles a turn here, 32 rows four: shallower rings
+        if (a.M <= 16) {
+            if (tiles >= 880) return launch_ring<MODE, XBS, 4, 1, 4, 2>(a, stream);
+            if (tiles >= 440) return launch_ring<MODE, XBS, 2, 1, 8, 2>(a, stream);
+            return launch_ring<MODE, XBS, 1, 1, 8, 2>(a, stream);
+        }
+        if (tiles >= 440) return launch_ring<MODE, XBS, 2, 2, 4, 2>(a, stream);
+        return launch_ring<MODE, XBS, 1, 2, 4, 3>(a, stream);
     } else {
         // 8-bit operands: an activation tile is as many bytes as a weight tile, and one tile per wave with many waves
         // does best (fp8 at 8 rows, 8192^2: 17.3 us with 1 tile x 16 waves x 2 turns, 17.6 with 1 x 8 x 4, 21.1 with
         // 2 x 8 x 2; 16384^2: 58.6 / 60.0 / 66.1) unless K is short and N long (14336 x 4096: 21.1 / 21.8 against 18.8
         // with 4 x 4 x 3)
+        constexpr int D1 = RingShape<MODE>::WBS ? 3 : 4;  // ring depth that fits with one tile each and 8 waves
         if (a.M <= 16) {
-            if (tiles >= 880 && a.Kb < 8192) return launch_ring<MODE, 4, 1, 4, 3>(a, stream);
-            if (tiles >= 440) return launch_ring<MODE, 1, 1, 16, 2>(a, stream);
-            return launch_ring<MODE, 1, 1, 8, 4>(a, stream);
+            if (tiles >= 880 && a.turns < 64) return launch_ring<MODE, XBS, 4, 1, 4, 3>(a, stream);
+            if (tiles >= 440) return launch_ring<MODE, XBS, 1, 1, 16, 2>(a, stream);
+            return launch_ring<MODE, XBS, 1, 1, 8, D1>(a, stream);
         }
-        if (tiles >= 440) return launch_ring<MODE, 2, 2, 8, 2>(a, stream);
-        return launch_ring<MODE, 1, 2, 8, 2>(a, stream);
+        if (tiles >= 440) return launch_ring<MODE, XBS, 2, 2, 8, 2>(a, stream);
+        return launch_ring<MODE, XBS, 1, 2, 8, 2>(a, stream);
     }
 }
 
@@ -285,6 +345,7 @@ int ring_mode(const gla_matmul_args& p) {
     if (p.input_dtype == GLA_DT_MXFP4) return R_MX44;
     if (p.input_dtype == GLA_DT_FP8 && p.w_dtype == GLA_DT_FP8) return R_FP8;
     if (p.input_dtype == GLA_DT_INT8 && p.w_dtype == GLA_DT_INT8) return R_INT8;
+    if (p.input_dtype == GLA_DT_MXFP8) return (p.W_nbits == 4 && p.elements_per_sample == 2) ? R_MX84 : R_MX88;
     return -1;
 }
 
@@ -295,13 +356,20 @@ bool kring_eligible(const gla_matmul_args& p) {
     if (mode < 0 || p.x_quant_from != 0 || p.M < 1 || p.M > 32) return false;
     if (p.x_stride_k != 1 || p.w_stride_k != 1 || p.out_stride_n != 1) return false;
     if (p.x_stride_m % 16 != 0 || p.w_stride_n % 16 != 0 || ((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
-    if (mode == R_MX44) {
-        if (p.group_size != 32 || p.channel_scale_mode != GLA_CSM_MX || !(p.W_nbits == 4 && p.elements_per_sample == 2)) return false;
-        if (p.scales == nullptr || p.scales_x == nullptr || p.sx_dtype != GLA_DT_UINT8) return false;
-        if (p.K % 256 != 0) return false;  // whole turns of 128 bytes
-        if (p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3) || p.sx_stride_m % 4 != 0 || ((uintptr_t)p.scales_x & 3)) return false;
-        if (p.meta_stride_g != 1 || p.sx_stride_g != 1) return false;
-        return p.output_dtype == GLA_DT_FP32 || p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16;
+    const bool float_out = p.output_dtype == GLA_DT_FP32 || p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16;
+    if (mode == R_MX44 || mode == R_MX88 || mode == R_MX84) {
+        if (p.group_size != 32 || p.scales == nullptr || p.scales_x == nullptr || !float_out) return false;
+        if (p.meta_stride_g != 1 || p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3)) return false;
+        const bool xbs = p.channel_scale_mode == GLA_CSM_MX;
+        if (xbs && (p.sx_dtype != GLA_DT_UINT8 || p.sx_stride_g != 1 || p.sx_stride_m % 4 != 0 || ((uintptr_t)p.scales_x & 3))) return false;
+        if (mode == R_MX44) {
+            if (!xbs || !(p.W_nbits == 4 && p.elements_per_sample == 2)) return false;
+            return p.K % 256 == 0;  // whole turns of 128 bytes
+        }
+        // fp8 activations with block scales or one scale per token
+        if (!xbs && p.channel_scale_mode != GLA_CSM_ACTIVATION) return false;
+        if (mode == R_MX88) return p.W_nbits == 8 && p.elements_per_sample == 1 && p.w_dtype == GLA_DT_FP8 && p.K % 128 == 0;
+        return p.K % 256 == 0;
     }
     // fp8 x fp8 and int8 x int8: what the tiled 8-bit GEMM takes, K in whole turns
     if (mode == R_FP8 && p.acc_dtype != GLA_DT_FP32) return false;
@@ -310,7 +378,7 @@ bool kring_eligible(const gla_matmul_args& p) {
     if (p.channel_scale_mode < GLA_CSM_NONE || p.channel_scale_mode > GLA_CSM_BOTH) return false;
     if (p.K % 128 != 0) return false;
     if (p.output_dtype == GLA_DT_INT32) return mode == R_INT8 && p.channel_scale_mode == GLA_CSM_NONE;
-    if (!(p.output_dtype == GLA_DT_FP32 || p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16)) return false;
+    if (!float_out) return false;
     if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
     if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
     return true;
@@ -318,23 +386,30 @@ bool kring_eligible(const gla_matmul_args& p) {
 
 int launch_kring(const gla_matmul_args& p, hipStream_t stream) {
     if (!kring_eligible(p)) {
-        set_error("kring: MXFP4 x MXFP4, fp8 x fp8 or int8 x int8 operands, K-contiguous with 16-byte aligned rows, up to 32 "
-                  "rows, K a multiple of 256 (MXFP4) or 128");
+        set_error("kring: MXFP4 x MXFP4, fp8 x fp8, int8 x int8 or fp8 x MXFP8 / MXFP4 operands, K-contiguous with 16-byte "
+                  "aligned rows, up to 32 rows, K a multiple of 256 (MXFP4 weights) or 128");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     const int mode = ring_mode(p);
+    const bool mx = mode == R_MX44 || mode == R_MX88 || mode == R_MX84;
+    const bool xbs = mx && p.channel_scale_mode == GLA_CSM_MX;
     KRingArgs a;
     a.x = (const uint8_t*)p.x; a.w = (const uint8_t*)p.w; a.out = p.out;
-    a.M = p.M; a.N = p.N; a.Kb = mode == R_MX44 ? p.K / 2 : p.K;
+    a.M = p.M; a.N = p.N;
+    a.turns = p.K / ((mode == R_MX44 || mode == R_MX84) ? 256 : 128);
     a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m;
-    a.bsx = mode == R_MX44 ? (const uint8_t*)p.scales_x : nullptr; a.bsw = mode == R_MX44 ? (const uint8_t*)p.scales : nullptr;
+    a.bsx = xbs ? (const uint8_t*)p.scales_x : nullptr; a.bsw = mx ? (const uint8_t*)p.scales : nullptr;
     a.bsxm = p.sx_stride_m; a.bswn = p.meta_stride_n;
     a.scales = p.scales; a.scales_x = p.scales_x; a.sxm = p.sx_stride_m;
     a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype; a.out_dt = p.output_dtype;
     a.bias = p.bias; a.bias_dt = p.bias_dtype;
-    if (mode == R_MX44) return launch_mode_ring<R_MX44>(a, stream);
-    if (mode == R_FP8) return launch_mode_ring<R_FP8>(a, stream);
-    return launch_mode_ring<R_INT8>(a, stream);
+    switch (mode) {
+        case R_MX44: return launch_mode_ring<R_MX44, true>(a, stream);
+        case R_FP8: return launch_mode_ring<R_FP8, false>(a, stream);
+        case R_INT8: return launch_mode_ring<R_INT8, false>(a, stream);
+        case R_MX88: return xbs ? launch_mode_ring<R_MX88, true>(a, stream) : launch_mode_ring<R_MX88, false>(a, stream);
+        default: return xbs ? launch_mode_ring<R_MX84, true>(a, stream) : launch_mode_ring<R_MX84, false>(a, stream);
+    }
 }
 
 }  // namespace gla

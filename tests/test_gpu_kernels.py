@@ -993,6 +993,47 @@ def test_a8w4_mxfp8_activations_mxfp4_weights(device, post_scale, K):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("post_scale", [True, False])
+@pytest.mark.parametrize("w4", [False, True])
+def test_fp8_activations_on_mx_weights_decode_batches_in_one_launch(device, post_scale, w4):
+    """fp8 activations (one scale per token, or MXFP8 micro-scales) x MXFP8 / MXFP4 weights at 3..32 rows: both
+    operands copied to LDS by lines and fed to the scaled MFMA as they are (the mixed fp8 x fp4 form for MXFP4
+    weights, whose activation rows are two tiles a turn).  Ragged N, few and many turns of K, block scales that
+    differ from block to block, every launch shape, a bias."""
+    from gemlite_amd import _ext
+    proc = helper.A8W4_MXFP_dynamic if w4 else helper.A8W8_MXFP_dynamic
+    for (N, K) in ((1040, 4096), (520, 2304), (72, 256), (7056, 768), (14096, 512)):
+        W = gen_x(N, K, torch.bfloat16, seed=N + 2, std=0.03)
+        W[:, 32:64] *= 8.0
+        W[:, 96:128] *= 0.125
+        if w4:
+            codes, e8 = orc.quantize_mxfp4_weights(to_np(W))
+            wq = torch.from_numpy(codes)
+        else:
+            codes, e8 = orc.quantize_mxfp8_weights(to_np(W))
+            wq = torch.from_numpy(codes).view(torch.float8_e4m3fn)
+        layer = proc(device=device, dtype=torch.bfloat16, post_scale=post_scale).from_weights(
+            wq, scales=torch.from_numpy(e8), bias=gen_x(1, N, torch.bfloat16, seed=3).reshape(-1) if N == 520 else None)
+        for M in (3, 5, 16, 17, 32, 33):
+            x = gen_x(M, K, torch.bfloat16, seed=90 + M)
+            x[:, 64:96] *= 16.0
+            x = x.to(device)
+            if post_scale:
+                xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn)
+            else:
+                xq, sx = gemlite_amd.scale_activations_mxfp8(x)
+            m = layer.get_meta_args()
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+            a = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, out, W_nbits=m[1], group_size=m[2],
+                                       unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                       acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                       data_contiguous=m[11])
+            ring = M <= 16 or (M <= 32 and N < 7040)
+            assert _ext.matmul_family(a) == ("K_SKINNY" if ring else "GEMM_MXFP8"), (N, K, M, _ext.matmul_family(a))
+            check_layer(layer, x, torch.bfloat16, types=["GEMM_SPLITK", "GEMM"])
+
+
+@pytest.mark.gpu
 def test_mxfp4_with_k_not_a_multiple_of_128_streams(device):
     """MXFP4 x MXFP4 at K = 96, 160: three and five 32-blocks (the matrix-core kernel needs K % 128 == 0)."""
     for K in (96, 160):

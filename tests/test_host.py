@@ -486,8 +486,10 @@ def test_weight_only_and_mixed_mx_processors():
             lin, del_orig=False)
         assert l.input_dtype == DType.MXFP8 and l.scaled_activations and (l.W_nbits, l.elements_per_sample) == (4, 2)
         assert (l.W_group_mode, l.channel_scale_mode) == (0, csm)
-        # streaming up to 4 rows; above (K = 256 is a multiple of 128) the mixed fp8 x fp4 matrix-core kernel
-        for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (4, "MX_STREAM"), (5, "GEMM_MXFP8"), (64, "GEMM_MXFP8")):
+        # streaming up to 2 rows; 3..32 rows (K = 256 is one turn of the skinny kernel) in one launch on the mixed
+        # fp8 x fp4 form of the scaled MFMA; the tiled GEMM above
+        for M, fam in ((1, "MX_STREAM"), (2, "MX_STREAM"), (4, "K_SKINNY"), (5, "K_SKINNY"), (32, "K_SKINNY"),
+                       (33, "GEMM_MXFP8"), (64, "GEMM_MXFP8")):
             xq = torch.zeros(M, K, dtype=torch.float8_e4m3fn)
             sx = torch.ones(M, 1) if post_scale else torch.full(((M + 31) // 32 * 32, K // 32), 127, dtype=torch.uint8)
             assert _family(l, M, None, scales_x=sx, x=xq) == fam
