@@ -53,7 +53,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
 
 constexpr int kMxStreamRows = 2;  // MXFP4 x MXFP4: rows up to which the streaming kernel is chosen
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY, F_K_SKINNY };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY, F_K_SKINNY, F_WN_MID };
 
 int validate_operands(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -270,14 +270,18 @@ Family choose(const gla_matmul_args& p, int type) {
     if (p.M >= 3 && p.M <= 32 && (p.M <= 16 || p.N < 7040) && !want_matrix && p.tile_config < 1000 &&
         !(want_stream && gemv_kmajor_eligible(p)) && kring_eligible(p))
         return F_K_SKINNY;
+    // a tile_config that names the mid-batch kernel: -4, or waves per workgroup (4 or 8) + 1000 * K splits
+    const bool mid_asked = p.tile_config == GLA_TILE_PREFER_MID || (p.tile_config > 0 && (p.tile_config % 1000 == 4 || p.tile_config % 1000 == 8));
+    if (mid_asked && wn_mid_eligible(p)) return F_WN_MID;
     const bool small = !want_matrix && (type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16 || want_stream);
     if (small) {
-        // 8-bit codes on very large layers from 6 rows: the tiled GEMM's split-K stream is ahead of the 16-row GEMV
-        // pass (16384^2 at 8 / 16 rows: 65.2 / 64.6 against 70.6 / 72.8 us; 8192^2: 27.3 against 21.5-22.3, so only
-        // from 256 M weights up)
-        const bool big8 = p.W_nbits == 8 && p.M >= 6 && !want_stream && p.tile_config <= 0 && (int64_t)p.N * p.K >= ((int64_t)1 << 28) &&
+        // 8-bit codes on large layers from 5 rows: the mid-batch kernel reads the weights once for all rows and shares
+        // the activations through LDS, where the 16-row GEMV pass has every wave fetch its own (16384^2 at 5 / 16 rows:
+        // 48.5 / 50.1 against 69.5 / 72.8 us; 8192 x 16384: 33.5 against 38-40; 8192^2: 23-24 against 21.6-22.7, left
+        // with the GEMV)
+        const bool big8 = p.W_nbits == 8 && p.M >= 5 && !want_stream && p.tile_config <= 0 && (int64_t)p.N * p.K >= ((int64_t)1 << 27) &&
                           type > GLA_MATMUL_GEMV_SPLITK;
-        if (big8 && gemv_packed_eligible(p) && gemm_wn_eligible(p)) return F_GEMM_WN;
+        if (big8 && wn_mid_eligible(p)) return F_WN_MID;
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
     }
@@ -286,6 +290,11 @@ Family choose(const gla_matmul_args& p, int type) {
     // groups of 32, K not a multiple of 64), and up to 64 rows it beats the tiled GEMM on small and medium layers,
     // where that one cannot fill the chip without a deep K split (4096^2 4-bit at 32 rows: 9 against 17 us; 8192^2:
     // 22 against 26 us; 16384^2: 69 against 56 us, so large layers stay with the GEMM).
+    // 17..64 rows of 8-bit codes on large layers: weights from registers into the MFMA, activations shared through LDS
+    // (16384^2 at 32 / 64 rows: 56 / 70 us against 66 / 78 of the tiled GEMM; 8192^2: 26 / 31 against 27 / 32, left there)
+    if (p.M > 16 && p.M <= 64 && p.W_nbits == 8 && (int64_t)p.N * p.K >= ((int64_t)1 << 27) && !want_matrix && !want_stream &&
+        p.tile_config <= 0 && wn_mid_eligible(p))
+        return F_WN_MID;
     if (p.M > 16 && gemv_packed_eligible(p)) {
         if (!gemm_wn_eligible(p)) return F_GEMV_PACKED;
         const int64_t chunks = (p.M + 15) / 16;
@@ -310,6 +319,7 @@ int64_t family_workspace(Family f, const gla_matmul_args& a) {
     switch (f) {
         case F_GEMV_PACKED: return gemv_packed_workspace_bytes(a);
         case F_GEMM_WN: return gemm_wn_workspace_bytes(a);
+        case F_WN_MID: return wn_mid_workspace_bytes(a);
         case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(a);
         case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(a);
         case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(a);
@@ -455,6 +465,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_GEMM_KBYTES_MX: return args->bias != nullptr ? launch_gemm_kbytes_mx_bias(*args, s) : launch_gemm_kbytes_mx(*args, s);
         case F_MX_SKINNY: return launch_mx_skinny(*args, s);
         case F_K_SKINNY: return launch_kring(*args, s);
+        case F_WN_MID: return launch_wn_mid(*args, s);
         default: rc2 = launch_generic(*args, s); break;
     }
     if (rc2 == GLA_OK && args->bias != nullptr) rc2 = launch_bias_add(*args, s);

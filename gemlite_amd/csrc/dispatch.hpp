@@ -131,6 +131,11 @@ int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p);
 // ---- weight-only MX layers at 3..16 rows: weights straight into registers, matrix cores (mx_skinny.hip)
 bool mx_skinny_eligible(const gla_matmul_args& p);
 int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream);
+// ---- fp16 / bf16 x packed codes at 17..64 rows: weights from registers into the MFMA, activations shared through LDS (wn_mid.hip)
+bool wn_mid_eligible(const gla_matmul_args& p);
+int64_t wn_mid_workspace_bytes(const gla_matmul_args& p);
+int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream);
+
 // ---- MXFP4 x MXFP4, fp8 x fp8, int8 x int8 at 3..32 rows: operands copied to per-wave LDS rings by lines, MFMA (kring.hip)
 bool kring_eligible(const gla_matmul_args& p);
 int launch_kring(const gla_matmul_args& p, hipStream_t stream);

@@ -26,7 +26,7 @@ from .quant_utils import (scale_activations_mxfp4, scale_activations_mxfp8, scal
                           scale_activations_per_token)
 
 
-PREFER_STREAMING, PREFER_MATRIX = -2, -3   # GLA_TILE_PREFER_STREAMING / GLA_TILE_PREFER_MATRIX of the C header
+PREFER_STREAMING, PREFER_MATRIX, PREFER_MID = -2, -3, -4   # GLA_TILE_PREFER_* of the C header
 HAND_OFF_ROWS = 128                        # batch sizes up to which both kinds of kernel are timed
 
 
@@ -38,6 +38,8 @@ def candidate_configs(family: str, M: int, K: int) -> List[int]:
         bms = [32, 64] if M <= 32 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 512)]
+    if family == "WN_MID":           # waves per workgroup + 1000 * K splits
+        return [-1] + [nw + 1000 * s for nw in (4, 8) for s in (2, 4, 8, 16) if s <= max(1, K // 512)]
     if family in ("GEMM_KBYTES", "GEMM_KBYTES_MX"):      # BM + 1000 * K splits
         bms = [64] if M <= 64 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
@@ -106,7 +108,7 @@ def tune_layer(layer: GemLiteLinear, batch_sizes: Iterable[int], reps: int = 20,
         if M <= HAND_OFF_ROWS:
             # around the hand-off between the streaming kernels and the matrix-core GEMMs the other side is timed too;
             # the library's thresholds there were fitted on one machine
-            candidates += [t for t in (PREFER_STREAMING, PREFER_MATRIX) if _ext.matmul_family(build(t)) != family]
+            candidates += [t for t in (PREFER_STREAMING, PREFER_MATRIX, PREFER_MID) if _ext.matmul_family(build(t)) != family]
         for tile in candidates:
             args = build(tile)
             need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))

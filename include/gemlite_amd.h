@@ -82,6 +82,9 @@ extern "C" {
  * and batch size and stores the winner under the reference's config-cache key (reference: gemlite/core.py:838-906). */
 #define GLA_TILE_PREFER_STREAMING (-2)
 #define GLA_TILE_PREFER_MATRIX (-3)
+/* fp16 / bf16 activations on 2-, 4- or 8-bit packed codes, up to 64 rows: the mid-batch kernel (weights from registers
+ * into the MFMA, activations shared through LDS), which the library itself takes for 8-bit codes on large layers only */
+#define GLA_TILE_PREFER_MID (-4)
 
 /*
  * Arguments of one quantized matmul  out[M,N] = x[M,K] * dequant(w)[K,N].
@@ -190,6 +193,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_GEMM_KBYTES_MX 11 /* weight-only MX layers above 16 rows: MFMA GEMM, block scale applied on conversion */
 #define GLA_FAMILY_MX_SKINNY 12     /* weight-only MX layers at 3..16 rows: weights read once into registers, MFMA */
 #define GLA_FAMILY_K_SKINNY 13      /* MXFP4 x MXFP4, fp8 x fp8, int8 x int8 at 3..32 rows: operands as they are into the MFMA, one launch */
+#define GLA_FAMILY_WN_MID 14        /* fp16 / bf16 x packed codes at 17..64 rows: weights from registers into the MFMA, activations shared through LDS */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of

@@ -249,6 +249,39 @@ def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
 
 
+@pytest.mark.parametrize("nbits,gs", [(2, 64), (2, 128), (4, 64), (4, 128), (4, 256), (8, 64), (8, 128), (4, None), (8, None)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_packed_codes_at_17_to_64_rows(device, nbits, gs, dtype):
+    """The mid-batch kernel (weights from registers into the MFMA, activations shared through an LDS ring): every code
+    width and activation type, groups of half a stage, one stage and several stages, channel-wise scales (gs None),
+    1..4 row tiles with ragged last tiles, N that ends inside a wave's 64 columns and inside a workgroup's 512, K of
+    few and many stages (with and without a K split, splits of unequal length), a bias."""
+    dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
+    for (N, K) in ((1000, 1280), (520, 4352), (2112, 512)):
+        g = K if gs is None else gs
+        W_q, scales, zeros = gen_int_case(N, K, nbits, g, dtype, seed=nbits * 100 + g % 1000 + N)
+        layer = GemLiteLinear(nbits, g, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device),
+                                                           bias=gen_x(1, N, dtype, seed=5).reshape(-1).to(device) if N == 520 else None)
+        m = layer.get_meta_args()
+        for M in (5, 17, 32, 33, 47, 64):
+            x = gen_x(M, K, dtype, seed=M)
+            y_ref = oracle_forward(layer, x)
+            x = x.to(device)
+            for tile in (-4, 2008, 1004):   # the library's plan; 8 waves and 2 splits; 4 waves, K in one piece
+                out = torch.empty(M, N, dtype=dtype, device=device)
+                a = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                           unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                           acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                           data_contiguous=m[11], tile_config=tile, bias=layer.bias)
+                assert _ext.matmul_family(a) == "WN_MID", (N, K, M, tile, _ext.matmul_family(a))
+                print(f"case: WN_MID tile={tile} M={M} N={N} K={K}", flush=True)
+                _ext.matmul(a, device)
+                torch.cuda.synchronize()
+                err = rel_frob(to_np(out), y_ref)
+                assert err <= TIGHT[dtype], (N, K, M, tile, err)
+                assert elementwise_excess(to_np(out), y_ref, kind_of(dtype)) <= 1.0, (N, K, M, tile)
+
+
 @pytest.mark.parametrize("nbits,gs", [(1, 32), (1, 64), (2, 16), (2, 32), (4, 16), (8, 16)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_packed_codes_in_short_groups(device, nbits, gs, dtype):
