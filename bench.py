@@ -325,6 +325,13 @@ def extra_points(lib, device, T, quick):
         fns = [(lambda xi=xi: _ext.scale_activations_per_token(xi, xq_o, sx_o)) for xi in xs]
         us = T.graph_us(fns, 6)
         out[f"actquant_per_token_{name}"] = bw_point(us, M * K * 3 + M * 4, M=M, K=K, copies=len(xs))
+        if name == "fp8":
+            # what a plain streaming kernel with the same traffic (2 bytes read, 1 written per element, no row reduction)
+            # reaches on this box: torch's elementwise cast bf16 -> uint8 of the same matrices
+            u8 = torch.empty((M, K), dtype=torch.uint8, device=device)
+            us_cast = T.graph_us([(lambda xi=xi: u8.copy_(xi)) for xi in xs], 6)
+            out[f"actquant_per_token_{name}"]["elementwise_cast_same_traffic_us"] = round(us_cast, 2)
+            out[f"actquant_per_token_{name}"]["frac_of_that_cast"] = round(us_cast / us, 3)
         # decode: one row through the K-major streaming kernel (8-bit activations), weights rotated
         wbytes = N * K + N * 4
         layers = [layer] + [clone_layer(layer) for _ in range(copies_for(wbytes) - 1)]

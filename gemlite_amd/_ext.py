@@ -427,7 +427,7 @@ def matmul_is_supported(args: MatmulArgs) -> bool:
     return load_library().gla_matmul_family(ctypes.byref(args)) >= 0
 
 
-FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM", "BLOCKQ_STREAM", "GEMM_BLOCKQ", "GEMM_KBYTES_MX", "MX_SKINNY", "K_SKINNY", "WN_MID"]
+FAMILIES = ["GENERIC", "GEMV_PACKED", "GEMV_KMAJOR", "GEMM_WN", "GEMM_8BIT", "GEMM_MXFP4", "GEMM_KBYTES", "GEMM_MXFP8", "MX_STREAM", "BLOCKQ_STREAM", "GEMM_BLOCKQ", "GEMM_KBYTES_MX", "MX_SKINNY", "K_SKINNY", "WN_MID", "GEMM_16BIT"]
 
 
 def matmul_family(args: MatmulArgs) -> str:

@@ -53,7 +53,7 @@ int matmul_type_for(int M, int W_nbits, int mx) {
 
 constexpr int kMxStreamRows = 2;  // MXFP4 x MXFP4: rows up to which the streaming kernel is chosen
 
-enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY, F_K_SKINNY, F_WN_MID };
+enum Family { F_GENERIC = 0, F_GEMV_PACKED, F_GEMV_KMAJOR, F_GEMM_WN, F_GEMM_8BIT, F_GEMM_MXFP4, F_GEMM_KBYTES, F_GEMM_MXFP8, F_MX_STREAM, F_BLOCKQ_STREAM, F_GEMM_BLOCKQ, F_GEMM_KBYTES_MX, F_MX_SKINNY, F_K_SKINNY, F_WN_MID, F_GEMM_16BIT };
 
 int validate_operands(const gla_matmul_args* p) {
     if (p == nullptr) {
@@ -275,12 +275,16 @@ Family choose(const gla_matmul_args& p, int type) {
     if (mid_asked && wn_mid_eligible(p)) return F_WN_MID;
     const bool small = !want_matrix && (type <= GLA_MATMUL_GEMV_SPLITK || p.M <= 16 || want_stream);
     if (small) {
-        // 8-bit codes on large layers from 5 rows: the mid-batch kernel reads the weights once for all rows and shares
-        // the activations through LDS, where the 16-row GEMV pass has every wave fetch its own (16384^2 at 5 / 16 rows:
-        // 48.5 / 50.1 against 69.5 / 72.8 us; 8192 x 16384: 33.5 against 38-40; 8192^2: 23-24 against 21.6-22.7, left
-        // with the GEMV)
-        const bool big8 = p.W_nbits == 8 && p.M >= 5 && !want_stream && p.tile_config <= 0 && (int64_t)p.N * p.K >= ((int64_t)1 << 27) &&
-                          type > GLA_MATMUL_GEMV_SPLITK;
+        // 8-bit codes on large layers: the mid-batch kernel reads the weights once for all rows and shares the
+        // activations through LDS, where the GEMV has every wave fetch its own and, under bf16, feeds a byte as two
+        // nibbles.  From 5 rows on layers of 128 M weights (16384 x 8192 at 5 / 16 rows: 29.8 / 30.9 against 37.5 / 39.3 us;
+        // 8192 x 16384: 33.5 against 38-40; below 5 rows and on 8192^2 the GEMV is level or ahead), at any row count
+        // from 256 M weights (16384^2 at 1 / 4 / 16 rows: 49.7 / 51.0 / 48.8 against 54.1 / 56.1 / 72.9)
+        const int64_t weights = (int64_t)p.N * p.K;
+        // (a caller that names a GEMV type gets the GEMV)
+        const bool big8 = p.W_nbits == 8 && !want_stream && p.tile_config <= 0 &&
+                          (type > GLA_MATMUL_GEMV_SPLITK || p.matmul_type == GLA_MATMUL_AUTO) &&
+                          (weights >= ((int64_t)1 << 28) || (p.M >= 5 && weights >= ((int64_t)1 << 27)));
         if (big8 && wn_mid_eligible(p)) return F_WN_MID;
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
@@ -304,6 +308,11 @@ Family choose(const gla_matmul_args& p, int type) {
     if (gemm_wn_eligible(p)) return F_GEMM_WN;
     if (gemm_8bit_eligible(p)) return F_GEMM_8BIT;  // also streams K-major 8-bit operands at small M (split-K)
     if (gemm_kbytes_eligible(p)) return F_GEMM_KBYTES;
+    // unquantised layers: the generic family's vector kernels serve decode; from 9 rows (5 on layers above 32 M weights),
+    // or when asked, the MFMA GEMM (4096^2 bf16 at 8 / 16 / 64 / 4096 rows: 17.1 / 16.7 / 19.9 / 130 us against 16.2 / 25.3 /
+    // 70 / 3505; 14336 x 4096 at 4 / 8 rows: 33.7 / 28.8 against 30.4 / 47.2)
+    if ((p.M > 8 || (p.M > 4 && (int64_t)p.N * p.K > ((int64_t)1 << 25)) || want_matrix) && !want_stream && gemm_16bit_eligible(p))
+        return F_GEMM_16BIT;
     if (want_matrix) {  // no matrix-core kernel takes the call: the streaming ones after all
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;
@@ -320,6 +329,7 @@ int64_t family_workspace(Family f, const gla_matmul_args& a) {
         case F_GEMV_PACKED: return gemv_packed_workspace_bytes(a);
         case F_GEMM_WN: return gemm_wn_workspace_bytes(a);
         case F_WN_MID: return wn_mid_workspace_bytes(a);
+        case F_GEMM_16BIT: return gemm_16bit_workspace_bytes(a);
         case F_GEMM_8BIT: case F_GEMM_MXFP4: return gemm_8bit_workspace_bytes(a);
         case F_GEMM_KBYTES: return gemm_kbytes_workspace_bytes(a);
         case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(a);
@@ -354,7 +364,7 @@ bool widen(const gla_matmul_args& p, Widened& w) {
     w.q.workspace = nullptr;
     w.q.workspace_bytes = 0;
     w.f = choose(w.q, resolve_type(w.q));
-    if (!(w.f == F_GEMV_PACKED || w.f == F_GEMM_WN)) return false;
+    if (!(w.f == F_GEMV_PACKED || w.f == F_GEMM_WN || w.f == F_WN_MID)) return false;
     // An int32 accumulator was asked for: the 16-bit kernels sum in fp32, which is the same number as long as every
     // partial sum of |x| (<= 128) times |q - z| (below 2^W_nbits for a zero point inside the code range) over K stays
     // below 2^24.  Longer sums go to the generic kernel, which adds integers.
@@ -446,7 +456,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         w.q.x = x16;
         w.q.workspace = args->workspace;
         w.q.workspace_bytes = (uint64_t)w.x_off;
-        return w.f == F_GEMV_PACKED ? launch_gemv_packed(w.q, s) : launch_gemm_wn(w.q, s);
+        return w.f == F_GEMV_PACKED ? launch_gemv_packed(w.q, s) : (w.f == F_WN_MID ? launch_wn_mid(w.q, s) : launch_gemm_wn(w.q, s));
     }
     int rc2;
     switch (f) {
@@ -466,6 +476,7 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         case F_MX_SKINNY: return launch_mx_skinny(*args, s);
         case F_K_SKINNY: return launch_kring(*args, s);
         case F_WN_MID: return launch_wn_mid(*args, s);
+        case F_GEMM_16BIT: return launch_gemm_16bit(*args, s);
         default: rc2 = launch_generic(*args, s); break;
     }
     if (rc2 == GLA_OK && args->bias != nullptr) rc2 = launch_bias_add(*args, s);

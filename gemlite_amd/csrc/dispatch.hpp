@@ -131,6 +131,11 @@ int64_t gemm_kbytes_workspace_bytes(const gla_matmul_args& p);
 // ---- weight-only MX layers at 3..16 rows: weights straight into registers, matrix cores (mx_skinny.hip)
 bool mx_skinny_eligible(const gla_matmul_args& p);
 int launch_mx_skinny(const gla_matmul_args& p, hipStream_t stream);
+// ---- unquantised layers above 16 rows: fp16 x fp16 / bf16 x bf16 MFMA GEMM, weights [N, K] K-contiguous (gemm_16bit.hip)
+bool gemm_16bit_eligible(const gla_matmul_args& p);
+int64_t gemm_16bit_workspace_bytes(const gla_matmul_args& p);
+int launch_gemm_16bit(const gla_matmul_args& p, hipStream_t stream);
+
 // ---- fp16 / bf16 x packed codes at 17..64 rows: weights from registers into the MFMA, activations shared through LDS (wn_mid.hip)
 bool wn_mid_eligible(const gla_matmul_args& p);
 int64_t wn_mid_workspace_bytes(const gla_matmul_args& p);

@@ -44,7 +44,9 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6, kMX84 = 7, kMX84T = 8 };
+enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6, kMX84 = 7, kMX84T = 8, kH16 = 9, kB16 = 10 };
+// kH16 / kB16: fp16 x fp16 / bf16 x bf16 (unquantised layers, W_nbits = 16): the byte geometry of the int8 mode (two
+// K-steps of 32 bytes per stage, here 16 values each) on v_mfma_f32_32x32x16; built in a translation unit of its own
 // kMXFP8T: MXFP8 weights whose activations carry no block scales (their per-token scale is applied in the
 // epilogue), so no registers are spent on activation scale words and the 256-row tile fits
 // kMX84 / kMX84T: fp8 activations (with MXFP8 micro-scales / per token) x MXFP4 weights: the mixed form of the
@@ -99,7 +101,7 @@ __device__ __forceinline__ void wait_vmcnt8() {
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
 constexpr int slot_bytes8(int mode, int bm) {
     const bool w4 = mode == kMX84 || mode == kMX84T;
-    return bm * kRowB8 + kBN * (w4 ? 32 : kRowB8) + (mode == kFP8 || mode == kINT8 ? 0 : (bm + kBN) * 4);
+    return bm * kRowB8 + kBN * (w4 ? 32 : kRowB8) + (mode == kFP8 || mode == kINT8 || mode == kH16 || mode == kB16 ? 0 : (bm + kBN) * 4);
 }
 
 // WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
@@ -122,6 +124,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr bool BQ = MODE == kBQF8 || MODE == kBQI8;     // fp32 block scales, applied by the vector unit
     constexpr bool F8 = MODE == kFP8 || MODE == kBQF8;      // plain fp8 operands, one 64-byte K-step per stage
     constexpr bool I8 = MODE == kINT8 || MODE == kBQI8;
+    constexpr bool H16 = MODE == kH16 || MODE == kB16;      // 16-bit float operands, two K-steps of 16 values per stage
     constexpr bool MX = MODE == kMXFP4 || M8 || BQ;         // block scales ride along with every stage
     // MXFP8 and the fp32 block scales: a 32-bit scale word of a row covers 128 values = two stages; MXFP4: one stage
     constexpr int SSH = (M8 || BQ) ? 1 : 0;
@@ -384,7 +387,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         } else {
             // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
             // must not live across control flow)
-            const bool valid = !I8 || s2 * 32 < limit;
+            const bool valid = !(I8 || H16) || s2 * 32 < limit;
             u32x4 af = fa[B][i].c[s2];
             if (!valid) af = u32x4{0, 0, 0, 0};
             const u32x4 bf = fb[B][j].c[s2];
@@ -396,6 +399,11 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
                 }
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(int4_t{(int)bf.x, (int)bf.y, (int)bf.z, (int)bf.w},
                                                                   int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w}, cin, 0, 0, 0);
+            } else if constexpr (H16) {
+                if constexpr (MODE == kB16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bf), __builtin_bit_cast(bf16x8_t, af), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, bf), __builtin_bit_cast(half8_t, af), acc[i][j], 0, 0, 0);
             } else {
                 // fp4 operands occupy the first four of the eight operand registers; the rest is not read
                 const int4_t a4 = int4_t{(int)af.x, (int)af.y, (int)af.z, (int)af.w};
@@ -776,6 +784,7 @@ int attach_plan(const gla_matmul_args& p, const Plan8& g, Gemm8Args& a) {
 
 }  // namespace
 
+#ifndef GLA_G8_16BIT
 bool gemm_8bit_eligible(const gla_matmul_args& p) {
     const bool fp8 = p.input_dtype == GLA_DT_FP8 && p.w_dtype == GLA_DT_FP8 && p.acc_dtype == GLA_DT_FP32;
     const bool i8 = p.input_dtype == GLA_DT_INT8 && p.w_dtype == GLA_DT_INT8;
@@ -1012,5 +1021,50 @@ int launch_gemm_mxfp8(const gla_matmul_args& p, hipStream_t stream) {
     if (p.elements_per_sample == 2) return act_blocks ? launch_mode<kMX84>(a, g.bm, stream) : launch_mode<kMX84T>(a, g.bm, stream);
     return act_blocks ? launch_mode<kMXFP8>(a, g.bm, stream) : launch_mode<kMXFP8T>(a, g.bm, stream);
 }
+
+#else  // GLA_G8_16BIT
+
+// ---- unquantised layers: fp16 x fp16 / bf16 x bf16, weights [N, K] with K contiguous (W_nbits = 16) ----------------
+// (reference: the same `tl.dot` GEMM with the unpacking switched off, gemlite/triton_kernels/gemm_kernels.py:285-496)
+bool gemm_16bit_eligible(const gla_matmul_args& p) {
+    const bool h = p.input_dtype == GLA_DT_FP16 && p.w_dtype == GLA_DT_FP16, b = p.input_dtype == GLA_DT_BF16 && p.w_dtype == GLA_DT_BF16;
+    if (!h && !b) return false;
+    if (p.elements_per_sample != 1 || p.W_nbits != 16 || p.W_group_mode != GLA_WGM_NONE || p.acc_dtype != GLA_DT_FP32) return false;
+    if (p.channel_scale_mode < GLA_CSM_NONE || p.channel_scale_mode > GLA_CSM_BOTH) return false;
+    if (p.w_stride_k != 1 || p.x_stride_k != 1 || p.out_stride_n != 1) return false;
+    // rows of whole 16-byte chunks, K in whole stages of 32 values
+    if (p.K % 32 != 0 || p.x_stride_m % 8 != 0 || p.w_stride_n % 8 != 0) return false;
+    if (((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
+    if ((int64_t)p.M * p.x_stride_m * 2 >= (1ll << 31) || (int64_t)p.N * p.w_stride_n * 2 >= (1ll << 31)) return false;
+    if (!(p.output_dtype == GLA_DT_FP16 || p.output_dtype == GLA_DT_BF16 || p.output_dtype == GLA_DT_FP32)) return false;
+    if ((p.channel_scale_mode & 1) && p.scales == nullptr) return false;
+    if ((p.channel_scale_mode & 2) && p.scales_x == nullptr) return false;
+    return true;
+}
+
+int64_t gemm_16bit_workspace_bytes(const gla_matmul_args& p) {
+    const Plan8 g = plan8(p.M, p.N, p.K * 2, p.tile_config);
+    return g.S > 1 ? kWsReserved8 + (int64_t)g.S * p.M * p.N * 4 : 0;
+}
+
+int launch_gemm_16bit(const gla_matmul_args& p, hipStream_t stream) {
+    if (!gemm_16bit_eligible(p)) {
+        set_error("gemm_16bit: fp16 x fp16 or bf16 x bf16, both K-contiguous with 16-byte aligned rows, K a multiple of 32");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    Gemm8Args a;
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
+    a.a = (const uint8_t*)p.x; a.b = (const uint8_t*)p.w; a.scales = p.scales; a.scales_x = p.scales_x; a.out = p.out;
+    a.M = p.M; a.N = p.N; a.Kb = p.K * 2; a.lda = p.x_stride_m * 2; a.ldb = p.w_stride_n * 2; a.osm = p.out_stride_m;
+    a.sxm = p.sx_stride_m; a.msn = 0; a.csm = p.channel_scale_mode; a.meta_dt = p.meta_dtype; a.sx_dt = p.sx_dtype;
+    a.out_dt = p.output_dtype; a.sx_stage = 0; a.sw_stage = 0; a.ascales = nullptr; a.asxm = 0;
+    const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
+    const int rc = attach_plan(p, g, a);
+    if (rc != GLA_OK) return rc;
+    if (p.input_dtype == GLA_DT_BF16) return launch_mode<kB16>(a, g.bm, stream);
+    return launch_mode<kH16>(a, g.bm, stream);
+}
+
+#endif
 
 }  // namespace gla

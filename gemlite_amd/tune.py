@@ -44,7 +44,7 @@ def candidate_configs(family: str, M: int, K: int) -> List[int]:
         bms = [64] if M <= 64 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 512)]
-    if family in ("GEMM_8BIT", "GEMM_MXFP4", "GEMM_MXFP8"):
+    if family in ("GEMM_8BIT", "GEMM_MXFP4", "GEMM_MXFP8", "GEMM_16BIT"):
         bms = [64] if M <= 64 else ([64, 128] if M <= 128 else [128, 256])
         splits = [1, 2, 4, 8, 16] if M <= 256 else [1, 2]
         return [-1] + [bm + 1000 * s for bm in bms for s in splits if s <= max(1, K // 1024)]

@@ -194,6 +194,7 @@ int gla_select_config(const gla_matmul_args* args);
 #define GLA_FAMILY_MX_SKINNY 12     /* weight-only MX layers at 3..16 rows: weights read once into registers, MFMA */
 #define GLA_FAMILY_K_SKINNY 13      /* MXFP4 x MXFP4, fp8 x fp8, int8 x int8 at 3..32 rows: operands as they are into the MFMA, one launch */
 #define GLA_FAMILY_WN_MID 14        /* fp16 / bf16 x packed codes at 17..64 rows: weights from registers into the MFMA, activations shared through LDS */
+#define GLA_FAMILY_GEMM_16BIT 15    /* unquantised layers above 16 rows: fp16 x fp16 / bf16 x bf16 MFMA GEMM */
 int gla_matmul_family(const gla_matmul_args* args);
 
 /* Diagnostic, no counterpart in the reference: launches a register-only loop of

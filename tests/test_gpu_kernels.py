@@ -401,6 +401,29 @@ def test_unpacked_16_bit_weights_both_layouts(device, contiguous, w_dtype, x_dty
             check_layer(layer, gen_x(M, K, x_dtype, seed=M).to(device), x_dtype, types=())
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_unquantised_layers_above_16_rows_on_matrix_cores(device, dtype):
+    """W_nbits = 16 at the reference's own test shape (tests/test_int.py:99-118: K = 3968, N = 2032) and its batch
+    sizes above 16 rows, and at a shape whose K is a few stages: the MFMA GEMM on both operands as they lie ([rows, K],
+    K contiguous), every tile height, with and without a K split, ragged M and N tiles, a bias."""
+    dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
+    for (N, K, with_bias) in ((2032, 3968, False), (520, 160, True)):
+        W = gen_x(N, K, dtype, seed=N, std=0.05)
+        bias = gen_x(1, N, dtype, seed=4).view(N).to(device) if with_bias else None
+        layer = GemLiteLinear(16, None, K, N, dt, dt).pack(W.to(device), None, None, bias)
+        assert layer.W_group_mode == 0 and layer.channel_scale_mode == 0 and not layer.data_contiguous
+        m = layer.get_meta_args()
+        for M in (17, 30, 65, 100, 250, 600):
+            x = gen_x(M, K, dtype, seed=M).to(device)
+            out = torch.empty(M, N, dtype=dtype, device=device)
+            a = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                       unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                       acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                       data_contiguous=m[11])
+            assert _ext.matmul_family(a) == "GEMM_16BIT", (N, K, M, _ext.matmul_family(a))
+            check_layer(layer, x, dtype, types=["GEMM_SPLITK", "GEMM"])
+
+
 @pytest.mark.parametrize("width", [8, 16, 64])
 def test_other_packing_widths(device, width):
     N, K, gs = 256, 512, 64
