@@ -260,7 +260,17 @@ def extra_points(lib, device, T, quick):
     run = Launch(lib, base, x, y, device)
     us = T.eager_us(run, 40)
     gemm_point("gemm_a16w4_gs128_fp16", M, N, K, us, 2500.0, "fp16", zeroed(run, x, base.W_q.data))
-    del base, x, y, run
+    del base, run
+    # an unquantised layer of the same shape (W_nbits = 16): fp16 x fp16 on the K-contiguous MFMA GEMM, and the vendor's
+    # plain GEMM on the same operands in the same run
+    W16 = (torch.randn((N, K), generator=g) * 0.02).to(torch.float16).to(device)
+    l16 = GemLiteLinear(16, None, K, N, DType.FP16, DType.FP16).pack(W16, None, None)
+    run = Launch(lib, l16, x, y, device)
+    us = T.eager_us(run, 40)
+    us_vendor = T.eager_us(lambda: torch.matmul(x, l16.W_q, out=y), 20)
+    gemm_point("gemm_a16w16_fp16", M, N, K, us, 2500.0, "fp16", zeroed(run, x, W16))
+    out["gemm_a16w16_fp16"]["vendor_library_same_operands"] = {"us": round(us_vendor, 1), "entry": "torch.matmul"}
+    del l16, W16, x, y, run
 
     # ---- C3: bf16 activations, K = N = 16384: 8-bit channel-wise and 2-bit group-64 weights, M = 1 / 16 / 64 / 512
     N = K = 16384
@@ -331,7 +341,7 @@ def extra_points(lib, device, T, quick):
             u8 = torch.empty((M, K), dtype=torch.uint8, device=device)
             us_cast = T.graph_us([(lambda xi=xi: u8.copy_(xi)) for xi in xs], 6)
             out[f"actquant_per_token_{name}"]["elementwise_cast_same_traffic_us"] = round(us_cast, 2)
-            out[f"actquant_per_token_{name}"]["frac_of_that_cast"] = round(us_cast / us, 3)
+            out[f"actquant_per_token_{name}"]["speed_vs_that_cast"] = round(us_cast / us, 3)
         # decode: one row through the K-major streaming kernel (8-bit activations), weights rotated
         wbytes = N * K + N * 4
         layers = [layer] + [clone_layer(layer) for _ in range(copies_for(wbytes) - 1)]

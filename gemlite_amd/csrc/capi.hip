@@ -300,6 +300,12 @@ Family choose(const gla_matmul_args& p, int type) {
         p.tile_config <= 0 && wn_mid_eligible(p))
         return F_WN_MID;
     if (p.M > 16 && gemv_packed_eligible(p)) {
+        // groups of 32, which the tiled GEMM does not take: the mid-batch kernel (row chunks of 64) once the GEMV's
+        // chunks of 16 have re-read the weights often enough (4-bit gs 32, 8192^2 at 64 / 256 rows: 36 / 85 against
+        // 42 / 164 us; 4096^2: 23 / 36 against 15 / 43)
+        if (!gemm_wn_eligible(p) && !want_stream && p.tile_config <= 0 && (p.M > 64 || (int64_t)p.N * p.K >= ((int64_t)1 << 26)) &&
+            wn_mid_eligible(p))
+            return F_WN_MID;
         if (!gemm_wn_eligible(p)) return F_GEMV_PACKED;
         const int64_t chunks = (p.M + 15) / 16;
         const int64_t restreamed = chunks * (int64_t)p.N * p.K * (p.W_nbits < 4 ? 4 : p.W_nbits) / 8;  // 2-bit codes cost what 4-bit ones do
@@ -313,6 +319,12 @@ Family choose(const gla_matmul_args& p, int type) {
     // 70 / 3505; 14336 x 4096 at 4 / 8 rows: 33.7 / 28.8 against 30.4 / 47.2)
     if ((p.M > 8 || (p.M > 4 && (int64_t)p.N * p.K > ((int64_t)1 << 25)) || want_matrix) && !want_stream && gemm_16bit_eligible(p))
         return F_GEMM_16BIT;
+    // 2-bit codes in groups of 32 and 1-bit codes in groups of 32 / 64 have no streaming kernel and no tiled GEMM: the
+    // mid-batch kernel at every row count (2-bit gs 32, 8192^2 at 1 / 64 / 256 rows: 19.5 / 30 / 63 us against 37 / 408 /
+    // 1592 of the generic kernels; 1-bit gs 64, 16384^2 at 64 rows: 72 us against 2.0 ms), except a single row of 1-bit
+    // codes on small and medium layers, where the generic K-split kernel is ahead (14336 x 4096: 15.2 against 19.3)
+    const bool one_row_1bit = p.W_nbits == 1 && p.M == 1 && (int64_t)p.N * p.K < ((int64_t)1 << 26);
+    if (p.tile_config <= 0 && !want_stream && !one_row_1bit && wn_mid_eligible(p)) return F_WN_MID;
     if (want_matrix) {  // no matrix-core kernel takes the call: the streaming ones after all
         if (gemv_packed_eligible(p)) return F_GEMV_PACKED;
         if (gemv_kmajor_eligible(p)) return F_GEMV_KMAJOR;

@@ -1,4 +1,4 @@
-// Mid-batch matmul (17..64 rows) for fp16/bf16 activations x 32-bit packed low-bit weights stored [K/e, N], N fastest:
+// Mid-batch matmul (up to 64 rows per pass) for fp16/bf16 activations x 32-bit packed low-bit weights stored [K/e, N], N fastest:
 // out[M,N] = x[M,K] * dequant(W)[K,N].  The batch sizes between the streaming GEMV (up to 16 rows) and the tiled GEMM,
 // where the weights are still read once but every weight meets 2-4 MFMA row tiles.
 //
@@ -15,6 +15,7 @@
 //    row >> 1, and each wave reads its A operands from there (one ds_read_b128 per row tile and K-step).
 //  * Weights and group metadata of the next D - 1 stages wait in registers; a wave waits on the vector-memory counter
 //    once per stage, then the workgroup meets at one bare barrier, behind which the slot read last is refilled.
+//  * 1-bit codes: a lane's word is 32 K-values, its share of all four K-steps of a 128-K stage (one load per stage).
 //  * Dequantisation as in the tiled GEMM (wn_dequant.hpp): fp16 in natural K order (one v_perm + one masked OR per code
 //    pair, packed fp16 subtract and fma), bf16 with codes paired (j, j + 4) or (j, j + 8) and the activation fragment
 //    permuted to match, 2-bit codes on bf16 through a four-entry table per column and group, byte codes on bf16 by
@@ -46,6 +47,9 @@ struct WnMidArgs {
     int S;
     int spg;        // stages per quantisation group when a group spans whole stages (else 1)
     int spg_shift;  // log2(spg) when it is a power of two, else -1
+    // groups that follow from the lane (a lane's word spans 16 or 32 K-values, so one MFMA K-step mixes 32-blocks):
+    // group of (stage st, metadata slot gi, K-quarter kb) = st gt + gi gmul + (kb >> kbs)
+    int lane_g, gt, gmul, kbs;
     int64_t xsm_b, wsk_b, msg_b, zsg_b;  // bytes per activation row, word row, group row of scales / zeros
     int64_t osm, sxm;
     int has_s, has_zt;  // the scales / zeros arrays are read per group
@@ -106,6 +110,7 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
     const bool col_ok = col < a.N;
     if (col > a.N - 4) col = a.N - 4;  // clamped lanes compute something and store nothing
     const int split = blockIdx.y;
+    const int m0 = blockIdx.z * (16 * RT);  // batches above 64 rows run as row chunks that each read the weights again
     const int st0 = split * a.sps;
     const int nst = (a.stages - st0) < a.sps ? (a.stages - st0) : a.sps;
     const int st_last = st0 + nst - 1;
@@ -122,7 +127,7 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
         const int rt = t / XT, h = t % XT;
         const int row = 8 * j + (lane >> 3);
         const int piece = ((lane & 7) ^ (row >> 1)) & 7;
-        int m = 16 * rt + row;
+        int m = m0 + 16 * rt + row;
         if (m > a.M - 1) m = a.M - 1;
         a_off[i] = (uint32_t)m * (uint32_t)a.xsm_b + (uint32_t)(h * 128 + piece * 16);
         a_dst[i] = t * TILE + j * 1024;
@@ -156,7 +161,9 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
         for (int u = 0; u < CW; ++u) f.w[u] = load_streaming_u4(wk + w_off[u]);
 #pragma unroll
         for (int gi = 0; gi < GPS; ++gi) {
-            const int g = GPS > 1 ? st * GPS + gi : group_of(st);
+            // (2-bit codes in groups of 32 and 1-bit codes in groups of 32 or 64: the lane's group follows from its
+            // K-quarter)
+            const int g = a.lane_g ? st * a.gt + gi * a.gmul + (kb >> a.kbs) : (GPS > 1 ? st * GPS + gi : group_of(st));
             f.s[gi] = load_streaming_u2(a.scales + (a.has_s ? (int64_t)g * a.msg_b + m_off : 0));
             f.z[gi] = load_streaming_u2(a.zeros + (a.has_zt ? (int64_t)g * a.zsg_b + m_off : 0));
         }
@@ -225,6 +232,15 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
                     const uint32_t w = word(2 * ks + q / 2);
                     t = __builtin_amdgcn_perm(w, w, q % 2 ? 0x0c030c02u : 0x0c010c00u) | 0x64006400u;
                     bq[q] = dequant_pair<BF16>(t, meta[j]);
+                } else if constexpr (BITS == 1) {
+                    // a word is 32 K-values = the lane's share of all four K-steps: step ks takes byte ks, whose bits 2q and
+                    // 2q + 1 land in the mantissas of 2^(10 - 2q) and 2^(9 - 2q)
+                    const uint32_t w = word(0);
+                    const uint32_t u = __builtin_amdgcn_perm(w, w, 0x0c000c00u | ((uint32_t)ks << 16) | (uint32_t)ks);
+                    const uint32_t mk = (1u << (2 * q)) | (1u << (2 * q + 17));
+                    const uint32_t mg = ((uint32_t)(25 - 2 * q) << 10) | ((uint32_t)(24 - 2 * q) << 26);
+                    t = (u & mk) | mg;
+                    bq[q] = dequant_pair<BF16>(t, meta[j], (float)(1024 >> (2 * q)), (float)(512 >> (2 * q)));
                 } else if constexpr (BITS == 4) {
                     const uint32_t w = word(ks);
                     t = (__builtin_amdgcn_perm(w, w, 0x0c000c00u | (q << 16) | q) & nat_mask0) | nat_magic0;
@@ -237,6 +253,9 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
                     if (q % 2 == 0) bq[q] = dequant_pair<BF16>((u & nat_mask0) | nat_magic0, meta[j], 1024.0f, 256.0f);
                     else bq[q] = dequant_pair<BF16>((u & nat_mask1) | nat_magic1, meta[j], 64.0f, 16.0f);
                 }
+            } else if constexpr (BITS == 1) {
+                t = ((word(0) >> (4 * ks + q)) & pair_mask) | magic;  // codes (4 ks + q, + 16) of the lane's 32
+                bq[q] = dequant_pair<BF16>(t, meta[j]);
             } else if constexpr (BITS == 4) {
                 t = ((word(ks) >> (q * 4)) & pair_mask) | magic;  // codes (q, q + 4)
                 bq[q] = dequant_pair<BF16>(t, meta[j]);
@@ -272,7 +291,7 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
                 if (ks % (KSTEPS / GPS) == 0) convert_meta(f.s[ks / (KSTEPS / GPS)], f.z[ks / (KSTEPS / GPS)]);
             } else {
                 if (ks == 0) {
-                    const int g = group_of(st);
+                    const int g = a.lane_g ? st : group_of(st);
                     if (g != g_have) convert_meta(f.s[0], f.z[0]);
                     g_have = g;
                 }
@@ -281,7 +300,21 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 const unsigned char* tile = base + (rt * XT + (XT > 1 ? ks / 2 : 0)) * TILE;
-                if constexpr (BF16 && BITS == 2) {
+                if constexpr (BITS == 1) {
+                    // the lane's 32 K-values are half a 64-K tile: tile kb / 2, pieces 4 (kb % 2) .. + 3
+                    const unsigned char* t1 = base + (rt * XT + (kb >> 1)) * TILE;
+                    if constexpr (BF16) {
+                        // codes (4 ks + r, + 16): activations 4 ks .. + 3 and 16 + 4 ks .. + 3 of the lane's 32
+                        if (ks % 2 == 0) {
+                            keep_lo[rt] = a_piece(t1, 4 * (kb & 1) + ks / 2);
+                            keep_hi[rt] = a_piece(t1, 4 * (kb & 1) + ks / 2 + 2);
+                        }
+                        const int t2 = 2 * (ks % 2);
+                        av[rt] = pair_order(keep_lo[rt][t2], keep_lo[rt][t2 + 1], keep_hi[rt][t2], keep_hi[rt][t2 + 1]);
+                    } else {
+                        av[rt] = a_piece(t1, 4 * (kb & 1) + ks);
+                    }
+                } else if constexpr (BF16 && BITS == 2) {
                     if (ks % 2 == 0) {
                         keep_lo[rt] = a_piece(tile, 2 * kb);
                         keep_hi[rt] = a_piece(tile, 2 * kb + 1);
@@ -337,7 +370,7 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
     (void)st_last;
     wait_vmcnt_m<0>();  // the surplus copies of the last iterations must have landed before the LDS is given back
 
-    // ---- lane (cg, kb) holds rows 16 rt + 4 kb + e of columns n0w + 4 cg + j in acc[rt][j][e]
+    // ---- lane (cg, kb) holds rows m0 + 16 rt + 4 kb + e of columns n0w + 4 cg + j in acc[rt][j][e]
     if (!col_ok) return;
     if (a.S > 1) {
         float* dst = a.partials + (size_t)split * a.M * a.N;
@@ -345,7 +378,7 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int m = 16 * rt + 4 * kb + e;
+                const int m = m0 + 16 * rt + 4 * kb + e;
                 if (m < a.M) *(float4_t*)(dst + (size_t)m * a.N + col) = float4_t{acc[rt][0][e], acc[rt][1][e], acc[rt][2][e], acc[rt][3][e]};
             }
         return;
@@ -360,7 +393,7 @@ __global__ __launch_bounds__(NW * 64) void wn_mid_kernel(WnMidArgs a) {
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int m = 16 * rt + 4 * kb + e;
+            const int m = m0 + 16 * rt + 4 * kb + e;
             if (m >= a.M) continue;
             const float sa = (a.csm & 2) ? load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm) : 1.0f;
 #pragma unroll
@@ -393,7 +426,8 @@ __global__ __launch_bounds__(256) void wn_mid_finish_kernel(WnMidArgs p) {
 }
 
 struct MidPlan {
-    int rt, nw, S, sps, stages, gps;
+    int rt, nw, S, sps, stages, gps, gt;
+    bool lane_groups;  // 2-bit codes in groups of 32, 1-bit codes in groups of 32 / 64: the lane picks its group (gt per stage)
 };
 
 int stage_k(int bits) { return bits == 8 ? 64 : 128; }
@@ -401,7 +435,7 @@ int stage_k(int bits) { return bits == 8 ? 64 : 128; }
 MidPlan mid_plan(const gla_matmul_args& p) {
     // tile_config: waves per workgroup (4 or 8) + 1000 * K splits; anything else leaves both to the rule below
     MidPlan g;
-    g.rt = ceil_div(p.M, 16);
+    g.rt = p.M > 64 ? 4 : ceil_div(p.M, 16);
     const int cfg = p.tile_config > 0 ? p.tile_config : 0;
     // Four waves (256 columns) per workgroup: half the K splits, and with them half the fp32 partials, of eight waves
     // for the same number of workgroups (8-bit codes, 16384^2 at 16 / 64 rows: 50 / 70 us against 60 / 75)
@@ -410,9 +444,15 @@ MidPlan mid_plan(const gla_matmul_args& p) {
     const bool grouped = p.W_group_mode >= GLA_WGM_SCALE || (p.W_group_mode == GLA_WGM_SHIFT && !p.zero_is_scalar);
     const int gs = grouped ? p.group_size : p.K;
     g.gps = gs < stage_k(p.W_nbits) ? stage_k(p.W_nbits) / gs : 1;
+    // a lane's word of 2-bit codes is 16 K-values, of 1-bit codes 32: below groups of 64 (128) the group follows
+    // from the lane
+    g.lane_groups = (p.W_nbits == 2 && g.gps == 4) || (p.W_nbits == 1 && g.gps > 1);
+    g.gt = g.gps;
+    if (g.lane_groups) g.gps = p.W_nbits == 2 ? 2 : 1;
     // one workgroup per CU; a split is at least 4 stages long
     const int blocks = ceil_div(p.N, 64 * g.nw);
-    int want = cfg >= 1000 ? cfg / 1000 : (256 + blocks - 1) / blocks;
+    const int chunks = ceil_div(p.M, 64);
+    int want = cfg >= 1000 ? cfg / 1000 : (256 + blocks * chunks - 1) / (blocks * chunks);
     if (want > g.stages / 4) want = g.stages / 4;
     if (want < 1) want = 1;
     g.sps = ceil_div(g.stages, want);
@@ -433,7 +473,7 @@ int launch_mid(const WnMidArgs& a, const MidPlan& g, hipStream_t stream) {
         if (rc != GLA_OK) return rc;
     }
     (void)g;
-    hipLaunchKernelGGL(kern, dim3(ceil_div(a.N, 64 * NW), a.S), dim3(NW * 64), smem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(ceil_div(a.N, 64 * NW), a.S, ceil_div(a.M, 16 * RT)), dim3(NW * 64), smem, stream, a);
     int rc = check_hip(hipGetLastError(), "wn_mid launch");
     if (rc == GLA_OK && a.S > 1) {
         const int64_t items = (int64_t)a.M * (a.N / 4);
@@ -445,6 +485,9 @@ int launch_mid(const WnMidArgs& a, const MidPlan& g, hipStream_t stream) {
 
 template <int BITS, bool BF16, int RT>
 int launch_mid_gps(const WnMidArgs& a, const MidPlan& g, hipStream_t stream) {
+    if constexpr (BITS == 4) {
+        if (g.gps == 4) return launch_mid<BITS, BF16, RT, 4, 4>(a, g, stream);  // groups of 32: four waves only
+    }
     if (g.nw == 4) {
         if (g.gps == 2) return launch_mid<BITS, BF16, RT, 2, 4>(a, g, stream);
         return launch_mid<BITS, BF16, RT, 1, 4>(a, g, stream);
@@ -466,21 +509,31 @@ int launch_mid_rt(const WnMidArgs& a, const MidPlan& g, hipStream_t stream) {
 }  // namespace
 
 bool wn_mid_eligible(const gla_matmul_args& p) {
-    if (!gemm_wn_eligible(p)) return false;  // operand types, layouts and alignments of the packed-weight kernels
-    if (p.M < 1 || p.M > 64) return false;
+    // operand types, layouts and alignments as for the tiled packed-weight GEMM, whose rule on groups (whole 64-K
+    // stages) is replaced by this kernel's own below; 1-bit codes, which that one does not take, pass as 2-bit ones
+    gla_matmul_args q = p;
+    q.group_size = p.K;
+    if (p.W_nbits == 1 && p.elements_per_sample == 32) {
+        q.W_nbits = 2;
+        q.elements_per_sample = 16;
+    }
+    if (p.K <= 0 || !gemm_wn_eligible(q)) return false;
+    if (p.M < 1) return false;
     const int ks = stage_k(p.W_nbits);
-    if (p.K % ks != 0 || p.K / ks < 1) return false;
+    if (p.K % ks != 0) return false;
     const bool uses_scales = p.W_group_mode >= GLA_WGM_SCALE;
     const bool zeros_tensor = (p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE) && !p.zero_is_scalar;
     const bool grouped = uses_scales || zeros_tensor;
     const int gs = grouped ? p.group_size : p.K;
-    // a group is whole stages, or a stage is two groups
-    if (!(gs % ks == 0 || 2 * gs == ks)) return false;
+    if (gs <= 0 || p.K % gs != 0) return false;
+    // a group is whole stages, or a stage is two groups, or (2- and 4-bit codes) four groups of one K-step each
+    if (!(gs % ks == 0 || 2 * gs == ks || (4 * gs == ks && p.W_nbits != 8))) return false;
+    if ((int64_t)(p.K / p.elements_per_sample) * p.w_stride_k >= (1ll << 31)) return false;
     // metadata is read as four adjacent 16-bit values per lane
     const bool one_group = gs == p.K;
     if (uses_scales && (((uintptr_t)p.scales & 7) || (!one_group && p.meta_stride_g % 4 != 0))) return false;
     if (zeros_tensor && (((uintptr_t)p.zeros & 7) || (!one_group && p.meta_stride_g % 4 != 0))) return false;
-    if ((int64_t)64 * p.x_stride_m * 2 >= (1ll << 31)) return false;
+    if ((int64_t)p.M * p.x_stride_m * 2 >= (1ll << 31)) return false;
     return true;
 }
 
@@ -491,8 +544,8 @@ int64_t wn_mid_workspace_bytes(const gla_matmul_args& p) {
 
 int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream) {
     if (!wn_mid_eligible(p)) {
-        set_error("wn_mid: fp16 / bf16 activations on 2-, 4- or 8-bit packed codes, up to 64 rows, groups of whole 128-K "
-                  "stages (8-bit: 64) or half a stage");
+        set_error("wn_mid: fp16 / bf16 activations on 2-, 4- or 8-bit packed codes, groups of whole 128-K stages (8-bit: 64), "
+                  "half a stage or (2-, 4-bit) a quarter");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     const MidPlan g = mid_plan(p);
@@ -510,6 +563,9 @@ int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream) {
     a.stages = g.stages; a.sps = g.sps; a.S = g.S;
     const int ks = stage_k(p.W_nbits);
     a.spg = gs >= ks ? gs / ks : 1;
+    a.lane_g = g.lane_groups; a.gt = g.gt;
+    a.gmul = p.W_nbits == 2 ? 2 : 0;                       // 2-bit: metadata slot gi is the 64-K load, two groups each
+    a.kbs = (p.W_nbits == 1 && g.gt == 4) ? 0 : 1;         // 1-bit gs 32: a group per K-quarter; otherwise per pair of them
     a.spg_shift = -1;
     for (int s = 0; s < 31; ++s)
         if ((1 << s) == a.spg) a.spg_shift = s;
@@ -531,6 +587,7 @@ int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream) {
     }
     const bool bf16 = p.input_dtype == GLA_DT_BF16;
     switch (p.W_nbits) {
+        case 1: return bf16 ? launch_mid_rt<1, true>(a, g, stream) : launch_mid_rt<1, false>(a, g, stream);
         case 2: return bf16 ? launch_mid_rt<2, true>(a, g, stream) : launch_mid_rt<2, false>(a, g, stream);
         case 4: return bf16 ? launch_mid_rt<4, true>(a, g, stream) : launch_mid_rt<4, false>(a, g, stream);
         default: return bf16 ? launch_mid_rt<8, true>(a, g, stream) : launch_mid_rt<8, false>(a, g, stream);

@@ -249,12 +249,12 @@ def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
 
 
-@pytest.mark.parametrize("nbits,gs", [(2, 64), (2, 128), (4, 64), (4, 128), (4, 256), (8, 64), (8, 128), (4, None), (8, None)])
+@pytest.mark.parametrize("nbits,gs", [(1, 32), (1, 64), (1, 128), (1, 256), (2, 32), (4, 32), (8, 32), (2, 64), (2, 128), (4, 64), (4, 128), (4, 256), (8, 64), (8, 128), (4, None), (8, None)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_packed_codes_at_17_to_64_rows(device, nbits, gs, dtype):
     """The mid-batch kernel (weights from registers into the MFMA, activations shared through an LDS ring): every code
-    width and activation type, groups of half a stage, one stage and several stages, channel-wise scales (gs None),
-    1..4 row tiles with ragged last tiles, N that ends inside a wave's 64 columns and inside a workgroup's 512, K of
+    width and activation type, groups of a quarter of a stage, half a stage, one stage and several stages, channel-wise
+    scales (gs None), 1..4 row tiles with ragged last tiles, batches above 64 rows as row chunks, N that ends inside a wave's 64 columns and inside a workgroup's 512, K of
     few and many stages (with and without a K split, splits of unequal length), a bias."""
     dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
     for (N, K) in ((1000, 1280), (520, 4352), (2112, 512)):
@@ -263,7 +263,7 @@ def test_packed_codes_at_17_to_64_rows(device, nbits, gs, dtype):
         layer = GemLiteLinear(nbits, g, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device),
                                                            bias=gen_x(1, N, dtype, seed=5).reshape(-1).to(device) if N == 520 else None)
         m = layer.get_meta_args()
-        for M in (5, 17, 32, 33, 47, 64):
+        for M in (5, 17, 32, 33, 47, 64, 150):
             x = gen_x(M, K, dtype, seed=M)
             y_ref = oracle_forward(layer, x)
             x = x.to(device)
