@@ -575,6 +575,16 @@ def run_point(name, lib, device, T):
         layer, _ = make_layer(N, K, seed=11, device=device)
         xq, sx = torch.randn((M, K), generator=g).to(torch.float16).to(device), None
         peak = 2500.0
+    elif name in ("gemv_a16w8_channelwise_16384sq_M16", "gemm_a16w8_channelwise_16384sq_M64"):
+        # 8-bit channel-wise codes under bf16 at 16 / 64 rows: the mid-batch kernel (one layer, a few launches)
+        M, N, K = (16 if name.endswith("M16") else 64), 16384, 16384
+        W_q = torch.randint(0, 256, (N, K), dtype=torch.uint8, device=device)
+        sc = (torch.randn((N, 1), device=device) * 0.01).abs().clamp_(min=1e-4).to(torch.bfloat16)
+        zr = (torch.rand((N, 1), device=device) * 64 + 96).to(torch.bfloat16)
+        layer = helper.A16Wn(device=device, post_scale=True).from_weights(W_q, sc, zr, 8, K)
+        del W_q
+        xq, sx = torch.randn((M, K), device=device).to(torch.bfloat16), None
+        peak = 2500.0
     else:
         sys.exit(f"bench.py: unknown --point {name}")
     y = torch.empty((M, N), dtype=torch.float16 if name == "gemm_a16w4_gs128_fp16" else torch.bfloat16, device=device)
