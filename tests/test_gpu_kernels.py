@@ -902,6 +902,28 @@ def test_a8w4_hqq_int_dynamic_fp8_activations(device, group_size):
 
 
 @pytest.mark.gpu
+def test_a8w2_hqq_int_dynamic_groups_of_32_widened_onto_the_mid_batch_kernel(device):
+    """fp8 activations quantised per token x 2-bit codes in groups of 32 (A8W2_HQQ_INT_dynamic): the activations are
+    widened to fp16 in the workspace and the packed-code kernel that takes groups of 32 runs on them, the mid-batch
+    one at every row count, per-token scales in its epilogue or split-K finishing launch."""
+    N, K = 520, 2048
+    W_q, scales, zeros = gen_int_case(N, K, 2, 32, torch.float16, seed=77)
+    layer = helper.A8W2_HQQ_INT_dynamic(device=device).from_weights(W_q, scales, zeros)
+    assert layer.scaled_activations and layer.input_dtype == DType.FP8 and layer.group_size == 32
+    m = layer.get_meta_args()
+    for M in (1, 7, 40, 100):
+        x = gen_x(M, K, torch.float16, seed=M).to(device)
+        xq, sx = gemlite_amd.scale_activations_per_token(x, torch.float8_e4m3fn)
+        out = torch.empty(M, N, dtype=gemlite_amd.DTYPE_TO_TORCH[m[6]], device=device)
+        a = _ext.build_matmul_args(xq, layer.W_q, layer.scales, layer.zeros, sx, out, W_nbits=m[1], group_size=m[2],
+                                   unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                   acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                   data_contiguous=m[11])
+        assert _ext.matmul_family(a) == "WN_MID", (M, _ext.matmul_family(a))
+        check_layer(layer, x, torch.bfloat16)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("K", [384, 1024])
 def test_a8w8_mxfp8_weights_per_token_activations(device, K):
     """MXFP8 weights x fp8 activations quantised per token, scale applied after the K sum

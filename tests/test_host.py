@@ -316,6 +316,49 @@ def _family(layer, M, x_dtype, scales_x=None, x=None):
     return _ext.matmul_family(a)
 
 
+def test_packed_layers_without_a_tiled_gemm_take_the_mid_batch_kernel():
+    # host logic only.  Groups of 32 and 1-bit codes have no tiled GEMM (and 2-bit gs 32 / 1-bit gs 32, 64 no streaming
+    # kernel either): which family takes them at each row count, and that the preferences only switch between kernels
+    # that accept the call.
+    g = torch.Generator().manual_seed(0)
+    N, K = 512, 1024
+    Ms = (1, 4, 16, 17, 64, 65, 300)
+
+    def layer(nbits, gs, dt=DType.BF16, tdt=torch.bfloat16):
+        W_q = torch.randint(0, 2 ** nbits, (N, K), generator=g).to(torch.uint8)
+        return GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q, torch.rand(N * K // gs, 1).to(tdt), torch.rand(N * K // gs, 1).to(tdt))
+
+    assert [_family(layer(2, 32), M, torch.bfloat16) for M in Ms] == ["WN_MID"] * 7
+    assert [_family(layer(1, 64), M, torch.bfloat16) for M in Ms] == ["GENERIC"] + ["WN_MID"] * 6   # one row: the K-split vector kernel
+    assert [_family(layer(1, 32), M, torch.bfloat16) for M in Ms] == ["GENERIC"] + ["WN_MID"] * 6
+    # 4- and 8-bit codes in groups of 32, 1-bit codes in groups of 128: the GEMV (row chunks) up to 64 rows on a small layer
+    for l in (layer(4, 32), layer(8, 32), layer(1, 128)):
+        assert [_family(l, M, torch.bfloat16) for M in Ms] == ["GEMV_PACKED"] * 5 + ["WN_MID"] * 2
+    # groups of 16 stay with the generic kernels
+    assert [_family(layer(4, 16), M, torch.bfloat16) for M in (1, 64)] == ["GENERIC"] * 2
+    # a preference for the mid-batch kernel is honoured where it is eligible (any row count) and ignored elsewhere
+    l4 = layer(4, 128, DType.FP16, torch.float16)
+    m = l4.get_meta_args()
+    for M, tile, fam in ((1, -4, "WN_MID"), (16, -4, "WN_MID"), (300, -4, "WN_MID"), (16, 2008, "WN_MID"), (16, -1, "GEMV_PACKED"),
+                         (300, -1, "GEMM_WN")):
+        a = _ext.build_matmul_args(torch.zeros(M, K, dtype=torch.float16), l4.W_q, l4.scales, l4.zeros, None,
+                                   torch.zeros(M, N, dtype=torch.float16), W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+                                   elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
+                                   channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11], tile_config=tile)
+        assert _ext.matmul_family(a) == fam, (M, tile, _ext.matmul_family(a))
+    lg = layer(4, 16)
+    mg = lg.get_meta_args()
+    a = _ext.build_matmul_args(torch.zeros(8, K, dtype=torch.bfloat16), lg.W_q, lg.scales, lg.zeros, None,
+                               torch.zeros(8, N, dtype=torch.bfloat16), W_nbits=mg[1], group_size=mg[2], unpack_mask=mg[3],
+                               elements_per_sample=mg[4], input_dtype=mg[5], output_dtype=mg[6], acc_dtype=mg[7], meta_dtype=mg[8],
+                               channel_scale_mode=mg[9], W_group_mode=mg[10], data_contiguous=mg[11], tile_config=-4)
+    assert _ext.matmul_family(a) == "GENERIC"
+    # unquantised layers: vector kernels for decode, the MFMA GEMM from 9 rows
+    W = torch.randn(N, K).to(torch.float16)
+    l16 = GemLiteLinear(16, None, K, N, DType.FP16, DType.FP16).pack(W, None, None)
+    assert [_family(l16, M, torch.float16) for M in (1, 8, 9, 64, 4096)] == ["GENERIC"] * 2 + ["GEMM_16BIT"] * 3
+
+
 def test_benchmark_configurations_take_a_tuned_kernel_family():
     # host logic only: which family gla_matmul would launch (the layout-agnostic kernel is correct but slow,
     # so none of the benchmark configurations may fall to it)
