@@ -246,8 +246,9 @@ int gla_matmul(const gla_matmul_args* args, void* stream);
  * library's code object carries (each GPU the library runs on holds its own copy until the process
  * ends).  The call allocates and frees nothing.  A problem whose gla_matmul_workspace_bytes()
  * exceeds GLA_STATIC_SCRATCH_BYTES is refused with GLA_ERR_WORKSPACE_TOO_SMALL.  The first call on
- * a device that needs scratch looks the array's address up and clears its ticket counters with a
- * small kernel on `stream`.  All calls on one GPU share the array: calls that may overlap in time
+ * a device that needs scratch looks the array's address up; nothing is cleared (the array is zero
+ * when the code object is loaded, and every kernel leaves the counters and slots it used at zero
+ * again), so that first call may itself be recorded into a graph.  All calls on one GPU share the array: calls that may overlap in time
  * on one GPU (two streams, two graphs replayed concurrently) race and must use gla_matmul with
  * workspaces of their own. */
 #define GLA_STATIC_SCRATCH_BYTES (72u << 20)
