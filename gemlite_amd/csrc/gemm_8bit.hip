@@ -44,7 +44,9 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6, kMX84 = 7, kMX84T = 8, kH16 = 9, kB16 = 10 };
+enum Mode { kFP8 = 0, kINT8 = 1, kMXFP4 = 2, kMXFP8 = 3, kMXFP8T = 4, kBQF8 = 5, kBQI8 = 6, kMX84 = 7, kMX84T = 8, kH16 = 9, kB16 = 10, kINT8R = 11 };
+// kINT8R: int8 x int8 whose K is not a multiple of 64 (a K-step past the end multiplies zeroed operands: a select per
+// operand register and K-step, 33 vector instructions per stage in front of the MFMAs that the other layers do without)
 // kH16 / kB16: fp16 x fp16 / bf16 x bf16 (unquantised layers, W_nbits = 16): the byte geometry of the int8 mode (two
 // K-steps of 32 bytes per stage, here 16 values each) on v_mfma_f32_32x32x16; built in a translation unit of its own
 // kMXFP8T: MXFP8 weights whose activations carry no block scales (their per-token scale is applied in the
@@ -101,7 +103,7 @@ __device__ __forceinline__ void wait_vmcnt8() {
 constexpr int kRing8 = 4;  // LDS ring of pipeline stages, all of them in flight
 constexpr int slot_bytes8(int mode, int bm) {
     const bool w4 = mode == kMX84 || mode == kMX84T;
-    return bm * kRowB8 + kBN * (w4 ? 32 : kRowB8) + (mode == kFP8 || mode == kINT8 || mode == kH16 || mode == kB16 ? 0 : (bm + kBN) * 4);
+    return bm * kRowB8 + kBN * (w4 ? 32 : kRowB8) + (mode == kFP8 || mode == kINT8 || mode == kINT8R || mode == kH16 || mode == kB16 ? 0 : (bm + kBN) * 4);
 }
 
 // WN = wave columns (4): 8 waves, wave tile (BM/2) x 64, up to 128 accumulator registers per lane.
@@ -123,7 +125,8 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     constexpr bool TOKEN = MODE == kMXFP8T || MODE == kMX84T;  // no activation block scales
     constexpr bool BQ = MODE == kBQF8 || MODE == kBQI8;     // fp32 block scales, applied by the vector unit
     constexpr bool F8 = MODE == kFP8 || MODE == kBQF8;      // plain fp8 operands, one 64-byte K-step per stage
-    constexpr bool I8 = MODE == kINT8 || MODE == kBQI8;
+    constexpr bool I8 = MODE == kINT8 || MODE == kINT8R || MODE == kBQI8;
+    constexpr bool RAGGED = MODE == kINT8R;                 // K ends inside a stage
     constexpr bool H16 = MODE == kH16 || MODE == kB16;      // 16-bit float operands, two K-steps of 16 values per stage
     constexpr bool MX = MODE == kMXFP4 || M8 || BQ;         // block scales ride along with every stage
     // MXFP8 and the fp32 block scales: a 32-bit scale word of a row covers 128 values = two stages; MXFP4: one stage
@@ -387,7 +390,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
         } else {
             // a K-step past the end of a ragged K multiplies zeros (no branch: the accumulators
             // must not live across control flow)
-            const bool valid = !(I8 || H16) || s2 * 32 < limit;
+            const bool valid = !RAGGED || s2 * 32 < limit;
             u32x4 af = fa[B][i].c[s2];
             if (!valid) af = u32x4{0, 0, 0, 0};
             const u32x4 bf = fb[B][j].c[s2];
@@ -523,7 +526,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void gemm_8bit_kernel(Gemm8Args 
     // 4g .. 4g+3, the four adjacent output columns 8g + 4kb .. + 3, which leave in one store.
     const int n_wave = n0 + wn * WNC + 4 * kb;
     if (p.S > 1) {  // partial tile, raw 32-bit accumulators; the reduction kernel finishes
-        typedef typename std::conditional<MODE == kINT8, int32_t, float>::type raw_t;  // BQ: the scaled fp32 sums
+        typedef typename std::conditional<MODE == kINT8 || MODE == kINT8R, int32_t, float>::type raw_t;  // BQ: the scaled fp32 sums
         typedef raw_t raw4_t __attribute__((ext_vector_type(4)));
         raw_t* part = (raw_t*)p.partials + (size_t)blockIdx.y * p.M * p.N;
         const bool wide = (p.N & 3) == 0;
@@ -697,7 +700,7 @@ int launch_bm(const Gemm8Args& a, hipStream_t stream) {
         const int64_t items = (int64_t)a.M * a.N;
         Gemm8Args f = a;
         if (MODE == kMXFP4 || MODE == kBQF8 || MODE == kBQI8) f.csm = 0;  // block scales were applied in the main kernel
-        hipLaunchKernelGGL((splitk_finish8_kernel<MODE == kINT8>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+        hipLaunchKernelGGL((splitk_finish8_kernel<MODE == kINT8 || MODE == kINT8R>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
                            stream, f);
         rc = check_hip(hipGetLastError(), "gemm_8bit split-K reduction launch");
     }
@@ -812,7 +815,7 @@ int launch_gemm_8bit(const gla_matmul_args& p, hipStream_t stream) {
     const Plan8 g = plan8(p.M, p.N, a.Kb, p.tile_config);
     const int rc = attach_plan(p, g, a);
     if (rc != GLA_OK) return rc;
-    if (p.input_dtype == GLA_DT_INT8) return launch_mode<kINT8>(a, g.bm, stream);
+    if (p.input_dtype == GLA_DT_INT8) return a.Kb % kRowB8 ? launch_mode<kINT8R>(a, g.bm, stream) : launch_mode<kINT8>(a, g.bm, stream);
     return launch_mode<kFP8>(a, g.bm, stream);
 }
 
