@@ -1031,9 +1031,18 @@ void launch_one(const GemvArgs& a, const Geometry& g, hipStream_t stream) {
                 hipLaunchKernelGGL((gemv_direct_kernel<BITS, BF16, RT, 4, true>), grid, dim3(256), g.smem, stream, a);
                 return;
             }
-            if constexpr (RT <= 4 && (BITS == 4 || BITS == 8)) {
+            if constexpr (BITS == 4 || BITS == 8) {
                 if (g.FL == 4) {  // groups of 128 (and channel-wise 8-bit codes): folds at fixed places of the batch
                     launch_direct<BITS, BF16, RT, 4>(a, g, grid, stream);
+                    return;
+                }
+            }
+            if constexpr (BITS == 2) {
+                // 2-bit codes in groups of 64: a fold after every iteration, so that the group sums start from the MFMA's
+                // zero operand instead of being cleared (16384^2 at 16 rows 36.0-37.0 -> 32.7-33.5 us, 8192^2 17.5 -> 16.8).
+                // (The same in the staged kernel, which serves up to 4 rows: 16384^2 at one row 26.7 -> 35 us; not kept.)
+                if (g.FL == 1) {
+                    launch_direct<BITS, BF16, RT, 1>(a, g, grid, stream);
                     return;
                 }
             }
