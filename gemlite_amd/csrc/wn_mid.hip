@@ -445,10 +445,12 @@ MidPlan mid_plan(const gla_matmul_args& p) {
     const int gs = grouped ? p.group_size : p.K;
     g.gps = gs < stage_k(p.W_nbits) ? stage_k(p.W_nbits) / gs : 1;
     // a lane's word of 2-bit codes is 16 K-values, of 1-bit codes 32: below groups of 64 (128) the group follows
-    // from the lane
-    g.lane_groups = (p.W_nbits == 2 && g.gps == 4) || (p.W_nbits == 1 && g.gps > 1);
+    // from the lane.  So it does in groups of 16, two of which share every K-step (a lane's eight codes of a K-step lie
+    // in one group): metadata per K-step (4- and 8-bit codes) or per word (2-bit codes).
+    const bool g16 = gs == 16;
+    g.lane_groups = g16 || (p.W_nbits == 2 && g.gps == 4) || (p.W_nbits == 1 && g.gps > 1);
     g.gt = g.gps;
-    if (g.lane_groups) g.gps = p.W_nbits == 2 ? 2 : 1;
+    if (g.lane_groups) g.gps = p.W_nbits == 2 ? 2 : (g16 ? (p.W_nbits == 4 ? 4 : 2) : 1);
     // one workgroup per CU; a split is at least 4 stages long
     const int blocks = ceil_div(p.N, 64 * g.nw);
     const int chunks = ceil_div(p.M, 64);
@@ -526,8 +528,9 @@ bool wn_mid_eligible(const gla_matmul_args& p) {
     const bool grouped = uses_scales || zeros_tensor;
     const int gs = grouped ? p.group_size : p.K;
     if (gs <= 0 || p.K % gs != 0) return false;
-    // a group is whole stages, or a stage is two groups, or (2- and 4-bit codes) four groups of one K-step each
-    if (!(gs % ks == 0 || 2 * gs == ks || (4 * gs == ks && p.W_nbits != 8))) return false;
+    // a group is whole stages, or a stage is a whole number of groups of at least 16 (1-bit codes: 32, a pair of
+    // the codes that share a register on bf16 lies 16 K-values apart)
+    if (!(gs % ks == 0 || (ks % gs == 0 && gs >= (p.W_nbits == 1 ? 32 : 16)))) return false;
     if ((int64_t)(p.K / p.elements_per_sample) * p.w_stride_k >= (1ll << 31)) return false;
     // metadata is read as four adjacent 16-bit values per lane
     const bool one_group = gs == p.K;
@@ -544,8 +547,8 @@ int64_t wn_mid_workspace_bytes(const gla_matmul_args& p) {
 
 int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream) {
     if (!wn_mid_eligible(p)) {
-        set_error("wn_mid: fp16 / bf16 activations on 2-, 4- or 8-bit packed codes, groups of whole 128-K stages (8-bit: 64), "
-                  "half a stage or (2-, 4-bit) a quarter");
+        set_error("wn_mid: fp16 / bf16 activations on 1-, 2-, 4- or 8-bit packed codes, groups of whole 128-K stages (8-bit: 64) "
+                  "or of 16 / 32 / 64 (1-bit: 32 / 64)");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
     const MidPlan g = mid_plan(p);
@@ -564,8 +567,15 @@ int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream) {
     const int ks = stage_k(p.W_nbits);
     a.spg = gs >= ks ? gs / ks : 1;
     a.lane_g = g.lane_groups; a.gt = g.gt;
-    a.gmul = p.W_nbits == 2 ? 2 : 0;                       // 2-bit: metadata slot gi is the 64-K load, two groups each
-    a.kbs = (p.W_nbits == 1 && g.gt == 4) ? 0 : 1;         // 1-bit gs 32: a group per K-quarter; otherwise per pair of them
+    if (gs == 16) {
+        // 2-bit: metadata slot gi is the 64-K load, a group per lane quarter; 4- and 8-bit: slot gi is the K-step, a
+        // group per pair of lane quarters
+        a.gmul = p.W_nbits == 2 ? 4 : 2;
+        a.kbs = p.W_nbits == 2 ? 0 : 1;
+    } else {
+        a.gmul = p.W_nbits == 2 ? 2 : 0;                   // 2-bit: metadata slot gi is the 64-K load, two groups each
+        a.kbs = (p.W_nbits == 1 && g.gt == 4) ? 0 : 1;     // 1-bit gs 32: a group per K-quarter; otherwise per pair of them
+    }
     a.spg_shift = -1;
     for (int s = 0; s < 31; ++s)
         if ((1 << s) == a.spg) a.spg_shift = s;

@@ -249,11 +249,11 @@ def test_a16wn_bits_and_groups(device, nbits, gs, dtype):
         check_layer(layer, gen_x(M, K, dtype, seed=M).to(device), dtype)
 
 
-@pytest.mark.parametrize("nbits,gs", [(1, 32), (1, 64), (1, 128), (1, 256), (2, 32), (4, 32), (8, 32), (2, 64), (2, 128), (4, 64), (4, 128), (4, 256), (8, 64), (8, 128), (4, None), (8, None)])
+@pytest.mark.parametrize("nbits,gs", [(2, 16), (4, 16), (8, 16), (1, 32), (1, 64), (1, 128), (1, 256), (2, 32), (4, 32), (8, 32), (2, 64), (2, 128), (4, 64), (4, 128), (4, 256), (8, 64), (8, 128), (4, None), (8, None)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_packed_codes_at_17_to_64_rows(device, nbits, gs, dtype):
     """The mid-batch kernel (weights from registers into the MFMA, activations shared through an LDS ring): every code
-    width and activation type, groups of a quarter of a stage, half a stage, one stage and several stages, channel-wise
+    width and activation type, groups of 16, of a quarter of a stage, half a stage, one stage and several stages, channel-wise
     scales (gs None), 1..4 row tiles with ragged last tiles, batches above 64 rows as row chunks, N that ends inside a wave's 64 columns and inside a workgroup's 512, K of
     few and many stages (with and without a K split, splits of unequal length), a bias."""
     dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
@@ -290,6 +290,8 @@ def test_packed_codes_in_short_groups(device, nbits, gs, dtype):
     between waves, rows 1 / 2 / 4 per lane and a ragged last block; scale-only, shift-only and scalar-zero modes."""
     dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
     for N, K in ((200, 320), (1000, 2112)):
+        if nbits == 8:
+            K += 32  # not a whole number of the mid-batch kernel's 64-K stages either
         W_q, scales, zeros = gen_int_case(N, K, nbits, gs, dtype, seed=nbits * 100 + gs)
         layer = GemLiteLinear(nbits, gs, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device))
         x1 = gen_x(1, K, dtype, seed=1).to(device)
@@ -313,8 +315,7 @@ def test_packed_codes_in_short_groups(device, nbits, gs, dtype):
 
 @pytest.mark.parametrize("nbits,gs", [(1, 32), (2, 16)])
 def test_short_group_codes_at_prefill_size(device, nbits, gs):
-    """1024 rows on packings no matrix-core kernel takes (the generic family's packed-word kernel walks the row
-    blocks, four rows at a time)."""
+    """1024 rows on packings the tiled GEMM does not take: sixteen row chunks of the mid-batch kernel."""
     N, K, M = 256, 1024, 1024
     W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.float16, seed=nbits + gs)
     layer = GemLiteLinear(nbits, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))

@@ -334,8 +334,10 @@ def test_packed_layers_without_a_tiled_gemm_take_the_mid_batch_kernel():
     # 4- and 8-bit codes in groups of 32, 1-bit codes in groups of 128: the GEMV (row chunks) up to 64 rows on a small layer
     for l in (layer(4, 32), layer(8, 32), layer(1, 128)):
         assert [_family(l, M, torch.bfloat16) for M in Ms] == ["GEMV_PACKED"] * 5 + ["WN_MID"] * 2
-    # groups of 16 stay with the generic kernels
-    assert [_family(layer(4, 16), M, torch.bfloat16) for M in (1, 64)] == ["GENERIC"] * 2
+    # groups of 16: the mid-batch kernel at any row count (2-, 4-, 8-bit codes); 1-bit codes stay with the generic kernels
+    for l in (layer(2, 16), layer(4, 16), layer(8, 16)):
+        assert [_family(l, M, torch.bfloat16) for M in Ms] == ["WN_MID"] * 7
+    assert [_family(layer(1, 16), M, torch.bfloat16) for M in (1, 64)] == ["GENERIC"] * 2
     # a preference for the mid-batch kernel is honoured where it is eligible (any row count) and ignored elsewhere
     l4 = layer(4, 128, DType.FP16, torch.float16)
     m = l4.get_meta_args()
@@ -346,7 +348,7 @@ def test_packed_layers_without_a_tiled_gemm_take_the_mid_batch_kernel():
                                    elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
                                    channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11], tile_config=tile)
         assert _ext.matmul_family(a) == fam, (M, tile, _ext.matmul_family(a))
-    lg = layer(4, 16)
+    lg = layer(1, 16)
     mg = lg.get_meta_args()
     a = _ext.build_matmul_args(torch.zeros(8, K, dtype=torch.bfloat16), lg.W_q, lg.scales, lg.zeros, None,
                                torch.zeros(8, N, dtype=torch.bfloat16), W_nbits=mg[1], group_size=mg[2], unpack_mask=mg[3],
