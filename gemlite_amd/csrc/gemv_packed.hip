@@ -904,10 +904,14 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true, i
     // one wave, one batch: 4 quarters x kBatch loads of word rows
     g.unit = 4 * kBatch;
     const int units = ceil_div(g.R, g.unit);  // wave-batches along K
-    // 2-bit codes: direct only for the 16-row tile (up to 4 rows the staged kernel measured a little faster)
-    const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8 || (p.W_nbits == 2 && g.RT == 16));
+    // 2-bit codes: direct for the 16-row tile, and up to 4 rows on layers of up to 64 M weights, where a launch is short
+    // and the staged kernel's fill of its LDS tables stands in front of the stream (bf16, groups of 64, one row: 8192^2
+    // 10.5 -> 8.9 us, 4096^2 7.2 -> 5.8, at 4 rows 12.6 -> 9.7 and 8.5 -> 6.7; 16384^2 27 -> 32, so larger layers stay
+    // staged).  Its 2-bit instantiations fit the register file at 4 and 8 waves only.
+    const bool w2_short = p.W_nbits == 2 && g.RT <= 4 && (int64_t)p.N * p.K <= ((int64_t)1 << 26);
+    const bool can_direct = allow_direct && (p.W_nbits == 4 || p.W_nbits == 8 || (p.W_nbits == 2 && g.RT == 16) || w2_short);
     // the cross-wave buffer is [waves][RT][64] floats; the staged 16-row kernel runs 4 waves
-    int max_waves = (g.RT == 16) ? (can_direct ? 16 : 4) : 16;
+    int max_waves = (g.RT == 16) ? (can_direct ? 16 : 4) : (w2_short && can_direct ? 8 : 16);
     // Large layers: once 8-wave workgroups still give every CU two or more, they stream better than
     // 16-wave ones (measured on 16384^2: 4-bit 27.9 against 32.2 us, 8-bit 44 against 53 us).
     if (max_waves > 8 && (int64_t)g.tiles * ceil_div(p.M, g.RT) * ceil_div(units, 8) >= 512) max_waves = 8;
@@ -918,7 +922,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true, i
     if (p.tile_config >= 1000) {
         waves = p.tile_config / 1000;
         nb = p.tile_config % 1000;
-        const bool any_count = can_direct && nb == 1 && waves >= (g.RT <= 4 ? 4 : 8) && waves <= 16;
+        const bool any_count = can_direct && !w2_short && nb == 1 && waves >= (g.RT <= 4 ? 4 : 8) && waves <= 16;
         if (!(waves == 4 || waves == 8 || waves == 16 || any_count) || waves > max_waves || nb < 1) return false;
     } else {
         // Slabs along K: enough workgroups to cover the CUs, and few enough wave-batches per
@@ -933,7 +937,7 @@ bool geometry(const gla_matmul_args& p, Geometry& g, bool allow_direct = true, i
         int per_wg = ceil_div(units, want_s);  // wave-batches per workgroup
         if (can_direct && per_wg <= max_waves && (g.RT <= 4 || per_wg > 8)) {
             // one batch per wave and exactly as many waves as batches: equal slabs
-            waves = per_wg < 4 ? 4 : per_wg;
+            waves = per_wg < 4 ? 4 : (w2_short && per_wg > 4 ? 8 : per_wg);
             nb = 1;
         } else {
             waves = per_wg <= 4 ? 4 : (per_wg <= 8 && max_waves >= 8 ? 8 : max_waves);
