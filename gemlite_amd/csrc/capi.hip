@@ -256,6 +256,22 @@ Family choose(const gla_matmul_args& p, int type) {
         // matrix cores (16384^2 MXFP4, 8 rows: 48 against 62 us of the tiled GEMM); above that the tiled GEMM
         if (want_stream) return F_MX_STREAM;
         if (want_matrix && gemm_kbytes_mx_eligible(p)) return F_GEMM_KBYTES_MX;
+        // ... unless the activations go as sums of e4m3 terms (two per bf16 value, three per fp16 value) into the skinny
+        // kernel of the narrow formats, which converts no weight: a small launch in front, so it pays on large layers
+        // while the terms of the batch fit one 16-row tile (bf16: 8 rows, fp16: 5), and with two tiles on long-K layers.
+        // Measured against the kernel below, 8 rows of bf16: MXFP4 16384^2 48.9 -> 40.8 us, 8192 x 28672 48.7 -> 39.4,
+        // 4096 x 14336 17.7 -> 13.2, 14336 x 4096 16.2 -> 14.1, 8192^2 16.5 -> 15.5, 4096^2 6.8 -> 8.6 (stays); MXFP8 8192 x
+        // 28672 85.5 -> 73.5, 4096 x 14336 27.1 -> 23.2, 8192^2 27.2 -> 25.3, 16384^2 78.3 -> 78.7 and 14336 x 4096 22.1 -> 23.0
+        // (stay); 16 rows of bf16: 4096 x 14336 20.7 -> 17.6, 8192 x 28672 54.7 -> 49.2, 16384^2 51.6 -> 57.9 (stays).
+        // GLA_TILE_PREFER_MID asks for it wherever it is eligible.
+        if (p.M > 2 && p.M <= 16 && p.tile_config < 1000 && kring_eligible(p)) {
+            const int terms = p.input_dtype == GLA_DT_MXBF16 ? 2 : 3;
+            const bool one_tile = terms * p.M <= 16, w4 = p.elements_per_sample == 2;
+            const bool long_k = p.K >= 14336 && p.N <= 8192;
+            const bool pays = one_tile ? (w4 ? (int64_t)p.N * p.K >= 50000000 : (p.K >= 8192 && p.N <= 8192))
+                                       : (terms == 2 && long_k);
+            if (p.tile_config == GLA_TILE_PREFER_MID || pays) return F_K_SKINNY;
+        }
         if (p.M > 2 && p.M <= 16 && p.tile_config < 1000 && mx_skinny_eligible(p)) return F_MX_SKINNY;
         return gemm_kbytes_mx_eligible(p) ? F_GEMM_KBYTES_MX : F_MX_STREAM;
     }
@@ -347,6 +363,7 @@ int64_t family_workspace(Family f, const gla_matmul_args& a) {
         case F_GEMM_MXFP8: return gemm_mxfp8_workspace_bytes(a);
         case F_GEMM_BLOCKQ: return gemm_blockq_workspace_bytes(a);
         case F_GEMM_KBYTES_MX: return gemm_kbytes_mx_workspace_bytes(a);
+        case F_K_SKINNY: return kring_workspace_bytes(a);
         default: return 0;
     }
 }

@@ -143,6 +143,7 @@ int launch_wn_mid(const gla_matmul_args& p, hipStream_t stream);
 
 // ---- MXFP4 x MXFP4, fp8 x fp8, int8 x int8 at 3..32 rows: operands copied to per-wave LDS rings by lines, MFMA (kring.hip)
 bool kring_eligible(const gla_matmul_args& p);
+int64_t kring_workspace_bytes(const gla_matmul_args& p);  // 16-bit activations on MX weights: their e4m3 terms
 int launch_kring(const gla_matmul_args& p, hipStream_t stream);
 bool gemm_kbytes_mx_eligible(const gla_matmul_args& p);
 int launch_gemm_kbytes_mx(const gla_matmul_args& p, hipStream_t stream);

@@ -8,6 +8,14 @@
 //                   same on the activations or one fp32 scale per token in the epilogue
 //   fp8 x MXFP4      the mixed form of the instruction (A e2m1, B e4m3): 256 K-values a turn, the activations of a
 //                   turn travelling as two tiles (4096^2 at 8 rows 5.2 us against 16.2 tiled, 16384^2 35.0 against 54.9)
+//   16-bit x MXFP8 / MXFP4 (weight-only layers)
+//                   the last two modes on activations written as a sum of e4m3 terms: a bf16 value is 8 significant
+//                   bits = two e4m3 values of 4 (an fp16 value three), each term with its own e8m0 scale per 32-block, 16
+//                   apart.  A small launch writes the terms as rows of their own (row T j + t of a 16-row tile = term
+//                   t of the tile's j-th activation row), the matmul multiplies them like any fp8 rows - the products
+//                   of the scaled MFMA are exact, so the sum of a row's terms is the product with the 16-bit value -
+//                   and the epilogue adds the T accumulator columns of a row.  No weight is converted.  What the terms
+//                   cannot hold is smaller than 2^-20 (fp16: 2^-24) of the block's largest magnitude.
 //
 // The decode-batch path of dynamically quantised A8W8 and A4W4 layers, between the streaming kernels (dot products
 // on the vector unit, 1-2 rows) and the tiled GEMMs (64-row tiles, K split over workgroups, a finishing launch and,
@@ -56,6 +64,7 @@ struct KRingArgs {
     const void* scales_x;     // per-token scales [M] (bit 1)
     void* out;
     int M, N, turns;          // turns = K / (K-values per turn)
+    int fold, Mo;             // fold T > 1: activation row T j + t of a tile is term t of output row (16 / T) tile + j; Mo output rows
     int64_t xsm, wsn, bsxm, bswn, sxm, osm;   // bytes (sxm, osm: elements)
     int csm, meta_dt, sx_dt, out_dt;
     const void* bias;
@@ -260,11 +269,25 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
             if (t || xt) __syncthreads();
             red[wave][lane] = acc[t][xt];
             __syncthreads();
-            const int m = 16 * xt + r16;
-            if (wave != 0 || m >= a.M) continue;
+            if (wave != 0) continue;
             acc_t D = {0, 0, 0, 0};
 #pragma unroll
             for (int w = 0; w < NW; ++w) D += red[w][lane];
+            int m = 16 * xt + r16;
+            if constexpr (MODE == R_MX88 || MODE == R_MX84) {
+                if (a.fold > 1) {
+                    // the terms of output row j are the accumulator columns T j .. T j + T - 1 of the same lane group
+                    const int T = a.fold, per_tile = 16 / T;
+                    const int src = 16 * kq + (r16 < per_tile ? T * r16 : 0);
+                    acc_t S = {0, 0, 0, 0};
+                    for (int t = 0; t < T; ++t)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) S[e] += __shfl(D[e], src + t, 64);
+                    D = S;
+                    m = r16 < per_tile ? per_tile * xt + r16 : a.Mo;
+                }
+            }
+            if (m >= a.Mo) continue;
             const float sa = row_scale ? load_as_float(a.scales_x, a.sx_dt, (int64_t)m * a.sxm) : 1.0f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -283,6 +306,79 @@ __global__ __launch_bounds__(NW * 64) void kring_kernel(KRingArgs a) {
                 store_from_float(a.out, a.out_dt, o, v);
             }
         }
+    }
+}
+
+// 16-bit activation rows as sums of T e4m3 terms with e8m0 block scales, in the row order the fold of the epilogue
+// expects.  One thread per (tile, row slot j, 32-block): term t = RNE_e4m3(r / s_t), r <- r - term s_t (exact), s_t =
+// 2^(floor(log2 amax) - 7 - 4 t), so the block's largest value lands in [128, 256).  Slots past M and the rows a tile
+// cannot use (16 - T (16 / T)) are written as zeros with the identity scale: the matmul reads all of them.
+template <bool BF16, int T>
+__global__ __launch_bounds__(256) void split_e4m3_kernel(const uint16_t* __restrict__ x, int64_t xsm, int M, int K, int tiles,
+                                                         uint8_t* __restrict__ y, uint8_t* __restrict__ sy) {
+    constexpr int PER = 16 / T, SLOTS = PER + (16 % T ? 1 : 0);
+    const int groups = K / 32;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (int64_t)tiles * SLOTS * groups) return;
+    const int g = (int)(id % groups), j = (int)((id / groups) % SLOTS), tile = (int)(id / groups / SLOTS);
+    const int m = tile * PER + j;
+    uint8_t* yrow = y + ((int64_t)tile * 16 + T * j) * K + g * 32;
+    uint8_t* srow = sy + ((int64_t)tile * 16 + T * j) * groups + g;
+    if (j >= PER || m >= M) {
+        const int rows = j >= PER ? 16 % T : T;
+        for (int t = 0; t < rows; ++t) {
+            *(uint4*)(yrow + (int64_t)t * K) = make_uint4(0, 0, 0, 0);
+            *(uint4*)(yrow + (int64_t)t * K + 16) = make_uint4(0, 0, 0, 0);
+            srow[(int64_t)t * groups] = 127;
+        }
+        return;
+    }
+    float r[32];
+    const uint4* src = (const uint4*)(x + (int64_t)m * xsm + g * 32);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint4 v = src[i];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if constexpr (BF16) {
+                r[8 * i + 2 * k] = __builtin_bit_cast(float, w[k] << 16);
+                r[8 * i + 2 * k + 1] = __builtin_bit_cast(float, w[k] & 0xffff0000u);
+            } else {
+                r[8 * i + 2 * k] = half_bits_to_float((uint16_t)(w[k] & 0xffffu));
+                r[8 * i + 2 * k + 1] = half_bits_to_float((uint16_t)(w[k] >> 16));
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(r[i]));
+    // floor(log2 amax) from the exponent field (a block of zeros, or of values below 2^-126, keeps the smallest scale)
+    const int e = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xffu) - 127;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        int se = e + 120 - 4 * t;  // biased exponent of s_t
+        se = se < 0 ? 0 : (se > 254 ? 254 : se);
+        const float s = __builtin_ldexpf(1.0f, se - 127);
+        uint32_t out[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float q[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) q[k] = __builtin_ldexpf(r[4 * i + k], 127 - se);  // below 256 in magnitude
+            const uint32_t w = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false) & 0xffffu;
+            const uint32_t w2 = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], 0, false) & 0xffffu;
+            out[i] = w | (w2 << 16);
+            if (t + 1 < T) {
+                r[4 * i + 0] = __builtin_fmaf(-__builtin_amdgcn_cvt_f32_fp8((int)out[i], 0), s, r[4 * i + 0]);
+                r[4 * i + 1] = __builtin_fmaf(-__builtin_amdgcn_cvt_f32_fp8((int)out[i], 1), s, r[4 * i + 1]);
+                r[4 * i + 2] = __builtin_fmaf(-__builtin_amdgcn_cvt_f32_fp8((int)out[i], 2), s, r[4 * i + 2]);
+                r[4 * i + 3] = __builtin_fmaf(-__builtin_amdgcn_cvt_f32_fp8((int)out[i], 3), s, r[4 * i + 3]);
+            }
+        }
+        *(uint4*)(yrow + (int64_t)t * K) = make_uint4(out[0], out[1], out[2], out[3]);
+        *(uint4*)(yrow + (int64_t)t * K + 16) = make_uint4(out[4], out[5], out[6], out[7]);
+        srow[(int64_t)t * groups] = (uint8_t)se;
     }
 }
 
@@ -349,9 +445,82 @@ int ring_mode(const gla_matmul_args& p) {
     return -1;
 }
 
+// Weight-only MX layers: terms per 16-bit activation value (0: not such a call)
+int split_terms(const gla_matmul_args& p) {
+    return p.input_dtype == GLA_DT_MXBF16 ? 2 : (p.input_dtype == GLA_DT_MXFP16 ? 3 : 0);
+}
+
+struct SplitPlan {
+    int T, tiles;         // terms; 16-row tiles of fp8 rows
+    int64_t y_off, s_off, total;   // workspace offsets of the terms and their scale bytes, bytes in all
+};
+
+SplitPlan split_plan(const gla_matmul_args& p) {
+    SplitPlan s;
+    s.T = split_terms(p);
+    s.tiles = ceil_div(p.M, 16 / s.T);
+    s.y_off = kWsPrivateBytes;
+    s.s_off = s.y_off + (int64_t)s.tiles * 16 * p.K;
+    s.total = s.s_off + (int64_t)s.tiles * 16 * (p.K / 32);
+    return s;
+}
+
+bool split_eligible(const gla_matmul_args& p) {
+    const int T = split_terms(p);
+    if (T == 0 || p.M < 1 || p.M > 2 * (16 / T) || p.x_quant_from != 0) return false;
+    if (p.group_size != 32 || p.channel_scale_mode != GLA_CSM_NONE || p.scales == nullptr) return false;
+    const bool w4 = p.W_nbits == 4 && p.elements_per_sample == 2;
+    const bool w8 = p.W_nbits == 8 && p.elements_per_sample == 1;
+    if (!w4 && !w8) return false;
+    if (p.K % (w4 ? 256 : 128) != 0) return false;
+    if (p.meta_stride_g != 1 || p.meta_stride_n % 4 != 0 || ((uintptr_t)p.scales & 3)) return false;
+    if (p.x_stride_k != 1 || p.w_stride_k != 1 || p.out_stride_n != 1) return false;
+    if (p.x_stride_m % 8 != 0 || p.w_stride_n % 16 != 0 || ((uintptr_t)p.x & 15) || ((uintptr_t)p.w & 15)) return false;
+    switch (p.output_dtype) {
+        case GLA_DT_FP32: case GLA_DT_FP16: case GLA_DT_BF16: case GLA_DT_MXFP16: case GLA_DT_MXBF16: return true;
+        default: return false;
+    }
+}
+
+int launch_split(const gla_matmul_args& p, hipStream_t stream) {
+    const SplitPlan sp = split_plan(p);
+    if (p.workspace == nullptr || (int64_t)p.workspace_bytes < sp.total) {
+        set_error("kring: workspace of %lld bytes required (the activations' e4m3 terms go there), %llu given", (long long)sp.total,
+                  (unsigned long long)p.workspace_bytes);
+        return GLA_ERR_WORKSPACE_TOO_SMALL;
+    }
+    uint8_t* y = (uint8_t*)p.workspace + sp.y_off;
+    uint8_t* sy = (uint8_t*)p.workspace + sp.s_off;
+    const int slots = sp.T == 2 ? 8 : 6;
+    const int64_t items = (int64_t)sp.tiles * slots * (p.K / 32);
+    const dim3 grid((unsigned)((items + 255) / 256));
+    if (sp.T == 2)
+        hipLaunchKernelGGL((split_e4m3_kernel<true, 2>), grid, dim3(256), 0, stream, (const uint16_t*)p.x, p.x_stride_m, p.M, p.K, sp.tiles, y, sy);
+    else
+        hipLaunchKernelGGL((split_e4m3_kernel<false, 3>), grid, dim3(256), 0, stream, (const uint16_t*)p.x, p.x_stride_m, p.M, p.K, sp.tiles, y, sy);
+    int rc = check_hip(hipGetLastError(), "kring: activation split launch");
+    if (rc != GLA_OK) return rc;
+    const bool w4 = p.elements_per_sample == 2;
+    KRingArgs a;
+    a.x = y; a.w = (const uint8_t*)p.w; a.out = p.out;
+    a.M = sp.tiles * 16; a.N = p.N; a.Mo = p.M; a.fold = sp.T;
+    a.turns = p.K / (w4 ? 256 : 128);
+    a.xsm = p.K; a.wsn = p.w_stride_n; a.osm = p.out_stride_m;
+    a.bsx = sy; a.bsw = (const uint8_t*)p.scales;
+    a.bsxm = p.K / 32; a.bswn = p.meta_stride_n;
+    a.scales = nullptr; a.scales_x = nullptr; a.sxm = 0;
+    a.csm = GLA_CSM_MX; a.meta_dt = GLA_DT_UINT8; a.sx_dt = GLA_DT_UINT8;
+    a.out_dt = p.output_dtype == GLA_DT_MXFP16 ? GLA_DT_FP16 : (p.output_dtype == GLA_DT_MXBF16 ? GLA_DT_BF16 : p.output_dtype);
+    a.bias = p.bias; a.bias_dt = p.bias_dtype;
+    return w4 ? launch_mode_ring<R_MX84, true>(a, stream) : launch_mode_ring<R_MX88, true>(a, stream);
+}
+
 }  // namespace
 
+int64_t kring_workspace_bytes(const gla_matmul_args& p) { return split_terms(p) ? split_plan(p).total : 0; }
+
 bool kring_eligible(const gla_matmul_args& p) {
+    if (split_terms(p)) return split_eligible(p);
     const int mode = ring_mode(p);
     if (mode < 0 || p.x_quant_from != 0 || p.M < 1 || p.M > 32) return false;
     if (p.x_stride_k != 1 || p.w_stride_k != 1 || p.out_stride_n != 1) return false;
@@ -387,15 +556,16 @@ bool kring_eligible(const gla_matmul_args& p) {
 int launch_kring(const gla_matmul_args& p, hipStream_t stream) {
     if (!kring_eligible(p)) {
         set_error("kring: MXFP4 x MXFP4, fp8 x fp8, int8 x int8 or fp8 x MXFP8 / MXFP4 operands, K-contiguous with 16-byte "
-                  "aligned rows, up to 32 rows, K a multiple of 256 (MXFP4 weights) or 128");
+                  "aligned rows, up to 32 rows (bf16 / fp16 on MX weights: 16 / 10), K a multiple of 256 (MXFP4 weights) or 128");
         return GLA_ERR_UNSUPPORTED_MODE;
     }
+    if (split_terms(p)) return launch_split(p, stream);
     const int mode = ring_mode(p);
     const bool mx = mode == R_MX44 || mode == R_MX88 || mode == R_MX84;
     const bool xbs = mx && p.channel_scale_mode == GLA_CSM_MX;
     KRingArgs a;
     a.x = (const uint8_t*)p.x; a.w = (const uint8_t*)p.w; a.out = p.out;
-    a.M = p.M; a.N = p.N;
+    a.M = p.M; a.N = p.N; a.Mo = p.M; a.fold = 1;
     a.turns = p.K / ((mode == R_MX44 || mode == R_MX84) ? 256 : 128);
     a.xsm = p.x_stride_m; a.wsn = p.w_stride_n; a.osm = p.out_stride_m;
     a.bsx = xbs ? (const uint8_t*)p.scales_x : nullptr; a.bsw = mx ? (const uint8_t*)p.scales : nullptr;

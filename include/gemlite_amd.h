@@ -83,7 +83,10 @@ extern "C" {
 #define GLA_TILE_PREFER_STREAMING (-2)
 #define GLA_TILE_PREFER_MATRIX (-3)
 /* fp16 / bf16 activations on 2-, 4- or 8-bit packed codes, up to 64 rows: the mid-batch kernel (weights from registers
- * into the MFMA, activations shared through LDS), which the library itself takes for 8-bit codes on large layers only */
+ * into the MFMA, activations shared through LDS), which the library itself takes for 8-bit codes on large layers only.
+ * fp16 / bf16 activations on MXFP8 / MXFP4 weights at 3..16 (fp16: 10) rows: the activations as sums of e4m3 terms
+ * through the skinny kernel of the narrow formats (family K_SKINNY; the call then needs a workspace), which the library
+ * itself takes on large layers only */
 #define GLA_TILE_PREFER_MID (-4)
 
 /*

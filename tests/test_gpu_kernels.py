@@ -1038,6 +1038,75 @@ def test_weight_only_mxfp_skinny_kernel_on_wide_layers(device, W_nbits):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("W_nbits", [8, 4])
+def test_weight_only_mxfp_batches_as_sums_of_e4m3_terms(device, dtype, W_nbits):
+    """3..16 rows (fp16: 10) of 16-bit activations on MX weights through the skinny kernel of the narrow formats: a launch
+    in front writes every activation as two (fp16: three) e4m3 terms with block scales of their own, the scaled MFMA
+    multiplies them with the weights as they are, the epilogue adds a row's terms.  Forced with the preference on a
+    small ragged layer (N = 2032 ends inside a 16-row weight tile; one and two activation tiles, a last tile with one
+    row; a bias), activations whose blocks differ by 2^12 in magnitude, a block of zeros, fp16 values down to the
+    subnormals; then one-hot rows, which must come out exactly; then a layer large enough to take the path unasked."""
+    N, K = 2032, 3840
+    W = gen_x(N, K, torch.bfloat16, seed=71, std=0.03)
+    W[:, 64:96] *= 16.0
+    W[7, 128:160] = 0.0
+    lin = torch.nn.Linear(K, N, bias=True, dtype=dtype)
+    lin.weight.data = W.to(dtype)
+    lin.bias.data = gen_x(1, N, dtype, seed=72).reshape(-1)
+    cls = helper.A16W8_MXFP if W_nbits == 8 else helper.A16W4_MXFP
+    layer = cls(device=device, dtype=dtype).from_linear(lin.to(device))
+    m = layer.get_meta_args()
+
+    def run(x, bias):
+        out = torch.empty(x.shape[0], N, dtype=dtype, device=device)
+        a = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                   unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                   acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                   data_contiguous=m[11], tile_config=-4, bias=bias)
+        assert _ext.matmul_family(a) == "K_SKINNY", (x.shape[0], _ext.matmul_family(a))
+        print(f"case: K_SKINNY on e4m3 terms M={x.shape[0]} N={N} K={K} W{W_nbits} {dtype}", flush=True)
+        _ext.matmul(a, device)
+        torch.cuda.synchronize()
+        return out
+
+    rows = (3, 5, 8, 9, 16) if dtype == torch.bfloat16 else (3, 5, 6, 10)
+    for M in rows:
+        x = gen_x(M, K, dtype, seed=M)
+        x[:, 96:160] *= 64.0
+        x[:, 160:192] /= 64.0
+        x[0, 256:288] = 0.0
+        if dtype == torch.float16:
+            x[1, 320:352] *= 2.0 ** -14      # down to fp16 subnormals
+        y_ref = oracle_forward(layer, x)
+        y = to_np(run(x.to(device), layer.bias))
+        err = rel_frob(y, y_ref)
+        assert err <= TIGHT[dtype], (M, err)
+        assert elementwise_excess(y, y_ref, kind_of(dtype)) <= 1.0, M
+    # one-hot rows pick single dequantised weights: exact, whatever the position inside its block and the row's slot
+    layer_bias, layer.bias = layer.bias, None
+    for M in rows[-2:]:
+        x = torch.zeros(M, K, dtype=dtype)
+        for r in range(M):
+            x[r, (97 * r + 5) % K] = 1.0 if r % 2 == 0 else -0.375
+        assert np.array_equal(to_np(run(x.to(device), None)), round_like(oracle_forward(layer, x), dtype))
+    layer.bias = layer_bias
+    # unasked: a long-K layer at 8 rows (MXFP4: 58.7 M weights; MXFP8: K >= 8192 and N <= 8192)
+    N2, K2 = 4096, 14336
+    lin2 = torch.nn.Linear(K2, N2, bias=False, dtype=dtype, device=device)
+    lin2.weight.data = gen_x(N2, K2, torch.bfloat16, seed=73, std=0.02).to(dtype).to(device)
+    big = cls(device=device, dtype=dtype).from_linear(lin2)
+    M = 8 if dtype == torch.bfloat16 else 5
+    x = gen_x(M, K2, dtype, seed=74).to(device)
+    m2 = big.get_meta_args()
+    a = _ext.build_matmul_args(x, big.W_q, big.scales, big.zeros, None, torch.empty(M, N2, dtype=dtype, device=device), W_nbits=m2[1],
+                               group_size=m2[2], unpack_mask=m2[3], elements_per_sample=m2[4], input_dtype=m2[5], output_dtype=m2[6],
+                               acc_dtype=m2[7], meta_dtype=m2[8], channel_scale_mode=m2[9], W_group_mode=m2[10], data_contiguous=m2[11])
+    assert _ext.matmul_family(a) == "K_SKINNY"
+    check_layer(big, x, dtype, types=["GEMM"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("W_nbits", [8, 4])
 def test_weight_only_mxfp_layers_k_not_a_multiple_of_128(device, dtype, W_nbits):
     """K = 1056 (33 blocks): every batch size stays on the streaming kernel."""
     N, K = 264, 1056

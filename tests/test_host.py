@@ -721,3 +721,45 @@ def test_patch_model_replaces_linears_and_skips_named_modules():
 
     with pytest.raises(ImportError):
         helper.patch_model(Model(), device="cpu", processor=HqqOnly())
+
+
+def test_weight_only_mx_batches_go_as_e4m3_terms_on_large_layers():
+    """Host logic only: 3..16 rows of fp16 / bf16 on MXFP4 / MXFP8 weights.  The skinny kernel of the narrow formats takes
+    them, as sums of e4m3 terms, where that measured faster: while the terms fit one 16-row tile (bf16 8 rows, fp16 5) on
+    MXFP4 layers of 50 M weights or more and on MXFP8 layers with K >= 8192 and N <= 8192, with two tiles (bf16 up to 16
+    rows) on long-K layers; GLA_TILE_PREFER_MID asks for it anywhere; the call then needs a workspace for the terms."""
+    def layer(cls, dtype, N, K):
+        e = 2 if cls is gemlite_amd.helper.A16W4_MXFP else 1
+        W_q = torch.zeros((N, K // e), dtype=torch.uint8)
+        if e == 1:
+            W_q = W_q.view(torch.float8_e4m3fn)
+        return cls(device="cpu", dtype=dtype).from_packed_weights(W_q, torch.full((N, K // 32), 127, dtype=torch.uint8))
+
+    def args(l, M, dtype, tile=-1):
+        m = l.get_meta_args()
+        return _ext.build_matmul_args(
+            torch.zeros(M, l.in_features, dtype=dtype), l.W_q, l.scales, l.zeros, None, torch.zeros(M, l.out_features, dtype=dtype),
+            W_nbits=m[1], group_size=m[2], unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+            acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11], tile_config=tile)
+
+    W4, W8 = gemlite_amd.helper.A16W4_MXFP, gemlite_amd.helper.A16W8_MXFP
+    bf, fp = torch.bfloat16, torch.float16
+    fams = lambda l, dtype, Ms: [_ext.matmul_family(args(l, M, dtype)) for M in Ms]
+    Ms = (2, 3, 5, 6, 8, 9, 16, 17)
+    long_k = layer(W4, bf, 4096, 14336)
+    assert fams(long_k, bf, Ms) == ["MX_STREAM"] + ["K_SKINNY"] * 6 + ["GEMM_KBYTES_MX"]
+    assert fams(layer(W4, fp, 4096, 14336), fp, Ms) == ["MX_STREAM", "K_SKINNY", "K_SKINNY"] + ["MX_SKINNY"] * 4 + ["GEMM_KBYTES_MX"]
+    assert fams(layer(W4, bf, 14336, 4096), bf, Ms) == ["MX_STREAM"] + ["K_SKINNY"] * 4 + ["MX_SKINNY"] * 2 + ["GEMM_KBYTES_MX"]
+    small = layer(W4, bf, 4096, 4096)
+    assert fams(small, bf, Ms) == ["MX_STREAM"] + ["MX_SKINNY"] * 6 + ["GEMM_KBYTES_MX"]
+    assert fams(layer(W8, bf, 4096, 14336), bf, Ms) == ["MX_STREAM"] + ["K_SKINNY"] * 6 + ["GEMM_KBYTES_MX"]
+    assert fams(layer(W8, bf, 14336, 4096), bf, Ms) == ["MX_STREAM"] + ["MX_SKINNY"] * 6 + ["GEMM_KBYTES_MX"]
+    # the preference: honoured up to 16 (fp16: 10) rows, ignored outside; the terms and their scale bytes go to the workspace
+    assert [_ext.matmul_family(args(small, M, bf, -4)) for M in (2, 3, 16, 17)] == ["MX_STREAM", "K_SKINNY", "K_SKINNY", "GEMM_KBYTES_MX"]
+    small_fp = layer(W4, fp, 4096, 4096)
+    assert [_ext.matmul_family(args(small_fp, M, fp, -4)) for M in (10, 11)] == ["K_SKINNY", "MX_SKINNY"]
+    private = 4 << 20
+    assert _ext.matmul_workspace_need(args(small, 8, bf, -4)) == private + 16 * 4096 + 16 * 128
+    assert _ext.matmul_workspace_need(args(small, 9, bf, -4)) == private + 32 * 4096 + 32 * 128
+    assert _ext.matmul_workspace_need(args(small_fp, 5, fp, -4)) == private + 16 * 4096 + 16 * 128
+    assert _ext.matmul_workspace_need(args(small, 8, bf)) == 0
