@@ -406,6 +406,50 @@ bool widen(const gla_matmul_args& p, Widened& w) {
     return true;
 }
 
+// Packed layers at prefill size: from 2048 rows of bf16 (4096 of fp16) the weights are first written out as 16-bit
+// values into the workspace (wn_unpack16.hip: once per call, at memory speed, 11.6 us for 4096^2) and the 16-bit GEMM
+// runs on them, at the rate of an unquantised layer, instead of the fused kernel that unpacks every weight once per
+// 128 or 256 rows beside its MFMAs.  Per-channel and per-token scales stay in the GEMM's epilogue.
+struct Unpacked {
+    gla_matmul_args q;   // the call the 16-bit GEMM sees (w and workspace filled in at launch)
+    int64_t w_off;       // where the 16-bit weights go in the workspace
+    int64_t total;       // workspace bytes of the whole call
+};
+
+bool unpack_first(const gla_matmul_args& p, Family f, Unpacked& u) {
+    const bool asked = p.tile_config == GLA_TILE_PREFER_UNPACKED && p.M > 16 && gemm_wn_eligible(p);
+    // same launches side by side, fused -> unpacked (us): 4-bit gs 128 bf16 4096^2 at 1024 / 2048 / 4096 / 8192 rows 72 ->
+    // 74, 107 -> 92, 161 -> 135, 297 -> 246; 8192^2 189 -> 179, 292 -> 261, 573 -> 474, 1179 -> 914; fp16, whose fused
+    // unpacking is cheaper: 66 -> 73, 94 -> 96, 146 -> 143, 280 -> 267; 8192^2 158 -> 186, 271 -> 278, 527 -> 505, 1052 -> 968
+    const int from_rows = p.input_dtype == GLA_DT_BF16 ? 2048 : 4096;
+    const bool by_rule = f == F_GEMM_WN && p.M >= from_rows && p.tile_config <= 0 && p.tile_config != GLA_TILE_PREFER_MATRIX;
+    if (!asked && !by_rule) return false;
+    if (p.acc_dtype != GLA_DT_FP32 || (p.W_group_mode >= GLA_WGM_SCALE && (p.channel_scale_mode & 1))) return false;
+    if ((int64_t)p.N * p.K >= ((int64_t)1 << 30)) return false;
+    u.q = p;
+    u.q.W_nbits = 16;
+    u.q.elements_per_sample = 1;
+    u.q.unpack_mask = 0xffff;
+    u.q.w_dtype = p.input_dtype;
+    u.q.W_group_mode = GLA_WGM_NONE;
+    u.q.group_size = p.K;
+    u.q.zeros = nullptr;
+    u.q.zero_is_scalar = 0;
+    if (!(p.channel_scale_mode & 1)) u.q.scales = nullptr;
+    u.q.w = (const void*)(uintptr_t)256;  // stands for an aligned pointer while the kernel's rules are asked
+    u.q.w_stride_k = 1;
+    u.q.w_stride_n = p.K;
+    u.q.tile_config = -1;
+    u.q.workspace = nullptr;
+    u.q.workspace_bytes = 0;
+    if (!gemm_16bit_eligible(u.q)) return false;
+    const int64_t inner = gemm_16bit_workspace_bytes(u.q);
+    if (inner < 0) return false;
+    u.w_off = ((inner > kWsPrivateBytes ? inner : kWsPrivateBytes) + 255) / 256 * 256;
+    u.total = u.w_off + (int64_t)p.N * p.K * 2;
+    return true;
+}
+
 }  // namespace
 }  // namespace gla
 
@@ -453,6 +497,8 @@ int gla_matmul_family(const gla_matmul_args* args) {
     const Family f = choose(*args, resolve_type(*args));
     Widened w;
     if (f == F_GENERIC && widen(*args, w)) return (int)w.f;  // the kernel that runs on the widened activations
+    Unpacked u;
+    if (unpack_first(*args, f, u)) return (int)F_GEMM_16BIT;   // ... on the unpacked weights
     return (int)f;
 }
 
@@ -463,6 +509,8 @@ int64_t gla_matmul_workspace_bytes(const gla_matmul_args* args) {
     const Family f = choose(*args, resolve_type(*args));
     Widened w;
     if (f == F_GENERIC && widen(*args, w)) return w.total;
+    Unpacked u;
+    if (unpack_first(*args, f, u)) return u.total;
     return family_workspace(f, *args);
 }
 
@@ -486,6 +534,21 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
         w.q.workspace = args->workspace;
         w.q.workspace_bytes = (uint64_t)w.x_off;
         return w.f == F_GEMV_PACKED ? launch_gemv_packed(w.q, s) : (w.f == F_WN_MID ? launch_wn_mid(w.q, s) : launch_gemm_wn(w.q, s));
+    }
+    Unpacked u;
+    if (unpack_first(*args, f, u)) {
+        if (args->workspace == nullptr || (int64_t)args->workspace_bytes < u.total) {
+            set_error("matmul: workspace of %lld bytes required (the weights are unpacked into it), %llu given", (long long)u.total,
+                      (unsigned long long)args->workspace_bytes);
+            return GLA_ERR_WORKSPACE_TOO_SMALL;
+        }
+        void* w16 = (char*)args->workspace + u.w_off;
+        const int rcu = launch_wn_unpack16(*args, w16, args->K, s);
+        if (rcu != GLA_OK) return rcu;
+        u.q.w = w16;
+        u.q.workspace = args->workspace;
+        u.q.workspace_bytes = (uint64_t)u.w_off;
+        return launch_gemm_16bit(u.q, s);
     }
     int rc2;
     switch (f) {

@@ -76,6 +76,8 @@ int launch_gemv_kmajor(const gla_matmul_args& p, hipStream_t stream);
 bool gemm_wn_eligible(const gla_matmul_args& p);
 int64_t gemm_wn_workspace_bytes(const gla_matmul_args& p);
 int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream);
+// the weights of such a call as fp16 / bf16 values, [N, ldo] with K contiguous (wn_unpack16.hip)
+int launch_wn_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hipStream_t stream);
 
 // ---- MFMA GEMM on 8-bit operands, both K-contiguous (gemm_8bit.hip) --------
 bool gemm_8bit_eligible(const gla_matmul_args& p);

@@ -1,0 +1,131 @@
+// Packed 2-, 4- and 8-bit codes written out as the fp16 / bf16 weights they stand for, [N, K] with K contiguous: the
+// first half of the prefill path of packed layers from 2048 rows of bf16 (4096 of fp16) up, whose second half is the
+// 16-bit matrix-core GEMM (gemm_16bit.hip).  The fused kernel (gemm_wn.hip) unpacks every weight once per 128 or 256
+// rows of the batch, and its vector work stands beside the MFMAs; here a weight is unpacked once per call, at memory
+// speed (4096^2 4-bit codes: 11.6 us), and the GEMM that follows runs at the rate of unquantised layers (4-bit codes in
+// groups of 128, bf16, M = N = K = 4096: 161 us fused, 135 us for the pair; 8192 rows: 297 -> 246).
+// Reference: gemlite/triton_kernels/gemm_kernels.py:405-452 with utils.py:73-105 - the same five W_group_mode forms,
+// evaluated with the same arithmetic as the fused kernels (wn_dequant.hpp), so a layer's weights round the same way
+// on either side of the hand-off.
+//
+// One thread: one column n and 64 consecutive K-values = 64 / e packed words of that column (a wave reads 256
+// contiguous bytes per word row) -> 128 contiguous bytes of row n of the output, which the wave transposes through LDS
+// so that its stores are whole lines too (16 bytes per lane at a stride of a row each ran at a third of the speed).
+// Groups are whole multiples of 64 K-values (the fused GEMM's rule), so a thread needs one (scale, zero) pair.
+#include "common.hpp"
+#include "dispatch.hpp"
+#include "wn_dequant.hpp"
+
+namespace gla {
+
+namespace {
+
+struct Unpack16Args {
+    const uint32_t* w;        // [K / e, N] packed words
+    const void* scales;       // [K / group, N]
+    const void* zeros;        // [K / group, N] or one value
+    uint16_t* out;            // [N, ldo]
+    int N, chunks;            // chunks = K / 64
+    int64_t wsk, msg, ldo;    // elements
+    int cpg;                  // 64-K chunks per group
+    int wgm, meta_dt, z_dt;
+    bool has_s, has_zt, z_scalar;
+};
+
+template <int BITS, bool BF16>
+__global__ __launch_bounds__(256) void wn_unpack16_kernel(Unpack16Args a) {
+    constexpr int E = 32 / BITS, WORDS = 64 / E;
+    constexpr int OFF = BITS == 8 ? 0 : 128;
+    __shared__ __align__(16) unsigned char tile[4][64 * 128];  // per wave: 64 columns x 128 bytes, 16-byte slots swizzled by row
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * 64;
+    const int chunk = blockIdx.y * 4 + wave;
+    const bool live = chunk < a.chunks;          // wave-uniform
+    int n = n0 + lane;
+    if (n > a.N - 1) n = a.N - 1;                // lanes past N unpack the last column again and store nothing
+    const int ch = live ? chunk : a.chunks - 1;
+    uint32_t w[WORDS];
+    const uint32_t* src = a.w + (int64_t)ch * WORDS * a.wsk + n;
+#pragma unroll
+    for (int j = 0; j < WORDS; ++j) w[j] = __builtin_nontemporal_load(src + (int64_t)j * a.wsk);
+    const int g = ch / a.cpg;
+    const float s = a.has_s ? load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + n) : 1.0f;
+    const float z = a.has_zt ? load_as_float(a.zeros, a.meta_dt, (int64_t)g * a.msg + n)
+                             : (a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0) : 0.0f);
+    const float c1 = a.wgm == GLA_WGM_SHIFT ? -1.0f : (a.wgm == GLA_WGM_FMA ? 1.0f : 0.0f);
+    const float c2 = a.wgm == GLA_WGM_SHIFT_SCALE ? -1.0f : 0.0f;
+    const ColMeta<BF16> meta = make_meta<BF16, OFF>(s, z * __builtin_fmaf(c2, s, c1));
+    uint32_t o[32];
+#pragma unroll
+    for (int j = 0; j < WORDS; ++j) {
+#pragma unroll
+        for (int i = 0; i < E / 2; ++i) {
+            const uint32_t lo = (w[j] >> (BITS * 2 * i)) & ((1u << BITS) - 1u);
+            const uint32_t hi = (w[j] >> (BITS * (2 * i + 1))) & ((1u << BITS) - 1u);
+            uint32_t r;
+            if constexpr (BF16 && BITS == 8) {
+                // 128 + q is not exact in bf16 above 127: bytes straight to fp32, scaled there, packed once
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                const f32x2 v = {__builtin_fmaf((float)lo, meta.s, meta.z), __builtin_fmaf((float)hi, meta.s, meta.z)};
+                r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+            } else {
+                const uint32_t magic = BF16 ? 0x43004300u : 0x64006400u;  // 128 + q in bf16, 1024 + q in fp16
+                r = dequant_pair<BF16>(magic | lo | (hi << 16), meta);
+            }
+            o[j * (E / 2) + i] = r;
+        }
+    }
+    // through LDS, so that a store instruction writes whole 128-byte lines: the lane's 128 bytes go to row `lane`,
+    // then lane (row l / 8 of eight, slot l % 8) stores 16 bytes and eight lanes together one row's line
+    unsigned char* mine = tile[wave];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        *(uint4*)(mine + lane * 128 + ((i ^ (lane & 7)) * 16)) = make_uint4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = 8 * i + (lane >> 3), c = lane & 7;
+        const uint4 v = *(const uint4*)(mine + r * 128 + ((c ^ (r & 7)) * 16));
+        if (live && n0 + r < a.N) *(uint4*)(a.out + (int64_t)(n0 + r) * a.ldo + (int64_t)chunk * 64 + c * 8) = v;
+    }
+}
+
+template <int BITS>
+void launch_bits(const Unpack16Args& a, bool bf16, hipStream_t stream) {
+    const dim3 grid(ceil_div(a.N, 64), ceil_div(a.chunks, 4));
+    if (bf16)
+        hipLaunchKernelGGL((wn_unpack16_kernel<BITS, true>), grid, dim3(256), 0, stream, a);
+    else
+        hipLaunchKernelGGL((wn_unpack16_kernel<BITS, false>), grid, dim3(256), 0, stream, a);
+}
+
+}  // namespace
+
+// The call must be one the fused packed-weight GEMM takes (gemm_wn_eligible: operand types, layouts, alignments, groups
+// of whole 64-K stages); out: [N, ldo] 16-bit values of the activation type, ldo >= K, 16-byte aligned rows.
+int launch_wn_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hipStream_t stream) {
+    if (!gemm_wn_eligible(p) || ldo < p.K || ldo % 8 != 0 || ((uintptr_t)out & 15)) {
+        set_error("wn_unpack16: a call of the packed-weight GEMM and an aligned [N, ldo >= K] output are required");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    const bool uses_scales = p.W_group_mode >= GLA_WGM_SCALE;
+    const bool uses_zeros = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
+    const bool grouped = uses_scales || (uses_zeros && !p.zero_is_scalar);
+    const int gs = grouped ? p.group_size : p.K;
+    Unpack16Args a;
+    a.w = (const uint32_t*)p.w; a.scales = p.scales; a.zeros = p.zeros; a.out = (uint16_t*)out;
+    a.N = p.N; a.chunks = p.K / 64;
+    a.wsk = p.w_stride_k; a.msg = gs == p.K ? 0 : p.meta_stride_g; a.ldo = ldo;
+    a.cpg = gs / 64;
+    a.wgm = p.W_group_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
+    a.has_s = uses_scales; a.has_zt = uses_zeros && !p.zero_is_scalar; a.z_scalar = uses_zeros && p.zero_is_scalar;
+    const bool bf16 = p.input_dtype == GLA_DT_BF16;
+    switch (p.W_nbits) {
+        case 2: launch_bits<2>(a, bf16, stream); break;
+        case 4: launch_bits<4>(a, bf16, stream); break;
+        default: launch_bits<8>(a, bf16, stream); break;
+    }
+    return check_hip(hipGetLastError(), "wn_unpack16 launch");
+}
+
+}  // namespace gla

@@ -26,7 +26,7 @@ from .quant_utils import (scale_activations_mxfp4, scale_activations_mxfp8, scal
                           scale_activations_per_token)
 
 
-PREFER_STREAMING, PREFER_MATRIX, PREFER_MID = -2, -3, -4   # GLA_TILE_PREFER_* of the C header
+PREFER_STREAMING, PREFER_MATRIX, PREFER_MID, PREFER_UNPACKED = -2, -3, -4, -5   # GLA_TILE_PREFER_* of the C header
 HAND_OFF_ROWS = 128                        # batch sizes up to which both kinds of kernel are timed
 
 
@@ -109,6 +109,9 @@ def tune_layer(layer: GemLiteLinear, batch_sizes: Iterable[int], reps: int = 20,
             # around the hand-off between the streaming kernels and the matrix-core GEMMs the other side is timed too;
             # the library's thresholds there were fitted on one machine
             candidates += [t for t in (PREFER_STREAMING, PREFER_MATRIX, PREFER_MID) if _ext.matmul_family(build(t)) != family]
+        if M >= 512 and family in ("GEMM_WN", "GEMM_16BIT"):
+            # prefill of packed layers: the fused kernel against weight unpacking + the 16-bit GEMM
+            candidates += [t for t in (PREFER_MATRIX, PREFER_UNPACKED) if _ext.matmul_family(build(t)) != family]
         for tile in candidates:
             args = build(tile)
             need = lib.gla_matmul_workspace_bytes(ctypes.byref(args))

@@ -282,6 +282,60 @@ def test_packed_codes_at_17_to_64_rows(device, nbits, gs, dtype):
                 assert elementwise_excess(to_np(out), y_ref, kind_of(dtype)) <= 1.0, (N, K, M, tile)
 
 
+@pytest.mark.parametrize("nbits,gs", [(4, 128), (4, 64), (2, 64), (8, 128), (8, None), (4, None)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_packed_layers_at_prefill_size_unpack_their_weights_first(device, nbits, gs, dtype):
+    """From 2048 rows of bf16, 4096 of fp16 (or on request) the packed codes are written out once as 16-bit weights and the 16-bit
+    matrix-core GEMM runs on them.  Every code width of the fused GEMM, groups of one and two 64-K chunks and one group
+    per channel (scales after the K sum), both activation types; N ends inside a wave's 64 columns, K inside a
+    workgroup's four chunks; a bias; the five dequantisation forms; and that the weights come out exactly as the fused
+    kernel makes them (one-hot rows: bit-identical outputs of both paths)."""
+    dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
+    N, K = (2032, 1088) if gs == 64 else (520, 1152)
+    g = K if gs is None else gs
+    W_q, scales, zeros = gen_int_case(N, K, nbits, g, dtype, seed=nbits * 100 + g % 1000)
+    layer = GemLiteLinear(nbits, g, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device),
+                                                       bias=gen_x(1, N, dtype, seed=5).reshape(-1).to(device))
+    l_scale = GemLiteLinear(nbits, g, K, N, dt, dt).pack(W_q.to(device), scales.to(device), None)                  # scales only
+    l_zero = GemLiteLinear(nbits, g, K, N, dt, dt).pack(W_q.to(device), scales.to(device), 1 if nbits < 4 else 3)   # one integer zero
+    l_shift = GemLiteLinear(nbits, g, K, N, dt, DType.FP32).pack(W_q.to(device), None, 1)                           # shift only
+
+    def run(l, x, tile):
+        m = l.get_meta_args()
+        out = torch.empty(x.shape[0], N, dtype=dtype if l is not l_shift else torch.float32, device=device)
+        a = _ext.build_matmul_args(x, l.W_q, l.scales, l.zeros, None, out, W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+                                   elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
+                                   channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11], tile_config=tile, bias=l.bias)
+        fam = _ext.matmul_family(a)
+        print(f"case: {fam} tile={tile} M={x.shape[0]} N={N} K={K} W{nbits} gs={gs} mode={l.W_group_mode}", flush=True)
+        _ext.matmul(a, device)
+        torch.cuda.synchronize()
+        return fam, out
+
+    for M, tile in ((40, -5), (300, -5), (2048 if dtype == torch.bfloat16 else 4096, -1)):
+        x = gen_x(M, K, dtype, seed=M)
+        y_ref = oracle_forward(layer, x)
+        fam, out = run(layer, x.to(device), tile)
+        assert fam == "GEMM_16BIT", (M, tile, fam)
+        err = rel_frob(to_np(out), y_ref)
+        assert err <= TIGHT[dtype], (M, err)
+        assert elementwise_excess(to_np(out), y_ref, kind_of(dtype)) <= 1.0, M
+    for l, tol in ((l_scale, dtype), (l_zero, dtype), (l_shift, torch.float32)):
+        x = (gen_x(70, K, dtype, seed=7) / 10)
+        fam, out = run(l, x.to(device), -5)
+        assert fam == "GEMM_16BIT", (l.W_group_mode, fam)
+        y_ref = oracle_forward(l, x)
+        assert rel_frob(to_np(out), y_ref) <= TIGHT[tol], l.W_group_mode
+    # one-hot rows read single weights: the fused kernel and this path must agree to the bit
+    x = torch.zeros(48, K, dtype=dtype)
+    for r in range(48):
+        x[r, (53 * r + 11) % K] = 1.0
+    layer.bias = None
+    (fa, ya), (fb, yb) = run(layer, x.to(device), -3), run(layer, x.to(device), -5)
+    assert (fa, fb) == ("GEMM_WN", "GEMM_16BIT")
+    assert torch.equal(ya, yb)
+
+
 @pytest.mark.parametrize("nbits,gs", [(1, 32), (1, 64), (2, 16), (2, 32), (4, 16), (8, 16)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_packed_codes_in_short_groups(device, nbits, gs, dtype):

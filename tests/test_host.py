@@ -371,7 +371,8 @@ def test_benchmark_configurations_take_a_tuned_kernel_family():
     s, z = torch.rand(N * K // 128, 1).half(), torch.rand(N * K // 128, 1).half()
     l = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q, s, z)
     # (up to 64 rows a layer this small stays with the streaming kernel, as row chunks of 16: see the next test)
-    assert [_family(l, M, torch.float16) for M in (1, 2, 4, 8, 16, 64, 65, 4096)] == ["GEMV_PACKED"] * 6 + ["GEMM_WN"] * 2
+    # (from 4096 rows of fp16 the weights are unpacked first and the 16-bit GEMM runs)
+    assert [_family(l, M, torch.float16) for M in (1, 2, 4, 8, 16, 64, 65, 1000, 4096)] == ["GEMV_PACKED"] * 6 + ["GEMM_WN"] * 2 + ["GEMM_16BIT"]
     # A16W8 channel-wise and A16W2 gs64, bf16
     W8 = torch.randint(0, 256, (N, K), generator=g).to(torch.uint8)
     l8 = GemLiteLinear(8, K, K, N, DType.BF16, DType.BF16).pack(W8, torch.rand(N, 1).bfloat16(), torch.rand(N, 1).bfloat16())
@@ -763,3 +764,28 @@ def test_weight_only_mx_batches_go_as_e4m3_terms_on_large_layers():
     assert _ext.matmul_workspace_need(args(small, 9, bf, -4)) == private + 32 * 4096 + 32 * 128
     assert _ext.matmul_workspace_need(args(small_fp, 5, fp, -4)) == private + 16 * 4096 + 16 * 128
     assert _ext.matmul_workspace_need(args(small, 8, bf)) == 0
+
+
+def test_packed_layers_unpack_their_weights_first_at_prefill_size():
+    """Host logic only: from 4096 rows of fp16, 2048 of bf16 (or with GLA_TILE_PREFER_UNPACKED above 16) a call of the fused packed-weight GEMM
+    becomes weight unpacking + the 16-bit GEMM, reported as that family, with N * K * 2 bytes more workspace; an explicit
+    tile keeps the fused kernel."""
+    g = torch.Generator().manual_seed(0)
+    N, K = 512, 1024
+    W_q = torch.randint(0, 16, (N, K), generator=g).to(torch.uint8)
+    l = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q, torch.rand(N * K // 128, 1).half(), torch.rand(N * K // 128, 1).half())
+    m = l.get_meta_args()
+
+    def args(M, tile=-1):
+        return _ext.build_matmul_args(torch.zeros(M, K, dtype=torch.float16), l.W_q, l.scales, l.zeros, None,
+                                      torch.zeros(M, N, dtype=torch.float16), W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+                                      elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7], meta_dtype=m[8],
+                                      channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11], tile_config=tile)
+
+    assert [_ext.matmul_family(args(M)) for M in (65, 4095, 4096, 9000)] == ["GEMM_WN", "GEMM_WN", "GEMM_16BIT", "GEMM_16BIT"]
+    assert _ext.matmul_family(args(4096, -3)) == "GEMM_WN"   # the preference for the tiled GEMM keeps the fused kernel
+    assert [_ext.matmul_family(args(M, -5)) for M in (16, 17, 300)] == ["GEMV_PACKED", "GEMM_16BIT", "GEMM_16BIT"]
+    assert _ext.matmul_family(args(2048, 2128)) == "GEMM_WN"
+    need = _ext.matmul_workspace_need(args(4096))
+    assert need >= (4 << 20) + N * K * 2 and need % 256 == 0
+    assert _ext.matmul_workspace_need(args(300, -5)) >= (4 << 20) + N * K * 2
