@@ -253,14 +253,21 @@ def extra_points(lib, device, T, quick):
             t.view(torch.uint8).zero_()
         return T.eager_us(run, 20)
 
-    # A16W4 gs128 fp16, M = 4096 (fused-dequant MFMA GEMM)
+    # A16W4 gs128 fp16, M = 4096: as the library runs it (weights unpacked into the workspace, then the 16-bit MFMA
+    # GEMM), and beside it the fused-dequant MFMA GEMM it hands over from (the preference for the tiled GEMM keeps it)
     M = 4096
     x = torch.randn((M, K), generator=g).to(torch.float16).to(device)
     y = torch.empty((M, N), dtype=torch.float16, device=device)
+    fused = Launch(lib, base, x, y, device)
+    fused.args.tile_config = -3  # GLA_TILE_PREFER_MATRIX
+    us_fused = T.eager_us(fused, 40)
     run = Launch(lib, base, x, y, device)
     us = T.eager_us(run, 40)
+    family = _ext.matmul_family(run.args)
     gemm_point("gemm_a16w4_gs128_fp16", M, N, K, us, 2500.0, "fp16", zeroed(run, x, base.W_q.data))
-    del base, run
+    out["gemm_a16w4_gs128_fp16"]["family"] = family
+    out["gemm_a16w4_gs128_fp16"]["us_fused_dequant_kernel"] = round(us_fused, 1)
+    del base, run, fused
     # an unquantised layer of the same shape (W_nbits = 16): fp16 x fp16 on the K-contiguous MFMA GEMM, and the vendor's
     # plain GEMM on the same operands in the same run
     W16 = (torch.randn((N, K), generator=g) * 0.02).to(torch.float16).to(device)
@@ -570,7 +577,9 @@ def run_point(name, lib, device, T):
         x = torch.randn((M, K), generator=g).to(torch.bfloat16).to(device)
         xq, sx = gemlite_amd.scale_activations_mxfp4(x)
         peak = 10100.0
-    elif name == "gemm_a16w4_gs128_fp16":
+    elif name in ("gemm_a16w4_gs128_fp16", "gemm_a16w4_gs128_fp16_fused"):
+        # as the library runs it (from 4096 rows of fp16: weights unpacked into the workspace, then the 16-bit GEMM), or
+        # kept on the fused-dequant kernel with the preference for the tiled GEMM
         M = N = K = 4096
         layer, _ = make_layer(N, K, seed=11, device=device)
         xq, sx = torch.randn((M, K), generator=g).to(torch.float16).to(device), None
@@ -587,8 +596,14 @@ def run_point(name, lib, device, T):
         peak = 2500.0
     else:
         sys.exit(f"bench.py: unknown --point {name}")
-    y = torch.empty((M, N), dtype=torch.float16 if name == "gemm_a16w4_gs128_fp16" else torch.bfloat16, device=device)
-    us = T.eager_us(Launch(lib, layer, xq, y, device, scales_x=sx), 10)
+    y = torch.empty((M, N), dtype=torch.float16 if name.startswith("gemm_a16w4_gs128_fp16") else torch.bfloat16, device=device)
+    launch = Launch(lib, layer, xq, y, device, scales_x=sx)
+    if name.endswith("_fused"):
+        launch.args.tile_config = -3  # GLA_TILE_PREFER_MATRIX
+        need = lib.gla_matmul_workspace_bytes(ctypes.byref(launch.args))
+        ws = _ext.get_workspace(device, max(need, 1), stream=0)
+        launch.args.workspace, launch.args.workspace_bytes = ws.data_ptr(), ws.numel()
+    us = T.eager_us(launch, 10)
     tf = 2.0 * M * N * K / us / 1e6
     print(json.dumps({"point": name, "M": M, "N": N, "K": K, "us": round(us, 1), "TFLOP/s": round(tf, 1),
                       "frac_of_peak": round(tf / peak, 4)}))
