@@ -628,15 +628,24 @@ extern "C" {
 int64_t gla_static_scratch_bytes(void) { return (int64_t)GLA_STATIC_SCRATCH_BYTES; }
 
 int gla_matmul_static(const gla_matmul_args* args, void* stream) {
-    const int64_t need = gla_matmul_workspace_bytes(args);
+    int64_t need = gla_matmul_workspace_bytes(args);
     if (need < 0) return (int)need;
+    gla_matmul_args a = *args;
+    if (need > (int64_t)GLA_STATIC_SCRATCH_BYTES && args->tile_config <= 0 && args->tile_config != GLA_TILE_PREFER_MATRIX) {
+        // a packed layer at prefill size whose unpacked weights do not fit the array stays on the fused kernel
+        a.tile_config = GLA_TILE_PREFER_MATRIX;
+        const int64_t fused = gla_matmul_workspace_bytes(&a);
+        if (fused >= 0 && fused <= (int64_t)GLA_STATIC_SCRATCH_BYTES)
+            need = fused;
+        else
+            a.tile_config = args->tile_config;
+    }
     if (need > (int64_t)GLA_STATIC_SCRATCH_BYTES) {
         set_error("gla_matmul_static: this problem (M=%d N=%d K=%d) needs %lld bytes of scratch; the built-in array holds "
                   "%lld. Use gla_matmul with a workspace of that size", args->M, args->N, args->K, (long long)need,
                   (long long)GLA_STATIC_SCRATCH_BYTES);
         return GLA_ERR_WORKSPACE_TOO_SMALL;
     }
-    gla_matmul_args a = *args;
     a.workspace = nullptr;
     a.workspace_bytes = 0;
     if (need > 0) {

@@ -252,7 +252,9 @@ int gla_matmul(const gla_matmul_args* args, void* stream);
  * the struct are ignored: the scratch is a device array of GLA_STATIC_SCRATCH_BYTES bytes that the
  * library's code object carries (each GPU the library runs on holds its own copy until the process
  * ends).  The call allocates and frees nothing.  A problem whose gla_matmul_workspace_bytes()
- * exceeds GLA_STATIC_SCRATCH_BYTES is refused with GLA_ERR_WORKSPACE_TOO_SMALL.  The first call on
+ * exceeds GLA_STATIC_SCRATCH_BYTES is refused with GLA_ERR_WORKSPACE_TOO_SMALL, with one exception: a
+ * packed layer at prefill size whose unpacked 16-bit weights (N * K * 2 bytes) would not fit runs on
+ * the fused kernel instead, as gla_matmul does with GLA_TILE_PREFER_MATRIX.  The first call on
  * a device that needs scratch looks the array's address up; nothing is cleared (the array is zero
  * when the code object is loaded, and every kernel leaves the counters and slots it used at zero
  * again), so that first call may itself be recorded into a graph.  All calls on one GPU share the array: calls that may overlap in time

@@ -112,6 +112,41 @@ def test_gemm_split_k_twice(device):
         assert rel_frob(to_np(yb), oracle_forward(layer, x)) <= 1.5e-3
 
 
+def test_unpacked_weights_in_the_array_twice_and_the_fused_kernel_when_they_do_not_fit(device):
+    """A packed layer at prefill size unpacks its weights into the scratch (N K 2 bytes) before the 16-bit GEMM; twice in
+    a row, the second call on a smaller layer, which finds the first one's weights there.  A layer whose unpacked weights
+    exceed the array is not refused: the entry point keeps it on the fused kernel, so it must equal gla_matmul with the
+    preference for the tiled GEMM bit for bit."""
+    lib = _ext.load_library()
+    for (N, K, M, seed) in ((4096, 4096, 4096, 7), (4096, 1024, 4096, 8)):   # 256 output tiles: K in one piece
+        print(f"case: static scratch, unpacked weights N={N} K={K} M={M}", flush=True)
+        W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16, seed=seed)
+        layer = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+        x = gen_x(M, K, torch.float16, seed=seed + 10).to(device)
+        ya, yb, need = _both(layer, x, None, N, torch.float16, device)
+        assert (4 << 20) + N * K * 2 <= need <= lib.gla_static_scratch_bytes(), "the case is meant to unpack the weights into the scratch"
+        assert _same(ya, yb)
+        assert rel_frob(to_np(yb), oracle_forward(layer, x)) <= 1.5e-3
+    N, K, M = 8192, 4608, 4096    # 75.5 MB of fp16 weights: more than the array holds
+    print(f"case: static scratch, fused kernel instead of unpacked weights N={N} K={K} M={M}", flush=True)
+    W_q, scales, zeros = gen_int_case(N, K, 4, 128, torch.float16, seed=9)
+    layer = GemLiteLinear(4, 128, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))
+    x = gen_x(M, K, torch.float16, seed=19).to(device)
+    out_a = torch.full((M, N), float("nan"), dtype=torch.float16, device=device)
+    out_b = torch.full((M, N), float("nan"), dtype=torch.float16, device=device)
+    a = _args(layer, x, None, out_a)
+    assert _ext.matmul_family(a) == "GEMM_16BIT" and _ext.matmul_workspace_need(a) > lib.gla_static_scratch_bytes()
+    a.tile_config = -3          # GLA_TILE_PREFER_MATRIX: the fused kernel
+    assert _ext.matmul_family(a) == "GEMM_WN"
+    _ext.matmul(a, device)
+    b = _args(layer, x, None, out_b)
+    b.workspace, b.workspace_bytes = None, 0
+    rc = lib.gla_matmul_static(ctypes.byref(b), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.gla_last_error().decode()
+    torch.cuda.synchronize()
+    assert _same(out_a, out_b)
+
+
 def test_mxfp4_regrouped_scales_twice(device):
     """MXFP4 x MXFP4 with 128+-row tiles: both scale arrays are regrouped by stage into the scratch."""
     for (N, K, M, seed) in ((4096, 4096, 2048, 5), (4096, 4096, 1100, 6)):   # sizes at which the 128-row tile is the one chosen
