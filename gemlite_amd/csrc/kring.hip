@@ -419,6 +419,8 @@ int launch_mode_ring(const KRingArgs& a, hipStream_t stream) {
             if (tiles >= 440) return launch_ring<MODE, XBS, 2, 1, 8, 2>(a, stream);
             return launch_ring<MODE, XBS, 1, 1, 8, 2>(a, stream);
         }
+        // (16-bit activations as e4m3 terms, 16 rows of bf16 = 32 fp8 rows, 16384^2: 58 us with 2 weight tiles per wave, 51 with 4)
+        if (tiles >= 880) return launch_ring<MODE, XBS, 4, 2, 4, 2>(a, stream);
         if (tiles >= 440) return launch_ring<MODE, XBS, 2, 2, 4, 2>(a, stream);
         return launch_ring<MODE, XBS, 1, 2, 4, 3>(a, stream);
     } else {

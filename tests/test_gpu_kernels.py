@@ -1143,6 +1143,27 @@ def test_weight_only_mxfp_batches_as_sums_of_e4m3_terms(device, dtype, W_nbits):
             x[r, (97 * r + 5) % K] = 1.0 if r % 2 == 0 else -0.375
         assert np.array_equal(to_np(run(x.to(device), None)), round_like(oracle_forward(layer, x), dtype))
     layer.bias = layer_bias
+    # a wide layer (881 tiles of 16 weight rows, the last one ragged): four weight tiles per wave against two activation tiles
+    if dtype == torch.bfloat16:
+        N3, K3 = 14088, 512
+        lin3 = torch.nn.Linear(K3, N3, bias=False, dtype=dtype)
+        lin3.weight.data = gen_x(N3, K3, torch.bfloat16, seed=75, std=0.03).to(dtype)
+        wide = cls(device=device, dtype=dtype).from_linear(lin3.to(device))
+        m3 = wide.get_meta_args()
+        for M in (7, 13):
+            x = gen_x(M, K3, dtype, seed=M + 40)
+            out = torch.empty(M, N3, dtype=dtype, device=device)
+            a = _ext.build_matmul_args(x.to(device), wide.W_q, wide.scales, wide.zeros, None, out, W_nbits=m3[1], group_size=m3[2],
+                                       unpack_mask=m3[3], elements_per_sample=m3[4], input_dtype=m3[5], output_dtype=m3[6],
+                                       acc_dtype=m3[7], meta_dtype=m3[8], channel_scale_mode=m3[9], W_group_mode=m3[10],
+                                       data_contiguous=m3[11], tile_config=-4)
+            assert _ext.matmul_family(a) == "K_SKINNY"
+            print(f"case: K_SKINNY on e4m3 terms M={M} N={N3} K={K3} W{W_nbits} {dtype}", flush=True)
+            _ext.matmul(a, device)
+            torch.cuda.synchronize()
+            y_ref = oracle_forward(wide, x)
+            assert rel_frob(to_np(out), y_ref) <= TIGHT[dtype], M
+            assert elementwise_excess(to_np(out), y_ref, kind_of(dtype)) <= 1.0, M
     # unasked: a long-K layer at 8 rows (MXFP4: 58.7 M weights; MXFP8: K >= 8192 and N <= 8192)
     N2, K2 = 4096, 14336
     lin2 = torch.nn.Linear(K2, N2, bias=False, dtype=dtype, device=device)
