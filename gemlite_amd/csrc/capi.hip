@@ -417,6 +417,38 @@ struct Unpacked {
 };
 
 bool unpack_first(const gla_matmul_args& p, Family f, Unpacked& u) {
+    // (unpacked weight bytes under 16-bit activations likewise: the bytes are converted once, the per-channel scale stays
+    // in the epilogue; int8 bytes x bf16, M = 4096, N = K = 8192: see below)
+    const bool bytes = p.w_dtype == GLA_DT_INT8 || p.w_dtype == GLA_DT_UINT8 || p.w_dtype == GLA_DT_FP8;
+    if (bytes) {
+        const bool asked_b = p.tile_config == GLA_TILE_PREFER_UNPACKED && p.M > 16 && gemm_kbytes_eligible(p);
+        const bool by_rule_b = f == F_GEMM_KBYTES && p.M >= 2048 && p.tile_config <= 0 && p.tile_config != GLA_TILE_PREFER_MATRIX;
+        if (!asked_b && !by_rule_b) return false;
+        if (p.K % 16 != 0 || (p.W_group_mode == GLA_WGM_SCALE && (p.channel_scale_mode & 1))) return false;
+        if ((p.W_group_mode == GLA_WGM_SCALE || (p.channel_scale_mode & 1)) && p.meta_stride_n != 1) return false;
+        if ((int64_t)p.N * p.K >= ((int64_t)1 << 30)) return false;
+        u.q = p;
+        u.q.W_nbits = 16;
+        u.q.unpack_mask = 0xffff;
+        u.q.w_dtype = p.input_dtype;
+        if (p.W_group_mode == GLA_WGM_SCALE) u.q.channel_scale_mode = p.channel_scale_mode | 1;  // one scale per channel, after the K sum as before
+        u.q.W_group_mode = GLA_WGM_NONE;
+        u.q.group_size = p.K;
+        u.q.zeros = nullptr;
+        u.q.zero_is_scalar = 0;
+        u.q.w = (const void*)(uintptr_t)256;
+        u.q.w_stride_k = 1;
+        u.q.w_stride_n = p.K;
+        u.q.tile_config = -1;
+        u.q.workspace = nullptr;
+        u.q.workspace_bytes = 0;
+        if (!gemm_16bit_eligible(u.q)) return false;
+        const int64_t inner_b = gemm_16bit_workspace_bytes(u.q);
+        if (inner_b < 0) return false;
+        u.w_off = ((inner_b > kWsPrivateBytes ? inner_b : kWsPrivateBytes) + 255) / 256 * 256;
+        u.total = u.w_off + (int64_t)p.N * p.K * 2;
+        return true;
+    }
     const bool asked = p.tile_config == GLA_TILE_PREFER_UNPACKED && p.M > 16 && gemm_wn_eligible(p);
     // same launches side by side, fused -> unpacked (us): 4-bit gs 128 bf16 4096^2 at 1024 / 2048 / 4096 / 8192 rows 72 ->
     // 74, 107 -> 92, 161 -> 135, 297 -> 246; 8192^2 189 -> 179, 292 -> 261, 573 -> 474, 1179 -> 914; fp16, whose fused
@@ -543,7 +575,8 @@ int gla_matmul(const gla_matmul_args* args, void* stream) {
             return GLA_ERR_WORKSPACE_TOO_SMALL;
         }
         void* w16 = (char*)args->workspace + u.w_off;
-        const int rcu = launch_wn_unpack16(*args, w16, args->K, s);
+        const bool bytes = args->w_dtype == GLA_DT_INT8 || args->w_dtype == GLA_DT_UINT8 || args->w_dtype == GLA_DT_FP8;
+        const int rcu = bytes ? launch_kbytes_unpack16(*args, w16, args->K, s) : launch_wn_unpack16(*args, w16, args->K, s);
         if (rcu != GLA_OK) return rcu;
         u.q.w = w16;
         u.q.workspace = args->workspace;

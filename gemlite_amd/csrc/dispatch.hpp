@@ -78,6 +78,8 @@ int64_t gemm_wn_workspace_bytes(const gla_matmul_args& p);
 int launch_gemm_wn(const gla_matmul_args& p, hipStream_t stream);
 // the weights of such a call as fp16 / bf16 values, [N, ldo] with K contiguous (wn_unpack16.hip)
 int launch_wn_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hipStream_t stream);
+// ... and the same for unpacked int8 / uint8 / fp8 weight bytes (a call of gemm_kbytes)
+int launch_kbytes_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hipStream_t stream);
 
 // ---- MFMA GEMM on 8-bit operands, both K-contiguous (gemm_8bit.hip) --------
 bool gemm_8bit_eligible(const gla_matmul_args& p);

@@ -99,7 +99,74 @@ void launch_bits(const Unpack16Args& a, bool bf16, hipStream_t stream) {
         hipLaunchKernelGGL((wn_unpack16_kernel<BITS, false>), grid, dim3(256), 0, stream, a);
 }
 
+// Unpacked int8 / uint8 / e4m3 weight bytes, [N, K] K-contiguous, as the same numbers in fp16 / bf16 (exact: every such
+// byte value is a 16-bit float of either kind): 16 bytes in, 32 bytes out per thread, both coalesced.
+template <int WDT, bool BF16>
+__global__ __launch_bounds__(256) void kbytes_unpack16_kernel(const uint8_t* __restrict__ w, int64_t wsn, int N, int K,
+                                                              uint16_t* __restrict__ out, int64_t ldo) {
+    const int pieces = K / 16;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (int64_t)N * pieces) return;
+    const int n = (int)(id / pieces), k = (int)(id % pieces) * 16;
+    const u32x4 v = __builtin_nontemporal_load((const u32x4*)(w + (int64_t)n * wsn + k));
+    const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float f[4];
+        if constexpr (WDT == GLA_DT_FP8) {
+            f[0] = __builtin_amdgcn_cvt_f32_fp8((int)in[i], 0);
+            f[1] = __builtin_amdgcn_cvt_f32_fp8((int)in[i], 1);
+            f[2] = __builtin_amdgcn_cvt_f32_fp8((int)in[i], 2);
+            f[3] = __builtin_amdgcn_cvt_f32_fp8((int)in[i], 3);
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const uint32_t byte = (in[i] >> (8 * b)) & 0xffu;
+                f[b] = WDT == GLA_DT_INT8 ? (float)(int)(int8_t)byte : (float)byte;
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if constexpr (BF16) {
+                // exact: at most 8 significant bits
+                o[2 * i + h] = (__builtin_bit_cast(uint32_t, f[2 * h]) >> 16) | (__builtin_bit_cast(uint32_t, f[2 * h + 1]) & 0xffff0000u);
+            } else {
+                o[2 * i + h] = (uint32_t)float_to_half_bits(f[2 * h]) | ((uint32_t)float_to_half_bits(f[2 * h + 1]) << 16);
+            }
+        }
+    }
+    uint4* dst = (uint4*)(out + (int64_t)n * ldo + k);
+    dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+    dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
 }  // namespace
+
+// The call must be one the byte-weight GEMM takes (gemm_kbytes_eligible); out: [N, ldo] values of the activation type.
+int launch_kbytes_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hipStream_t stream) {
+    if (!gemm_kbytes_eligible(p) || p.K % 16 != 0 || ldo < p.K || ldo % 8 != 0 || ((uintptr_t)out & 15)) {
+        set_error("kbytes_unpack16: a call of the byte-weight GEMM and an aligned [N, ldo >= K] output are required");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
+    const int64_t items = (int64_t)p.N * (p.K / 16);
+    const dim3 grid((unsigned)((items + 255) / 256));
+    const bool bf16 = p.input_dtype == GLA_DT_BF16;
+    const uint8_t* w = (const uint8_t*)p.w;
+    uint16_t* o = (uint16_t*)out;
+#define GLA_LAUNCH_KB16(WDT)                                                                                                 \
+    if (bf16)                                                                                                                \
+        hipLaunchKernelGGL((kbytes_unpack16_kernel<WDT, true>), grid, dim3(256), 0, stream, w, p.w_stride_n, p.N, p.K, o, ldo); \
+    else                                                                                                                     \
+        hipLaunchKernelGGL((kbytes_unpack16_kernel<WDT, false>), grid, dim3(256), 0, stream, w, p.w_stride_n, p.N, p.K, o, ldo)
+    switch (p.w_dtype) {
+        case GLA_DT_FP8: GLA_LAUNCH_KB16(GLA_DT_FP8); break;
+        case GLA_DT_INT8: GLA_LAUNCH_KB16(GLA_DT_INT8); break;
+        default: GLA_LAUNCH_KB16(GLA_DT_UINT8); break;
+    }
+#undef GLA_LAUNCH_KB16
+    return check_hip(hipGetLastError(), "kbytes_unpack16 launch");
+}
 
 // The call must be one the fused packed-weight GEMM takes (gemm_wn_eligible: operand types, layouts, alignments, groups
 // of whole 64-K stages); out: [N, ldo] 16-bit values of the activation type, ldo >= K, 16-byte aligned rows.

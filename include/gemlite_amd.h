@@ -88,9 +88,9 @@ extern "C" {
  * through the skinny kernel of the narrow formats (family K_SKINNY; the call then needs a workspace), which the library
  * itself takes on large layers only */
 #define GLA_TILE_PREFER_MID (-4)
-/* fp16 / bf16 activations on 2-, 4- or 8-bit packed codes above 16 rows: the weights are first written out as 16-bit
- * values into the workspace (N * K * 2 bytes of it), then the 16-bit matrix-core GEMM runs (family GEMM_16BIT); the
- * library itself does so from 2048 rows of bf16 and 4096 rows of fp16 */
+/* fp16 / bf16 activations on 2-, 4- or 8-bit packed codes, or on unpacked int8 / uint8 / fp8 weight bytes, above 16
+ * rows: the weights are first written out as 16-bit values into the workspace (N * K * 2 bytes of it), then the 16-bit
+ * matrix-core GEMM runs (family GEMM_16BIT); the library itself does so from 2048 rows (packed codes under fp16: 4096) */
 #define GLA_TILE_PREFER_UNPACKED (-5)
 
 /*

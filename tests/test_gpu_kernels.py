@@ -894,6 +894,50 @@ def test_a16w8_weight_only_unpacked_bytes(device, fp8, post_scale, dtype, K):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("post_scale", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_byte_weights_at_prefill_size_are_converted_first(device, fp8, post_scale, dtype):
+    """From 2048 rows (or on request) unpacked int8 / fp8 weight bytes are written out once as fp16 / bf16 values (exact)
+    and the 16-bit GEMM runs on them with the per-channel scale in its epilogue, as the byte-weight GEMM has it.  N is
+    no multiple of the kernels' tiles; one-hot rows: bit-identical outputs of both paths."""
+    N, K = 1028, 2112
+    W = gen_x(N, K, dtype, seed=21, std=0.02)
+    proc = (helper.A16W8_FP8 if fp8 else helper.A16W8_INT8)(device=device, post_scale=post_scale)
+    W_q_cpu, s_cpu = gemlite_amd.quantize_weights_per_channel(W, torch.float8_e4m3fn if fp8 else torch.int8)
+    proc.dtype = dtype
+    layer = proc.from_weights(W_q_cpu, scales=s_cpu)
+    m = layer.get_meta_args()
+
+    def run(x, tile):
+        out = torch.empty((x.shape[0], N), dtype=dtype, device=device)
+        a = _ext.build_matmul_args(x, layer.W_q, layer.scales, layer.zeros, None, out, W_nbits=m[1], group_size=m[2],
+                                   unpack_mask=m[3], elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6],
+                                   acc_dtype=m[7], meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10],
+                                   data_contiguous=m[11], tile_config=tile)
+        fam = _ext.matmul_family(a)
+        print(f"case: {fam} tile={tile} M={x.shape[0]} N={N} K={K} fp8={fp8} post_scale={post_scale} {dtype}", flush=True)
+        _ext.matmul(a, device)
+        torch.cuda.synchronize()
+        return fam, out
+
+    for M, tile in ((40, -5), (300, -5), (2048, -1)):
+        x = gen_x(M, K, dtype, seed=M)
+        y_ref = oracle_forward(layer, x)
+        fam, out = run(x.to(device), tile)
+        assert fam == "GEMM_16BIT", (M, tile, fam)
+        err = rel_frob(to_np(out), y_ref)
+        assert err <= TIGHT[dtype], (M, err)
+        assert elementwise_excess(to_np(out), y_ref, kind_of(dtype)) <= 1.0, M
+    x = torch.zeros(48, K, dtype=dtype)
+    for r in range(48):
+        x[r, (53 * r + 11) % K] = 1.0
+    (fa, ya), (fb, yb) = run(x.to(device), -3), run(x.to(device), -5)
+    assert (fa, fb) == ("GEMM_KBYTES", "GEMM_16BIT")
+    assert torch.equal(ya, yb)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("zeros_kind", ["tensor_fma", "tensor_shift_scale", "scalar"])
 def test_int8_bytes_with_zero_point_channelwise(device, dtype, zeros_kind):
