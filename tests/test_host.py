@@ -789,3 +789,29 @@ def test_packed_layers_unpack_their_weights_first_at_prefill_size():
     need = _ext.matmul_workspace_need(args(4096))
     assert need >= (4 << 20) + N * K * 2 and need % 256 == 0
     assert _ext.matmul_workspace_need(args(300, -5)) >= (4 << 20) + N * K * 2
+
+
+def test_byte_weight_layers_convert_their_weights_first_from_2048_rows():
+    """Host logic only: unpacked int8 weight bytes under 16-bit activations.  From 2048 rows (or with
+    GLA_TILE_PREFER_UNPACKED above 16) the bytes are converted into the workspace and the 16-bit GEMM runs; the preference
+    for the tiled GEMM keeps the byte-weight kernel."""
+    N, K = 512, 1024
+    W = (torch.randn(N, K) * 0.02).to(torch.bfloat16)
+    for post_scale in (True, False):
+        proc = gemlite_amd.helper.A16W8_INT8(device="cpu", post_scale=post_scale)
+        W_q, s = gemlite_amd.quantize_weights_per_channel(W, torch.int8)
+        proc.dtype = torch.bfloat16
+        l = proc.from_weights(W_q, scales=s)
+        m = l.get_meta_args()
+
+        def args(M, tile=-1):
+            return _ext.build_matmul_args(torch.zeros(M, K, dtype=torch.bfloat16), l.W_q, l.scales, l.zeros, None,
+                                          torch.zeros(M, N, dtype=torch.bfloat16), W_nbits=m[1], group_size=m[2], unpack_mask=m[3],
+                                          elements_per_sample=m[4], input_dtype=m[5], output_dtype=m[6], acc_dtype=m[7],
+                                          meta_dtype=m[8], channel_scale_mode=m[9], W_group_mode=m[10], data_contiguous=m[11],
+                                          tile_config=tile)
+
+        assert [_ext.matmul_family(args(M)) for M in (16, 17, 2047, 2048)] == ["GEMV_KMAJOR", "GEMM_KBYTES", "GEMM_KBYTES", "GEMM_16BIT"]
+        assert [_ext.matmul_family(args(M, -5)) for M in (16, 17)] == ["GEMV_KMAJOR", "GEMM_16BIT"]
+        assert _ext.matmul_family(args(4096, -3)) == "GEMM_KBYTES"
+        assert _ext.matmul_workspace_need(args(2048)) >= (4 << 20) + N * K * 2
