@@ -449,12 +449,20 @@ bool unpack_first(const gla_matmul_args& p, Family f, Unpacked& u) {
         u.total = u.w_off + (int64_t)p.N * p.K * 2;
         return true;
     }
-    const bool asked = p.tile_config == GLA_TILE_PREFER_UNPACKED && p.M > 16 && gemm_wn_eligible(p);
+    // Layers without a tiled GEMM (groups of 16 / 32, 1-bit codes) run the mid-batch kernel as chunks of 64 rows, each
+    // of which streams and unpacks the weights again: they unpack first from 512 rows (1- and 2-bit codes: 1024).
+    const bool tiled = gemm_wn_eligible(p);
+    const bool asked = p.tile_config == GLA_TILE_PREFER_UNPACKED && p.M > 16 && (tiled || wn_mid_eligible(p));
     // same launches side by side, fused -> unpacked (us): 4-bit gs 128 bf16 4096^2 at 1024 / 2048 / 4096 / 8192 rows 72 ->
     // 74, 107 -> 92, 161 -> 135, 297 -> 246; 8192^2 189 -> 179, 292 -> 261, 573 -> 474, 1179 -> 914; fp16, whose fused
     // unpacking is cheaper: 66 -> 73, 94 -> 96, 146 -> 143, 280 -> 267; 8192^2 158 -> 186, 271 -> 278, 527 -> 505, 1052 -> 968
     const int from_rows = p.input_dtype == GLA_DT_BF16 ? 2048 : 4096;
-    const bool by_rule = f == F_GEMM_WN && p.M >= from_rows && p.tile_config <= 0 && p.tile_config != GLA_TILE_PREFER_MATRIX;
+    // (bf16, mid-batch chunks -> unpacked, us: 8192^2 4-bit gs 32 at 512 / 1024 / 4096 rows 157 -> 133, 254 -> 190, 892 -> 483;
+    // 2-bit gs 32 125 -> 131, 197 -> 189, 698 -> 481; 1-bit gs 64 138 -> 124, 216 -> 181, 745 -> 470; 4096^2 4-bit gs 32 51 -> 48,
+    // 85 -> 66, 256 -> 132; 2-bit 42 -> 47, 68 -> 66, 209 -> 132)
+    const int kMidUnpackRows = p.W_nbits >= 4 ? 512 : 1024;
+    const bool free_choice = p.tile_config <= 0 && p.tile_config != GLA_TILE_PREFER_MATRIX && p.tile_config != GLA_TILE_PREFER_MID;
+    const bool by_rule = free_choice && ((f == F_GEMM_WN && p.M >= from_rows) || (f == F_WN_MID && !tiled && p.M >= kMidUnpackRows));
     if (!asked && !by_rule) return false;
     if (p.acc_dtype != GLA_DT_FP32 || (p.W_group_mode >= GLA_WGM_SCALE && (p.channel_scale_mode & 1))) return false;
     if ((int64_t)p.N * p.K >= ((int64_t)1 << 30)) return false;

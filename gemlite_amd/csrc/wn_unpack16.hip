@@ -1,4 +1,4 @@
-// Packed 2-, 4- and 8-bit codes written out as the fp16 / bf16 weights they stand for, [N, K] with K contiguous: the
+// Packed 1-, 2-, 4- and 8-bit codes written out as the fp16 / bf16 weights they stand for, [N, K] with K contiguous: the
 // first half of the prefill path of packed layers from 2048 rows of bf16 (4096 of fp16) up, whose second half is the
 // 16-bit matrix-core GEMM (gemm_16bit.hip).  The fused kernel (gemm_wn.hip) unpacks every weight once per 128 or 256
 // rows of the batch, and its vector work stands beside the MFMAs; here a weight is unpacked once per call, at memory
@@ -11,7 +11,9 @@
 // One thread: one column n and 64 consecutive K-values = 64 / e packed words of that column (a wave reads 256
 // contiguous bytes per word row) -> 128 contiguous bytes of row n of the output, which the wave transposes through LDS
 // so that its stores are whole lines too (16 bytes per lane at a stride of a row each ran at a third of the speed).
-// Groups are whole multiples of 64 K-values (the fused GEMM's rule), so a thread needs one (scale, zero) pair.
+// With groups of whole multiples of 64 K-values (the fused GEMM's rule) a thread needs one (scale, zero) pair; groups of
+// 16 / 32 (layers only the mid-batch kernel takes, which at thousands of rows would stream and unpack the weights once
+// per 64 rows) change inside a thread's chunk, between words.
 #include "common.hpp"
 #include "dispatch.hpp"
 #include "wn_dequant.hpp"
@@ -27,7 +29,7 @@ struct Unpack16Args {
     uint16_t* out;            // [N, ldo]
     int N, chunks;            // chunks = K / 64
     int64_t wsk, msg, ldo;    // elements
-    int cpg;                  // 64-K chunks per group
+    int gs;                   // K-values per group (a multiple of 64, or 16 / 32)
     int wgm, meta_dt, z_dt;
     bool has_s, has_zt, z_scalar;
 };
@@ -48,16 +50,27 @@ __global__ __launch_bounds__(256) void wn_unpack16_kernel(Unpack16Args a) {
     const uint32_t* src = a.w + (int64_t)ch * WORDS * a.wsk + n;
 #pragma unroll
     for (int j = 0; j < WORDS; ++j) w[j] = __builtin_nontemporal_load(src + (int64_t)j * a.wsk);
-    const int g = ch / a.cpg;
-    const float s = a.has_s ? load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + n) : 1.0f;
-    const float z = a.has_zt ? load_as_float(a.zeros, a.meta_dt, (int64_t)g * a.msg + n)
-                             : (a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0) : 0.0f);
     const float c1 = a.wgm == GLA_WGM_SHIFT ? -1.0f : (a.wgm == GLA_WGM_FMA ? 1.0f : 0.0f);
     const float c2 = a.wgm == GLA_WGM_SHIFT_SCALE ? -1.0f : 0.0f;
-    const ColMeta<BF16> meta = make_meta<BF16, OFF>(s, z * __builtin_fmaf(c2, s, c1));
+    auto meta_of = [&](int g) __attribute__((always_inline)) {
+        const float s = a.has_s ? load_as_float(a.scales, a.meta_dt, (int64_t)g * a.msg + n) : 1.0f;
+        const float z = a.has_zt ? load_as_float(a.zeros, a.meta_dt, (int64_t)g * a.msg + n)
+                                 : (a.z_scalar ? load_as_float(a.zeros, a.z_dt, 0) : 0.0f);
+        return make_meta<BF16, OFF>(s, z * __builtin_fmaf(c2, s, c1));
+    };
+    // groups of 64 K-values or more: one per chunk; groups of 16 / 32: a word lies in one of them
+    int g_have = ch * 64 / a.gs;
+    ColMeta<BF16> meta = meta_of(g_have);
     uint32_t o[32];
 #pragma unroll
     for (int j = 0; j < WORDS; ++j) {
+        if (a.gs < 64) {
+            const int g = (ch * 64 + j * E) / a.gs;
+            if (g != g_have) {
+                g_have = g;
+                meta = meta_of(g);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < E / 2; ++i) {
             const uint32_t lo = (w[j] >> (BITS * 2 * i)) & ((1u << BITS) - 1u);
@@ -168,26 +181,31 @@ int launch_kbytes_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hip
     return check_hip(hipGetLastError(), "kbytes_unpack16 launch");
 }
 
-// The call must be one the fused packed-weight GEMM takes (gemm_wn_eligible: operand types, layouts, alignments, groups
-// of whole 64-K stages); out: [N, ldo] 16-bit values of the activation type, ldo >= K, 16-byte aligned rows.
+// The call must be one the fused packed-weight GEMM or the mid-batch kernel takes (operand types, layouts, alignments;
+// groups of whole 64-K chunks, or of 16 / 32 with a packed word inside one group; 1-bit codes in groups of 32 or more);
+// out: [N, ldo] 16-bit values of the activation type, ldo >= K, 16-byte aligned rows.
 int launch_wn_unpack16(const gla_matmul_args& p, void* out, int64_t ldo, hipStream_t stream) {
-    if (!gemm_wn_eligible(p) || ldo < p.K || ldo % 8 != 0 || ((uintptr_t)out & 15)) {
-        set_error("wn_unpack16: a call of the packed-weight GEMM and an aligned [N, ldo >= K] output are required");
-        return GLA_ERR_UNSUPPORTED_MODE;
-    }
     const bool uses_scales = p.W_group_mode >= GLA_WGM_SCALE;
     const bool uses_zeros = p.W_group_mode == GLA_WGM_SHIFT || p.W_group_mode >= GLA_WGM_SHIFT_SCALE;
     const bool grouped = uses_scales || (uses_zeros && !p.zero_is_scalar);
     const int gs = grouped ? p.group_size : p.K;
+    const int e = p.elements_per_sample;
+    const bool groups_ok = gs > 0 && e > 0 && (gs % 64 == 0 || (64 % gs == 0 && gs % e == 0));
+    if (!(gemm_wn_eligible(p) || wn_mid_eligible(p)) || p.K % 64 != 0 || !groups_ok || ldo < p.K || ldo % 8 != 0 ||
+        ((uintptr_t)out & 15)) {
+        set_error("wn_unpack16: a call of the packed-weight GEMM or the mid-batch kernel and an aligned [N, ldo >= K] output are required");
+        return GLA_ERR_UNSUPPORTED_MODE;
+    }
     Unpack16Args a;
     a.w = (const uint32_t*)p.w; a.scales = p.scales; a.zeros = p.zeros; a.out = (uint16_t*)out;
     a.N = p.N; a.chunks = p.K / 64;
     a.wsk = p.w_stride_k; a.msg = gs == p.K ? 0 : p.meta_stride_g; a.ldo = ldo;
-    a.cpg = gs / 64;
+    a.gs = gs;
     a.wgm = p.W_group_mode; a.meta_dt = p.meta_dtype; a.z_dt = p.zeros_dtype;
     a.has_s = uses_scales; a.has_zt = uses_zeros && !p.zero_is_scalar; a.z_scalar = uses_zeros && p.zero_is_scalar;
     const bool bf16 = p.input_dtype == GLA_DT_BF16;
     switch (p.W_nbits) {
+        case 1: launch_bits<1>(a, bf16, stream); break;
         case 2: launch_bits<2>(a, bf16, stream); break;
         case 4: launch_bits<4>(a, bf16, stream); break;
         default: launch_bits<8>(a, bf16, stream); break;

@@ -282,16 +282,18 @@ def test_packed_codes_at_17_to_64_rows(device, nbits, gs, dtype):
                 assert elementwise_excess(to_np(out), y_ref, kind_of(dtype)) <= 1.0, (N, K, M, tile)
 
 
-@pytest.mark.parametrize("nbits,gs", [(4, 128), (4, 64), (2, 64), (8, 128), (8, None), (4, None)])
+@pytest.mark.parametrize("nbits,gs", [(4, 128), (4, 64), (2, 64), (8, 128), (8, None), (4, None), (4, 32), (2, 32), (1, 64), (1, 32), (1, 128),
+                                      (2, 16), (4, 16), (8, 16)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_packed_layers_at_prefill_size_unpack_their_weights_first(device, nbits, gs, dtype):
     """From 2048 rows of bf16, 4096 of fp16 (or on request) the packed codes are written out once as 16-bit weights and the 16-bit
     matrix-core GEMM runs on them.  Every code width of the fused GEMM, groups of one and two 64-K chunks and one group
     per channel (scales after the K sum), both activation types; N ends inside a wave's 64 columns, K inside a
     workgroup's four chunks; a bias; the five dequantisation forms; and that the weights come out exactly as the fused
-    kernel makes them (one-hot rows: bit-identical outputs of both paths)."""
+    kernel makes them (one-hot rows: bit-identical outputs of both paths).  Groups of 16 / 32 and 1-bit codes, which have
+    no tiled GEMM and would run the mid-batch kernel once per 64 rows, take the same path (from 512 rows unasked)."""
     dt = gemlite_amd.TORCH_TO_DTYPE[dtype]
-    N, K = (2032, 1088) if gs == 64 else (520, 1152)
+    N, K = (2032, 1088) if gs == 64 and nbits > 1 else (520, 1152)
     g = K if gs is None else gs
     W_q, scales, zeros = gen_int_case(N, K, nbits, g, dtype, seed=nbits * 100 + g % 1000)
     layer = GemLiteLinear(nbits, g, K, N, dt, dt).pack(W_q.to(device), scales.to(device), zeros.to(device),
@@ -331,8 +333,9 @@ def test_packed_layers_at_prefill_size_unpack_their_weights_first(device, nbits,
     for r in range(48):
         x[r, (53 * r + 11) % K] = 1.0
     layer.bias = None
-    (fa, ya), (fb, yb) = run(layer, x.to(device), -3), run(layer, x.to(device), -5)
-    assert (fa, fb) == ("GEMM_WN", "GEMM_16BIT")
+    tiled = (gs is None or gs % 64 == 0) and nbits > 1
+    (fa, ya), (fb, yb) = run(layer, x.to(device), -3 if tiled else -4), run(layer, x.to(device), -5)
+    assert (fa, fb) == ("GEMM_WN" if tiled else "WN_MID", "GEMM_16BIT")
     assert torch.equal(ya, yb)
 
 
@@ -369,7 +372,8 @@ def test_packed_codes_in_short_groups(device, nbits, gs, dtype):
 
 @pytest.mark.parametrize("nbits,gs", [(1, 32), (2, 16)])
 def test_short_group_codes_at_prefill_size(device, nbits, gs):
-    """1024 rows on packings the tiled GEMM does not take: sixteen row chunks of the mid-batch kernel."""
+    """1024 rows on packings the tiled GEMM does not take: the weights are unpacked into the workspace and the 16-bit GEMM runs
+    (below 1024 rows: row chunks of the mid-batch kernel)."""
     N, K, M = 256, 1024, 1024
     W_q, scales, zeros = gen_int_case(N, K, nbits, gs, torch.float16, seed=nbits + gs)
     layer = GemLiteLinear(nbits, gs, K, N, DType.FP16, DType.FP16).pack(W_q.to(device), scales.to(device), zeros.to(device))

@@ -334,6 +334,10 @@ def test_packed_layers_without_a_tiled_gemm_take_the_mid_batch_kernel():
     # 4- and 8-bit codes in groups of 32, 1-bit codes in groups of 128: the GEMV (row chunks) up to 64 rows on a small layer
     for l in (layer(4, 32), layer(8, 32), layer(1, 128)):
         assert [_family(l, M, torch.bfloat16) for M in Ms] == ["GEMV_PACKED"] * 5 + ["WN_MID"] * 2
+    # (at prefill size such layers unpack their weights first and run the 16-bit GEMM: from 512 rows, 1- and 2-bit codes from 1024)
+    assert [_family(layer(4, 32), M, torch.bfloat16) for M in (511, 512)] == ["WN_MID", "GEMM_16BIT"]
+    assert [_family(layer(2, 32), M, torch.bfloat16) for M in (1023, 1024)] == ["WN_MID", "GEMM_16BIT"]
+    assert [_family(layer(1, 64), M, torch.bfloat16) for M in (1023, 1024)] == ["WN_MID", "GEMM_16BIT"]
     # groups of 16: the mid-batch kernel at any row count (2-, 4-, 8-bit codes); 1-bit codes stay with the generic kernels
     for l in (layer(2, 16), layer(4, 16), layer(8, 16)):
         assert [_family(l, M, torch.bfloat16) for M in Ms] == ["WN_MID"] * 7
